@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+A "step" is one decode-shaped product of BASELINE.json's configs[1]: affine 4-bit g64,
+x bf16 [1,4096], W [14336,4096] (packed uint32 + bf16 scales and biases), y bf16 [1,14336].
+`value` is the weight stream rate in GB/s: the algorithmic bytes of one product
+(packed 29,360,128 + scales 1,835,008 + biases 1,835,008 = 33,030,144 B) over the average
+time of one launch, with every operand resident in HBM.  Launches go back to back on one
+stream through the C ABI and rotate through enough distinct weight copies that no launch finds
+its weights in the 256 MB last-level cache.  The prefill-shaped product (configs[2], M = 2048)
+is timed the same way and reported in the same line as `qmm`.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-qmm]
+
+Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
+N, K = 14336, 4096
+GROUP, BITS = 64, 4
+WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
+METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
+
+
+def make_weights(copies, device):
+    import torch
+
+    import nuvec_amd as nv
+    out = []
+    gen = torch.Generator(device=device)
+    for i in range(copies):
+        gen.manual_seed(1234 + i)
+        w = (torch.randn(N, K, device=device, generator=gen) * 0.02).to(torch.bfloat16)
+        out.append(nv.quantize(w, nv.Quant.affine(GROUP, BITS)))
+        del w
+    torch.cuda.synchronize()
+    return out
+
+
+class Product:
+    """One prepared nvq_quantized_matmul call: descriptor and pointers built once, so the timed
+    loop is a bare C-ABI call per launch."""
+
+    def __init__(self, lib, m, x, q, y):
+        from nuvec_amd import _lib
+        d = _lib.QmmDescC()
+        d.quant = q.quant._c()
+        d.dtype, d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = _lib.BF16, 1, m, N, K, m, 0
+        self.d, self.fn = d, lib.nvq_quantized_matmul
+        self.args = (C.byref(d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),
+                     C.c_void_p(q.scales.data_ptr()), C.c_void_p(q.biases.data_ptr()), C.c_void_p(y.data_ptr()),
+                     C.c_void_p(None))
+        self.keep = (x, q, y)
+
+    def __call__(self, stream):
+        rc = self.fn(*self.args, stream)
+        if rc:
+            from nuvec_amd import _lib
+            _lib.check(rc)
+
+
+def time_launches(calls, steps, warmup, graph=True):
+    """Average milliseconds per launch over `steps` launches, after `warmup` untimed ones, between
+    two HIP events recorded on the stream the kernels run on.  `calls` are rotated.
+
+    graph=True: one rotation of the calls is captured into a HIP graph (the same C-ABI calls, made
+    once on the capturing stream) and the graph is replayed, so the launches reach the GPU back
+    to back without a Python call between them; `steps` is rounded to whole rotations.
+    graph=False: one C-ABI call per launch from the Python loop (host-bound for kernels this short)."""
+    import torch
+    n = len(calls)
+    stream = torch.cuda.current_stream()
+    for i in range(warmup):
+        calls[i % n](C.c_void_p(stream.cuda_stream))
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if not graph:
+        start.record()
+        for i in range(steps):
+            calls[i % n](C.c_void_p(stream.cuda_stream))
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps, steps
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        cap = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for c in calls:
+            c(cap)
+    reps = max(1, round(steps / n))
+    g.replay()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        g.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / (reps * n), reps * n
+
+
+def cpu_baseline(seconds_budget=20.0):
+    """The CPU restatement of nuvec's path (dequantize the whole matrix, then the fixed-order
+    few-row product) on this host's cores, on a bounded sample of the same workload."""
+    import numpy as np
+
+    from oracle import ref
+    rng = np.random.default_rng(0)
+    w = ref.from_f32((rng.standard_normal((N, K)) * 0.02).astype(np.float32), ref.BF16)
+    x = ref.from_f32(rng.standard_normal((1, K)).astype(np.float32), ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, GROUP, BITS)
+    threads = max(1, min(ref.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1)))
+    run = lambda: ref.quantized_matmul(x, packed, scales, biases, group=GROUP, bits=BITS, dtype=ref.BF16, threads=threads)
+    run()
+    done, t0 = 0, time.perf_counter()
+    while done < 3 or (time.perf_counter() - t0 < seconds_budget / 2 and done < 50):
+        run()
+        done += 1
+    dt = (time.perf_counter() - t0) / done
+    return {"value": WEIGHT_BYTES / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "ms_per_step": dt * 1e3,
+            "sample": f"{done} products of the same workload (x bf16 [1,{K}], W [{N},{K}] affine 4-bit g64): whole-matrix "
+                      f"dequantize on one thread as the reference does, then the 8-lane fixed-order product over "
+                      f"64-column blocks on {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--copies", type=int, default=24, help="distinct weight copies rotated through (24 x 33 MB = 793 MB)")
+    ap.add_argument("--qmm-steps", type=int, default=40)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-qmm", action="store_true", help="skip the M=2048 leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N without exchange, "
+                 "see DESIGN.md)")
+
+    import torch
+
+    import nuvec_amd  # noqa: F401
+    from nuvec_amd import _lib
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU")
+    device = torch.device("cuda:0")
+    lib = _lib.load()
+    _lib.check(lib.nvq_init(0))
+
+    qs = make_weights(args.copies, device)
+    x1 = torch.randn(1, K, device=device).to(torch.bfloat16)
+    ys = [torch.empty(1, N, dtype=torch.bfloat16, device=device) for _ in qs]
+    calls = [Product(lib, 1, x1, q, y) for q, y in zip(qs, ys)]
+
+    ms, steps = time_launches(calls, args.steps, args.warmup)
+    gbps = WEIGHT_BYTES / (ms * 1e-3) / 1e9
+    direct_ms, _ = time_launches(calls, min(args.steps, 2000), 50, graph=False)
+    hot_ms, _ = time_launches(calls[:1] * len(calls), min(args.steps, 2000), 50)
+
+    record = {
+        "metric": METRIC, "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: decode QMV, affine 4-bit g64, x bf16 [1,4096], W [14336,4096], M=1",
+                   "weight_copies_rotated": args.copies, "submission": "one HIP graph per rotation of the weight copies, replayed back to back on one stream"},
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": None, "kernel": "qmv", "bytes_per_launch": WEIGHT_BYTES, "us_per_launch": ms * 1e3},
+        "direct_launch": {"us_per_launch": direct_ms * 1e3, "gbps": WEIGHT_BYTES / (direct_ms * 1e-3) / 1e9,
+                          "note": "one C-ABI call per launch from the Python loop: bounded by the host's call rate"},
+        "cache_hot": {"us_per_launch": hot_ms * 1e3, "gbps": WEIGHT_BYTES / (hot_ms * 1e-3) / 1e9,
+                      "note": "one weight buffer reused: served from the last-level cache, not an HBM figure"},
+    }
+
+    if not args.no_qmm:
+        m = 2048
+        xm = torch.randn(m, K, device=device).to(torch.bfloat16)
+        ym = torch.empty(m, N, dtype=torch.bfloat16, device=device)
+        qcalls = [Product(lib, m, xm, q, ym) for q in qs[:4]]
+        qms, qsteps = time_launches(qcalls, args.qmm_steps, 4, graph=False)
+        flop = 2.0 * m * N * K
+        tflops = flop / (qms * 1e-3) / 1e12
+        record["qmm"] = {"workload": "configs[2]: prefill QMM, affine 4-bit g64, x bf16 [2048,4096], W [14336,4096]",
+                         "value": tflops, "unit": "TFLOP/s", "ms_per_step": qms, "steps": qsteps,
+                         "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "qmm",
+                                      "flop_per_launch": flop}}
+
+    if not args.no_cpu:
+        record["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(record))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,193 @@
+/*
+ * nuvec_hip.h — C ABI of the MI355X (gfx950) backend for nuvec's quantized-matmul path.
+ *
+ * This is the surface a `hip` arm of nuvec's device boundary binds: the counterpart of
+ * `GpuEval::{supports, run}` for the five primitives of the path
+ * (reference: crates/nuvec-core/src/gpu.rs:1571-1799; the stub with the same surface is
+ * gpu.rs:154-281).  Every entry point cites the reference routine it replaces.
+ *
+ * Conventions (they mirror what the reference's boundary already does):
+ *  - Plain C: pointers, sizes and small POD structs.  No exceptions or panics cross it;
+ *    every call returns an `nvq_status` and `nvq_last_error()` holds the message of the
+ *    calling thread's last failure (nuvec maps it to `Error::Backend`, error.rs:29-34).
+ *  - Ownership: the caller allocates every operand, output and workspace with the exact
+ *    byte size and owns them (gpu.rs:1696, 6256-6258).  These entry points allocate nothing
+ *    and free nothing.
+ *  - Pointers are device pointers of the device given to `nvq_init` (any memory the HIP
+ *    runtime can read from a kernel).  Operands are row-contiguous in their last two
+ *    dimensions; batch dimensions are described by element strides (gpu.rs:7042-7051).
+ *  - Asynchrony: a call validates on the host, enqueues kernels on `stream` (a `hipStream_t`
+ *    passed as `void*`; NULL is the default stream) and returns.  Completion is the caller's
+ *    stream or event synchronisation (the reference's `run` likewise only encodes,
+ *    gpu.rs:1-11).  Empty products never reach the backend (gpu.rs:1640,1665,1667); here they
+ *    return NVQ_OK without launching.
+ *  - Re-entrant: no mutable global state besides a once-initialised device record.
+ *  - dtype codes are nuvec's fixture order (crates/nuvec-core/tests/common/fixture.rs:15-30).
+ *  - Packed layout is MLX's: per row a little-endian bit stream, value i at bit i*bits,
+ *    stored as uint32 (crates/nuvec-core/src/kernels.rs:749-756, 808-817).
+ */
+#ifndef NUVEC_HIP_H
+#define NUVEC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NVQ_MAX_BATCH_DIMS 6
+
+#if defined(__GNUC__)
+#define NVQ_API __attribute__((visibility("default")))
+#else
+#define NVQ_API
+#endif
+
+typedef enum nvq_status {
+    NVQ_OK = 0,
+    NVQ_INVALID_ARGUMENT = 1, /* Error::InvalidArgument / shape / dtype mismatch (error.rs) */
+    NVQ_UNSUPPORTED = 2,      /* `supports()` would be false: the caller falls back to its CPU path */
+    NVQ_OUT_OF_MEMORY = 3,    /* Error::OutOfMemory */
+    NVQ_BACKEND = 4,          /* Error::Backend: a HIP call failed */
+    NVQ_NO_DEVICE = 5         /* Error::UnsupportedDevice */
+} nvq_status;
+
+typedef enum nvq_dtype {
+    NVQ_U8 = 1, NVQ_U32 = 3, NVQ_I32 = 7, NVQ_F16 = 9, NVQ_BF16 = 10, NVQ_F32 = 11
+} nvq_dtype;
+
+/* QuantMode (crates/nuvec-core/src/quantized.rs:22-35). */
+typedef enum nvq_mode { NVQ_AFFINE = 0, NVQ_MXFP4 = 1, NVQ_MXFP8 = 2, NVQ_NVFP4 = 3 } nvq_mode;
+
+/* Quant (quantized.rs:93-101). */
+typedef struct nvq_quant {
+    int32_t mode;       /* nvq_mode */
+    int32_t group_size; /* affine 32/64/128; mxfp4, mxfp8 32; nvfp4 16 */
+    int32_t bits;       /* affine 1-6 or 8; mxfp4, nvfp4 4; mxfp8 8 */
+} nvq_quant;
+
+typedef struct nvq_device_info {
+    int32_t device;
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_block;
+    int64_t global_memory_bytes;
+    char arch[64]; /* e.g. "gfx950:sramecc+:xnack-" */
+    char name[128];
+} nvq_device_info;
+
+/* Primitive::QuantizedMatmul operands (crates/nuvec-core/src/primitive.rs:466-494) as the
+ * device routine receives them (gpu.rs:6934-7060):
+ *   x       dtype  [batch..., m, k]
+ *   w       u32    [batch..., n, k*bits/32]   (transpose)  or [batch..., k, n*bits/32]
+ *   scales  dtype  [batch..., n, k/group]     (affine)     or u8 for the fp modes
+ *   biases  dtype  like scales (affine), NULL for the fp modes
+ *   y       dtype  [batch..., m, n], row-contiguous
+ * `batch_shape` is the output's batch shape; each operand's batch strides are in elements
+ * of that operand (0 = broadcast).  With a 2-D `w` and row-contiguous `x` the caller folds
+ * all leading rows into `m` and passes batch_ndim = 0 (the reference's "flat" rule,
+ * gpu.rs:6948-6950); `item_rows` then carries x's second-to-last dimension, which is what
+ * routing between the few-row and the tiled kernels looks at (gpu.rs:6975-6981). */
+typedef struct nvq_qmm_desc {
+    nvq_quant quant;
+    int32_t dtype;     /* NVQ_F16 / NVQ_BF16 / NVQ_F32: x, y and (affine) scales, biases */
+    int32_t transpose; /* 1: y = x . dequantize(w)^T  (MLX's default) */
+    int32_t row_exact; /* Primitive::QuantizedMatmul::row_exact (primitive.rs:491-493) */
+    int32_t rows;      /* Primitive::QuantizedMatmul::rows (primitive.rs:489-490) */
+    int64_t m, n, k;
+    int64_t item_rows; /* 0 = m */
+    int32_t batch_ndim;
+    int64_t batch_shape[NVQ_MAX_BATCH_DIMS];
+    int64_t x_strides[NVQ_MAX_BATCH_DIMS];
+    int64_t w_strides[NVQ_MAX_BATCH_DIMS];
+    int64_t s_strides[NVQ_MAX_BATCH_DIMS]; /* scales and biases share a shape and strides */
+} nvq_qmm_desc;
+
+/* FastOp::GatherQmm operands (crates/nuvec-core/src/quantized.rs:539-587, gpu.rs:7174-7294):
+ *   x [x_batches, m, k]; w [experts, n, k*bits/32] (transpose); scales/biases [experts, n, k/group];
+ *   lhs, rhs u32[pairs]; y [pairs, m, n] = x[lhs[i]] . dequantize(w[rhs[i]])^T.
+ * `offsets` (i32[experts], from nvq_sorted_offsets) is given when the caller took the grouped
+ * route: rhs sorted, lhs = arange, m == 1 (quantized.rs:646-651, 772-782). */
+typedef struct nvq_gather_desc {
+    nvq_quant quant;
+    int32_t dtype;
+    int32_t transpose;
+    int64_t m, n, k;
+    int64_t pairs;
+    int64_t x_batches;
+    int64_t experts;
+} nvq_gather_desc;
+
+/* ── runtime ─────────────────────────────────────────────────────────────────────── */
+
+/* Binds the library to HIP device `device` (idempotent; the process-wide device record,
+ * as `Device::shared()`, crates/nuvec-gpu/src/cuda/device.rs:79-82).  NVQ_NO_DEVICE when
+ * there is no gfx950 device: `GpuEval::available` (gpu.rs:1571-1573) is then false. */
+NVQ_API int32_t nvq_init(int32_t device);
+NVQ_API int32_t nvq_get_device_info(nvq_device_info *info);
+/* The calling thread's last error message ("" if none).  Valid until its next failing call. */
+NVQ_API const char *nvq_last_error(void);
+NVQ_API const char *nvq_version(void);
+
+/* ── validation mirrors (usable without a device) ────────────────────────────────── */
+
+/* Quant::checked (quantized.rs:133-168): NVQ_OK or NVQ_INVALID_ARGUMENT with the
+ * reference's message, prefixed by `op`. */
+NVQ_API int32_t nvq_quant_check(const nvq_quant *quant, const char *op);
+
+/* GatherQmm::groups / grouped (quantized.rs:724-735): 1 if a sorted gather of `rows` index
+ * rows over `experts` weight batches takes the grouped kernel. */
+NVQ_API int32_t nvq_gather_grouped(int64_t rows, int64_t experts, int32_t row_exact);
+
+/* GpuEval::supports for Primitive::QuantizedMatmul (gpu.rs:1665): 1 if nvq_quantized_matmul
+ * has a kernel for `desc`, else 0 (the caller then runs its CPU path, eval.rs:738-748). */
+NVQ_API int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *desc);
+
+/* ── the path ────────────────────────────────────────────────────────────────────── */
+
+/* GpuEval::quantize / fp_quantize (gpu.rs:6247-6275, 6302-6324); arithmetic of
+ * kernels::quantize / fp_quantize (kernels.rs:774-831, 914-971), bit for bit.
+ *   w       dtype [rows, cols] row-contiguous (leading dims folded into rows), cols % group == 0
+ *   packed  u32   [rows, cols*bits/32]
+ *   scales  dtype [rows, cols/group] (affine) or u8 (fp modes)
+ *   biases  dtype [rows, cols/group] (affine), NULL for the fp modes */
+NVQ_API int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols,
+                     void *packed, void *scales, void *biases, void *stream);
+
+/* GpuEval::dequantize / fp_dequantize (gpu.rs:6905-6930, 6879-6902) with the CPU's
+ * arithmetic (kernels.rs:835-859: two roundings in the scales' dtype; 976-1009), bit for bit.
+ *   affine: `dtype` is the dtype of scales, biases and out.
+ *   fp modes: `dtype` is the output dtype (f16, bf16 or f32); scales are u8, biases NULL.
+ *   out dtype [rows, cols]. */
+NVQ_API int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
+                       const void *biases, int64_t rows, int64_t cols, void *out, void *stream);
+
+/* Bytes of scratch nvq_quantized_matmul needs for `desc` (split-K partials; the reference
+ * allocates them on its side of the boundary, gpu.rs:7562).  0 = none. */
+NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
+
+/* GpuEval::quantized_matmul / fp_quantized_matmul (gpu.rs:6934-7168, 6336-6577); values of
+ * kernels::quantized_matmul (kernels.rs:1091-1142) within the stated tolerance.
+ * `workspace` may be NULL when nvq_quantized_matmul_workspace_bytes(desc) == 0. */
+NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
+                             const void *biases, void *y, void *workspace, void *stream);
+
+/* GpuEval::sorted_offsets (gpu.rs:6732-6756); kernels::sorted_offsets (kernels.rs:873-892):
+ * per row of `indices` u32[rows, m], offsets[row, g] = first position whose value is >= g. */
+NVQ_API int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
+                           int32_t *offsets, void *stream);
+
+NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);
+
+/* GpuEval::gather_qmm / fp_gather_qmm (gpu.rs:7174-7294, 6758-6876); values of the gathered
+ * products of quantized::gather_qmm_graph (quantized.rs:679-719).
+ * `offsets` NULL = one product per pair; non-NULL = grouped route (see nvq_gather_desc). */
+NVQ_API int32_t nvq_gather_qmm(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
+                       const void *biases, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                       void *y, void *workspace, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NUVEC_HIP_H */

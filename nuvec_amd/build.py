@@ -1,0 +1,69 @@
+"""Compiles the gfx950 kernels and the C ABI into `nuvec_amd/libnuvec_hip.so` with hipcc.
+
+Cross-compiles without a GPU.  Run as `python -m nuvec_amd.build` or through
+`__graft_entry__.build()`.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(HERE, "..", "include")
+LIB = os.path.join(HERE, "libnuvec_hip.so")
+SOURCES = ["nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmv.hip", "gather.hip"]
+
+# -ffp-contract=off: the quantizers must round every operation as the CPU does; fused
+# multiply-adds are written explicitly where wanted.  Correctly rounded f32 division is
+# hipcc's default and is spelled out because the bit-exact quantizers depend on it.
+# Packed-FP32 instructions are switched off for all device code.
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-gpu-flush-denormals-to-zero",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-fvisibility=hidden",
+    f"-I{INCLUDE}", f"-I{CSRC}",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build(verbose: bool = False, jobs: int = 4) -> str:
+    hipcc = _hipcc()
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{proc.stdout}\n{proc.stderr}")
+        # hipcc's host pass warns that it does not know the packed-fp32 feature: harmless.
+        noise = "is not a recognized feature for this target"
+        err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l and l.strip())
+        if verbose and err:
+            print(err, file=sys.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,331 @@
+// Host side of the C ABI: device record, error reporting, the reference's argument checks and
+// the routing from an operation to a gfx950 kernel.
+//
+// Validation restates nuvec's record-time checks so that a caller binding this library gets the
+// same refusals with the same wording (reference: crates/nuvec-core/src/quantized.rs:133-168,
+// 363-379; crates/nuvec-core/src/primitive.rs:1223-1320, 1412-1460).
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "nvq_internal.h"
+
+namespace nvq {
+
+namespace {
+thread_local char g_error[512] = "";
+
+struct DeviceRecord {
+    std::mutex mutex;
+    bool ready = false;
+    int device = -1;
+    hipDeviceProp_t prop;
+} g_device;
+
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+}  // namespace
+
+int32_t fail(int32_t status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+const char *dtype_name(int32_t d) {
+    switch (d) {
+    case NVQ_U8: return "uint8";
+    case NVQ_U32: return "uint32";
+    case NVQ_I32: return "int32";
+    case NVQ_F16: return "float16";
+    case NVQ_BF16: return "bfloat16";
+    case NVQ_F32: return "float32";
+    default: return "unknown";
+    }
+}
+
+const char *mode_name(int32_t m) {
+    switch (m) {
+    case NVQ_AFFINE: return "affine";
+    case NVQ_MXFP4: return "mxfp4";
+    case NVQ_MXFP8: return "mxfp8";
+    case NVQ_NVFP4: return "nvfp4";
+    default: return "unknown";
+    }
+}
+
+int32_t require_device() {
+    if (!g_device.ready) return fail(NVQ_NO_DEVICE, "no device bound: call nvq_init first");
+    return NVQ_OK;
+}
+
+int32_t compute_units() { return g_device.ready ? g_device.prop.multiProcessorCount : 0; }
+
+// Quant::checked (quantized.rs:133-168), messages included.
+int32_t check_quant(const nvq_quant *q, const char *op) {
+    if (q == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null quant", op);
+    const int g = q->group_size, b = q->bits;
+    if (q->mode == NVQ_AFFINE) {
+        if (!(g == 32 || g == 64 || g == 128))
+            return fail(NVQ_INVALID_ARGUMENT, "%s: group size %d is not supported (32, 64 or 128)", op, g);
+        if (!((b >= 1 && b <= 6) || b == 8))
+            return fail(NVQ_INVALID_ARGUMENT, "%s: %d bits are not supported (1, 2, 3, 4, 5, 6 or 8)", op, b);
+        return NVQ_OK;
+    }
+    int eg, eb;
+    switch (q->mode) {
+    case NVQ_MXFP4: eg = 32; eb = 4; break;
+    case NVQ_MXFP8: eg = 32; eb = 8; break;
+    case NVQ_NVFP4: eg = 16; eb = 4; break;
+    default: return fail(NVQ_INVALID_ARGUMENT, "%s: invalid quantization mode %d (affine, mxfp4, mxfp8 or nvfp4)", op, q->mode);
+    }
+    if (g != eg)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: %s quantization requires group size %d but got %d", op, mode_name(q->mode), eg, g);
+    if (b != eb)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: %s quantization requires bits to be %d but got %d", op, mode_name(q->mode), eb, b);
+    return NVQ_OK;
+}
+
+namespace {
+
+// check_groups (quantized.rs:363-379) as far as pointers can tell: affine needs biases, the
+// floating-point modes must not have them.
+int32_t check_groups(const char *op, int32_t mode, const void *biases) {
+    if (mode == NVQ_AFFINE && biases == nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: biases must be provided for affine quantization", op);
+    if (mode != NVQ_AFFINE && biases != nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: biases must be null for quantization mode '%s'", op, mode_name(mode));
+    return NVQ_OK;
+}
+
+int32_t check_float(const char *op, int32_t dtype) {
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "%s: unsupported dtype %s", op, dtype_name(dtype));
+    return NVQ_OK;
+}
+
+// The kernels use 16-byte vector accesses on every operand; allocations from hipMalloc (and
+// any sub-buffer at a multiple of 16 bytes) satisfy this.
+int32_t check_aligned(const char *op, const char *what, const void *p) {
+    if (p != nullptr && !aligned(p, 16))
+        return fail(NVQ_UNSUPPORTED, "%s: %s is not 16-byte aligned", op, what);
+    return NVQ_OK;
+}
+
+#define NVQ_TRY(expr)                     \
+    do {                                  \
+        int32_t nvq_rc_ = (expr);         \
+        if (nvq_rc_ != NVQ_OK) return nvq_rc_; \
+    } while (0)
+
+// The product's argument checks (primitive.rs:1279-1320 after quantized_columns,
+// primitive.rs:1412-1460): K must be whole groups and whole packed words.
+int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose, int64_t m, int64_t n, int64_t k) {
+    if (m < 0 || n < 0 || k < 0) return fail(NVQ_INVALID_ARGUMENT, "%s: negative dimension", op);
+    const int64_t cols = transpose ? k : n;  // values per packed row
+    if (cols % q.group_size != 0 || (cols * q.bits) % 32 != 0)
+        return fail(NVQ_INVALID_ARGUMENT,
+                    "%s: packed weights [.., %lld] and scales [.., %lld] do not match group size %d and %d bits", op,
+                    (long long)(cols * q.bits / 32), (long long)(cols / q.group_size), q.group_size, q.bits);
+    if (m >= (1LL << 31) || n >= (1LL << 31) || k >= (1LL << 31))
+        return fail(NVQ_UNSUPPORTED, "%s: dimensions beyond 2^31", op);
+    return NVQ_OK;
+}
+
+}  // namespace
+}  // namespace nvq
+
+using namespace nvq;
+
+extern "C" {
+
+const char *nvq_last_error(void) { return g_error; }
+
+const char *nvq_version(void) { return "nuvec-hip 0.1.0 (gfx950)"; }
+
+int32_t nvq_init(int32_t device) {
+    std::lock_guard<std::mutex> lock(g_device.mutex);
+    if (g_device.ready && g_device.device == device) return NVQ_OK;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(NVQ_NO_DEVICE, "no HIP device is visible");
+    }
+    if (device < 0 || device >= count) return fail(NVQ_NO_DEVICE, "device %d of %d does not exist", device, count);
+    hipDeviceProp_t prop;
+    NVQ_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(NVQ_NO_DEVICE, "device %d is %s: this library holds gfx950 code only", device, prop.gcnArchName);
+    g_device.prop = prop;
+    g_device.device = device;
+    g_device.ready = true;
+    return NVQ_OK;
+}
+
+int32_t nvq_get_device_info(nvq_device_info *info) {
+    if (info == nullptr) return fail(NVQ_INVALID_ARGUMENT, "device_info: null output");
+    NVQ_TRY(require_device());
+    memset(info, 0, sizeof *info);
+    info->device = g_device.device;
+    info->compute_units = g_device.prop.multiProcessorCount;
+    info->wavefront_size = g_device.prop.warpSize;
+    info->lds_bytes_per_block = (int32_t)g_device.prop.sharedMemPerBlock;
+    info->global_memory_bytes = (int64_t)g_device.prop.totalGlobalMem;
+    snprintf(info->arch, sizeof info->arch, "%s", g_device.prop.gcnArchName);
+    snprintf(info->name, sizeof info->name, "%s", g_device.prop.name);
+    return NVQ_OK;
+}
+
+int32_t nvq_quant_check(const nvq_quant *quant, const char *op) { return check_quant(quant, op ? op : "quant"); }
+
+// quantized.rs:724-735 (`ROW_TOKENS` = ROW_INDEPENDENT_ROWS * 8 = 64: crates/nuvec-core/src/lib.rs).
+int32_t nvq_gather_grouped(int64_t rows, int64_t experts, int32_t row_exact) {
+    const int64_t least = row_exact ? 65 : 16;
+    return rows >= least && rows / (experts > 1 ? experts : 1) >= 4;
+}
+
+int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols, void *packed,
+                     void *scales, void *biases, void *stream) {
+    NVQ_TRY(check_quant(quant, "quantize"));
+    // primitive.rs:1234-1243
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "quantize: unsupported dtype %s", dtype_name(dtype));
+    if (rows < 0 || cols < 0 || cols % quant->group_size != 0)
+        return fail(NVQ_INVALID_ARGUMENT,
+                    "quantize: needs at least 2 dimensions with the last divisible by the group size %d, got shape [%lld, %lld]",
+                    quant->group_size, (long long)rows, (long long)cols);
+    NVQ_TRY(check_groups("quantize", quant->mode, quant->mode == NVQ_AFFINE ? biases : nullptr));
+    if (quant->mode != NVQ_AFFINE && biases != nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "quantize: biases must be null for quantization mode '%s'", mode_name(quant->mode));
+    if (rows == 0 || cols == 0) return NVQ_OK;
+    if (w == nullptr || packed == nullptr || scales == nullptr) return fail(NVQ_INVALID_ARGUMENT, "quantize: null operand");
+    NVQ_TRY(require_device());
+    NVQ_TRY(check_aligned("quantize", "w", w));
+    NVQ_TRY(check_aligned("quantize", "packed", packed));
+    const int64_t n = rows * cols;
+    if (quant->mode == NVQ_AFFINE)
+        return launch_affine_quantize(dtype, quant->group_size, quant->bits, w, n, packed, scales, biases, (hipStream_t)stream);
+    return launch_fp_quantize(quant->mode, dtype, w, n, packed, scales, (hipStream_t)stream);
+}
+
+int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales, const void *biases,
+                       int64_t rows, int64_t cols, void *out, void *stream) {
+    NVQ_TRY(check_quant(quant, "dequantize"));
+    NVQ_TRY(check_groups("dequantize", quant->mode, biases));
+    // primitive.rs:1272-1276
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "dequantize: unsupported dtype %s", dtype_name(dtype));
+    if (rows < 0 || cols < 0 || cols % quant->group_size != 0 || (cols * quant->bits) % 32 != 0)
+        return fail(NVQ_INVALID_ARGUMENT,
+                    "dequantize: packed weights [%lld, %lld] and scales [%lld, %lld] do not match group size %d and %d bits",
+                    (long long)rows, (long long)(cols * quant->bits / 32), (long long)rows,
+                    (long long)(cols / quant->group_size), quant->group_size, quant->bits);
+    if (rows == 0 || cols == 0) return NVQ_OK;
+    if (packed == nullptr || scales == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "dequantize: null operand");
+    NVQ_TRY(require_device());
+    NVQ_TRY(check_aligned("dequantize", "packed", packed));
+    NVQ_TRY(check_aligned("dequantize", "out", out));
+    const int64_t n = rows * cols;
+    if (quant->mode == NVQ_AFFINE)
+        return launch_affine_dequantize(dtype, quant->group_size, quant->bits, packed, scales, biases, n, out, (hipStream_t)stream);
+    return launch_fp_dequantize(quant->mode, dtype, packed, scales, n, out, (hipStream_t)stream);
+}
+
+static int32_t check_qmm(const nvq_qmm_desc *d, const char *op) {
+    if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null descriptor", op);
+    NVQ_TRY(check_quant(&d->quant, op));
+    NVQ_TRY(check_float(op, d->dtype));
+    NVQ_TRY(check_product_dims(op, d->quant, d->transpose, d->m, d->n, d->k));
+    if (d->batch_ndim < 0 || d->batch_ndim > NVQ_MAX_BATCH_DIMS)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: %d batch dimensions (at most %d)", op, d->batch_ndim, NVQ_MAX_BATCH_DIMS);
+    for (int i = 0; i < d->batch_ndim; i++)
+        if (d->batch_shape[i] < 0 || d->x_strides[i] < 0 || d->w_strides[i] < 0 || d->s_strides[i] < 0)
+            return fail(NVQ_INVALID_ARGUMENT, "%s: negative batch shape or stride", op);
+    return NVQ_OK;
+}
+
+int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
+    if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
+    if (!d->transpose) return 0;  // x . w (qvm / qmm_n) has no gfx950 kernel yet
+    if (d->quant.mode != NVQ_AFFINE && d->quant.mode != NVQ_MXFP4) return 0;
+    return 1;
+}
+
+size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *) { return 0; }
+
+int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                             void *y, void *workspace, void *stream) {
+    (void)workspace;
+    NVQ_TRY(check_qmm(d, "quantized_matmul"));
+    NVQ_TRY(check_groups("quantized_matmul", d->quant.mode, biases));
+    int64_t batch = 1;
+    for (int i = 0; i < d->batch_ndim; i++) batch *= d->batch_shape[i];
+    if (batch == 0 || d->m == 0 || d->n == 0) return NVQ_OK;
+    if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "quantized_matmul: null operand");
+    NVQ_TRY(require_device());
+    if (!nvq_quantized_matmul_supported(d))
+        return fail(NVQ_UNSUPPORTED, "quantized_matmul: no gfx950 kernel for mode %s, transpose=%d", mode_name(d->quant.mode), d->transpose);
+    NVQ_TRY(check_aligned("quantized_matmul", "x", x));
+    NVQ_TRY(check_aligned("quantized_matmul", "w", w));
+    NVQ_TRY(check_aligned("quantized_matmul", "y", y));
+    if (d->k == 0) {  // an empty reduction is zero (crates/nuvec-cpu/src/matmul.rs:237-240)
+        return launch_fill_zero(y, batch * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
+    }
+    ProductArgs a{};
+    a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
+    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
+    a.m = d->m; a.n = d->n; a.k = d->k;
+    a.batch = batch;
+    a.batch_ndim = d->batch_ndim;
+    for (int i = 0; i < d->batch_ndim; i++) {
+        a.batch_shape[i] = d->batch_shape[i];
+        a.x_strides[i] = d->x_strides[i];
+        a.w_strides[i] = d->w_strides[i];
+        a.s_strides[i] = d->s_strides[i];
+    }
+    return launch_qmv(a, (hipStream_t)stream);
+}
+
+int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups, int32_t *offsets, void *stream) {
+    if (rows < 0 || m < 0 || groups < 0) return fail(NVQ_INVALID_ARGUMENT, "sorted_offsets: negative size");
+    if (rows == 0 || groups == 0) return NVQ_OK;
+    if (offsets == nullptr || (indices == nullptr && m > 0)) return fail(NVQ_INVALID_ARGUMENT, "sorted_offsets: null operand");
+    NVQ_TRY(require_device());
+    return launch_sorted_offsets(indices, rows, m, groups, offsets, (hipStream_t)stream);
+}
+
+size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *) { return 0; }
+
+int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                       const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
+    (void)workspace;
+    (void)offsets;
+    if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
+    NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
+    NVQ_TRY(check_groups("gather_qmm", d->quant.mode, biases));
+    NVQ_TRY(check_float("gather_qmm", d->dtype));
+    NVQ_TRY(check_product_dims("gather_qmm", d->quant, d->transpose, d->m, d->n, d->k));
+    if (d->pairs < 0 || d->x_batches < 0 || d->experts < 0) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: negative size");
+    if (d->pairs == 0 || d->m == 0 || d->n == 0) return NVQ_OK;
+    if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr || lhs == nullptr || rhs == nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null operand");
+    NVQ_TRY(require_device());
+    if (!d->transpose || (d->quant.mode != NVQ_AFFINE && d->quant.mode != NVQ_MXFP4))
+        return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for mode %s, transpose=%d", mode_name(d->quant.mode), d->transpose);
+    NVQ_TRY(check_aligned("gather_qmm", "x", x));
+    NVQ_TRY(check_aligned("gather_qmm", "w", w));
+    NVQ_TRY(check_aligned("gather_qmm", "y", y));
+    if (d->k == 0) {
+        return launch_fill_zero(y, d->pairs * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
+    }
+    ProductArgs a{};
+    a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
+    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
+    a.m = d->m; a.n = d->n; a.k = d->k;
+    a.batch = d->pairs;
+    a.lhs = lhs; a.rhs = rhs;
+    a.x_batches = d->x_batches; a.experts = d->experts;
+    return launch_qmv(a, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,106 @@
+// Device-side scalar helpers: element types, exact conversions, the small float codecs.
+// Everything here is written so that the bits equal nuvec's CPU arithmetic
+// (reference: crates/nuvec-core/src/cast.rs:49-98, crates/nuvec-core/src/fp8.rs:11-129).
+// The library is compiled with floating-point contraction off: a fused multiply-add appears
+// only where it is written.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nvq {
+
+struct bf16_t { uint16_t bits; };   // bfloat16 storage
+typedef _Float16 f16_t;             // IEEE half: native arithmetic, round to nearest even
+
+__device__ __forceinline__ uint32_t f2u(float x) { return __float_as_uint(x); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+
+// bf16 <- f32: round to nearest even; a NaN keeps its high bits and is quieted
+// (the `half` crate's bf16::from_f32, which cast.rs:85-98 calls).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+    uint32_t u = f2u(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    uint32_t up = ((u & 0x8000u) != 0u) && ((u & 0x17FFFu) != 0u);
+    return (uint16_t)((u >> 16) + up);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int code = 11;
+    __device__ static __forceinline__ float load(const float *p, int64_t i) { return p[i]; }
+    __device__ static __forceinline__ void store(float *p, int64_t i, float v) { p[i] = v; }
+    // round(a*b) and round(a+b) in the element type
+    __device__ static __forceinline__ float mul(float a, float b) { return a * b; }
+    __device__ static __forceinline__ float add(float a, float b) { return a + b; }
+};
+template <> struct Elem<bf16_t> {
+    static constexpr int code = 10;
+    __device__ static __forceinline__ float load(const bf16_t *p, int64_t i) { return bf16_bits_to_f32(p[i].bits); }
+    __device__ static __forceinline__ void store(bf16_t *p, int64_t i, float v) { p[i].bits = f32_to_bf16_bits(v); }
+    __device__ static __forceinline__ float mul(float a, float b) { return bf16_bits_to_f32(f32_to_bf16_bits(a * b)); }
+    __device__ static __forceinline__ float add(float a, float b) { return bf16_bits_to_f32(f32_to_bf16_bits(a + b)); }
+};
+template <> struct Elem<f16_t> {
+    static constexpr int code = 9;
+    __device__ static __forceinline__ float load(const f16_t *p, int64_t i) { return (float)p[i]; }
+    __device__ static __forceinline__ void store(f16_t *p, int64_t i, float v) { p[i] = (f16_t)v; }
+    // Both operands are exact halves: native half arithmetic rounds the exact result once.
+    __device__ static __forceinline__ float mul(float a, float b) { return (float)((f16_t)a * (f16_t)b); }
+    __device__ static __forceinline__ float add(float a, float b) { return (float)((f16_t)a + (f16_t)b); }
+};
+
+// Rust's f32::min / f32::max as the reference's hosts evaluate them: the other operand
+// when one is NaN, and -0 ordered below +0.
+__device__ __forceinline__ float rs_min(float a, float b) {
+    float m = fminf(a, b);
+    if (a == 0.0f && b == 0.0f) m = u2f(f2u(a) | f2u(b));
+    return m;
+}
+__device__ __forceinline__ float rs_max(float a, float b) {
+    float m = fmaxf(a, b);
+    if (a == 0.0f && b == 0.0f) m = u2f(f2u(a) & f2u(b));
+    return m;
+}
+
+// fp8.rs:103-112: a float32 subnormal becomes a zero of its sign.
+__device__ __forceinline__ float ftz(float x) {
+    uint32_t u = f2u(x);
+    return ((u & 0x7F800000u) == 0u) ? u2f(u & 0x80000000u) : x;
+}
+// fp8.rs:114-118
+__device__ __forceinline__ float canonical(float x) { return x != x ? u2f(0x7FC00000u) : x; }
+
+// fp8.rs:47-73
+__device__ __forceinline__ uint32_t e2m1_from_f32(float x) {
+    if (x != x) return 0x7u;
+    uint32_t sign = (f2u(x) >> 28) & 0x8u;
+    float a = fabsf(x);
+    uint32_t code = a > 5.0f ? 7u : a >= 3.5f ? 6u : a > 2.5f ? 5u : a >= 1.75f ? 4u
+                  : a > 1.25f ? 3u : a >= 0.75f ? 2u : a > 0.25f ? 1u : 0u;
+    return code | sign;
+}
+// fp8.rs:75-80: 0, 0.5, 1, 1.5, 2, 3, 4, 6 and their negatives
+__device__ __forceinline__ float e2m1_to_f32(uint32_t code) {
+    uint32_t m = code & 7u;
+    // magnitudes as float32 bit patterns, built from the code: m < 2 -> m/2; else 2^((m>>1)-1) * (1 + (m&1)/2)
+    float v = m == 0u ? 0.0f : m == 1u ? 0.5f : u2f(((126u + (m >> 1)) << 23) | ((m & 1u) << 22));
+    return (code & 8u) ? -v : v;
+}
+// fp8.rs:95-102
+__device__ __forceinline__ float e8m0_to_f32(uint32_t code) {
+    return code == 0u ? u2f(0x400000u) : u2f(code << 23);
+}
+// e8m0_from_f32(mx_scale_round_up(x)) for x = ftz(amax / max_element) >= 0 (fp8.rs:82-93,
+// 120-129 as composed at kernels.rs:940-943): the smallest power of two not below x, i.e.
+// exponent field + (mantissa != 0), at most 254; 0 for zero; 0xFF for +Inf.
+__device__ __forceinline__ uint32_t e8m0_round_up_code(float x) {
+    uint32_t u = f2u(x);
+    if (u >= 0x7F800000u) return 0xFFu;
+    if (u == 0u) return 0u;
+    uint32_t c = (u >> 23) + ((u & 0x7FFFFFu) != 0u);
+    return c > 254u ? 254u : c;
+}
+
+}  // namespace nvq

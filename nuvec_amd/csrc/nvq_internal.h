@@ -1,0 +1,67 @@
+// Internal declarations shared by the host entry points and the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "nuvec_hip.h"
+
+namespace nvq {
+
+// ── errors ──────────────────────────────────────────────────────────────────────────
+// Records `status` and a printf-style message for the calling thread; returns `status`.
+int32_t fail(int32_t status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define NVQ_HIP_TRY(expr)                                                                      \
+    do {                                                                                       \
+        hipError_t nvq_e_ = (expr);                                                            \
+        if (nvq_e_ != hipSuccess)                                                              \
+            return ::nvq::fail(nvq_e_ == hipErrorOutOfMemory ? NVQ_OUT_OF_MEMORY : NVQ_BACKEND, \
+                               "%s: %s", #expr, hipGetErrorString(nvq_e_));                    \
+    } while (0)
+
+// Launch check: a bad configuration is reported by the launch itself.
+#define NVQ_LAUNCH_CHECK(what)                                                                  \
+    do {                                                                                        \
+        hipError_t nvq_e_ = hipGetLastError();                                                  \
+        if (nvq_e_ != hipSuccess)                                                               \
+            return ::nvq::fail(NVQ_BACKEND, "%s launch: %s", what, hipGetErrorString(nvq_e_));   \
+    } while (0)
+
+int32_t require_device();          // NVQ_OK once nvq_init succeeded
+int32_t compute_units();           // of the bound device
+int32_t check_quant(const nvq_quant *q, const char *op);
+inline bool float_dtype(int32_t d) { return d == NVQ_F16 || d == NVQ_BF16 || d == NVQ_F32; }
+inline int dtype_size(int32_t d) { return d == NVQ_F32 ? 4 : (d == NVQ_U8 ? 1 : (d == NVQ_U32 || d == NVQ_I32 ? 4 : 2)); }
+const char *dtype_name(int32_t d);
+const char *mode_name(int32_t m);
+
+// ── kernel launchers (each validates nothing: the entry points did) ─────────────────────
+int32_t launch_affine_quantize(int32_t dtype, int group, int bits, const void *w, int64_t n_values,
+                               void *packed, void *scales, void *biases, hipStream_t s);
+int32_t launch_affine_dequantize(int32_t dtype, int group, int bits, const void *packed, const void *scales,
+                                 const void *biases, int64_t n_values, void *out, hipStream_t s);
+int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n_values, void *packed,
+                           void *scales, hipStream_t s);
+int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales,
+                             int64_t n_values, void *out, hipStream_t s);
+int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
+                              int32_t *offsets, hipStream_t s);
+
+// One transposed product per batch/pair.  `lhs`/`rhs` NULL = batch strides from `desc`.
+struct ProductArgs {
+    const void *x, *w, *scales, *biases;
+    void *y;
+    int32_t mode, group, bits, dtype;
+    int64_t m, n, k;
+    int64_t batch;                  // grid z
+    int32_t batch_ndim;             // 0: single product
+    int64_t batch_shape[NVQ_MAX_BATCH_DIMS];
+    int64_t x_strides[NVQ_MAX_BATCH_DIMS], w_strides[NVQ_MAX_BATCH_DIMS], s_strides[NVQ_MAX_BATCH_DIMS];
+    const uint32_t *lhs, *rhs;      // gather: batch z reads x batch lhs[z] and weight batch rhs[z]
+    int64_t x_batches, experts;     // gather: index bounds (an index beyond them is clamped)
+};
+int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
+int32_t launch_fill_zero(void *p, int64_t bytes, hipStream_t s);
+
+}  // namespace nvq

@@ -1,0 +1,522 @@
+// Few-row quantized products y = x . dequantize(w)^T for gfx950: the decode-shaped path.
+// Values follow nuvec's CPU product (reference: crates/nuvec-core/src/kernels.rs:1091-1142)
+// within the stated tolerance; the factored form per group,
+//     scale * sum(x * code) + bias * sum(x),
+// is the one the reference's device kernels use (crates/nuvec-kernels/src/metal/quantized.h:247-360).
+//
+// Work split.  A wavefront owns RN consecutive weight rows and walks K in steps of 2048
+// values; inside a step lane l owns the 32 values [32 l, 32 l + 32), which are `bits`
+// consecutive dwords of the packed row (one 128-bit load at 4 bits) and lie inside one
+// quantization group (groups are 32, 64 or 128 values).  A wavefront-wide load therefore
+// reads 64*4*bits contiguous bytes of one row.  The x slice of the step is decoded once and
+// reused for the RN rows; the RN*RM partial sums stay in registers and are folded across
+// the wavefront once, at the end.  No LDS and no barriers: HBM latency is covered by the RN
+// independent row loads each lane has in flight.
+#include "nvq_device.h"
+#include "nvq_internal.h"
+
+namespace nvq {
+namespace {
+
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+
+constexpr int kWaves = 4;             // wavefronts per block
+constexpr int kStep = 64 * 32;        // values of K per wavefront step
+
+// Element offsets of batch `z` for x, w (in packed dwords), scales/biases and y.
+struct BatchOffsets { int64_t x, w, s, y; };
+
+__device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int64_t z, int64_t kwords, int64_t kgroups) {
+    BatchOffsets o{0, 0, 0, z * a.m * a.n};
+    if (a.rhs != nullptr) {  // gathered pairs
+        // An index outside its operand is the caller's error; it is clamped so that it cannot
+        // fault the device.
+        const int64_t l = min((int64_t)a.lhs[z], a.x_batches - 1), r = min((int64_t)a.rhs[z], a.experts - 1);
+        o.x = l * a.m * a.k;
+        o.w = r * a.n * kwords;
+        o.s = r * a.n * kgroups;
+        return o;
+    }
+    if (a.batch_ndim == 0) return o;
+    int64_t rest = z;
+#pragma unroll
+    for (int d = NVQ_MAX_BATCH_DIMS - 1; d >= 0; d--) {  // constant indices: the arrays stay in kernel arguments
+        if (d < a.batch_ndim) {
+            const int64_t i = rest % a.batch_shape[d];
+            rest /= a.batch_shape[d];
+            o.x += i * a.x_strides[d];
+            o.w += i * a.w_strides[d];
+            o.s += i * a.s_strides[d];
+        }
+    }
+    return o;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    return v;
+}
+
+// v + (v moved across lanes by a DPP control); lanes the control does not feed add 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, true);
+    return v + __int_as_float(moved);
+}
+
+// Sum over the wavefront in VALU data-parallel-primitive steps (no LDS traffic): shifts by
+// 1, 2, 4, 8 inside each row of 16 lanes, then the row totals carried into the next rows.
+// The total is valid in lane 63 only.
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v = dpp_add<0x111, 0xF>(v);  // row_shr:1
+    v = dpp_add<0x112, 0xF>(v);  // row_shr:2
+    v = dpp_add<0x114, 0xF>(v);  // row_shr:4
+    v = dpp_add<0x118, 0xF>(v);  // row_shr:8
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// (a & mask) | magic in one instruction.  The mask travels in a scalar register and the
+// constant in a vector register: a three-operand VALU instruction of this ISA takes no
+// literal and at most one scalar operand, so the compiler would otherwise emit an AND and an OR.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_sgpr, uint32_t magic_vgpr) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask_sgpr), "v"(magic_vgpr));
+    return d;
+}
+
+// Loads the lane's `BITS` dwords of a packed row.
+template <int BITS>
+__device__ __forceinline__ void load_words(const uint32_t *p, uint32_t (&d)[BITS]) {
+    if constexpr (BITS == 4) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(p);
+        d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+    } else if constexpr (BITS == 8) {
+        const uint4 q0 = reinterpret_cast<const uint4 *>(p)[0], q1 = reinterpret_cast<const uint4 *>(p)[1];
+        d[0] = q0.x; d[1] = q0.y; d[2] = q0.z; d[3] = q0.w;
+        d[4] = q1.x; d[5] = q1.y; d[6] = q1.z; d[7] = q1.w;
+    } else if constexpr (BITS == 2) {
+        const uint2 q = *reinterpret_cast<const uint2 *>(p);
+        d[0] = q.x; d[1] = q.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < BITS; i++) d[i] = p[i];
+    }
+}
+
+// Code `i` (0..31) of the lane's BITS dwords: value i sits at bit i*BITS of the stream
+// (reference: kernels.rs:749-756).
+template <int BITS>
+__device__ __forceinline__ uint32_t code_at(const uint32_t (&d)[BITS], int i) {
+    constexpr uint32_t mask = (1u << BITS) - 1u;
+    const int bit = i * BITS, word = bit >> 5, sh = bit & 31;
+    uint32_t v = d[word] >> sh;
+    if (sh + BITS > 32) v |= d[word + 1] << (32 - sh);
+    return v & mask;
+}
+
+// ── generic kernel: any bit width, any element type, affine or MXFP4 ──────────────────────
+template <typename T, int BITS, bool FP4, int RM, int RN>
+__global__ void __launch_bounds__(kWaves * 64) qmv_generic_kernel(const ProductArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t n0 = ((int64_t)blockIdx.x * kWaves + wave) * RN;
+    if (n0 >= a.n) return;
+    const int64_t m0 = (int64_t)blockIdx.y * RM;
+    const int64_t kwords = a.k * BITS / 32, kgroups = a.k / a.group;
+    const BatchOffsets o = batch_offsets(a, blockIdx.z, kwords, kgroups);
+    const T *x = (const T *)a.x + o.x;
+    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    T *y = (T *)a.y + o.y;
+
+    float acc[RN][RM];
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) acc[r][i] = 0.0f;
+
+    for (int64_t k0 = 0; k0 < a.k; k0 += kStep) {
+        const int64_t kb = k0 + lane * 32;
+        if (kb >= a.k) continue;  // K is a multiple of 32: a lane's slice is whole or absent
+        float xv[RM][32], xs[RM];
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            xs[i] = 0.0f;
+            const bool row = m0 + i < a.m;
+#pragma unroll
+            for (int j = 0; j < 32; j++) {
+                xv[i][j] = row ? Elem<T>::load(x, (m0 + i) * a.k + kb + j) : 0.0f;
+                xs[i] += xv[i][j];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RN; r++) {
+            const int64_t n = n0 + r;
+            if (n >= a.n) break;
+            uint32_t d[BITS];
+            load_words<BITS>(w + n * kwords + kb * BITS / 32, d);
+            const int64_t g = n * kgroups + kb / a.group;
+            float dot[RM];
+#pragma unroll
+            for (int i = 0; i < RM; i++) dot[i] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; j++) {
+                const uint32_t c = code_at<BITS>(d, j);
+                const float v = FP4 ? e2m1_to_f32(c) : (float)c;
+#pragma unroll
+                for (int i = 0; i < RM; i++) dot[i] = __builtin_fmaf(xv[i][j], v, dot[i]);
+            }
+            if constexpr (FP4) {
+                const float s = ftz(e8m0_to_f32(((const uint8_t *)a.scales)[o.s + g]));
+#pragma unroll
+                for (int i = 0; i < RM; i++) acc[r][i] = __builtin_fmaf(s, dot[i], acc[r][i]);
+            } else {
+                const float s = Elem<T>::load((const T *)a.scales + o.s, g);
+                const float b = Elem<T>::load((const T *)a.biases + o.s, g);
+#pragma unroll
+                for (int i = 0; i < RM; i++)
+                    acc[r][i] = __builtin_fmaf(s, dot[i], __builtin_fmaf(b, xs[i], acc[r][i]));
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float v = wave_sum(acc[r][i]);
+            if (lane == 0 && n0 + r < a.n && m0 + i < a.m) Elem<T>::store(y, (m0 + i) * a.n + n0 + r, v);
+        }
+}
+
+// ── 4-bit affine, bf16 / f16: packed-pair dot products ────────────────────────────────────
+// Two codes become two element-type values in one instruction: code c in the low mantissa
+// bits of the constant 128 (bf16, 0x4300) or 1024 (f16, 0x6400) is exactly 128 + c or 1024 + c.
+// `v_dot2_f32_{bf16,f16}` then accumulates x0*(B + c0) + x1*(B + c1) in float32, and the
+// offset is removed with the group's sum of x:  sum x*c = dot - B * sum x.
+template <typename T> struct Pair;
+template <> struct Pair<bf16_t> {
+    static constexpr uint32_t magic = 0x43004300u;
+    static constexpr float base = 128.0f;
+    __device__ static __forceinline__ float dot2(uint32_t x, uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, w), acc, false);
+    }
+    __device__ static __forceinline__ float lo(uint32_t p) { return u2f(p << 16); }
+    __device__ static __forceinline__ float hi(uint32_t p) { return u2f(p & 0xFFFF0000u); }
+};
+template <> struct Pair<f16_t> {
+    static constexpr uint32_t magic = 0x64006400u;
+    static constexpr float base = 1024.0f;
+    __device__ static __forceinline__ float dot2(uint32_t x, uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, x), __builtin_bit_cast(f16x2_t, w), acc, false);
+    }
+    __device__ static __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[0]; }
+    __device__ static __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[1]; }
+};
+
+// One wavefront per block, RN weight rows per wavefront, KU steps of 2048 values per loop
+// iteration with every load of the iteration issued before the first use: at K = 4096 the
+// whole product of a wavefront is one round trip to memory (KU*RN 128-bit loads per lane in
+// flight), and the block count (N / RN) spreads evenly over the compute units.
+template <typename T, int RM, int RN, int KU>
+__global__ void __launch_bounds__(64) qmv4_pair_kernel(const ProductArgs a) {
+    const int lane = threadIdx.x;
+    const int64_t n0 = (int64_t)blockIdx.x * RN;
+    const int64_t m0 = (int64_t)blockIdx.y * RM;
+    const int64_t kwords = a.k / 8, kgroups = a.k / a.group;
+    const BatchOffsets o = batch_offsets(a, blockIdx.z, kwords, kgroups);
+    const T *x = (const T *)a.x + o.x;
+    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
+    T *y = (T *)a.y + o.y;
+    constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
+
+    float acc[RN][RM];
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) acc[r][i] = 0.0f;
+
+    for (int64_t k0 = 0; k0 < a.k; k0 += (int64_t)KU * kStep) {
+        uint4 xq[KU][RM][4], wq[KU][RN];
+        T sraw[KU][RN], braw[KU][RN];
+        bool live[KU];
+#pragma unroll
+        for (int u = 0; u < KU; u++) {
+            const int64_t kb = k0 + (int64_t)u * kStep + lane * 32;
+            live[u] = kb < a.k;  // K is a multiple of 32: a lane's slice is whole or absent
+            const int64_t kc = live[u] ? kb : 0;
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                const int64_t row = m0 + i < a.m ? m0 + i : a.m - 1;
+                const uint4 *px = reinterpret_cast<const uint4 *>(x + row * a.k + kc);
+#pragma unroll
+                for (int j = 0; j < 4; j++) xq[u][i][j] = px[j];
+            }
+#pragma unroll
+            for (int r = 0; r < RN; r++) {
+                const int64_t n = n0 + r < a.n ? n0 + r : a.n - 1;  // clamp: tail rows are computed, not stored
+                wq[u][r] = *reinterpret_cast<const uint4 *>(w + n * kwords + kc / 8);
+                const int64_t g = n * kgroups + kc / a.group;
+                sraw[u][r] = scales[g];
+                braw[u][r] = biases[g];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < KU; u++) {
+            // x pairs in the order the nibbles pair up: word j holds values 8j..8j+7, and
+            // (w >> 4t) & 0x000F000F picks values 8j+t (low half) and 8j+t+4 (high half).
+            uint32_t xp[RM][16];
+            float xs[RM];
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                xs[i] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint4 q = xq[u][i][j];  // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
+                    xp[i][4 * j + 0] = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+                    xp[i][4 * j + 1] = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+                    xp[i][4 * j + 2] = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+                    xp[i][4 * j + 3] = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xs[i] = Pair<T>::dot2(xp[i][4 * j + t], ones, xs[i]);
+                }
+                if (!live[u] || m0 + i >= a.m) {  // an absent slice or row contributes nothing
+                    xs[i] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 16; j++) xp[i][j] = 0u;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RN; r++) {
+                const uint32_t d[4] = {wq[u][r].x, wq[u][r].y, wq[u][r].z, wq[u][r].w};
+                float dot[RM];
+#pragma unroll
+                for (int i = 0; i < RM; i++) dot[i] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const uint32_t pair = ((d[j] >> (4 * t)) & 0x000F000Fu) | Pair<T>::magic;
+#pragma unroll
+                        for (int i = 0; i < RM; i++) dot[i] = Pair<T>::dot2(xp[i][4 * j + t], pair, dot[i]);
+                    }
+                // scale * (dot - B * sum x) + bias * sum x
+                const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
+                const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+                for (int i = 0; i < RM; i++)
+                    acc[r][i] = __builtin_fmaf(sc, dot[i], __builtin_fmaf(bb, xs[i], acc[r][i]));
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float v = wave_sum(acc[r][i]);
+            if (lane == 0 && n0 + r < a.n && m0 + i < a.m) Elem<T>::store(y, (m0 + i) * a.n + n0 + r, v);
+        }
+}
+
+// ── 4-bit affine, bf16 / f16, one or two rows of x: the decode kernel ─────────────────────
+// A block of WAVES wavefronts shares the x slice of one K step (4096 values) through LDS, stored
+// once in the pair order the nibbles need together with the sums of its 32-value slices, so the
+// per-row work of a wavefront is only: two 128-bit weight loads per lane, the nibble expansion,
+// the packed dot products and one data-parallel-primitive reduction.  Every load of a step is
+// issued before the first use; blocks are small (WAVES*RN weight rows) so that tens of
+// thousands of independent loads are in flight on the chip.
+template <typename T, int RM, int RN, int WAVES, bool BATCHED>
+__global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs a) {
+    constexpr int kThreads = WAVES * 64;
+    constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
+    static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
+    __shared__ uint4 x_pairs[RM][2][4][64];  // [row][chunk][word][lane]: 4 pairs of a packed word
+    __shared__ float x_sums[RM][2][64];      // [row][chunk][lane]: sum of the lane's 32 values
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Sizes fit 32 bits (checked on the host); only row bases are 64-bit, and they are uniform.
+    const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
+    const int gshift = a.group == 32 ? 5 : a.group == 64 ? 6 : 7;
+    const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * WAVES + wave) * RN);
+    const int m0 = blockIdx.y * RM;
+    const int kwords = K >> 3, kgroups = K >> gshift;
+    // The single-product instantiation carries no batch arithmetic at all.
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
+    const T *x = (const T *)a.x + o.x;
+    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
+    T *y = (T *)a.y + o.y;
+    constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
+    uint32_t mask, magic;
+    asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
+
+    float acc[RN][RM];
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) acc[r][i] = 0.0f;
+
+    for (int k0 = 0; k0 < K; k0 += 2 * kStep) {
+        // x first: it is needed first and arrives from the cache.
+        uint4 xg[RM][kXPerThread];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int p = 0; p < kXPerThread; p++) {
+                const int kx = k0 + (tid + p * kThreads) * 8;
+                xg[i][p] = (kx < K && m0 + i < M) ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + kx)
+                                                      : make_uint4(0, 0, 0, 0);  // absent x: contributes nothing
+            }
+        uint4 wq[2][RN];
+        T sraw[2][RN], braw[2][RN];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int kb = k0 + u * kStep + lane * 32;
+            const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
+#pragma unroll
+            for (int r = 0; r < RN; r++) {
+                const int n = n0 + r < N ? n0 + r : N - 1;  // tail rows are computed, not stored
+                wq[u][r] = *reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 3));
+                const T *ps = scales + (int64_t)n * kgroups, *pb = biases + (int64_t)n * kgroups;
+                sraw[u][r] = ps[kc >> gshift];
+                braw[u][r] = pb[kc >> gshift];
+            }
+        }
+        if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int p = 0; p < kXPerThread; p++) {
+                const int idx = tid + p * kThreads;  // 128-bit piece: chunk idx/256, lane (idx%256)/4, word idx%4
+                const uint4 q = xg[i][p];            // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
+                uint4 pr;
+                pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+                pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+                pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+                pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+                x_pairs[i][idx >> 8][idx & 3][(idx & 255) >> 2] = pr;
+                float sum = Pair<T>::dot2(pr.x, ones, 0.0f);
+                sum = Pair<T>::dot2(pr.y, ones, sum);
+                sum = Pair<T>::dot2(pr.z, ones, sum);
+                sum = Pair<T>::dot2(pr.w, ones, sum);
+                sum += __shfl_xor(sum, 1);  // the four pieces of a lane's slice sit in adjacent threads
+                sum += __shfl_xor(sum, 2);
+                if ((idx & 3) == 0) x_sums[i][idx >> 8][(idx & 255) >> 2] = sum;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            uint4 xp[RM][4];
+            float xs[RM];
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) xp[i][j] = x_pairs[i][u][j][lane];
+                xs[i] = x_sums[i][u][lane];
+            }
+#pragma unroll
+            for (int r = 0; r < RN; r++) {
+                const uint32_t d[4] = {wq[u][r].x, wq[u][r].y, wq[u][r].z, wq[u][r].w};
+                float dot[RM][4];
+#pragma unroll
+                for (int i = 0; i < RM; i++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t p0 = and_or(d[j], mask, magic), p1 = and_or(d[j] >> 4, mask, magic);
+                    const uint32_t p2 = and_or(d[j] >> 8, mask, magic), p3 = and_or(d[j] >> 12, mask, magic);
+#pragma unroll
+                    for (int i = 0; i < RM; i++) {
+                        dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                        dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                        dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                        dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+                    }
+                }
+                // scale * (dot - B * sum x) + bias * sum x
+                const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
+                const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+                for (int i = 0; i < RM; i++) {
+                    const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+                    acc[r][i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[r][i]));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RN; r++)
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float v = wave_sum_lane63(acc[r][i]);
+            if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, v);
+        }
+}
+
+template <typename T, int RM, int RN, int WAVES>
+int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
+    const int64_t rows = (int64_t)WAVES * RN;
+    dim3 grid((unsigned)((a.n + rows - 1) / rows), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
+    if (a.batch == 1 && a.rhs == nullptr)
+        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, false>), grid, dim3(WAVES * 64), 0, s, a);
+    else
+        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, true>), grid, dim3(WAVES * 64), 0, s, a);
+    NVQ_LAUNCH_CHECK("qmv4_lds");
+    return NVQ_OK;
+}
+
+template <typename T, int BITS, bool FP4, int RM, int RN>
+int32_t run_generic(const ProductArgs &a, hipStream_t s) {
+    dim3 grid((unsigned)((a.n + kWaves * RN - 1) / (kWaves * RN)), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
+    hipLaunchKernelGGL((qmv_generic_kernel<T, BITS, FP4, RM, RN>), grid, dim3(kWaves * 64), 0, s, a);
+    NVQ_LAUNCH_CHECK("qmv");
+    return NVQ_OK;
+}
+
+template <typename T, int RM, int RN, int KU>
+int32_t run_pair4(const ProductArgs &a, hipStream_t s) {
+    dim3 grid((unsigned)((a.n + RN - 1) / RN), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
+    hipLaunchKernelGGL((qmv4_pair_kernel<T, RM, RN, KU>), grid, dim3(64), 0, s, a);
+    NVQ_LAUNCH_CHECK("qmv4_pair");
+    return NVQ_OK;
+}
+
+template <typename T>
+int32_t run_typed(const ProductArgs &a, hipStream_t s) {
+    if (a.mode == NVQ_MXFP4) return a.m == 1 ? run_generic<T, 4, true, 1, 4>(a, s) : run_generic<T, 4, true, 2, 4>(a, s);
+    if constexpr (!std::is_same<T, float>::value) {
+        if (a.bits == 4) {
+            if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
+            if (a.m == 2) return run_lds4<T, 2, 1, 8>(a, s);
+            return run_pair4<T, 4, 4, 1>(a, s);
+        }
+    }
+#define NVQ_GENERIC(B) (a.m == 1 ? run_generic<T, B, false, 1, 4>(a, s) : run_generic<T, B, false, 2, 4>(a, s))
+    switch (a.bits) {
+    case 1: return NVQ_GENERIC(1);
+    case 2: return NVQ_GENERIC(2);
+    case 3: return NVQ_GENERIC(3);
+    case 4: return NVQ_GENERIC(4);
+    case 5: return NVQ_GENERIC(5);
+    case 6: return NVQ_GENERIC(6);
+    case 8: return NVQ_GENERIC(8);
+    default: return fail(NVQ_INVALID_ARGUMENT, "quantized_matmul: %d bits are not supported", a.bits);
+    }
+#undef NVQ_GENERIC
+}
+
+}  // namespace
+
+int32_t launch_qmv(const ProductArgs &a, hipStream_t s) {
+    if (a.batch > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld batches exceed the grid limit", (long long)a.batch);
+    switch (a.dtype) {
+    case NVQ_F32: return run_typed<float>(a, s);
+    case NVQ_BF16: return run_typed<bf16_t>(a, s);
+    default: return run_typed<f16_t>(a, s);
+    }
+}
+
+}  // namespace nvq

@@ -1,0 +1,359 @@
+"""The public quantization ops with nuvec's (MLX-compatible) signatures, on torch device tensors.
+
+This is the host-side mirror of crates/nuvec-core/src/quantized.rs and ops.rs:965-1074:
+same names, argument meaning and refusals.  torch supplies device memory and the stream;
+every computation runs in libnuvec_hip.so through the C ABI.
+
+    q = quantize(w, Quant.affine(64, 4))          # Quantized(weight u32, scales, biases)
+    w2 = dequantize(q)                            # or q.dequantize(dtype)
+    y = quantized_matmul(x, q, transpose=True)    # x . dequantize(w)^T
+    y = gather_qmm(x, q, None, rhs, GatherQmm(sorted_indices=True))
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, replace
+from enum import IntEnum
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import InvalidArgument, Unsupported  # noqa: F401  (re-exported)
+
+
+class QuantMode(IntEnum):
+    """quantized.rs:22-35; `name` strings are MLX's."""
+    AFFINE = _lib.AFFINE
+    MXFP4 = _lib.MXFP4
+    MXFP8 = _lib.MXFP8
+    NVFP4 = _lib.NVFP4
+
+    @property
+    def mlx_name(self) -> str:
+        return self.name.lower()
+
+    @staticmethod
+    def parse(s: str) -> "QuantMode":
+        try:
+            return {"affine": QuantMode.AFFINE, "mxfp4": QuantMode.MXFP4, "mxfp8": QuantMode.MXFP8,
+                    "nvfp4": QuantMode.NVFP4}[s]
+        except KeyError:
+            raise InvalidArgument(f"invalid quantization mode '{s}' (affine, mxfp4, mxfp8 or nvfp4)") from None
+
+
+_DEFAULTS = {QuantMode.AFFINE: (64, 4), QuantMode.MXFP4: (32, 4), QuantMode.MXFP8: (32, 8), QuantMode.NVFP4: (16, 4)}
+
+
+@dataclass(frozen=True)
+class Quant:
+    """quantized.rs:93-168: a mode, a group size and a bit width."""
+    mode: QuantMode = QuantMode.AFFINE
+    group_size: int = 64
+    bits: int = 4
+
+    @staticmethod
+    def new(mode: QuantMode) -> "Quant":
+        g, b = _DEFAULTS[QuantMode(mode)]
+        return Quant(QuantMode(mode), g, b)
+
+    @staticmethod
+    def affine(group_size: int, bits: int) -> "Quant":
+        return Quant(QuantMode.AFFINE, group_size, bits)
+
+    def checked(self, op: str):
+        """Quant::checked: raises InvalidArgument with the reference's message."""
+        _lib.check(_lib.load().nvq_quant_check(C.byref(self._c()), op.encode()))
+        return self.group_size, self.bits
+
+    def _c(self) -> _lib.QuantC:
+        return _lib.QuantC(int(self.mode), int(self.group_size), int(self.bits))
+
+
+@dataclass
+class Quantized:
+    """quantized.rs:194-278: packed codes, scales, (affine) biases and how they were quantized."""
+    weight: torch.Tensor
+    scales: torch.Tensor
+    biases: Optional[torch.Tensor]
+    quant: Quant
+
+    @staticmethod
+    def affine(weight, scales, biases, group_size, bits) -> "Quantized":
+        return Quantized(weight, scales, biases, Quant.affine(group_size, bits))
+
+    @staticmethod
+    def fp(weight, scales, mode) -> "Quantized":
+        return Quantized(weight, scales, None, Quant.new(mode))
+
+    def dequantize(self, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return dequantize(self, dtype)
+
+
+@dataclass(frozen=True)
+class GatherQmm:
+    """quantized.rs:314-359."""
+    transpose: bool = True
+    sorted_indices: bool = False
+
+    @staticmethod
+    def groups(rows: int, experts: int, row_exact: bool = False) -> bool:
+        return bool(_lib.load().nvq_gather_grouped(rows, experts, int(row_exact)))
+
+
+_CODE = {torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float32: _lib.F32}
+_FLOATS = tuple(_CODE)
+
+
+def _init(t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise _lib.NoDevice("operands must live on the GPU: this backend has no CPU path")
+    _lib.check(_lib.load().nvq_init(t.device.index or 0))
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> C.c_void_p:
+    """The tensor's device address; NULL means "operand absent" in the C ABI, so an empty
+    tensor (torch gives it address 0) is passed as a never-dereferenced aligned non-null value."""
+    if t is None:
+        return C.c_void_p(None)
+    return C.c_void_p(t.data_ptr() or 16)
+
+
+def _u32(t: torch.Tensor) -> torch.Tensor:
+    return t.view(torch.uint32) if t.dtype == torch.int32 else t
+
+
+def _name(dtype) -> str:
+    return str(dtype).replace("torch.", "")
+
+
+def _check_groups(op: str, mode: QuantMode, scales: torch.Tensor, biases) -> None:
+    """quantized.rs:363-379."""
+    if mode == QuantMode.AFFINE:
+        if biases is None:
+            raise InvalidArgument(f"{op}: biases must be provided for affine quantization")
+    elif biases is not None:
+        raise InvalidArgument(f"{op}: biases must be null for quantization mode '{mode.mlx_name}'")
+    elif scales.dtype != torch.uint8:
+        raise InvalidArgument(f"{op}: scale type must be uint8 but received type {_name(scales.dtype)}")
+
+
+def _quantized_columns(op: str, w, scales, biases, quant: Quant) -> int:
+    """primitive.rs:1412-1460: values per packed row, after MLX's validate_quantized_input."""
+    group, bits = quant.checked(op)
+    w = _u32(w)
+    if w.dtype != torch.uint32:
+        raise InvalidArgument(f"{op}: packed weights must be uint32, got {_name(w.dtype)}")
+    if quant.mode == QuantMode.AFFINE:
+        if scales.dtype not in _FLOATS or biases.dtype != scales.dtype or biases.shape != scales.shape:
+            raise InvalidArgument(
+                f"{op}: scales and biases must share a float dtype and shape, got {_name(scales.dtype)} "
+                f"{list(scales.shape)} and {_name(biases.dtype)} {list(biases.shape)}")
+    elif scales.dtype != torch.uint8:
+        raise InvalidArgument(f"{op}: scale type must be uint8 but received type {_name(scales.dtype)}")
+    packed = (w.shape[-1] if w.ndim else 0) * 32
+    groups = (scales.shape[-1] if scales.ndim else 0) * group
+    if w.ndim < 2 or scales.ndim != w.ndim or w.shape[:-1] != scales.shape[:-1] or packed != groups * bits:
+        raise InvalidArgument(f"{op}: packed weights {list(w.shape)} and scales {list(scales.shape)} do not match "
+                              f"group size {group} and {bits} bits")
+    return groups
+
+
+def quantize(w: torch.Tensor, quant: Quant | QuantMode = Quant()) -> Quantized:
+    """ops.rs:965-1008, primitive.rs:1223-1259: quantizes the last axis of `w`."""
+    quant = Quant.new(quant) if isinstance(quant, QuantMode) else quant
+    group, bits = quant.checked("quantize")
+    if w.dtype not in _FLOATS:
+        raise InvalidArgument(f"quantize: unsupported dtype {_name(w.dtype)}")
+    if w.ndim < 2 or w.shape[-1] % group != 0:
+        raise InvalidArgument(f"quantize: needs at least 2 dimensions with the last divisible by the group size "
+                              f"{group}, got shape {list(w.shape)}")
+    _init(w)
+    w = w.contiguous()
+    last = w.shape[-1]
+    rows = w.numel() // last if last else 0
+    packed = torch.empty(w.shape[:-1] + (last * bits // 32,), dtype=torch.uint32, device=w.device)
+    affine = quant.mode == QuantMode.AFFINE
+    scales = torch.empty(w.shape[:-1] + (last // group,), dtype=w.dtype if affine else torch.uint8, device=w.device)
+    biases = torch.empty_like(scales) if affine else None
+    _lib.check(_lib.load().nvq_quantize(C.byref(quant._c()), _CODE[w.dtype], _ptr(w), rows, last, _ptr(packed),
+                                        _ptr(scales), _ptr(biases), _stream()))
+    return Quantized(packed, scales, biases, quant)
+
+
+def dequantize(q: Quantized, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """ops.rs:1014-1027, quantized.rs:401-444: affine computes in the scales' dtype, then casts;
+    the floating-point modes default to bfloat16."""
+    quant = q.quant
+    quant.checked("dequantize")
+    _check_groups("dequantize", quant.mode, q.scales, q.biases)
+    if dtype is not None and not dtype.is_floating_point:
+        raise InvalidArgument(f"dequantize: only real floating types are supported but the output dtype is {_name(dtype)}")
+    affine = quant.mode == QuantMode.AFFINE
+    cols = _quantized_columns("dequantize", q.weight, q.scales, q.biases, quant)
+    compute = q.scales.dtype if affine else (dtype or torch.bfloat16)
+    if compute not in _FLOATS:
+        raise InvalidArgument(f"dequantize: unsupported dtype {_name(compute)}")
+    _init(q.weight)
+    w, s = _u32(q.weight).contiguous(), q.scales.contiguous()
+    b = q.biases.contiguous() if affine else None
+    out = torch.empty(w.shape[:-1] + (cols,), dtype=compute, device=w.device)
+    rows = out.numel() // cols if cols else 0
+    _lib.check(_lib.load().nvq_dequantize(C.byref(quant._c()), _CODE[compute], _ptr(w), _ptr(s), _ptr(b), rows, cols,
+                                          _ptr(out), _stream()))
+    if affine and dtype is not None and dtype != out.dtype:
+        out = out.to(dtype)
+    return out
+
+
+def _promoted(op: str, x, scales, biases) -> torch.dtype:
+    """quantized.rs:491-497: affine promotes x, scales and biases; fp modes keep x's dtype."""
+    dtype = x.dtype
+    if biases is not None:
+        dtype = torch.promote_types(torch.promote_types(x.dtype, scales.dtype), biases.dtype)
+    if dtype not in _FLOATS:
+        raise InvalidArgument(f"{op}: unsupported dtype {_name(dtype)}")
+    return dtype
+
+
+def _strides(t: torch.Tensor, nbatch: int):
+    return [int(t.stride(i)) for i in range(nbatch)]
+
+
+def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, row_exact: bool = False) -> torch.Tensor:
+    """ops.rs:1031-1045, quantized.rs:446-537, primitive.rs:1279-1320."""
+    op = "quantized_matmul"
+    quant = q.quant
+    group, bits = quant.checked(op)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    affine = quant.mode == QuantMode.AFFINE
+    dtype = _promoted(op, x, q.scales, q.biases)
+    x = x.to(dtype)
+    w = _u32(q.weight)
+    scales = q.scales.to(dtype) if affine else q.scales
+    biases = q.biases.to(dtype) if affine else None
+    vector = x.ndim == 1
+    if vector:
+        x = x.unsqueeze(0)
+    columns = _quantized_columns(op, w, scales, biases, quant)
+    rows = w.shape[-2]
+    inner, outer = (columns, rows) if transpose else (rows, columns)
+    # Dense last two dimensions for every operand; batch dimensions broadcast by stride 0.
+    x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
+    biases = biases.contiguous() if affine else None
+    if w.ndim > 2 and x.ndim >= 2:
+        try:
+            batch = torch.broadcast_shapes(x.shape[:-2], w.shape[:-2])
+        except RuntimeError:
+            raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not broadcast") from None
+        full = lambda a: a.expand(batch + a.shape[-2:])
+        x, w, scales = full(x), full(w), full(scales)
+        biases = full(biases) if affine else None
+    xn, wn = x.ndim, w.ndim
+    batch_ok = wn == 2 or (xn == wn and x.shape[:-2] == w.shape[:-2])
+    if xn == 0 or x.shape[-1] != inner or not batch_ok:
+        raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not match")
+    _init(x)
+    out = torch.empty(x.shape[:-1] + (outer,), dtype=dtype, device=x.device)
+    d = _lib.QmmDescC()
+    d.quant, d.dtype, d.transpose, d.row_exact, d.rows = quant._c(), _CODE[dtype], int(transpose), int(row_exact), 0
+    d.n, d.k = outer, inner
+    if wn == 2:  # the reference's "flat" rule: every leading row of x is a row of one product
+        d.m = 1
+        for dim in x.shape[:-1]:
+            d.m *= dim
+        d.item_rows = x.shape[-2]
+        d.batch_ndim = 0
+    else:
+        d.m = d.item_rows = x.shape[-2]
+        nb = xn - 2
+        if nb > _lib.MAX_BATCH_DIMS:
+            raise Unsupported(f"{op}: {nb} batch dimensions")
+        d.batch_ndim = nb
+        for i in range(nb):
+            d.batch_shape[i] = x.shape[i]
+            d.x_strides[i], d.w_strides[i], d.s_strides[i] = x.stride(i), w.stride(i), scales.stride(i)
+    lib = _lib.load()
+    need = lib.nvq_quantized_matmul_workspace_bytes(C.byref(d))
+    workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    _lib.check(lib.nvq_quantized_matmul(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
+                                        _ptr(workspace), _stream()))
+    return out.squeeze(-2) if vector else out
+
+
+def sorted_offsets(rhs: torch.Tensor, groups: int) -> torch.Tensor:
+    """kernels.rs:873-892: per row of the last axis, where each group's indices start."""
+    _init(rhs)
+    rhs = rhs.contiguous()
+    m = rhs.shape[-1]
+    rows = rhs.numel() // m if m else 0
+    out = torch.empty(rhs.shape[:-1] + (groups,), dtype=torch.int32, device=rhs.device)
+    _lib.check(_lib.load().nvq_sorted_offsets(_ptr(rhs), rows, m, groups, _ptr(out), _stream()))
+    return out
+
+
+def _indices(op: str, a: torch.Tensor, given: Optional[torch.Tensor]) -> torch.Tensor:
+    """quantized.rs:739-767: integer indices as uint32 (carried as int32 bit patterns)."""
+    batch = a.shape[:-2]
+    if given is None:
+        n = 1
+        for s in batch:
+            n *= s
+        return torch.arange(n, dtype=torch.int32, device=a.device).reshape(batch)
+    if given.dtype.is_floating_point or given.dtype == torch.bool:
+        raise InvalidArgument(f"{op}: indices must be integers")
+    return given.to(device=a.device).to(torch.int32) if given.dtype != torch.uint32 else given.view(torch.int32)
+
+
+def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor] = None,
+               rhs_indices: Optional[torch.Tensor] = None, options: GatherQmm = GatherQmm(), *,
+               row_exact: bool = False) -> torch.Tensor:
+    """ops.rs:1050-1074, quantized.rs:589-673: output batch i = x[lhs[i]] . dequantize(w)[rhs[i]]^T."""
+    op = "gather_qmm"
+    quant = q.quant
+    quant.checked(op)
+    if lhs_indices is None and rhs_indices is None:
+        return quantized_matmul(x, q, options.transpose, row_exact=row_exact)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    affine = quant.mode == QuantMode.AFFINE
+    dtype = _promoted(op, x, q.scales, q.biases)
+    w = _u32(q.weight)
+    if x.ndim < 2 or w.ndim < 2 or (q.biases is not None and q.scales.shape != q.biases.shape):
+        raise InvalidArgument(f"{op}: x must be [..., M, K] and w [..., N, K'], got {list(x.shape)} and {list(w.shape)}")
+    x = x.to(dtype).contiguous()
+    scales = (q.scales.to(dtype) if affine else q.scales).contiguous()
+    biases = q.biases.to(dtype).contiguous() if affine else None
+    w = w.contiguous()
+    columns = _quantized_columns(op, w, scales, biases, quant)
+    rows = w.shape[-2]
+    inner, outer = (columns, rows) if options.transpose else (rows, columns)
+    if x.shape[-1] != inner:
+        raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not match")
+    lhs, rhs = _indices(op, x, lhs_indices), _indices(op, w, rhs_indices)
+    try:
+        lhs, rhs = torch.broadcast_tensors(lhs, rhs)
+    except RuntimeError:
+        raise InvalidArgument(f"{op}: index shapes {list(lhs.shape)} and {list(rhs.shape)} do not broadcast") from None
+    lhs, rhs = lhs.contiguous(), rhs.contiguous()
+    _init(x)
+    m = x.shape[-2]
+    x_batches = x.numel() // (m * inner) if m * inner else 0
+    experts = 1
+    for s in w.shape[:-2]:
+        experts *= s
+    is_sorted = lhs_indices is None and options.sorted_indices and GatherQmm.groups(rhs.numel(), experts, row_exact)
+    offsets = None
+    if is_sorted and m == 1 and x.ndim == 3 and rhs.ndim == 1:  # quantized.rs:772-782
+        offsets = sorted_offsets(rhs, experts)
+    out = torch.empty(tuple(rhs.shape) + (m, outer), dtype=dtype, device=x.device)
+    d = _lib.GatherDescC(quant._c(), _CODE[dtype], int(options.transpose), m, outer, inner, rhs.numel(), x_batches, experts)
+    lib = _lib.load()
+    need = lib.nvq_gather_qmm_workspace_bytes(C.byref(d))
+    workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    _lib.check(lib.nvq_gather_qmm(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs),
+                                  _ptr(offsets), _ptr(out), _ptr(workspace), _stream()))
+    return out

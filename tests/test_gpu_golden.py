@@ -1,0 +1,100 @@
+"""Replays the reference's golden vectors on the MI355X through the C ABI.
+
+Criteria as the reference applies them to its own device backend (tests/mlx.rs:55-147):
+quantize and the MXFP4 codecs bit for bit; affine dequantize exact against MLX's CPU vectors
+(the backend keeps the CPU's two roundings); products and gathers within FR-008's bound
+against MLX's device outputs and within the CPU-fixture bound against MLX's CPU outputs.
+"""
+import numpy as np
+import pytest
+
+from oracle import ref
+from tests import replay
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from tests.hip_backend import HipBackend
+    return HipBackend()
+
+
+def _supported(c):
+    """transpose=0 (x . w) and bits the first kernels do not cover are refused by the backend."""
+    return c.params.get("transpose", "1") == "1"
+
+
+def _failures(cases, check):
+    out = []
+    for c in cases:
+        msg = check(c)
+        if msg:
+            out.append(f"{c.name}: {msg}")
+    return out
+
+
+def test_affine_quantize_bits(hip, golden_cpu):
+    cases = [c for c in golden_cpu[1] if c.op == "quantize"]
+    assert len(cases) == 70
+    assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+
+
+def test_affine_dequantize_bits(hip, golden_cpu):
+    cases = [c for c in golden_cpu[1] if c.op == "dequantize"]
+    assert len(cases) == 21
+    assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+
+
+def test_affine_dequantize_equals_oracle_on_device_vectors(hip, golden_gpu):
+    """The 54 device-recorded inputs: the backend equals the CPU oracle bit for bit."""
+    cases = [c for c in golden_gpu[1] if c.name.startswith("affine-dequantize-")]
+    oracle = replay.OracleBackend()
+
+    def check(c):
+        want = replay.run_case(c, oracle)
+        got = replay.run_case(c, hip)
+        same = np.array_equal(got[0][0].view(np.uint8), want[0][0].view(np.uint8))
+        return None if same and got[0][1] == want[0][1] else "differs from the CPU oracle"
+
+    assert len(cases) == 54
+    assert not _failures(cases, check)
+
+
+def test_mxfp4_quantize_bits(hip, golden_gpu):
+    cases = [c for c in golden_gpu[1] if c.op == "quantize"]
+    assert len(cases) == 18
+    assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+
+
+def test_mxfp4_dequantize_bits(hip, golden_gpu):
+    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == "mxfp4"]
+    assert len(cases) == 15
+    assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+
+
+def test_products_against_mlx_cpu(hip, golden_cpu):
+    cases = [c for c in golden_cpu[1] if c.op == "quantized_matmul" and _supported(c)]
+    assert len(cases) >= 20
+    assert not _failures(cases, lambda c: replay.by_value(replay.run_case(c, hip), c.outputs, replay.product_bound(c)))
+
+
+def test_products_against_mlx_gpu(hip, golden_gpu):
+    cases = [c for c in golden_gpu[1] if c.op == "quantized_matmul" and _supported(c)]
+    assert len(cases) >= 40
+    assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
+
+
+def test_gathers_against_mlx_gpu(hip, golden_gpu):
+    cases = [c for c in golden_gpu[1] if c.op == "gather_qmm" and _supported(c)]
+    assert len(cases) >= 12
+    assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
+
+
+def test_untransposed_products_are_refused_not_faked(hip, golden_cpu):
+    """x . w has no gfx950 kernel yet: the backend must say so (the caller then takes its CPU
+    path) instead of answering from anywhere else."""
+    import nuvec_amd as nv
+    case = next(c for c in golden_cpu[1] if c.name == "qmm-n")
+    with pytest.raises(nv.Unsupported):
+        replay.run_case(case, hip)

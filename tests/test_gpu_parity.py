@@ -1,0 +1,157 @@
+"""HIP path against the CPU oracle on the same seeded inputs (the BASELINE configurations).
+
+Bars: packed words, scales and biases bit-exact; dequantize bit-exact; product outputs within
+1e-2 * max|row| for bfloat16, 1e-3 * max|row| for float16 and 1e-4 * max|row| for float32
+(float32 accumulation), `row` being the oracle's output row.
+"""
+import numpy as np
+import pytest
+import torch
+
+import nuvec_amd as nv
+from oracle import ref
+from tests.hip_backend import TORCH, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+TOL = {ref.BF16: 1e-2, ref.F16: 1e-3, ref.F32: 1e-4}
+
+
+def make_w(rng, n, k, dtype):
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    return ref.from_f32(w, dtype)
+
+
+def make_x(rng, m, k, dtype):
+    return ref.from_f32(rng.standard_normal((m, k)).astype(np.float32), dtype)
+
+
+def assert_rows_close(got, want, dtype, what):
+    g, w = ref.to_f32(got, dtype).astype(np.float64), ref.to_f32(want, dtype).astype(np.float64)
+    g, w = g.reshape(-1, g.shape[-1]), w.reshape(-1, w.shape[-1])
+    bound = TOL[dtype] * np.max(np.abs(w), axis=1, keepdims=True)
+    err = np.abs(g - w)
+    worst = float(np.max(err / np.maximum(bound, 1e-30)))
+    assert np.all(err <= bound), f"{what}: max error is {worst:.3f} x the bound"
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(64, 4), (64, 3), (32, 8), (128, 2), (32, 6), (64, 5), (128, 1)])
+def test_affine_quantize_dequantize_bit_exact(dtype, group, bits):
+    rng = np.random.default_rng(1000 + bits * 7 + group)
+    w = make_w(rng, 96, 1024, dtype)
+    w.reshape(-1)[::97] = ref.from_f32(np.zeros(1, np.float32), dtype)[0]  # exact zeros among the values
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(group, bits))
+    assert np.array_equal(to_host(q.weight), packed)
+    assert np.array_equal(to_host(q.scales).view(np.uint8), scales.view(np.uint8))
+    assert np.array_equal(to_host(q.biases).view(np.uint8), biases.view(np.uint8))
+    want = ref.affine_dequantize(packed, scales, biases, dtype, group, bits)
+    got = to_host(nv.dequantize(q))
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_config1_fp32_4bit_g64():
+    """BASELINE config 1: W f32 [4096,4096] ~ N(0,0.02), x f32 [1,4096], 4-bit g64."""
+    rng = np.random.default_rng(20260101)
+    w, x = make_w(rng, 4096, 4096, ref.F32), make_x(rng, 1, 4096, ref.F32)
+    packed, scales, biases = ref.affine_quantize(w, ref.F32, 64, 4)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(64, 4))
+    assert np.array_equal(to_host(q.weight), packed)
+    assert np.array_equal(to_host(q.scales), scales) and np.array_equal(to_host(q.biases), biases)
+    want_dense = ref.affine_dequantize(packed, scales, biases, ref.F32, 64, 4)
+    assert np.array_equal(to_host(nv.dequantize(q)), want_dense)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.F32, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert got.shape == (1, 4096)
+    assert_rows_close(got, want, ref.F32, "config 1")
+
+
+@pytest.mark.parametrize("m", [1, 4, 8])
+def test_config2_decode_bf16_4bit_g64(m):
+    """BASELINE config 2: W [14336,4096] bf16 scales/biases, x bf16 [M,4096]."""
+    rng = np.random.default_rng(20260102)
+    w, x = make_w(rng, 14336, 4096, ref.BF16), make_x(rng, m, 4096, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(64, 4))
+    assert np.array_equal(to_host(q.weight), packed)
+    assert np.array_equal(to_host(q.scales), scales) and np.array_equal(to_host(q.biases), biases)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, ref.BF16, f"config 2, M={m}")
+
+
+@pytest.mark.parametrize("group,bits", [(64, 3), (32, 8)])
+@pytest.mark.parametrize("m", [1, 16])
+def test_config4_odd_bit_widths(group, bits, m):
+    """BASELINE config 4: 3-bit g64 (codes cross word boundaries) and 8-bit g32, W [4096,4096]."""
+    rng = np.random.default_rng(20260104 + bits)
+    w, x = make_w(rng, 4096, 4096, ref.BF16), make_x(rng, m, 4096, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, group, bits)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(group, bits))
+    assert np.array_equal(to_host(q.weight), packed)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=ref.BF16, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, ref.BF16, f"config 4 b{bits} g{group} M={m}")
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(64, 4), (32, 2), (128, 6), (64, 5), (128, 1), (32, 3), (64, 8)])
+def test_ragged_shapes_every_width(dtype, group, bits):
+    """N not a multiple of the rows per block, K not a multiple of the wavefront step, M = 3."""
+    rng = np.random.default_rng(7 + bits)
+    n, k, m = 77, 2 * 2048 + 3 * group, 3
+    w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, dtype, f"ragged b{bits} g{group}")
+
+
+def test_mxfp4_quantize_and_products():
+    rng = np.random.default_rng(5)
+    n, k = 360, 2880
+    w = make_w(rng, n, k, ref.BF16)
+    packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+    q = nv.quantize(to_dev(w), nv.QuantMode.MXFP4)
+    assert np.array_equal(to_host(q.weight), packed) and np.array_equal(to_host(q.scales), scales)
+    for out in (ref.BF16, ref.F32, ref.F16):
+        want = ref.fp_dequantize(packed, scales, ref.MXFP4, out)
+        assert np.array_equal(to_host(nv.dequantize(q, TORCH[out])).view(np.uint8), want.view(np.uint8))
+    for m in (1, 5):
+        x = make_x(rng, m, k, ref.BF16)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, ref.BF16, f"mxfp4 M={m}")
+
+
+def test_empty_and_degenerate_products():
+    dev = torch.device("cuda")
+    q = nv.Quantized(torch.zeros((8, 16), dtype=torch.uint32, device=dev), torch.ones((8, 2), device=dev),
+                     torch.zeros((8, 2), device=dev), nv.Quant.affine(64, 4))
+    y = nv.quantized_matmul(torch.zeros((0, 128), device=dev), q)
+    assert y.shape == (0, 8)
+    q0 = nv.Quantized(torch.zeros((8, 0), dtype=torch.uint32, device=dev), torch.ones((8, 0), device=dev),
+                      torch.zeros((8, 0), device=dev), nv.Quant.affine(64, 4))
+    y = nv.quantized_matmul(torch.ones((3, 0), device=dev), q0)
+    assert y.shape == (3, 8) and float(y.abs().sum()) == 0.0
+
+
+def test_sorted_offsets_and_gather_pairs():
+    rng = np.random.default_rng(11)
+    experts, n, k, rows = 8, 64, 512, 40
+    w = make_w(rng, experts * n, k, ref.BF16).reshape(experts, n, k)
+    packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+    rhs = np.sort(rng.integers(0, experts, rows)).astype(np.uint32)
+    x = make_x(rng, rows, k, ref.BF16).reshape(rows, 1, k)
+    off = to_host(nv.sorted_offsets(torch.from_numpy(rhs.astype(np.int32)).cuda(), experts))
+    assert np.array_equal(off, ref.sorted_offsets(rhs, experts))
+    assert np.array_equal(off, np.searchsorted(rhs, np.arange(experts), side="left").astype(np.int32))
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(nv.QuantMode.MXFP4))
+    got = to_host(nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs.astype(np.int64)).cuda(),
+                                nv.GatherQmm(sorted_indices=True)))
+    want = ref.gather_qmm(x, packed, scales, None, np.arange(rows, dtype=np.uint32), rhs, mode=ref.MXFP4, group=32,
+                          bits=4, dtype=ref.BF16)
+    assert got.shape == (rows, 1, n)
+    assert_rows_close(got, want, ref.BF16, "sorted gather")
