@@ -283,6 +283,9 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
         a.w_strides[i] = d->w_strides[i];
         a.s_strides[i] = d->s_strides[i];
     }
+    // Routed by one item's rows, as the reference does (gpu.rs:6975-6981).
+    const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
+    if (item >= kQmmMinRows && qmm_supported(a)) return launch_qmm(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }
 

@@ -62,6 +62,13 @@ struct ProductArgs {
     int64_t x_batches, experts;     // gather: index bounds (an index beyond them is clamped)
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
+// The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
+bool qmm_supported(const ProductArgs &a);
+int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
+// Rows of x from which a product goes to the tiled kernel rather than the few-row kernels
+// (the counterpart of the reference's device-specific `qmv_batch_limit`,
+// crates/nuvec-core/src/gpu.rs:1506-1538).
+constexpr int64_t kQmmMinRows = 12;
 int32_t launch_fill_zero(void *p, int64_t bytes, hipStream_t s);
 
 }  // namespace nvq
