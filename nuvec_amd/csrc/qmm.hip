@@ -4,17 +4,21 @@
 // device kernels the weight tile is dequantized into on-chip memory in the element type and the
 // products accumulate in float32 (crates/nuvec-kernels/src/metal/quantized.h:583-817, 1358-1485).
 //
-// One block of 256 threads (four wavefronts, 2 x 2) owns a BM x BN = 256 x 256 tile of y and walks K in
-// steps of BK = 64.  Per step and block:
+// One block of 512 threads (eight wavefronts, 2 x 4, each 128 x 64 of y) owns a BM x BN = 256 x 256 tile
+// and walks K in steps of BK = 64.  Per step and block:
 //   * x tile   256 x 64 elements (32 KB): copied global -> registers -> LDS, 16 bytes per access;
-//   * w tile   256 rows x 32 packed bytes: thread t owns row t, i.e. exactly one quantization group
-//              of 64 values (or two of 32): 64 codes -> float (v_cvt_f32_ubyte) -> fma(code, scale,
-//              bias) -> packed element type -> 128 B of LDS;
-//   * 64 MFMA 32x32x16 per wavefront (4 x 4 accumulator tiles of 32 x 32, 256 accumulator registers).
+//   * w tile   256 rows x 32 packed bytes: thread t owns half a row (32 codes, inside one quantization
+//              group): codes -> float (v_cvt_f32_ubyte) -> fma(code, scale, bias) -> packed element type
+//              -> 64 B of LDS;
+//   * 32 MFMA 32x32x16 per wavefront (4 x 2 accumulator tiles of 32 x 32, 128 accumulator registers).
 // LDS rows are 128 B (64 elements) with the 16-byte chunk index XOR-ed with (row & 7), which makes the
-// 16-byte fragment reads of the matrix instruction and the tile writes bank-conflict free.  Two LDS
-// stages: the loads of step i+1 are issued before the matrix work of step i and their LDS writes
-// follow it; one barrier per step.
+// 16-byte fragment reads of the matrix instruction and the tile writes bank-conflict free.
+//
+// Overlap.  Each SIMD holds two wavefronts of the block.  LDS tiles are double-buffered and there is
+// one barrier per step; inside a step wavefronts 0-3 first dequantize step s+1 into the other buffer
+// and then run the matrix instructions of step s, while wavefronts 4-7 do the two phases in the
+// opposite order.  So on every SIMD one wavefront issues matrix instructions while the other issues
+// the conversion arithmetic, and the two pipes work at the same time.
 #include "nvq_device.h"
 #include "nvq_internal.h"
 
@@ -29,7 +33,7 @@ typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
 constexpr int kRowBytes = BK * 2;                       // 128 B per LDS row
 constexpr int kTileBytes = (BM + BN) * kRowBytes;       // one stage: x tile then w tile
 constexpr int kLdsBytes = 2 * kTileBytes;               // 128 KB
@@ -74,107 +78,112 @@ __device__ __forceinline__ uint4 dequant8(uint32_t word, float s, float b) {
 }
 
 template <typename T, bool BATCHED>
-__global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a, const int64_t xo, const int64_t wo, const int64_t so, const int64_t yo) {
+__global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // wavefront grid 2 x 2: 128 x 128 each
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = (wave >> 2) & 1, wn = wave & 3;  // wavefront grid 2 x 4: 128 x 64 each
+    const bool convert_first = wave < 4;            // the two wavefronts of a SIMD run the phases in opposite order
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = a.group == 32 ? 5 : a.group == 64 ? 6 : 7;
     const int kwords = K >> 3, kgroups = K >> gshift;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    int64_t bx = xo, bw = wo, bs = so, by = yo;
-    if constexpr (BATCHED) {
-        // batch z of a strided batch: offsets are multiples of the per-batch strides
-        bx += (int64_t)blockIdx.z * a.x_strides[0];
-        bw += (int64_t)blockIdx.z * a.w_strides[0];
-        bs += (int64_t)blockIdx.z * a.s_strides[0];
-        by += (int64_t)blockIdx.z * M * N;
+    int64_t bx = 0, bw = 0, bs = 0, by = 0;
+    if constexpr (BATCHED) {  // a batch with one stride per operand
+        bx = (int64_t)blockIdx.z * a.x_strides[0];
+        bw = (int64_t)blockIdx.z * a.w_strides[0];
+        bs = (int64_t)blockIdx.z * a.s_strides[0];
+        by = (int64_t)blockIdx.z * M * N;
     }
     const T *x = (const T *)a.x + bx;
     const uint32_t *w = (const uint32_t *)a.w + bw;
     const T *scales = (const T *)a.scales + bs, *biases = (const T *)a.biases + bs;
     T *y = (T *)a.y + by;
 
-    // Global-load assignment.  x: 8 chunks per row; thread t copies chunk t%8 of rows t/8 + 32 i.
+    // Global-load assignment.  x: 8 chunks of 16 B per row; thread t copies chunk t%8 of rows t/8 + 64 i.
     const int xc = tid & 7, xr = tid >> 3;
-    const T *xrow[8];
+    const T *xrow[4];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int row = m0 + xr + 32 * i;
+    for (int i = 0; i < 4; i++) {
+        const int row = m0 + xr + 64 * i;
         xrow[i] = x + (int64_t)(row < M ? row : M - 1) * K + xc * 8;  // tail rows are computed, not stored
     }
-    // w: thread t owns row t of the tile.
-    const int wrow = n0 + tid < N ? n0 + tid : N - 1;
+    // w: thread t owns half h = t%2 (32 codes = 16 packed bytes) of tile row t/2.
+    const int wr = tid >> 1, wh = tid & 1;
+    const int wrow = n0 + wr < N ? n0 + wr : N - 1;
     const uint32_t *wp = w + (int64_t)wrow * kwords;
     const T *sp = scales + (int64_t)wrow * kgroups, *bp = biases + (int64_t)wrow * kgroups;
 
-    floatx16_t acc[4][4];
+    floatx16_t acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    uint4 xg[8], wg[2];
-    float sc[2], bi[2];
+    uint4 xg[4], wg;
+    float sc, bi;
     auto load_step = [&](int k0) {
         const bool xlive = k0 + xc * 8 < K;  // K is a multiple of 32: a chunk of 8 is whole or absent
 #pragma unroll
-        for (int i = 0; i < 8; i++) xg[i] = xlive ? *reinterpret_cast<const uint4 *>(xrow[i] + k0) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int kh = k0 + 32 * h < K ? k0 + 32 * h : K - 32;  // an absent half reads valid data; its x is zero
-            wg[h] = *reinterpret_cast<const uint4 *>(wp + (kh >> 3));
-            sc[h] = Elem<T>::load(sp, kh >> gshift);
-            bi[h] = Elem<T>::load(bp, kh >> gshift);
-        }
+        for (int i = 0; i < 4; i++) xg[i] = xlive ? *reinterpret_cast<const uint4 *>(xrow[i] + k0) : make_uint4(0, 0, 0, 0);
+        const int kh = k0 + 32 * wh < K ? k0 + 32 * wh : K - 32;  // an absent half reads valid data; its x is zero
+        wg = *reinterpret_cast<const uint4 *>(wp + (kh >> 3));
+        sc = Elem<T>::load(sp, kh >> gshift);
+        bi = Elem<T>::load(bp, kh >> gshift);
     };
     auto store_step = [&](int stage) {
         unsigned char *xs = lds + stage * kTileBytes, *ws = xs + BM * kRowBytes;
 #pragma unroll
-        for (int i = 0; i < 8; i++) *reinterpret_cast<uint4 *>(xs + lds_offset(xr + 32 * i, xc)) = xg[i];
+        for (int i = 0; i < 4; i++) *reinterpret_cast<uint4 *>(xs + lds_offset(xr + 64 * i, xc)) = xg[i];
+        const uint32_t d[4] = {wg.x, wg.y, wg.z, wg.w};
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const uint32_t d[4] = {wg[h].x, wg[h].y, wg[h].z, wg[h].w};
+        for (int j = 0; j < 4; j++) *reinterpret_cast<uint4 *>(ws + lds_offset(wr, 4 * wh + j)) = dequant8<T>(d[j], sc, bi);
+    };
+    auto mma_step = [&](int stage) {
+        const unsigned char *xs = lds + stage * kTileBytes, *ws = xs + BM * kRowBytes;
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                *reinterpret_cast<uint4 *>(ws + lds_offset(tid, 4 * h + j)) = dequant8<T>(d[j], sc[h], bi[h]);
+        for (int kk = 0; kk < BK / 16; kk++) {
+            uint4 af[4], bf[2];
+            const int chunk = 2 * kk + (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + (lane & 31), chunk));
+#pragma unroll
+            for (int j = 0; j < 2; j++) bf[j] = *reinterpret_cast<const uint4 *>(ws + lds_offset(wn * 64 + j * 32 + (lane & 31), chunk));
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = Mma<T>::mfma(af[i], bf[j], acc[i][j]);
         }
     };
 
     const int steps = (K + BK - 1) / BK;
     load_step(0);
     store_step(0);
+    if (steps > 1) load_step(BK);  // the registers now hold step 1
     __syncthreads();
-    for (int step = 0; step < steps; step++) {
-        const int stage = step & 1;
-        const bool more = step + 1 < steps;
-        if (more) load_step((step + 1) * BK);
-        const unsigned char *xs = lds + stage * kTileBytes, *ws = xs + BM * kRowBytes;
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
-            uint4 af[4], bf[4];
-            const int chunk = 2 * kk + (lane >> 5);
-#pragma unroll
-            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + (lane & 31), chunk));
-#pragma unroll
-            for (int j = 0; j < 4; j++) bf[j] = *reinterpret_cast<const uint4 *>(ws + lds_offset(wn * 128 + j * 32 + (lane & 31), chunk));
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = Mma<T>::mfma(af[i], bf[j], acc[i][j]);
+    // Two half-steps per step, a barrier after the second.  In step s every wavefront converts step
+    // s+1 into the other LDS stage and multiplies step s, in the order its group prescribes; one copy
+    // of each phase's code serves both groups.
+    for (int half = 0; half < 2 * steps; half++) {
+        const int step = half >> 1, stage = step & 1;
+        const bool convert = ((half & 1) == 0) == convert_first;
+        if (convert) {
+            if (step + 1 < steps) store_step(stage ^ 1);
+            if (step + 2 < steps) load_step((step + 2) * BK);
+        } else {
+            mma_step(stage);
         }
-        if (more) store_step(stage ^ 1);
-        __syncthreads();
+        if (half & 1) __syncthreads();
     }
 
     // Epilogue: accumulator element e of a 32 x 32 tile is row 8 (e / 4) + 4 (lane / 32) + e % 4, column lane % 32.
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+        for (int j = 0; j < 2; j++) {
+            const int col = n0 + wn * 64 + j * 32 + (lane & 31);
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int row = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
@@ -193,7 +202,7 @@ int32_t run_qmm4(const ProductArgs &a, hipStream_t s) {
         configured[batched] = true;
     }
     dim3 grid((unsigned)((a.n + BN - 1) / BN), (unsigned)((a.m + BM - 1) / BM), (unsigned)a.batch);
-    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes, s, a, (int64_t)0, (int64_t)0, (int64_t)0, (int64_t)0);
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), kLdsBytes, s, a);
     NVQ_LAUNCH_CHECK("qmm4");
     return NVQ_OK;
 }
