@@ -24,7 +24,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-gpu-flush-denormals-to-zero",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-fvisibility=hidden",
+    "-Wall", "-Wno-unused-function", "-Wno-inline-asm", "-fvisibility=hidden",
     f"-I{INCLUDE}", f"-I{CSRC}",
 ]
 
