@@ -70,19 +70,27 @@ template <> struct Mma<f16_t> {
 // Byte offset of 16-byte chunk `chunk` (0..7) of LDS row `row`.
 __device__ __forceinline__ int lds_offset(int row, int chunk) { return row * kRowBytes + ((chunk ^ (row & 7)) << 4); }
 
+// Byte `B` of `v` as float: one instruction (the compiler otherwise extracts the byte first).
+template <int B>
+__device__ __forceinline__ float ubyte_to_float(uint32_t v) {
+    float f;
+    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+
 // Eight 4-bit codes of `word` (value i in bits 4i..4i+3) as fma(code, s, b), packed to the element
 // type in stream order.
 template <typename T>
 __device__ __forceinline__ uint4 dequant8(uint32_t word, float s, float b) {
     const uint32_t even = word & 0x0F0F0F0Fu, odd = (word >> 4) & 0x0F0F0F0Fu;  // codes 0,2,4,6 and 1,3,5,7
-    float e[4], o[4];
-    e[0] = (float)(even & 0xFFu); e[1] = (float)((even >> 8) & 0xFFu); e[2] = (float)((even >> 16) & 0xFFu); e[3] = (float)(even >> 24);
-    o[0] = (float)(odd & 0xFFu);  o[1] = (float)((odd >> 8) & 0xFFu);  o[2] = (float)((odd >> 16) & 0xFFu);  o[3] = (float)(odd >> 24);
     uint4 r;
-    r.x = Mma<T>::pack(__builtin_fmaf(e[0], s, b), __builtin_fmaf(o[0], s, b));
-    r.y = Mma<T>::pack(__builtin_fmaf(e[1], s, b), __builtin_fmaf(o[1], s, b));
-    r.z = Mma<T>::pack(__builtin_fmaf(e[2], s, b), __builtin_fmaf(o[2], s, b));
-    r.w = Mma<T>::pack(__builtin_fmaf(e[3], s, b), __builtin_fmaf(o[3], s, b));
+    r.x = Mma<T>::pack(__builtin_fmaf(ubyte_to_float<0>(even), s, b), __builtin_fmaf(ubyte_to_float<0>(odd), s, b));
+    r.y = Mma<T>::pack(__builtin_fmaf(ubyte_to_float<1>(even), s, b), __builtin_fmaf(ubyte_to_float<1>(odd), s, b));
+    r.z = Mma<T>::pack(__builtin_fmaf(ubyte_to_float<2>(even), s, b), __builtin_fmaf(ubyte_to_float<2>(odd), s, b));
+    r.w = Mma<T>::pack(__builtin_fmaf(ubyte_to_float<3>(even), s, b), __builtin_fmaf(ubyte_to_float<3>(odd), s, b));
     return r;
 }
 
@@ -137,12 +145,16 @@ __global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
     const int wrow = n0 + (wslot >> 1) < N ? n0 + (wslot >> 1) : N - 1;
     const uint32_t *wsrc = w + (int64_t)wrow * kwords + (wslot & 1) * 4;
     const int steps = K / BK;  // K is a multiple of 64 (checked on the host)
-    auto issue = [&](int step) {
+    // Load `part` (0..3: x, 4: w) of `step`; five parts per step and lane.
+    auto issue_part = [&](int step, int part) {
         const int k0 = (step < steps ? step : steps - 1) * BK;  // past the end: a harmless reload, keeps the wait counts uniform
         const uint32_t base = lds0 + (step % kStages) * kStageBytes;
+        if (part < 4) dma16(xsrc[part] + k0, base + (part * 512 + wave * 64) * 16);
+        else dma16(wsrc + (k0 >> 3), base + kXBytes + wave * 64 * 16);
+    };
+    auto issue = [&](int step) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) dma16(xsrc[i] + k0, base + (i * 512 + wave * 64) * 16);
-        dma16(wsrc + (k0 >> 3), base + kXBytes + wave * 64 * 16);
+        for (int part = 0; part < 5; part++) issue_part(step, part);
     };
 
     // Scale/bias tables: thread t < 256 owns tile row t.
@@ -193,7 +205,7 @@ __global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
         // The table of the next 256 values of K is loaded two steps ahead and written one step ahead.
         // Its loads go before this step's direct-to-LDS loads so that the wait above never covers them.
         if ((step & 3) == 1 && step + 3 < steps) sb_load((step + 3) >> 2);
-        issue(step + 2);
+        issue_part(step + 2, 4);  // the remaining four parts are spread over the matrix work below
         const unsigned char *xs = lds + (step % kStages) * kStageBytes, *ws = xs + kXBytes;
         const uint32_t *sbt = sb_table + ((step >> 2) & 1) * (kSbBytes / 4) + ((((step & 3) * BK + 32 * h) >> gshift) * BN);
         uint4 raw[2];
@@ -221,21 +233,28 @@ __global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) acc[i][j] = Mma<T>::mfma(af[i], bf[j], acc[i][j]);
+            issue_part(step + 2, kk);
         }
         if ((step & 3) == 2 && step + 2 < steps) sb_store((step + 2) >> 2);
     }
     dma_wait<0>();
 
     // Epilogue: accumulator element e of a 32 x 32 tile is row 8 (e / 4) + 4 (lane / 32) + e % 4, column lane % 32.
+    // The 32 lanes of a half-wavefront store 32 consecutive elements of one row.
+    const bool full = m0 + BM <= M && n0 + BN <= N;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int col = n0 + wn * 64 + j * 32 + l32;
+            const int row0 = m0 + wm * 128 + i * 32 + 4 * h;
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                if (row < M && col < N) Elem<T>::store(y, (int64_t)row * N + col, acc[i][j][e]);
+            for (int e = 0; e < 16; e += 2) {
+                const uint32_t pair = Mma<T>::pack(acc[i][j][e], acc[i][j][e + 1]);  // rounded to nearest even
+                const int row = row0 + 8 * (e >> 2) + (e & 3);
+                uint16_t *out = reinterpret_cast<uint16_t *>(y) + (int64_t)row * N + col;
+                if (full || (row < M && col < N)) out[0] = (uint16_t)pair;
+                if (full || (row + 1 < M && col < N)) out[N] = (uint16_t)(pair >> 16);
             }
         }
 }
