@@ -218,12 +218,18 @@ __global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
             sc[j] = Mma<T>::lo(sbv);
             bi[j] = Mma<T>::hi(sbv);
         }
+        // x fragments are read one substep ahead of the matrix instructions that use them.
+        uint4 af[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) af[0][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + l32, 4 * h));
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
-            uint4 af[4], bf[2];
-            const int chunk = 4 * h + kk;
+            uint4 bf[2];
+            if (kk < 3) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + l32, chunk));
+                for (int i = 0; i < 4; i++)
+                    af[(kk + 1) & 1][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + l32, 4 * h + kk + 1));
+            }
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const uint32_t word = kk == 0 ? raw[j].x : kk == 1 ? raw[j].y : kk == 2 ? raw[j].z : raw[j].w;
@@ -232,7 +238,7 @@ __global__ void __launch_bounds__(kThreads) qmm4_kernel(const ProductArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = Mma<T>::mfma(af[i], bf[j], acc[i][j]);
+                for (int j = 0; j < 2; j++) acc[i][j] = Mma<T>::mfma(af[kk & 1][i], bf[j], acc[i][j]);
             issue_part(step + 2, kk);
         }
         if ((step & 3) == 2 && step + 2 < steps) sb_store((step + 2) >> 2);

@@ -491,7 +491,8 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
         if (a.bits == 4) {
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
             if (a.m == 2) return run_lds4<T, 2, 1, 8>(a, s);
-            return run_pair4<T, 4, 4, 1>(a, s);
+            if (a.m == 3) return run_lds4<T, 3, 1, 8>(a, s);
+            return run_lds4<T, 4, 1, 8>(a, s);  // more rows: passes of four over grid.y
         }
     }
 #define NVQ_GENERIC(B) (a.m == 1 ? run_generic<T, B, false, 1, 4>(a, s) : run_generic<T, B, false, 2, 4>(a, s))
