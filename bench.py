@@ -31,6 +31,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
 N, K = 14336, 4096
 GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
+# what the same counters read for a plain device copy of known size; None until measured.
+QMV_TRAFFIC_BYTES = 33_202_176   # read 32,368 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
+QMM_TRAFFIC_BYTES = 276_716_544  # read 212,688 KiB + written 57,543 KiB (profiles/qmm4_kernel__prefill_c3_m2048.txt)
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -143,6 +147,9 @@ def main():
     ap.add_argument("--qmm-steps", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the M=2048 leg")
+    ap.add_argument("--only", choices=["qmv", "qmm", "copy"], default=None,
+                    help="profiling aid: run just the rotating decode leg, just the prefill leg, or a plain 1 GiB "
+                         "device copy (the known-size kernel the HBM counters are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N without exchange, "
@@ -157,32 +164,44 @@ def main():
     device = torch.device("cuda:0")
     lib = _lib.load()
     _lib.check(lib.nvq_init(0))
+    if args.only == "copy":
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=device).fill_(1.0)  # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 2, "copy_bytes_written": dst.numel() * 2, "launches": 10}))
+        return
 
-    qs = make_weights(args.copies, device)
-    x1 = torch.randn(1, K, device=device).to(torch.bfloat16)
-    ys = [torch.empty(1, N, dtype=torch.bfloat16, device=device) for _ in qs]
-    calls = [Product(lib, 1, x1, q, y) for q, y in zip(qs, ys)]
+    only = args.only
+    qs = make_weights(args.copies if only != "qmm" else 4, device)
+    record = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
 
-    ms, steps = time_launches(calls, args.steps, args.warmup)
-    gbps = WEIGHT_BYTES / (ms * 1e-3) / 1e9
-    direct_ms, _ = time_launches(calls, min(args.steps, 2000), 50, graph=False)
-    hot_ms, _ = time_launches(calls[:1] * len(calls), min(args.steps, 2000), 50)
+    if only != "qmm":
+        x1 = torch.randn(1, K, device=device).to(torch.bfloat16)
+        ys = [torch.empty(1, N, dtype=torch.bfloat16, device=device) for _ in qs]
+        calls = [Product(lib, 1, x1, q, y) for q, y in zip(qs, ys)]
+        ms, steps = time_launches(calls, args.steps, args.warmup, graph=False)
+        gbps = WEIGHT_BYTES / (ms * 1e-3) / 1e9
+        record.update({
+            "value": gbps, "steps": steps, "warmup": args.warmup, "ms_per_step": ms,
+            "config": {"workload": "configs[1]: decode QMV, affine 4-bit g64, x bf16 [1,4096], W [14336,4096], M=1",
+                       "weight_copies_rotated": args.copies,
+                       "submission": "one C-ABI call per launch, back to back on one stream"},
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": gbps / HBM_PEAK_GBPS, "traffic": QMV_TRAFFIC_BYTES, "kernel": "qmv4_lds_kernel",
+                         "bytes_per_launch": WEIGHT_BYTES, "us_per_launch": ms * 1e3},
+        })
+        if only is None:
+            graph_ms, _ = time_launches(calls, min(args.steps, 2000), 50, graph=True)
+            hot_ms, _ = time_launches(calls[:1] * len(calls), min(args.steps, 2000), 50, graph=False)
+            record["graph_replay"] = {"us_per_launch": graph_ms * 1e3, "gbps": WEIGHT_BYTES / (graph_ms * 1e-3) / 1e9,
+                                      "note": "the same launches captured once into a HIP graph per rotation and replayed"}
+            record["cache_hot"] = {"us_per_launch": hot_ms * 1e3, "gbps": WEIGHT_BYTES / (hot_ms * 1e-3) / 1e9,
+                                   "note": "one weight buffer reused: served from the last-level cache, not an HBM figure"}
 
-    record = {
-        "metric": METRIC, "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": "configs[1]: decode QMV, affine 4-bit g64, x bf16 [1,4096], W [14336,4096], M=1",
-                   "weight_copies_rotated": args.copies, "submission": "one HIP graph per rotation of the weight copies, replayed back to back on one stream"},
-        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "qmv", "bytes_per_launch": WEIGHT_BYTES, "us_per_launch": ms * 1e3},
-        "direct_launch": {"us_per_launch": direct_ms * 1e3, "gbps": WEIGHT_BYTES / (direct_ms * 1e-3) / 1e9,
-                          "note": "one C-ABI call per launch from the Python loop: bounded by the host's call rate"},
-        "cache_hot": {"us_per_launch": hot_ms * 1e3, "gbps": WEIGHT_BYTES / (hot_ms * 1e-3) / 1e9,
-                      "note": "one weight buffer reused: served from the last-level cache, not an HBM figure"},
-    }
-
-    if not args.no_qmm:
+    if only == "qmm" or (only is None and not args.no_qmm):
         m = 2048
         xm = torch.randn(m, K, device=device).to(torch.bfloat16)
         ym = torch.empty(m, N, dtype=torch.bfloat16, device=device)
@@ -193,10 +212,10 @@ def main():
         record["qmm"] = {"workload": "configs[2]: prefill QMM, affine 4-bit g64, x bf16 [2048,4096], W [14336,4096]",
                          "value": tflops, "unit": "TFLOP/s", "ms_per_step": qms, "steps": qsteps,
                          "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "kernel": "qmm",
-                                      "flop_per_launch": flop}}
+                                      "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": QMM_TRAFFIC_BYTES,
+                                      "kernel": "qmm4_kernel", "flop_per_launch": flop}}
 
-    if not args.no_cpu:
+    if only is None and not args.no_cpu:
         record["cpu_baseline"] = cpu_baseline()
     print(json.dumps(record))
 

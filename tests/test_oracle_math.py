@@ -1,0 +1,174 @@
+"""Pins of the CPU oracle that do not come from recorded vectors: the known answers the
+reference's unit tests hold, closed forms, invariants and brute force on small inputs."""
+import ctypes as C
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from oracle import ref
+
+L = ref.lib()
+
+
+def test_e2m1_known_answers():
+    """fp8.rs:185-214: round trips, values, tie thresholds, signed zero, NaN."""
+    values = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for code, v in enumerate(values):
+        assert L.nvq_ref_e2m1_to_f32(code) == v and L.nvq_ref_e2m1_to_f32(code | 8) == -v
+    for code in range(16):
+        assert L.nvq_ref_e2m1_from_f32(L.nvq_ref_e2m1_to_f32(code)) == code
+    for x, code in [(0.25, 0), (0.75, 2), (1.25, 2), (1.75, 4), (2.5, 4), (3.5, 6), (5.0, 6), (7.0, 7)]:
+        assert L.nvq_ref_e2m1_from_f32(x) == code
+    assert L.nvq_ref_e2m1_from_f32(-0.0) == 8
+    assert L.nvq_ref_e2m1_from_f32(float("nan")) == 7
+
+
+def test_e8m0_known_answers():
+    """fp8.rs:216-233."""
+    tiny = np.array([0x400000], np.uint32).view(np.float32)[0]
+    assert L.nvq_ref_e8m0_from_f32(1.0) == 127 and L.nvq_ref_e8m0_from_f32(0.25) == 125
+    assert L.nvq_ref_e8m0_from_f32(0.0) == 0 and L.nvq_ref_e8m0_from_f32(-1.0) == 0
+    assert L.nvq_ref_e8m0_from_f32(float("inf")) == 0xFF and L.nvq_ref_e8m0_from_f32(float("nan")) == 0xFF
+    assert L.nvq_ref_e8m0_to_f32(0) == tiny and L.nvq_ref_e8m0_to_f32(0xFF) == float("inf")
+    assert L.nvq_ref_mx_scale_round_up(1.0 / 6.0) == 0.25
+    assert L.nvq_ref_mx_scale_round_up(0.0) == tiny
+    assert L.nvq_ref_mx_scale_round_up(0.5) == 0.5
+
+
+def test_e4m3_known_answers():
+    """fp8.rs:137-183: MLX's probes and every code's round trip."""
+    nan, inf = float("nan"), float("inf")
+    values = [0.1, 1.0, 448.0, 500.0, -3.3, 1e-4, 0.0, -0.0, inf, -inf, nan, 2.0 ** -9, 2.0 ** -10, 0.0029296875, 464.0,
+              465.0, 1.0625, 1.1875]
+    expected = [29, 56, 126, 126, 197, 0, 0, 128, 126, 254, 126, 1, 0, 2, 126, 126, 56, 58]
+    assert [L.nvq_ref_e4m3_from_f32(v) for v in values] == expected
+    for code, v in [(0, 0.0), (1, 0.001953125), (7, 0.013671875), (8, 0.015625), (56, 1.0), (126, 448.0), (254, -448.0)]:
+        assert L.nvq_ref_e4m3_to_f32(code) == v
+    for code in range(256):
+        if code & 0x7F != 0x7F:
+            assert L.nvq_ref_e4m3_from_f32(L.nvq_ref_e4m3_to_f32(code)) == code
+
+
+def test_mx_scale_is_the_smallest_power_of_two_not_below():
+    """Closed form of mx_scale_round_up on normal inputs: exponent + (mantissa != 0)."""
+    rng = np.random.default_rng(3)
+    xs = np.concatenate([np.exp2(rng.uniform(-100, 100, 2000)).astype(np.float32), np.exp2(np.arange(-100, 100)).astype(np.float32)])
+    for x in xs:
+        u = int(np.array([x], np.float32).view(np.uint32)[0])
+        want = min((u >> 23) + ((u & 0x7FFFFF) != 0), 254)
+        assert L.nvq_ref_e8m0_from_f32(L.nvq_ref_mx_scale_round_up(float(x))) == want
+
+
+def test_code_is_a_little_endian_bit_stream():
+    """kernels.rs:749-756 against brute force over an integer made of the bytes."""
+    rng = np.random.default_rng(4)
+    data = rng.integers(0, 256, 64, dtype=np.uint8)
+    big = int.from_bytes(data.tobytes(), "little")
+    for bits in (1, 2, 3, 4, 5, 6, 8):
+        for i in range(64 * 8 // bits - 1):
+            got = L.nvq_ref_code(data.ctypes.data_as(C.POINTER(C.c_uint8)), C.c_int64(i), bits)
+            assert got == (big >> (i * bits)) & ((1 << bits) - 1)
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+@pytest.mark.parametrize("group", [32, 64, 128])
+def test_round_trip_within_one_step(dtype, bits, group):
+    """crates/nuvec-core/tests/quantized.rs:69-96: error at most one step, mean at most half a step."""
+    rng = np.random.default_rng(bits * 131 + group)
+    w = ref.from_f32(rng.standard_normal((8, 4 * group)).astype(np.float32), dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+    back = ref.to_f32(ref.affine_dequantize(packed, scales, biases, dtype, group, bits), dtype)
+    step = np.repeat(np.abs(ref.to_f32(scales, dtype)), group, axis=-1)
+    err = np.abs(back - ref.to_f32(w, dtype))
+    eps = {ref.F32: 1e-6, ref.BF16: 2.0 ** -7, ref.F16: 2.0 ** -10}[dtype]
+    slack = eps * (np.abs(back) + step * ((1 << bits) - 1))
+    assert np.all(err <= step + slack)
+    assert float(np.mean(err / step)) <= 0.5 + 0.05
+
+
+def test_constant_and_zero_groups():
+    """quantized.rs:98-125: a constant group and an exact zero are representable."""
+    w = np.full((2, 64), 0.375, np.float32)
+    p, s, b = ref.affine_quantize(w, ref.F32, 64, 4)
+    assert np.array_equal(ref.affine_dequantize(p, s, b, ref.F32, 64, 4), w)
+    w = np.linspace(-1, 2, 128, dtype=np.float32).reshape(2, 64)
+    w[0, 5] = 0.0
+    p, s, b = ref.affine_quantize(w, ref.F32, 64, 4)
+    assert ref.affine_dequantize(p, s, b, ref.F32, 64, 4)[0, 5] == 0.0
+
+
+def exact_dot(x, w):
+    return float(sum(Fraction(float(a)) * Fraction(float(b)) for a, b in zip(x, w)))
+
+
+def test_few_rows_order_invariants():
+    """few_rows.rs:336-395: close to the exact dot product (1e-5 sqrt K), independent of the weight
+    layout (stride), and unchanged by zero padding of the reduction."""
+    rng = np.random.default_rng(9)
+    for k in (1, 7, 8, 9, 64, 100, 1000):
+        x = rng.standard_normal(k).astype(np.float32)
+        w = rng.standard_normal(k).astype(np.float32)
+        fp = lambda a: a.ctypes.data_as(C.POINTER(C.c_float))
+        got = L.nvq_ref_dot_few_rows(fp(x), fp(w), C.c_int64(1), C.c_int64(k))
+        assert abs(got - exact_dot(x, w)) <= 1e-5 * np.sqrt(k) * max(1.0, float(np.max(np.abs(x)) * np.max(np.abs(w))))
+        strided = np.zeros(3 * k, np.float32)
+        strided[::3] = w
+        assert L.nvq_ref_dot_few_rows(fp(x), fp(strided), C.c_int64(3), C.c_int64(k)) == got
+        xp, wp = np.concatenate([x, np.zeros(13, np.float32)]), np.concatenate([w, np.ones(13, np.float32)])
+        assert L.nvq_ref_dot_few_rows(fp(xp), fp(wp), C.c_int64(1), C.c_int64(k + 13)) == got
+    # the fixed tree: partial p mod 8, combined ((s0+s4)+(s2+s6))+((s1+s5)+(s3+s7))
+    x = np.array([1e8, 1, -1e8, 1, 1, 1, 1, 1], np.float32)
+    w = np.ones(8, np.float32)
+    f = np.float32
+    want = ((f(1e8) + f(1)) + (f(-1e8) + f(1))) + ((f(1) + f(1)) + (f(1) + f(1)))
+    assert L.nvq_ref_dot_few_rows(x.ctypes.data_as(C.POINTER(C.c_float)), w.ctypes.data_as(C.POINTER(C.c_float)), C.c_int64(1), C.c_int64(8)) == want
+
+
+def test_product_equals_x_times_dequantized_weights():
+    """quantized.rs:168-215: quantized_matmul == x . dequantize(w)^T, here against an exact rational product."""
+    rng = np.random.default_rng(12)
+    for bits, group, dtype in [(4, 64, ref.F32), (3, 32, ref.BF16), (8, 128, ref.F16), (2, 64, ref.BF16)]:
+        n, k, m = 5, 2 * group, 3
+        w = ref.from_f32((rng.standard_normal((n, k)) * 0.1).astype(np.float32), dtype)
+        x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32), dtype)
+        p, s, b = ref.affine_quantize(w, dtype, group, bits)
+        dense = ref.to_f32(ref.affine_dequantize(p, s, b, dtype, group, bits), dtype)
+        y = ref.to_f32(ref.quantized_matmul(x, p, s, b, group=group, bits=bits, dtype=dtype), dtype)
+        x32 = ref.to_f32(x, dtype)
+        for i in range(m):
+            for j in range(n):
+                want = exact_dot(x32[i], dense[j])
+                tol = {ref.F32: 1e-6, ref.BF16: 2.0 ** -8, ref.F16: 2.0 ** -11}[dtype] * max(1.0, abs(want)) + 1e-5
+                assert abs(float(y[i, j]) - want) <= tol
+    # transpose=False reads the same dense matrix the other way
+    w = (rng.standard_normal((64, 64)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((2, 64)).astype(np.float32)
+    p, s, b = ref.affine_quantize(w, ref.F32, 64, 4)
+    dense = ref.affine_dequantize(p, s, b, ref.F32, 64, 4)
+    y = ref.quantized_matmul(x, p, s, b, group=64, bits=4, dtype=ref.F32, transpose=False)
+    assert np.allclose(y, x.astype(np.float64) @ dense.astype(np.float64), rtol=1e-5, atol=1e-5)
+
+
+def test_sorted_offsets_is_a_lower_bound():
+    rng = np.random.default_rng(5)
+    for rows, groups in [(0, 4), (1, 1), (40, 8), (1024, 32)]:
+        rhs = np.sort(rng.integers(0, groups, rows)).astype(np.uint32)
+        got = ref.sorted_offsets(rhs, groups)
+        assert np.array_equal(got, np.searchsorted(rhs, np.arange(groups), side="left").astype(np.int32))
+        assert np.array_equal(got, np.array([int(np.sum(rhs < g)) for g in range(groups)], np.int32))
+
+
+def test_gather_equals_per_pair_products():
+    """quantized.rs:506-527."""
+    rng = np.random.default_rng(6)
+    e, n, k, m = 4, 6, 64, 2
+    w = (rng.standard_normal((e, n, k)) * 0.1).astype(np.float32)
+    x = rng.standard_normal((3, m, k)).astype(np.float32)
+    p, s = ref.fp_quantize(w, ref.F32, ref.MXFP4)
+    lhs, rhs = np.array([2, 0, 1, 1], np.uint32), np.array([3, 3, 0, 2], np.uint32)
+    y = ref.gather_qmm(x, p, s, None, lhs, rhs, mode=ref.MXFP4, group=32, bits=4, dtype=ref.F32)
+    for i in range(4):
+        one = ref.quantized_matmul(x[lhs[i]], p[rhs[i]], s[rhs[i]], None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.F32)
+        assert np.array_equal(y[i], one)
