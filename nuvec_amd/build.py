@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(HERE, "..", "include")
 LIB = os.path.join(HERE, "libnuvec_hip.so")
-SOURCES = ["nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmv.hip", "qmm.hip", "gather.hip"]
+SOURCES = ["nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmv.hip", "qmf.hip", "qmm.hip", "gather.hip"]
 
 # -ffp-contract=off: the quantizers must round every operation as the CPU does; fused
 # multiply-adds are written explicitly where wanted.  Correctly rounded f32 division is

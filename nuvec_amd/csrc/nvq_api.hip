@@ -286,6 +286,10 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     // Routed by one item's rows, as the reference does (gpu.rs:6975-6981).
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
     if (item >= kQmmMinRows && qmm_supported(a)) return launch_qmm(a, (hipStream_t)stream);
+    // One or two rows of 4-bit affine weights: the decode kernel; more rows share one weight decode on the
+    // matrix cores.
+    const bool decode = a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32 && a.m <= 2;
+    if (!decode && a.m >= 3 && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }
 
@@ -302,7 +306,6 @@ size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *) { return 0; }
 int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                        const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
     (void)workspace;
-    (void)offsets;
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
     NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
     NVQ_TRY(check_groups("gather_qmm", d->quant.mode, biases));
@@ -328,6 +331,11 @@ int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, c
     a.batch = d->pairs;
     a.lhs = lhs; a.rhs = rhs;
     a.x_batches = d->x_batches; a.experts = d->experts;
+    // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
+    // weight decoded once.  Otherwise one product per pair.
+    a.offsets = offsets;
+    if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
+    a.offsets = nullptr;
     return launch_qmv(a, (hipStream_t)stream);
 }
 

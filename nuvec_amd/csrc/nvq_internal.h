@@ -60,6 +60,7 @@ struct ProductArgs {
     int64_t x_strides[NVQ_MAX_BATCH_DIMS], w_strides[NVQ_MAX_BATCH_DIMS], s_strides[NVQ_MAX_BATCH_DIMS];
     const uint32_t *lhs, *rhs;      // gather: batch z reads x batch lhs[z] and weight batch rhs[z]
     int64_t x_batches, experts;     // gather: index bounds (an index beyond them is clamped)
+    const int32_t *offsets;         // grouped gather: rows of expert e are [offsets[e], offsets[e+1]) of `batch` rows
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
@@ -68,7 +69,10 @@ int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
 // Rows of x from which a product goes to the tiled kernel rather than the few-row kernels
 // (the counterpart of the reference's device-specific `qmv_batch_limit`,
 // crates/nuvec-core/src/gpu.rs:1506-1538).
-constexpr int64_t kQmmMinRows = 12;
+constexpr int64_t kQmmMinRows = 128;
+// The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
+bool qmf_supported(const ProductArgs &a);
+int32_t launch_qmf(const ProductArgs &a, hipStream_t s);
 int32_t launch_fill_zero(void *p, int64_t bytes, hipStream_t s);
 
 }  // namespace nvq

@@ -211,3 +211,60 @@ def test_config3_prefill_bf16_4bit_g64():
     for i in (0, 777, m - 1):
         one = ref.to_f32(to_host(nv.quantized_matmul(xd[i:i + 1], q)), ref.BF16)[0]
         assert np.all(np.abs(one - g32[i]) <= 1e-2 * row_max[i])
+
+
+def moe_inputs(rng, experts, n, k, tokens, top):
+    w = make_w(rng, experts * n, k, ref.BF16).reshape(experts, n, k)
+    packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+    x_tok = make_x(rng, tokens, k, ref.BF16)
+    choice = np.stack([rng.permutation(experts)[:top] for _ in range(tokens)])  # distinct experts per token
+    pair_expert, pair_token = choice.reshape(-1), np.repeat(np.arange(tokens), top)
+    order = np.argsort(pair_expert, kind="stable")  # the caller's sort by expert (model.rs:2195-2210)
+    rhs = pair_expert[order].astype(np.uint32)
+    x = np.ascontiguousarray(x_tok[pair_token[order]]).reshape(-1, 1, k)
+    return packed, scales, x, rhs
+
+
+def test_config5_moe_gather_mxfp4():
+    """BASELINE config 5: 32 experts [2880,2880] MXFP4, 256 tokens x top-4 sorted by expert -> x [1024,1,2880].
+    Every output row against the oracle's per-pair product; grouped route == per-pair route within the bar."""
+    rng = np.random.default_rng(20260105)
+    experts, n, k = 32, 2880, 2880
+    packed, scales, x, rhs = moe_inputs(rng, experts, n, k, 256, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(nv.QuantMode.MXFP4))
+    rhs_dev = torch.from_numpy(rhs.astype(np.int64)).cuda()
+    assert nv.GatherQmm.groups(rhs.size, experts)
+    got = to_host(nv.gather_qmm(to_dev(x), q, None, rhs_dev, nv.GatherQmm(sorted_indices=True)))
+    assert got.shape == (1024, 1, n)
+    want = ref.gather_qmm(x, packed, scales, None, np.arange(1024, dtype=np.uint32), rhs, mode=ref.MXFP4, group=32, bits=4,
+                          dtype=ref.BF16, threads=8)
+    assert_rows_close(got, want, ref.BF16, "config 5 grouped")
+    unsorted = to_host(nv.gather_qmm(to_dev(x[:40]), q, None, rhs_dev[:40], nv.GatherQmm(sorted_indices=False)))
+    assert_rows_close(unsorted, want[:40], ref.BF16, "config 5 per pair")
+
+
+def test_grouped_gather_edge_cases():
+    """Experts without rows, an expert with more than 32 rows (two passes), affine 4-bit weights."""
+    rng = np.random.default_rng(8)
+    experts, n, k = 6, 72, 256
+    w = make_w(rng, experts * n, k, ref.BF16).reshape(experts, n, k)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+    rhs = np.sort(np.array([0] * 3 + [2] * 45 + [5] * 20, np.uint32))
+    x = make_x(rng, rhs.size, k, ref.BF16).reshape(-1, 1, k)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+    got = to_host(nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs.astype(np.int64)).cuda(), nv.GatherQmm(sorted_indices=True)))
+    want = ref.gather_qmm(x, packed, scales, biases, np.arange(rhs.size, dtype=np.uint32), rhs, group=64, bits=4, dtype=ref.BF16)
+    assert_rows_close(got, want, ref.BF16, "grouped affine")
+
+
+@pytest.mark.parametrize("m", [3, 16, 33, 100])
+def test_few_rows_on_matrix_cores(m):
+    """3 <= M < 128 of BASELINE's decode weights: one weight decode shared by all rows."""
+    rng = np.random.default_rng(40 + m)
+    n, k = 1000, 4096
+    w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, ref.BF16, f"few rows M={m}")
