@@ -14,7 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(HERE, "..", "include")
 LIB = os.path.join(HERE, "libnuvec_hip.so")
-SOURCES = ["nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmv.hip", "qmf.hip", "qmm.hip", "gather.hip"]
+SOURCES = ["qmf_b8.hip", "qmf_b6.hip", "qmf_b4.hip", "qmf_fp4.hip", "qmf_b3.hip", "qmf_b2.hip", "qmm.hip", "qmv.hip",
+           "nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmf.hip", "gather.hip"]  # slowest to compile first
 
 # -ffp-contract=off: the quantizers must round every operation as the CPU does; fused
 # multiply-adds are written explicitly where wanted.  Correctly rounded f32 division is
@@ -36,7 +37,7 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose: bool = False, jobs: int = 4) -> str:
+def build(verbose: bool = False, jobs: int = 8) -> str:
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)

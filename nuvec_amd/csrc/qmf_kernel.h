@@ -1,0 +1,503 @@
+// Few-row quantized products on the gfx950 matrix cores: y[m, n] = x[m, :] . dequantize(w[n, :]) for up to
+// 32 rows of x per pass, and the grouped (sorted) gathered product of mixture-of-experts layers, where
+// each expert's rows are such a product against that expert's weights.  Values follow nuvec's CPU product
+// (reference: crates/nuvec-core/src/kernels.rs:1091-1142, crates/nuvec-core/src/quantized.rs:679-719) within
+// the stated tolerance; the grouped route is the counterpart of the reference's `gather_qmm_rhs`
+// (crates/nuvec-kernels/src/metal/quantized.h:3301-3449, schedule at 2866-2906).
+//
+// This header holds the kernel template; qmf_b*.hip instantiate it per code width (affine 2, 3, 4, 6, 8 bits
+// and MXFP4) so that the widths compile in parallel.
+//
+// The weights are the large operand and each weight is decoded exactly once per pass.  The kernel is bound
+// by the memory instructions it issues, so everything is arranged to issue few, wide, coalesced ones:
+//   * a block of eight wavefronts owns 32 RG weight rows (RG = 1 or 2 groups of 32) and splits K into
+//     contiguous ranges, one per wavefront.  A wavefront takes its range in windows of two steps
+//     (128 values = 16 BITS bytes of every row, i.e. BITS chunks of 16 bytes): its loads, each a wavefront of
+//     consecutive chunks, fetch a window into registers several windows ahead; the window then goes through
+//     a private piece of LDS (chunks XOR-swizzled by row where BITS is a power of two) to reach the matrix
+//     operand layout, in which a lane (row n = lane % 32, half h = lane / 32) holds the 32 codes (BITS
+//     dwords) of its half of a step for every row group;
+//   * the scales and biases of the block's rows are one contiguous piece of memory: it is copied once,
+//     coalesced, into an LDS table laid out [group][row], and read from there;
+//   * the pieces of x are shared by the row groups, and a pass of at most 8 (16) rows of x packs four
+//     (two) of a step's pieces into one load: lane (row r = l % XR, slot q = l / XR) of a half loads the
+//     pieces q NL .. q NL + NL - 1 (NL = XR / 8), the matrix instruction of piece kk takes that register with the
+//     lanes of other slots cleared, so row r + XR q of the accumulator holds the share of piece kk and the
+//     shares are added when the tile is written.
+// Codes are expanded into matrix operands in registers (affine: code -> float -> fma -> packed convert;
+// MXFP4: one scaled FP4 -> element-type conversion per two codes).  The K order inside a step is permuted
+// consistently for both operands (piece kk of half h holds values 32 h + 8 kk .. + 8 of the step).  The
+// wavefronts' partial tiles are summed through LDS in a fixed order, so results do not depend on scheduling.
+#pragma once
+
+#include "nvq_device.h"
+#include "nvq_internal.h"
+
+#include <type_traits>
+#include <utility>
+
+namespace nvq {
+namespace qmf {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2v_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2v_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef u32x4_t u32x4_a4_t __attribute__((aligned(4)));  // 16 bytes in memory at any dword
+
+constexpr int kWaves = 8;  // wavefronts per block, each with its own range of K
+constexpr int kThreads = 64 * kWaves;
+constexpr int kLdsLimit = 160 * 1024;
+
+// Sizes that follow from the code width and the rows per block; shared by the kernel and its launcher.
+template <int BITS, int RG>
+struct Geometry {
+    static constexpr int kRows = 32 * RG;                  // weight rows per block = columns of y
+    static constexpr int kChunks = kRows * BITS;           // 16-byte chunks of one window
+    static constexpr int kLoads = (kChunks + 63) / 64;     // loads per lane and window
+    static constexpr int kDepth = kLoads <= 4 ? 4 : 2;     // windows of weights in flight per lane
+    static constexpr int kRowBytes = 16 * BITS;            // of one row in a window
+    static constexpr int kStageBytes = kChunks * 16;       // one window of one wavefront
+    static constexpr int kPartialBytes = 4 * RG * 16 * 64 * 4;  // four wavefronts' tiles
+    static constexpr int kFixedLdsBytes = kPartialBytes + kWaves * kStageBytes;
+    static constexpr bool kPow2 = (BITS & (BITS - 1)) == 0;
+    // 16-byte chunk c of row `row` sits at chunk position c ^ swizzle(row)
+    __host__ __device__ static constexpr int swizzle(int row) { return kPow2 ? (row / (BITS >= 16 ? 1 : 16 / BITS)) % BITS : 0; }
+};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant in the body
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+template <int B>
+__device__ __forceinline__ float ubyte_to_float(uint32_t v) {
+    float f;
+    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
+    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
+    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
+    return f;
+}
+
+template <typename T> struct Ops;
+template <> struct Ops<bf16_t> {
+    __device__ static __forceinline__ floatx16_t mfma(uint4 a, uint4 b, floatx16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
+        const floatx2_t f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2v_t));
+    }
+    // The two E2M1 codes of byte B of `word` times `scale`, as two elements (low nibble first).
+    template <int B> __device__ static __forceinline__ uint32_t fp4_pair(uint32_t word, float scale) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, B));
+    }
+};
+template <> struct Ops<f16_t> {
+    __device__ static __forceinline__ floatx16_t mfma(uint4 a, uint4 b, floatx16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
+        const floatx2_t f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2v_t));
+    }
+    template <int B> __device__ static __forceinline__ uint32_t fp4_pair(uint32_t word, float scale) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, B));
+    }
+};
+
+// Code J of a lane's 32 codes (BITS dwords, value i in bits i BITS .. of the stream) as a float.
+template <int BITS, int J>
+__device__ __forceinline__ float code_to_float(const uint32_t (&dw)[BITS]) {
+    constexpr int bit = J * BITS, d = bit / 32, s = bit % 32;
+    constexpr uint32_t mask = (1u << BITS) - 1u;
+    if constexpr (BITS == 8) {
+        return ubyte_to_float<s / 8>(dw[d]);
+    } else if constexpr (s + BITS <= 32) {
+        return (float)((dw[d] >> s) & mask);
+    } else {
+        return (float)(((dw[d] >> s) | (dw[d + 1] << (32 - s))) & mask);
+    }
+}
+
+// Piece KK (eight codes, stream order) of a lane's 32 codes as one matrix operand.
+template <typename T, int BITS, bool FP4, int KK>
+__device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float s, float b) {
+    uint4 r;
+    if constexpr (FP4) {
+        const uint32_t word = dw[KK];
+        r.x = Ops<T>::template fp4_pair<0>(word, s);
+        r.y = Ops<T>::template fp4_pair<1>(word, s);
+        r.z = Ops<T>::template fp4_pair<2>(word, s);
+        r.w = Ops<T>::template fp4_pair<3>(word, s);
+    } else if constexpr (BITS == 4) {
+        const uint32_t word = dw[KK];
+        const uint32_t even = word & 0x0F0F0F0Fu, odd = (word >> 4) & 0x0F0F0F0Fu;
+        r.x = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<0>(even), s, b), __builtin_fmaf(ubyte_to_float<0>(odd), s, b));
+        r.y = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<1>(even), s, b), __builtin_fmaf(ubyte_to_float<1>(odd), s, b));
+        r.z = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<2>(even), s, b), __builtin_fmaf(ubyte_to_float<2>(odd), s, b));
+        r.w = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<3>(even), s, b), __builtin_fmaf(ubyte_to_float<3>(odd), s, b));
+    } else {
+        constexpr int J = 8 * KK;
+        r.x = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 0>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 1>(dw), s, b));
+        r.y = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 2>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 3>(dw), s, b));
+        r.z = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 4>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 5>(dw), s, b));
+        r.w = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 6>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 7>(dw), s, b));
+    }
+    return r;
+}
+
+// GROUPED: blockIdx.z is an expert; its rows of x / y are [offsets[z], offsets[z+1]) (the last expert ends at
+// `pairs`), taken in passes of up to 32.  Otherwise blockIdx.z is a batch with one stride per operand and
+// blockIdx.y a pass of 32 rows.
+template <typename T, int BITS, bool FP4, int RG, bool GROUPED>
+__global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
+    using G = Geometry<BITS, RG>;
+    constexpr int kRows = G::kRows, kDepth = G::kDepth, kLoads = G::kLoads;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    float *partial = reinterpret_cast<float *>(lds);  // [4][RG][values][64]
+    using S = std::conditional_t<FP4, uint8_t, T>;    // stored scale type
+    S *table_s = reinterpret_cast<S *>(lds + G::kFixedLdsBytes);  // [group][rows]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, l32 = lane & 31;
+    const int K = (int)a.k, N = (int)a.n;
+    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int kgroups = K >> gshift;
+    const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
+    S *table_b = table_s + kRows * kgroups;
+    const int n0 = blockIdx.x * kRows;
+
+    int row_begin, row_end;  // rows of x (and of y) this block multiplies
+    int64_t xo = 0, wo = 0, so = 0, yo = 0;
+    if constexpr (GROUPED) {
+        const int e = blockIdx.z;
+        row_begin = a.offsets[e];
+        row_end = e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch;
+        if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
+        wo = (int64_t)e * N * row_bytes;
+        so = (int64_t)e * N * kgroups;
+    } else {
+        row_begin = blockIdx.y * 32;
+        row_end = row_begin + 32 < (int)a.m ? row_begin + 32 : (int)a.m;
+        if (a.batch_ndim > 0) {
+            xo = (int64_t)blockIdx.z * a.x_strides[0];
+            wo = (int64_t)blockIdx.z * a.w_strides[0] * 4;  // the stride counts packed words
+            so = (int64_t)blockIdx.z * a.s_strides[0];
+            yo = (int64_t)blockIdx.z * a.m * N;
+        }
+    }
+    const T *x = (const T *)a.x + xo;
+    T *y = (T *)a.y + yo;
+
+    // K in steps of 64 values, split over the wavefronts in windows of two steps.
+    const int steps = K >> 6;
+    const int windows = (steps + 1) >> 1;
+    const int s_begin = 2 * (windows * wave / kWaves);
+    const int s_end = 2 * (windows * (wave + 1) / kWaves) < steps ? 2 * (windows * (wave + 1) / kWaves) : steps;
+
+    // Window loads: load j of this lane is chunk q = 64 j + lane of the window, i.e. chunk q % BITS of
+    // row q / BITS.  Chunks of the window's second step begin at BITS / 2 (a window that ends the range
+    // early exists only for even BITS; its lanes fetch the first step again).
+    const unsigned char *wload[kLoads];
+    int wstore[kLoads];  // byte offset of the chunk within the wavefront's stage
+    bool second[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; j++) {
+        const int q = 64 * j + lane, qc = q < G::kChunks ? q : G::kChunks - 1;
+        const int row = qc / BITS, c = qc % BITS;
+        const int n = n0 + row < N ? n0 + row : N - 1;  // tail rows are computed, not stored
+        wload[j] = (const unsigned char *)a.w + wo + (int64_t)n * row_bytes + 16 * c;
+        wstore[j] = row * G::kRowBytes + 16 * (c ^ G::swizzle(row));
+        second[j] = 2 * c >= BITS;
+    }
+    auto load_window = [&](int step, u32x4_t (&w)[kLoads]) {
+        const bool half = step + 1 >= s_end;
+#pragma unroll
+        for (int j = 0; j < kLoads; j++) {
+            const int off = step * 8 * BITS - ((half && second[j]) ? 8 * BITS : 0);
+            if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) w[j] = *reinterpret_cast<const u32x4_a4_t *>(wload[j] + off);
+        }
+    };
+    unsigned char *stage = lds + G::kPartialBytes + wave * G::kStageBytes;
+    // Operand reads: the BITS dwords of half h of step t of row l32 (row group 0), in pieces that do not
+    // straddle a chunk.
+    constexpr int kPiece = BITS % 4 == 0 ? 4 : BITS % 2 == 0 ? 2 : 1;  // dwords per LDS read
+    constexpr int kPieces = BITS / kPiece;
+    int wread[2][kPieces];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int p = 0; p < kPieces; p++) {
+            const int byte = (2 * t + h) * 4 * BITS + 4 * kPiece * p;  // within the row
+            wread[t][p] = l32 * G::kRowBytes + 16 * ((byte >> 4) ^ G::swizzle(l32)) + (byte & 15);
+        }
+    static_assert(G::swizzle(32) == 0 && G::swizzle(33) == G::swizzle(1), "row groups share the swizzle of their rows");
+
+    auto load_scales = [&](int step, float (&scale)[RG], float (&bias)[RG]) {
+        const int g = (step * 64 + 32 * h) >> gshift;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const S *sp = table_s + g * kRows + 32 * rg + l32, *bp = table_b + g * kRows + 32 * rg + l32;
+            if constexpr (FP4) {
+                scale[rg] = ftz(e8m0_to_f32(*sp));
+                bias[rg] = 0.0f;
+            } else {
+                scale[rg] = Elem<T>::load(sp, 0);
+                bias[rg] = Elem<T>::load(bp, 0);
+            }
+        }
+    };
+
+    {
+        // The scales (and biases) of rows n0 .. n0 + kRows - 1 are contiguous: copy them in aligned 16-byte
+        // pieces and scatter the elements to [group][row].  Bytes of a piece outside the rows are dropped.
+        constexpr int kPer = 16 / (int)sizeof(S);
+        const int valid_rows = N - n0 < kRows ? N - n0 : kRows;
+        const int count = valid_rows * kgroups;
+        const int tensors = FP4 ? 1 : 2;
+        for (int t = 0; t < tensors; t++) {
+            const S *src = (t == 0 ? (const S *)a.scales : (const S *)a.biases) + so + (int64_t)n0 * kgroups;
+            S *dst = t == 0 ? table_s : table_b;
+            const int skew = (int)((uintptr_t)src & 15) / (int)sizeof(S);  // elements before src in its first piece
+            const uint4 *pieces = reinterpret_cast<const uint4 *>(src - skew);
+            const int n_pieces = (skew + count + kPer - 1) / kPer;
+            for (int p = tid; p < n_pieces; p += kThreads) {
+                const uint4 v = pieces[p];
+                S elems[kPer];
+                __builtin_memcpy(elems, &v, 16);
+                int idx = p * kPer - skew;  // element index of elems[0] within the block's rows
+                int row = idx >= 0 ? idx / kgroups : 0, g = idx >= 0 ? idx - row * kgroups : 0;
+#pragma unroll
+                for (int e = 0; e < kPer; e++, idx++) {
+                    if (idx >= 0 && idx < count) {
+                        dst[g * kRows + row] = elems[e];
+                        if (++g == kgroups) g = 0, row++;
+                    }
+                }
+            }
+        }
+    }
+
+    // One pass over at most XR rows of x (XR = 8, 16 or 32).
+    auto run_pass = [&](auto xr_tag, int pass, int rows) {
+        constexpr int XR = decltype(xr_tag)::value;
+        constexpr int NL = XR / 8;        // loads of x per step
+        constexpr int XD = (32 / XR) < kDepth ? (32 / XR) : kDepth;  // windows of x in flight (kDepth is a multiple of it)
+        constexpr int NV = XR / 2;        // values of the tile per lane and row group once the slots are added
+        const int r = l32 % XR, slot = l32 / XR;
+        const bool live = r < rows;  // this lane's row of x exists
+        // x row of this lane; in the grouped route rows are gathered through lhs (arange for sorted gathers)
+        int64_t xr = pass + (live ? r : 0);
+        if constexpr (GROUPED) xr = a.lhs != nullptr ? (int64_t)a.lhs[xr] : xr;
+        const T *xrow = x + xr * K + 32 * h + 8 * NL * slot;  // piece kk of half h covers k0 + 32 h + 8 kk .. + 8
+
+        floatx16_t acc[RG];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[rg][e] = 0.0f;
+
+        u32x4_t ring[kDepth][kLoads] = {};  // windows in flight
+        uint4 xring[XD][2][NL] = {};        // x pieces, XD windows ahead (they come from the cache)
+        auto load_x = [&](int step, uint4 (&xf)[2][NL]) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int sc = step + t < s_end ? step + t : step;
+#pragma unroll
+                for (int j = 0; j < NL; j++)
+                    xf[t][j] = live ? *reinterpret_cast<const uint4 *>(xrow + sc * 64 + 8 * j) : make_uint4(0, 0, 0, 0);
+            }
+        };
+        static_for<kDepth>([&](auto d_tag) {
+            constexpr int d = decltype(d_tag)::value;
+            if (s_begin + 2 * d < s_end) {
+                load_window(s_begin + 2 * d, ring[d]);
+                if constexpr (d < XD) load_x(s_begin + 2 * d, xring[d]);
+            }
+        });
+        __syncthreads();  // first pass: the table is written; later passes: nothing pending
+
+        for (int s0 = s_begin; s0 < s_end; s0 += 2 * kDepth) {
+            static_for<kDepth>([&](auto d_tag) {
+                constexpr int d = decltype(d_tag)::value;
+                const int step = s0 + 2 * d;
+                if (step < s_end) {
+                    // through LDS into the operand layout; the wavefront's LDS accesses execute in order
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int j = 0; j < kLoads; j++)
+                        if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) *reinterpret_cast<u32x4_t *>(stage + wstore[j]) = ring[d][j];
+                    __builtin_amdgcn_wave_barrier();
+                    asm volatile("" ::: "memory");
+                    uint32_t codes[2][RG][BITS];
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+#pragma unroll
+                        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+                            for (int p = 0; p < kPieces; p++) {
+                                const unsigned char *src = stage + wread[t][p] + rg * 32 * G::kRowBytes;
+                                if constexpr (kPiece == 4) {
+                                    const u32x4_t v = *reinterpret_cast<const u32x4_t *>(src);
+                                    codes[t][rg][4 * p] = v.x, codes[t][rg][4 * p + 1] = v.y, codes[t][rg][4 * p + 2] = v.z, codes[t][rg][4 * p + 3] = v.w;
+                                } else if constexpr (kPiece == 2) {
+                                    const u32x2_t v = *reinterpret_cast<const u32x2_t *>(src);
+                                    codes[t][rg][2 * p] = v.x, codes[t][rg][2 * p + 1] = v.y;
+                                } else {
+                                    codes[t][rg][p] = *reinterpret_cast<const uint32_t *>(src);
+                                }
+                            }
+                    asm volatile("" ::: "memory");
+                    uint4 xf[2][NL];
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+#pragma unroll
+                        for (int j = 0; j < NL; j++) xf[t][j] = xring[d % XD][t][j];
+                    if (step + 2 * kDepth < s_end) load_window(step + 2 * kDepth, ring[d]);
+                    if (step + 2 * XD < s_end) load_x(step + 2 * XD, xring[d % XD]);
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        if (step + t < s_end) {
+                            float scale[RG], bias[RG];
+                            load_scales(step + t, scale, bias);
+                            static_for<4>([&](auto kk_tag) {
+                                constexpr int kk = decltype(kk_tag)::value;
+                                uint4 xa = xf[t][kk % NL];
+                                if constexpr (XR < 32) {
+                                    const bool mine = slot == kk / NL;
+                                    xa.x = mine ? xa.x : 0u, xa.y = mine ? xa.y : 0u, xa.z = mine ? xa.z : 0u, xa.w = mine ? xa.w : 0u;
+                                }
+#pragma unroll
+                                for (int rg = 0; rg < RG; rg++)
+                                    acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg], bias[rg]), acc[rg]);
+                            });
+                        }
+                    }
+                }
+            });
+        }
+
+        // Accumulator element e of lane l is tile row 8 (e / 4) + 4 (l / 32) + e % 4, column l % 32; tile rows
+        // r, r + XR, ... are the slots' shares of row r of x.
+        float vals[RG][NV];
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                float sum = acc[rg][v];
+#pragma unroll
+                for (int q = 1; q < 32 / XR; q++) sum += acc[rg][v + NV * q];
+                vals[rg][v] = sum;
+            }
+        // Sum the wavefronts' partial tiles in a fixed order: the upper four hand theirs to the lower four,
+        // whose tiles are then added in wavefront order.
+        auto slot_of = [&](int w, int rg, int v) -> float * { return partial + ((w * RG + rg) * NV + v) * 64; };
+        if (wave >= 4) {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+                for (int v = 0; v < NV; v++) slot_of(wave - 4, rg, v)[lane] = vals[rg][v];
+        }
+        __syncthreads();
+        if (wave < 4) {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+                for (int v = 0; v < NV; v++) vals[rg][v] += slot_of(wave, rg, v)[lane];
+        }
+        __syncthreads();
+        if (wave < 4) {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+                for (int v = 0; v < NV; v++) slot_of(wave, rg, v)[lane] = vals[rg][v];
+        }
+        __syncthreads();
+        for (int idx = tid; idx < RG * NV * 64; idx += kThreads) {
+            const int l = idx & 63, v = (idx >> 6) % NV, rg = idx / (64 * NV);
+            const float sum = ((slot_of(0, rg, v)[l] + slot_of(1, rg, v)[l]) + slot_of(2, rg, v)[l]) + slot_of(3, rg, v)[l];
+            const int m = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), col = n0 + 32 * rg + (l & 31);
+            if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, sum);
+        }
+        __syncthreads();
+    };
+
+    for (int pass = row_begin; pass < row_end; pass += 32) {
+        const int rows = row_end - pass < 32 ? row_end - pass : 32;
+        if (rows <= 8) run_pass(std::integral_constant<int, 8>{}, pass, rows);
+        else if (rows <= 16) run_pass(std::integral_constant<int, 16>{}, pass, rows);
+        else run_pass(std::integral_constant<int, 32>{}, pass, rows);
+    }
+}
+
+// Bytes of the LDS table of scales (and biases) for `rows` weight rows.
+inline size_t table_bytes(const ProductArgs &a, int rows) {
+    const int64_t group = a.mode == NVQ_MXFP4 ? 32 : a.group;
+    const int64_t bytes = a.mode == NVQ_MXFP4 ? rows * (a.k / group) : 2 * rows * (a.k / group) * 2;
+    return (size_t)((bytes + 15) & ~(int64_t)15);
+}
+
+// Groups of 32 weight rows per block: two, unless that leaves most compute units without a block.
+inline int row_groups(const ProductArgs &a) {
+    if (a.offsets != nullptr) return 2;
+    const int64_t blocks = ((a.n + 63) / 64) * ((a.m + 31) / 32) * a.batch;
+    return blocks >= 192 ? 2 : 1;
+}
+
+template <typename T, int BITS, bool FP4, int RG, bool GROUPED>
+int32_t run_variant(const ProductArgs &a, hipStream_t s) {
+    using G = Geometry<BITS, RG>;
+    static bool configured = false;
+    auto kernel = qmf_kernel<T, BITS, FP4, RG, GROUPED>;
+    if (!configured) {
+        NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+        configured = true;
+    }
+    const size_t lds_bytes = G::kFixedLdsBytes + table_bytes(a, G::kRows);
+    if (lds_bytes > (size_t)kLdsLimit) return fail(NVQ_UNSUPPORTED, "quantized_matmul: K = %lld needs a %zu-byte LDS table", (long long)a.k, lds_bytes);
+    const unsigned gx = (unsigned)((a.n + G::kRows - 1) / G::kRows);
+    const dim3 grid = GROUPED ? dim3(gx, 1, (unsigned)a.experts) : dim3(gx, (unsigned)((a.m + 31) / 32), (unsigned)a.batch);
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
+    NVQ_LAUNCH_CHECK("qmf");
+    return NVQ_OK;
+}
+
+template <typename T, int BITS, bool FP4>
+int32_t run_width(const ProductArgs &a, hipStream_t s) {
+    if (a.offsets != nullptr) return run_variant<T, BITS, FP4, 2, true>(a, s);
+    return row_groups(a) == 2 ? run_variant<T, BITS, FP4, 2, false>(a, s) : run_variant<T, BITS, FP4, 1, false>(a, s);
+}
+
+template <int BITS, bool FP4>
+int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
+    return a.dtype == NVQ_BF16 ? run_width<bf16_t, BITS, FP4>(a, s) : run_width<f16_t, BITS, FP4>(a, s);
+}
+
+// LDS bytes of the variant `launch_qmf` would pick (for `qmf_supported`).
+template <int BITS>
+inline size_t lds_needed(const ProductArgs &a) {
+    return row_groups(a) == 2 ? Geometry<BITS, 2>::kFixedLdsBytes + table_bytes(a, 64) : Geometry<BITS, 1>::kFixedLdsBytes + table_bytes(a, 32);
+}
+
+}  // namespace qmf
+
+// One per code width, each in its own translation unit.
+int32_t launch_qmf_b2(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b3(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b4(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b6(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b8(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_fp4(const ProductArgs &a, hipStream_t s);
+
+}  // namespace nvq

@@ -98,6 +98,8 @@ def from_f32(a: np.ndarray, dtype: int) -> np.ndarray:
 def affine_quantize(w: np.ndarray, dtype: int, group: int, bits: int):
     w = _c(w)
     n, last = w.size, w.shape[-1]
+    if last % group != 0 or (last * bits) % 32 != 0:
+        raise ValueError(f"affine_quantize: last dimension {last} is not whole groups of {group} and whole words")
     packed = np.zeros(w.shape[:-1] + (last * bits // 32,), np.uint32)
     scales = np.zeros(w.shape[:-1] + (last // group,), NP_OF[dtype])
     biases = np.zeros_like(scales)

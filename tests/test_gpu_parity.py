@@ -268,3 +268,34 @@ def test_few_rows_on_matrix_cores(m):
     want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16, threads=8)
     got = to_host(nv.quantized_matmul(to_dev(x), q))
     assert_rows_close(got, want, ref.BF16, f"few rows M={m}")
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(32, 2), (64, 3), (128, 3), (64, 6), (32, 8), (128, 8), (32, 4)])
+def test_few_rows_every_width(dtype, group, bits):
+    """The few-row matrix-core kernel at every code width it takes: K of whole and of half windows
+    (128 and 64 values), N off the rows per block, passes of 8, 16 and 32 rows of x."""
+    rng = np.random.default_rng(900 + 10 * bits + group)
+    for m, n, k in [(1, 200, 256), (5, 77, 1152), (16, 130, 2048 + 128), (33, 64, 128), (2, 96, 576 if group < 128 else 640)]:
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, dtype, f"few rows b{bits} g{group} M={m} N={n} K={k}")
+
+
+@pytest.mark.parametrize("bits,group", [(3, 64), (8, 32)])
+def test_few_rows_batched_widths(bits, group):
+    """A batch of weight matrices with one stride per operand, 3- and 8-bit codes."""
+    rng = np.random.default_rng(77 + bits)
+    b, m, n, k = 3, 4, 96, 512
+    w, x = make_w(rng, b * n, k, ref.BF16), make_x(rng, b * m, k, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, group, bits)
+    q = nv.Quantized(to_dev(packed.reshape(b, n, -1)), to_dev(scales.reshape(b, n, -1)), to_dev(biases.reshape(b, n, -1)),
+                     nv.Quant.affine(group, bits))
+    got = to_host(nv.quantized_matmul(to_dev(x.reshape(b, m, k)), q))
+    for i in range(b):
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n],
+                                    biases[i * n:(i + 1) * n], group=group, bits=bits, dtype=ref.BF16)
+        assert_rows_close(got[i], want, ref.BF16, f"batched b{bits} item {i}")
