@@ -286,9 +286,10 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     // Routed by one item's rows, as the reference does (gpu.rs:6975-6981).
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
     if (item >= kQmmMinRows && qmm_supported(a)) return launch_qmm(a, (hipStream_t)stream);
-    // One or two rows of 4-bit affine weights: the decode kernel.  Other few-row products share one weight
-    // decode on the matrix cores where that kernel takes them.
-    const bool decode = a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32 && a.m <= 2;
+    // Up to four rows of 4-bit affine weights: the decode kernel (per-row work on the vector units, which is
+    // cheaper than the matrix-core kernel's full dequantization up to there).  Other few-row products share
+    // one weight decode on the matrix cores where that kernel takes them.
+    const bool decode = a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32 && a.m <= 4;
     if (!decode && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }

@@ -221,12 +221,16 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         wstore[j] = row * G::kRowBytes + 16 * (c ^ G::swizzle(row));
         second[j] = 2 * c >= BITS;
     }
+    // Every load of the K loop is issued on every path, so that the number of loads in flight is known where
+    // a window is consumed and the wait leaves the younger windows' loads outstanding.  A window past the
+    // range loads the first 16 bytes of the weights instead (one address for all lanes).
     auto load_window = [&](int step, u32x4_t (&w)[kLoads]) {
-        const bool half = step + 1 >= s_end;
+        const bool real = step < s_end, half = step + 1 >= s_end;
 #pragma unroll
         for (int j = 0; j < kLoads; j++) {
             const int off = step * 8 * BITS - ((half && second[j]) ? 8 * BITS : 0);
-            if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) w[j] = *reinterpret_cast<const u32x4_a4_t *>(wload[j] + off);
+            const unsigned char *src = real ? wload[j] + off : (const unsigned char *)a.w;
+            w[j] = *reinterpret_cast<const u32x4_a4_t *>(src);
         }
     };
     unsigned char *stage = lds + G::kPartialBytes + wave * G::kStageBytes;
@@ -310,21 +314,19 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
 
         u32x4_t ring[kDepth][kLoads] = {};  // windows in flight
         uint4 xring[XD][2][NL] = {};        // x pieces, XD windows ahead (they come from the cache)
+        // Lanes without a row of x read the pass's first row: their tile rows are never stored.
         auto load_x = [&](int step, uint4 (&xf)[2][NL]) {
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const int sc = step + t < s_end ? step + t : step;
+                const int sc = step + t < s_end ? step + t : (step < s_end ? step : s_begin);
 #pragma unroll
-                for (int j = 0; j < NL; j++)
-                    xf[t][j] = live ? *reinterpret_cast<const uint4 *>(xrow + sc * 64 + 8 * j) : make_uint4(0, 0, 0, 0);
+                for (int j = 0; j < NL; j++) xf[t][j] = *reinterpret_cast<const uint4 *>(xrow + sc * 64 + 8 * j);
             }
         };
         static_for<kDepth>([&](auto d_tag) {
             constexpr int d = decltype(d_tag)::value;
-            if (s_begin + 2 * d < s_end) {
-                load_window(s_begin + 2 * d, ring[d]);
-                if constexpr (d < XD) load_x(s_begin + 2 * d, xring[d]);
-            }
+            load_window(s_begin + 2 * d, ring[d]);
+            if constexpr (d < XD) load_x(s_begin + 2 * d, xring[d]);
         });
         __syncthreads();  // first pass: the table is written; later passes: nothing pending
 
@@ -332,59 +334,54 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
             static_for<kDepth>([&](auto d_tag) {
                 constexpr int d = decltype(d_tag)::value;
                 const int step = s0 + 2 * d;
-                if (step < s_end) {
-                    // through LDS into the operand layout; the wavefront's LDS accesses execute in order
-                    asm volatile("" ::: "memory");
+                // through LDS into the operand layout; the wavefront's LDS accesses execute in order
+                asm volatile("" ::: "memory");
 #pragma unroll
-                    for (int j = 0; j < kLoads; j++)
-                        if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) *reinterpret_cast<u32x4_t *>(stage + wstore[j]) = ring[d][j];
-                    __builtin_amdgcn_wave_barrier();
-                    asm volatile("" ::: "memory");
-                    uint32_t codes[2][RG][BITS];
+                for (int j = 0; j < kLoads; j++)
+                    if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) *reinterpret_cast<u32x4_t *>(stage + wstore[j]) = ring[d][j];
+                load_window(step + 2 * kDepth, ring[d]);  // the registers are free again: refill them
+                __builtin_amdgcn_wave_barrier();
+                asm volatile("" ::: "memory");
+                uint32_t codes[2][RG][BITS];
 #pragma unroll
-                    for (int t = 0; t < 2; t++)
+                for (int t = 0; t < 2; t++)
 #pragma unroll
-                        for (int rg = 0; rg < RG; rg++)
+                    for (int rg = 0; rg < RG; rg++)
 #pragma unroll
-                            for (int p = 0; p < kPieces; p++) {
-                                const unsigned char *src = stage + wread[t][p] + rg * 32 * G::kRowBytes;
-                                if constexpr (kPiece == 4) {
-                                    const u32x4_t v = *reinterpret_cast<const u32x4_t *>(src);
-                                    codes[t][rg][4 * p] = v.x, codes[t][rg][4 * p + 1] = v.y, codes[t][rg][4 * p + 2] = v.z, codes[t][rg][4 * p + 3] = v.w;
-                                } else if constexpr (kPiece == 2) {
-                                    const u32x2_t v = *reinterpret_cast<const u32x2_t *>(src);
-                                    codes[t][rg][2 * p] = v.x, codes[t][rg][2 * p + 1] = v.y;
-                                } else {
-                                    codes[t][rg][p] = *reinterpret_cast<const uint32_t *>(src);
-                                }
+                        for (int p = 0; p < kPieces; p++) {
+                            const unsigned char *src = stage + wread[t][p] + rg * 32 * G::kRowBytes;
+                            if constexpr (kPiece == 4) {
+                                const u32x4_t v = *reinterpret_cast<const u32x4_t *>(src);
+                                codes[t][rg][4 * p] = v.x, codes[t][rg][4 * p + 1] = v.y, codes[t][rg][4 * p + 2] = v.z, codes[t][rg][4 * p + 3] = v.w;
+                            } else if constexpr (kPiece == 2) {
+                                const u32x2_t v = *reinterpret_cast<const u32x2_t *>(src);
+                                codes[t][rg][2 * p] = v.x, codes[t][rg][2 * p + 1] = v.y;
+                            } else {
+                                codes[t][rg][p] = *reinterpret_cast<const uint32_t *>(src);
                             }
-                    asm volatile("" ::: "memory");
-                    uint4 xf[2][NL];
-#pragma unroll
-                    for (int t = 0; t < 2; t++)
-#pragma unroll
-                        for (int j = 0; j < NL; j++) xf[t][j] = xring[d % XD][t][j];
-                    if (step + 2 * kDepth < s_end) load_window(step + 2 * kDepth, ring[d]);
-                    if (step + 2 * XD < s_end) load_x(step + 2 * XD, xring[d % XD]);
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        if (step + t < s_end) {
-                            float scale[RG], bias[RG];
-                            load_scales(step + t, scale, bias);
-                            static_for<4>([&](auto kk_tag) {
-                                constexpr int kk = decltype(kk_tag)::value;
-                                uint4 xa = xf[t][kk % NL];
-                                if constexpr (XR < 32) {
-                                    const bool mine = slot == kk / NL;
-                                    xa.x = mine ? xa.x : 0u, xa.y = mine ? xa.y : 0u, xa.z = mine ? xa.z : 0u, xa.w = mine ? xa.w : 0u;
-                                }
-#pragma unroll
-                                for (int rg = 0; rg < RG; rg++)
-                                    acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg], bias[rg]), acc[rg]);
-                            });
                         }
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    if (step + t < s_end) {
+                        float scale[RG], bias[RG];
+                        load_scales(step + t, scale, bias);
+                        static_for<4>([&](auto kk_tag) {
+                            constexpr int kk = decltype(kk_tag)::value;
+                            uint4 xa = xring[d % XD][t][kk % NL];
+                            if constexpr (XR < 32) {
+                                const bool mine = slot == kk / NL;
+                                xa.x = mine ? xa.x : 0u, xa.y = mine ? xa.y : 0u, xa.z = mine ? xa.z : 0u, xa.w = mine ? xa.w : 0u;
+                            }
+#pragma unroll
+                            for (int rg = 0; rg < RG; rg++)
+                                acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg], bias[rg]), acc[rg]);
+                        });
                     }
                 }
+                // x of this window is used up: refill its registers (only now, so that the same registers serve
+                // and no copy, which would have to wait for the data, is needed at the loop's end)
+                load_x(step + 2 * XD, xring[d % XD]);
             });
         }
 
