@@ -57,16 +57,39 @@ class Product:
     """One prepared nvq_quantized_matmul call: descriptor and pointers built once, so the timed
     loop is a bare C-ABI call per launch."""
 
-    def __init__(self, lib, m, x, q, y):
+    def __init__(self, lib, m, x, q, y, n=N, k=K, dtype=None):
         from nuvec_amd import _lib
         d = _lib.QmmDescC()
         d.quant = q.quant._c()
-        d.dtype, d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = _lib.BF16, 1, m, N, K, m, 0
+        d.dtype = _lib.BF16 if dtype is None else dtype
+        d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = 1, m, n, k, m, 0
         self.d, self.fn = d, lib.nvq_quantized_matmul
+        biases = q.biases.data_ptr() if q.biases is not None else None
         self.args = (C.byref(d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),
-                     C.c_void_p(q.scales.data_ptr()), C.c_void_p(q.biases.data_ptr()), C.c_void_p(y.data_ptr()),
+                     C.c_void_p(q.scales.data_ptr()), C.c_void_p(biases), C.c_void_p(y.data_ptr()),
                      C.c_void_p(None))
         self.keep = (x, q, y)
+
+    def __call__(self, stream):
+        rc = self.fn(*self.args, stream)
+        if rc:
+            from nuvec_amd import _lib
+            _lib.check(rc)
+
+
+class GatherProduct:
+    """One prepared grouped nvq_gather_qmm call (sorted pairs, one row of x per pair)."""
+
+    def __init__(self, lib, x, q, lhs, rhs, offsets, y, n, k, experts):
+        from nuvec_amd import _lib
+        pairs = rhs.numel()
+        self.d = _lib.GatherDescC(q.quant._c(), _lib.BF16, 1, 1, n, k, pairs, x.shape[0], experts)
+        self.fn = lib.nvq_gather_qmm
+        biases = q.biases.data_ptr() if q.biases is not None else None
+        self.args = (C.byref(self.d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),
+                     C.c_void_p(q.scales.data_ptr()), C.c_void_p(biases), C.c_void_p(lhs.data_ptr()),
+                     C.c_void_p(rhs.data_ptr()), C.c_void_p(offsets.data_ptr()), C.c_void_p(y.data_ptr()), C.c_void_p(None))
+        self.keep = (x, q, lhs, rhs, offsets, y)
 
     def __call__(self, stream):
         rc = self.fn(*self.args, stream)
@@ -138,6 +161,60 @@ def cpu_baseline(seconds_budget=20.0):
                       f"64-column blocks on {threads} threads"}
 
 
+def all_configs(lib, device, qs):
+    """Every BASELINE configuration, each timed like the headline: rotating weight copies beyond the
+    last-level cache, one C-ABI call per launch, best of three event-timed runs.  `qs` are the C2 weights."""
+    import numpy as np
+    import torch
+
+    import nuvec_amd as nv
+    from nuvec_amd import _lib
+    out = []
+
+    def best_of(calls, steps):
+        return min(time_launches(calls, steps, len(calls), graph=False)[0] for _ in range(3))
+
+    def products(label, n, k, quant, tdtype, code, ms_list, copies, wbytes, weights=None):
+        if weights is None:
+            gen = torch.Generator(device=device)
+            weights = []
+            for i in range(copies):
+                gen.manual_seed(4321 + i)
+                weights.append(nv.quantize((torch.randn(n, k, device=device, generator=gen) * 0.02).to(tdtype), quant))
+        for m in ms_list:
+            x = torch.randn(m, k, device=device).to(tdtype)
+            ys = [torch.empty(m, n, dtype=tdtype, device=device) for _ in weights]
+            calls = [Product(lib, m, x, q, y, n, k, code) for q, y in zip(weights, ys)]
+            ms = best_of(calls, 600 if m <= 64 else 48)
+            out.append({"config": label, "m": m, "us_per_launch": ms * 1e3, "weight_gbps": wbytes / (ms * 1e-3) / 1e9,
+                        "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12})
+
+    products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1], 48, 10_485_760)
+    products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 2048], 0, WEIGHT_BYTES,
+             weights=qs)
+    products("C4 bf16 3-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 3), torch.bfloat16, _lib.BF16, [1, 16, 512], 48,
+             7_340_032)
+    products("C4 bf16 8-bit g32 W[4096,4096]", 4096, 4096, nv.Quant.affine(32, 8), torch.bfloat16, _lib.BF16, [1, 16, 512], 32,
+             18_874_368)
+    # C5: 32 MXFP4 experts [2880,2880], 256 tokens x 4 distinct experts, pairs sorted by expert
+    experts, n, k, tokens, top = 32, 2880, 2880, 256, 4
+    weights = [nv.quantize((torch.randn(experts, n, k, device=device) * 0.02).to(torch.bfloat16), nv.QuantMode.MXFP4)
+               for _ in range(4)]
+    rng = np.random.default_rng(0)
+    choice = np.stack([rng.permutation(experts)[:top] for _ in range(tokens)]).reshape(-1)
+    rhs = torch.from_numpy(np.sort(choice).astype(np.int32)).to(device)
+    lhs = torch.arange(tokens * top, dtype=torch.int32, device=device)
+    x = torch.randn(tokens * top, 1, k, device=device).to(torch.bfloat16)
+    y = torch.empty(tokens * top, 1, n, dtype=torch.bfloat16, device=device)
+    offsets = nv.sorted_offsets(rhs, experts)
+    calls = [GatherProduct(lib, x, q, lhs, rhs, offsets, y, n, k, experts) for q in weights]
+    ms = best_of(calls, 200)
+    out.append({"config": "C5 MXFP4 gather_qmm 32 experts W[2880,2880], 1024 sorted rows", "m": tokens * top,
+                "us_per_launch": ms * 1e3, "weight_gbps": 141_004_800 / (ms * 1e-3) / 1e9,
+                "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -147,6 +224,8 @@ def main():
     ap.add_argument("--qmm-steps", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the M=2048 leg")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time every BASELINE configuration (C1..C5) and report them under \"configs\"")
     ap.add_argument("--only", choices=["qmv", "qmm", "copy"], default=None,
                     help="profiling aid: run just the rotating decode leg, just the prefill leg, or a plain 1 GiB "
                          "device copy (the known-size kernel the HBM counters are scaled by)")
@@ -215,6 +294,8 @@ def main():
                                       "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": QMM_TRAFFIC_BYTES,
                                       "kernel": "qmm4_kernel", "flop_per_launch": flop}}
 
+    if only is None and args.all_configs:
+        record["configs"] = all_configs(lib, device, qs)
     if only is None and not args.no_cpu:
         record["cpu_baseline"] = cpu_baseline()
     print(json.dumps(record))

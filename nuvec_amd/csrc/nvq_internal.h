@@ -69,7 +69,7 @@ int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
 // Rows of x from which a product goes to the tiled kernel rather than the few-row kernels
 // (the counterpart of the reference's device-specific `qmv_batch_limit`,
 // crates/nuvec-core/src/gpu.rs:1506-1538).
-constexpr int64_t kQmmMinRows = 128;
+constexpr int64_t kQmmMinRows = 193;  // seven passes of the few-row kernel cost about one tile of the tiled kernel
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
 bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);

@@ -167,6 +167,28 @@ def quantized_matmul(x, w, scales, biases, *, mode=AFFINE, group=64, bits=4, dty
     return y
 
 
+def quantized_matmul_device(x, w, scales, biases, *, group=64, bits=4, dtype=F32, rounded_weights=True):
+    """The affine product in the arithmetic of the reference's device kernels, which comes in two forms.
+    rounded_weights=True, the tiled kernels: the weights are dequantized in the element type with ONE
+    rounding of fma(code, scale, bias) (crates/nuvec-kernels/src/metal/quantized.h:583-817; the same
+    values as `affine_dequantize(fma=True)`, which the reference's device fixtures pin bit for bit).
+    rounded_weights=False, the vector kernels: scale * sum(x * code) + bias * sum(x) per group, the
+    weights never rounded (quantized.h:1358-1485).  Either way the products accumulate wider than the
+    element type (float64 here) and the sum is rounded once.  The CPU path differs in rounding the
+    weights twice (crates/nuvec-core/src/kernels.rs:835-859).  x [M, K], w [N, Kp]."""
+    x, w = _c(x), _c(w, np.uint32)
+    if rounded_weights:
+        wd = to_f32(affine_dequantize(w, scales, biases, dtype, group, bits, fma=True), dtype).astype(np.float64)
+    else:
+        codes = to_f32(affine_dequantize(w, np.ones_like(_c(scales), np.float32), np.zeros_like(_c(scales), np.float32),
+                                         F32, group, bits), F32).astype(np.float64)
+        s64 = np.repeat(to_f32(_c(scales), dtype).astype(np.float64), group, axis=-1)
+        b64 = np.repeat(to_f32(_c(biases), dtype).astype(np.float64), group, axis=-1)
+        wd = codes * s64 + b64
+    y = to_f32(x, dtype).astype(np.float64) @ wd.T
+    return from_f32(y.astype(np.float32), dtype)
+
+
 def gather_qmm(x, w, scales, biases, lhs, rhs, *, mode=AFFINE, group=64, bits=4, dtype=F32, transpose=True,
                threads=1):
     """x [xb..., M, K]; w [e..., N, Kp]; lhs/rhs broadcast-equal integer arrays of one shape."""
