@@ -1,6 +1,6 @@
-// Routing of the few-row matrix-core kernel (qmf_kernel.h): which products it takes and the
-// per-width entry points.
-#include "qmf_kernel.h"
+// Routing of the few-row and the grouped matrix-core kernels (qmf_kernel.h, qmg_kernel.h): which products
+// they take and the per-width entry points.
+#include "qmg_kernel.h"
 
 namespace nvq {
 
@@ -27,8 +27,9 @@ bool qmf_supported(const ProductArgs &a) {
     } else {
         return false;
     }
+    if (a.offsets != nullptr)  // the grouped kernel: one row of x per pair, its scale table within its LDS budget
+        return a.m == 1 && a.experts <= 65535 && qmg::table_bytes(a) <= (size_t)qmg::kTableMaxBytes;
     if (lds > (size_t)qmf::kLdsLimit) return false;
-    if (a.offsets != nullptr) return a.m == 1 && a.experts <= 65535;
     if (a.rhs != nullptr) return false;
     return (a.batch == 1 || a.batch_ndim == 1) && a.batch <= 65535 && (a.m + 31) / 32 <= 65535;
 }

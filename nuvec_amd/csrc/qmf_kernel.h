@@ -1,9 +1,7 @@
 // Few-row quantized products on the gfx950 matrix cores: y[m, n] = x[m, :] . dequantize(w[n, :]) for up to
-// 32 rows of x per pass, and the grouped (sorted) gathered product of mixture-of-experts layers, where
-// each expert's rows are such a product against that expert's weights.  Values follow nuvec's CPU product
-// (reference: crates/nuvec-core/src/kernels.rs:1091-1142, crates/nuvec-core/src/quantized.rs:679-719) within
-// the stated tolerance; the grouped route is the counterpart of the reference's `gather_qmm_rhs`
-// (crates/nuvec-kernels/src/metal/quantized.h:3301-3449, schedule at 2866-2906).
+// 32 rows of x per pass.  Values follow nuvec's CPU product (reference:
+// crates/nuvec-core/src/kernels.rs:1091-1142) within the stated tolerance.  (The grouped gathered product
+// of mixture-of-experts layers has its own kernel, qmg_kernel.h, which shares the code expansion below.)
 //
 // This header holds the kernel template; qmf_b*.hip instantiate it per code width (affine 2, 3, 4, 6, 8 bits
 // and MXFP4) so that the widths compile in parallel.
@@ -18,7 +16,7 @@
 //     operand layout, in which a lane (row n = lane % 32, half h = lane / 32) holds the 32 codes (BITS
 //     dwords) of its half of a step for every row group;
 //   * the scales and biases of the block's rows are one contiguous piece of memory: it is copied once,
-//     coalesced, into an LDS table laid out [group][row], and read from there;
+//     coalesced, into an LDS table (rows padded against bank conflicts), and read from there;
 //   * the pieces of x are shared by the row groups, and a pass of at most 8 (16) rows of x packs four
 //     (two) of a step's pieces into one load: lane (row r = l % XR, slot q = l / XR) of a half loads the
 //     pieces q NL .. q NL + NL - 1 (NL = XR / 8), the matrix instruction of piece kk takes that register with the
@@ -157,17 +155,44 @@ __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float 
     return r;
 }
 
-// GROUPED: blockIdx.z is an expert; its rows of x / y are [offsets[z], offsets[z+1]) (the last expert ends at
-// `pairs`), taken in passes of up to 32.  Otherwise blockIdx.z is a batch with one stride per operand and
-// blockIdx.y a pass of 32 rows.
-template <typename T, int BITS, bool FP4, int RG, bool GROUPED>
+// The LDS table of scales (or biases) of a block's rows keeps the memory order [row][group] with rows padded
+// to an odd number of dwords, so that the coalesced copy in writes neighbouring addresses and lanes reading
+// one group of consecutive rows fall on different banks.
+__host__ __device__ inline int table_stride(int kgroups, int elem_bytes) { return 4 * (((kgroups * elem_bytes + 3) / 4) | 1); }
+
+// Copies `count` elements (whole rows of `kgroups`) starting at `src` into the table: aligned 16-byte pieces,
+// each thread scattering its piece's elements; bytes of a piece outside the rows are dropped.
+template <typename S, int THREADS>
+__device__ __forceinline__ void fill_table(unsigned char *table, const S *src, int count, int kgroups, int stride, int tid) {
+    constexpr int kPer = 16 / (int)sizeof(S);
+    const int skew = (int)((uintptr_t)src & 15) / (int)sizeof(S);  // elements before src in its first piece
+    const uint4 *pieces = reinterpret_cast<const uint4 *>(src - skew);
+    const int n_pieces = (skew + count + kPer - 1) / kPer;
+    for (int p = tid; p < n_pieces; p += THREADS) {
+        const uint4 v = pieces[p];
+        S elems[kPer];
+        __builtin_memcpy(elems, &v, 16);
+        int idx = p * kPer - skew;  // element index of elems[0] within the block's rows
+        int row = idx >= 0 ? idx / kgroups : 0, g = idx >= 0 ? idx - row * kgroups : 0;
+#pragma unroll
+        for (int e = 0; e < kPer; e++, idx++) {
+            if (idx >= 0 && idx < count) {
+                *reinterpret_cast<S *>(table + row * stride + g * (int)sizeof(S)) = elems[e];
+                if (++g == kgroups) g = 0, row++;
+            }
+        }
+    }
+}
+
+// blockIdx.z is a batch with one stride per operand and blockIdx.y a pass of 32 rows.
+template <typename T, int BITS, bool FP4, int RG>
 __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     using G = Geometry<BITS, RG>;
     constexpr int kRows = G::kRows, kDepth = G::kDepth, kLoads = G::kLoads;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     float *partial = reinterpret_cast<float *>(lds);  // [4][RG][values][64]
     using S = std::conditional_t<FP4, uint8_t, T>;    // stored scale type
-    S *table_s = reinterpret_cast<S *>(lds + G::kFixedLdsBytes);  // [group][rows]
+    unsigned char *table_s = lds + G::kFixedLdsBytes;  // scales [rows][groups, padded]; the biases follow
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = lane >> 5, l32 = lane & 31;
@@ -175,27 +200,19 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int kgroups = K >> gshift;
     const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
-    S *table_b = table_s + kRows * kgroups;
+    const int tstride = table_stride(kgroups, (int)sizeof(S));
+    unsigned char *table_b = table_s + kRows * tstride;
     const int n0 = blockIdx.x * kRows;
 
     int row_begin, row_end;  // rows of x (and of y) this block multiplies
     int64_t xo = 0, wo = 0, so = 0, yo = 0;
-    if constexpr (GROUPED) {
-        const int e = blockIdx.z;
-        row_begin = a.offsets[e];
-        row_end = e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch;
-        if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
-        wo = (int64_t)e * N * row_bytes;
-        so = (int64_t)e * N * kgroups;
-    } else {
-        row_begin = blockIdx.y * 32;
-        row_end = row_begin + 32 < (int)a.m ? row_begin + 32 : (int)a.m;
-        if (a.batch_ndim > 0) {
-            xo = (int64_t)blockIdx.z * a.x_strides[0];
-            wo = (int64_t)blockIdx.z * a.w_strides[0] * 4;  // the stride counts packed words
-            so = (int64_t)blockIdx.z * a.s_strides[0];
-            yo = (int64_t)blockIdx.z * a.m * N;
-        }
+    row_begin = blockIdx.y * 32;
+    row_end = row_begin + 32 < (int)a.m ? row_begin + 32 : (int)a.m;
+    if (a.batch_ndim > 0) {
+        xo = (int64_t)blockIdx.z * a.x_strides[0];
+        wo = (int64_t)blockIdx.z * a.w_strides[0] * 4;  // the stride counts packed words
+        so = (int64_t)blockIdx.z * a.s_strides[0];
+        yo = (int64_t)blockIdx.z * a.m * N;
     }
     const T *x = (const T *)a.x + xo;
     T *y = (T *)a.y + yo;
@@ -252,7 +269,8 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         const int g = (step * 64 + 32 * h) >> gshift;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
-            const S *sp = table_s + g * kRows + 32 * rg + l32, *bp = table_b + g * kRows + 32 * rg + l32;
+            const int at = (32 * rg + l32) * tstride + g * (int)sizeof(S);
+            const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
             if constexpr (FP4) {
                 scale[rg] = ftz(e8m0_to_f32(*sp));
                 bias[rg] = 0.0f;
@@ -264,33 +282,11 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     };
 
     {
-        // The scales (and biases) of rows n0 .. n0 + kRows - 1 are contiguous: copy them in aligned 16-byte
-        // pieces and scatter the elements to [group][row].  Bytes of a piece outside the rows are dropped.
-        constexpr int kPer = 16 / (int)sizeof(S);
+        // The scales (and biases) of rows n0 .. n0 + kRows - 1 are contiguous in memory.
         const int valid_rows = N - n0 < kRows ? N - n0 : kRows;
-        const int count = valid_rows * kgroups;
-        const int tensors = FP4 ? 1 : 2;
-        for (int t = 0; t < tensors; t++) {
-            const S *src = (t == 0 ? (const S *)a.scales : (const S *)a.biases) + so + (int64_t)n0 * kgroups;
-            S *dst = t == 0 ? table_s : table_b;
-            const int skew = (int)((uintptr_t)src & 15) / (int)sizeof(S);  // elements before src in its first piece
-            const uint4 *pieces = reinterpret_cast<const uint4 *>(src - skew);
-            const int n_pieces = (skew + count + kPer - 1) / kPer;
-            for (int p = tid; p < n_pieces; p += kThreads) {
-                const uint4 v = pieces[p];
-                S elems[kPer];
-                __builtin_memcpy(elems, &v, 16);
-                int idx = p * kPer - skew;  // element index of elems[0] within the block's rows
-                int row = idx >= 0 ? idx / kgroups : 0, g = idx >= 0 ? idx - row * kgroups : 0;
-#pragma unroll
-                for (int e = 0; e < kPer; e++, idx++) {
-                    if (idx >= 0 && idx < count) {
-                        dst[g * kRows + row] = elems[e];
-                        if (++g == kgroups) g = 0, row++;
-                    }
-                }
-            }
-        }
+        fill_table<S, kThreads>(table_s, (const S *)a.scales + so + (int64_t)n0 * kgroups, valid_rows * kgroups, kgroups, tstride, tid);
+        if constexpr (!FP4)
+            fill_table<S, kThreads>(table_b, (const S *)a.biases + so + (int64_t)n0 * kgroups, valid_rows * kgroups, kgroups, tstride, tid);
     }
 
     // One pass over at most XR rows of x (XR = 8, 16 or 32).
@@ -301,9 +297,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         constexpr int NV = XR / 2;        // values of the tile per lane and row group once the slots are added
         const int r = l32 % XR, slot = l32 / XR;
         const bool live = r < rows;  // this lane's row of x exists
-        // x row of this lane; in the grouped route rows are gathered through lhs (arange for sorted gathers)
-        int64_t xr = pass + (live ? r : 0);
-        if constexpr (GROUPED) xr = a.lhs != nullptr ? (int64_t)a.lhs[xr] : xr;
+        const int64_t xr = pass + (live ? r : 0);  // x row of this lane
         const T *xrow = x + xr * K + 32 * h + 8 * NL * slot;  // piece kk of half h covers k0 + 32 h + 8 kk .. + 8
 
         floatx16_t acc[RG];
@@ -440,23 +434,22 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
 
 // Bytes of the LDS table of scales (and biases) for `rows` weight rows.
 inline size_t table_bytes(const ProductArgs &a, int rows) {
-    const int64_t group = a.mode == NVQ_MXFP4 ? 32 : a.group;
-    const int64_t bytes = a.mode == NVQ_MXFP4 ? rows * (a.k / group) : 2 * rows * (a.k / group) * 2;
+    const bool fp4 = a.mode == NVQ_MXFP4;
+    const int64_t bytes = (int64_t)rows * table_stride((int)(a.k / (fp4 ? 32 : a.group)), fp4 ? 1 : 2) * (fp4 ? 1 : 2);
     return (size_t)((bytes + 15) & ~(int64_t)15);
 }
 
 // Groups of 32 weight rows per block: two, unless that leaves most compute units without a block.
 inline int row_groups(const ProductArgs &a) {
-    if (a.offsets != nullptr) return 2;
     const int64_t blocks = ((a.n + 63) / 64) * ((a.m + 31) / 32) * a.batch;
     return blocks >= 192 ? 2 : 1;
 }
 
-template <typename T, int BITS, bool FP4, int RG, bool GROUPED>
+template <typename T, int BITS, bool FP4, int RG>
 int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS, RG>;
     static bool configured = false;
-    auto kernel = qmf_kernel<T, BITS, FP4, RG, GROUPED>;
+    auto kernel = qmf_kernel<T, BITS, FP4, RG>;
     if (!configured) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
         configured = true;
@@ -464,7 +457,7 @@ int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     const size_t lds_bytes = G::kFixedLdsBytes + table_bytes(a, G::kRows);
     if (lds_bytes > (size_t)kLdsLimit) return fail(NVQ_UNSUPPORTED, "quantized_matmul: K = %lld needs a %zu-byte LDS table", (long long)a.k, lds_bytes);
     const unsigned gx = (unsigned)((a.n + G::kRows - 1) / G::kRows);
-    const dim3 grid = GROUPED ? dim3(gx, 1, (unsigned)a.experts) : dim3(gx, (unsigned)((a.m + 31) / 32), (unsigned)a.batch);
+    const dim3 grid(gx, (unsigned)((a.m + 31) / 32), (unsigned)a.batch);
     hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmf");
     return NVQ_OK;
@@ -472,8 +465,7 @@ int32_t run_variant(const ProductArgs &a, hipStream_t s) {
 
 template <typename T, int BITS, bool FP4>
 int32_t run_width(const ProductArgs &a, hipStream_t s) {
-    if (a.offsets != nullptr) return run_variant<T, BITS, FP4, 2, true>(a, s);
-    return row_groups(a) == 2 ? run_variant<T, BITS, FP4, 2, false>(a, s) : run_variant<T, BITS, FP4, 1, false>(a, s);
+    return row_groups(a) == 2 ? run_variant<T, BITS, FP4, 2>(a, s) : run_variant<T, BITS, FP4, 1>(a, s);
 }
 
 template <int BITS, bool FP4>

@@ -1,0 +1,285 @@
+// The grouped (sorted) gathered product of mixture-of-experts layers on the gfx950 matrix cores: the rows of
+// x that belong to expert e, [offsets[e], offsets[e+1]), times that expert's weights, every weight decoded
+// once per pass of 64 rows.  Counterpart of the reference's `gather_qmm_rhs`
+// (crates/nuvec-kernels/src/metal/quantized.h:3301-3449, schedule at 2866-2906); values follow nuvec's CPU
+// product (crates/nuvec-core/src/quantized.rs:679-719, crates/nuvec-core/src/kernels.rs:1091-1142) within the
+// stated tolerance.
+//
+// Experts give the launch its parallelism, so a block does not split K: a block of four wavefronts owns
+// 128 weight rows of one expert (32 per wavefront) and all wavefronts walk K together in windows of 128
+// values.  Per window
+//   * the block's 256 threads bring the x tile (up to 64 rows x 256 bytes, rows gathered through lhs) with
+//     four coalesced 16-byte loads each, one window ahead, into one of two LDS stages (chunks XOR-swizzled
+//     by row), from which every wavefront reads its matrix operands (one or two tiles of 32 rows): x leaves
+//     the cache once per 128 weight rows;
+//   * each wavefront fetches its own 32 weight rows of the window (16 BITS bytes per row) with coalesced
+//     loads into registers several windows ahead and passes them through a private piece of LDS into the
+//     operand layout, exactly as the few-row kernel does (qmf_kernel.h), and expands them in registers;
+//   * scales (and biases) of the block's rows come from an LDS table filled once per block.
+// A wavefront owns its 32 x 32 tiles of y outright, so nothing is reduced across wavefronts.
+#pragma once
+
+#include "qmf_kernel.h"
+
+namespace nvq {
+namespace qmg {
+
+using namespace qmf;  // element operations, code expansion, static_for
+
+constexpr int kWaves = 4;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kRows = 32 * kWaves;            // weight rows per block
+constexpr int kPassRows = 64;                 // rows of x per pass: two tiles of 32
+constexpr int kXStageBytes = kPassRows * 256;  // one window of x: 64 rows x 128 values
+constexpr int kTableMaxBytes = 48 * 1024;
+
+template <int BITS>
+struct Geometry {
+    static constexpr int kChunks = 32 * BITS;              // 16-byte chunks of one wavefront's window
+    static constexpr int kLoads = (kChunks + 63) / 64;     // loads per lane and window
+    static constexpr int kDepth = 2;                       // windows of weights in flight per lane
+    static constexpr int kRowBytes = 16 * BITS;            // of one row in a window
+    static constexpr int kStageBytes = kChunks * 16;       // one window of one wavefront
+    static constexpr int kFixedLdsBytes = 2 * kXStageBytes + kWaves * kStageBytes;
+    static constexpr bool kPow2 = (BITS & (BITS - 1)) == 0;
+    __host__ __device__ static constexpr int swizzle(int row) { return kPow2 ? (row / (BITS >= 16 ? 1 : 16 / BITS)) % BITS : 0; }
+};
+
+template <typename T, int BITS, bool FP4>
+__global__ void __launch_bounds__(kThreads) qmg_kernel(const ProductArgs a) {
+    using G = Geometry<BITS>;
+    constexpr int kDepth = G::kDepth, kLoads = G::kLoads;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    using S = std::conditional_t<FP4, uint8_t, T>;  // stored scale type
+    unsigned char *table_s = lds + G::kFixedLdsBytes;  // scales [rows][groups, padded]; the biases follow
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, l32 = lane & 31;
+    const int K = (int)a.k, N = (int)a.n;
+    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int kgroups = K >> gshift;
+    const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
+    const int tstride = table_stride(kgroups, (int)sizeof(S));
+    unsigned char *table_b = table_s + kRows * tstride;
+    const int n0 = blockIdx.x * kRows;
+    const int e = blockIdx.z;
+    const int row_begin = a.offsets[e];
+    const int row_end = e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch;
+    if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
+    const int64_t wo = (int64_t)e * N * row_bytes, so = (int64_t)e * N * kgroups;
+    const T *x = (const T *)a.x;
+    T *y = (T *)a.y;
+
+    const int steps = K >> 6;             // K is a multiple of 64 (checked on the host)
+    const int windows = (steps + 1) >> 1;  // the last window may hold one step
+
+    // Weight window loads of this wavefront: load j of a lane is chunk q = 64 j + lane, i.e. chunk q % BITS of
+    // row q / BITS of the wavefront's 32 rows.  Chunks of the window's second step begin at BITS / 2 (a window
+    // of one step exists only for even BITS; its lanes fetch the first step again).
+    const unsigned char *wload[kLoads];
+    int wstore[kLoads];
+    bool second[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; j++) {
+        const int q = 64 * j + lane, qc = q < G::kChunks ? q : G::kChunks - 1;
+        const int row = qc / BITS, c = qc % BITS;
+        const int n = n0 + 32 * wave + row < N ? n0 + 32 * wave + row : N - 1;  // tail rows are computed, not stored
+        wload[j] = (const unsigned char *)a.w + wo + (int64_t)n * row_bytes + 16 * c;
+        wstore[j] = row * G::kRowBytes + 16 * (c ^ G::swizzle(row));
+        second[j] = 2 * c >= BITS;
+    }
+    // Every load of the K loop is issued on every path (a window past the end loads one 16-byte piece, the
+    // same for all lanes), so that the waits can leave the younger windows' loads in flight.
+    auto load_window = [&](int win, u32x4_t (&w)[kLoads]) {
+        const bool real = win < windows, half = 2 * win + 1 >= steps;
+#pragma unroll
+        for (int j = 0; j < kLoads; j++) {
+            const int off = win * 16 * BITS - ((half && second[j]) ? 8 * BITS : 0);
+            const unsigned char *src = real ? wload[j] + off : (const unsigned char *)a.w;
+            w[j] = *reinterpret_cast<const u32x4_a4_t *>(src);
+        }
+    };
+    unsigned char *stage = lds + 2 * kXStageBytes + wave * G::kStageBytes;
+    constexpr int kPiece = BITS % 4 == 0 ? 4 : BITS % 2 == 0 ? 2 : 1;  // dwords per LDS read
+    constexpr int kPieces = BITS / kPiece;
+    int wread[2][kPieces];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int p = 0; p < kPieces; p++) {
+            const int byte = (2 * t + h) * 4 * BITS + 4 * kPiece * p;  // within the row
+            wread[t][p] = l32 * G::kRowBytes + 16 * ((byte >> 4) ^ G::swizzle(l32)) + (byte & 15);
+        }
+
+    auto load_scales = [&](int step, float &scale, float &bias) {
+        const int g = (step * 64 + 32 * h) >> gshift;
+        const int at = (32 * wave + l32) * tstride + g * (int)sizeof(S);
+        const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
+        if constexpr (FP4) {
+            scale = ftz(e8m0_to_f32(*sp));
+            bias = 0.0f;
+        } else {
+            scale = Elem<T>::load(sp, 0);
+            bias = Elem<T>::load(bp, 0);
+        }
+    };
+
+    {
+        // The scales (and biases) of rows n0 .. n0 + 127 are contiguous in memory.
+        const int valid_rows = N - n0 < kRows ? N - n0 : kRows;
+        fill_table<S, kThreads>(table_s, (const S *)a.scales + so + (int64_t)n0 * kgroups, valid_rows * kgroups, kgroups, tstride, tid);
+        if constexpr (!FP4)
+            fill_table<S, kThreads>(table_b, (const S *)a.biases + so + (int64_t)n0 * kgroups, valid_rows * kgroups, kgroups, tstride, tid);
+    }
+
+    // x tile loads: thread t brings chunks t + 256 i (i < 4) of a window's 1024 (chunk q: row q / 16, 16-byte
+    // piece q % 16); piece c of row r is stored at position c ^ (r % 16).  The operand of piece kk of step t
+    // for lane (row r = lane % 32, half h) of tile u is piece 8 t + 4 h + kk of row 32 u + r.
+    const int xc = tid & 15;
+    int xstore[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int r = (tid >> 4) + 16 * i;
+        xstore[i] = r * 256 + 16 * (xc ^ (r & 15));
+    }
+    int xread[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) xread[t][kk] = l32 * 256 + 16 * ((8 * t + 4 * h + kk) ^ (l32 & 15));
+
+    for (int pass = row_begin; pass < row_end; pass += kPassRows) {
+        const int rows = row_end - pass < kPassRows ? row_end - pass : kPassRows;
+        const bool two = rows > 32;  // the pass has a second tile of rows
+        // rows of x behind this thread's four chunks, gathered through lhs; a row past the pass reads the
+        // start of x (its tile row is never stored)
+        const T *xsrc[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = (tid >> 4) + 16 * i;
+            int64_t g = pass + (r < rows ? r : 0);
+            g = a.lhs != nullptr ? (int64_t)a.lhs[g] : g;
+            xsrc[i] = x + (r < rows ? g * K : 0) + 8 * xc;
+        }
+        auto load_x = [&](int win, u32x4_t (&xq)[4]) {
+            // a window of one step has no second half: those chunks (pieces 8..15) fetch the first half again
+            const int k0 = win < windows ? win * 128 - ((2 * win + 1 >= steps && xc >= 8) ? 64 : 0) : 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) xq[i] = *reinterpret_cast<const u32x4_t *>(xsrc[i] + k0);
+        };
+        auto store_x = [&](int win, const u32x4_t (&xq)[4]) {
+            unsigned char *dst = lds + (win & 1) * kXStageBytes;
+#pragma unroll
+            for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4_t *>(dst + xstore[i]) = xq[i];
+        };
+
+        floatx16_t acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int el = 0; el < 16; el++) acc[u][el] = 0.0f;
+
+        u32x4_t xq[2][4];                   // x chunks of the next two windows
+        u32x4_t ring[kDepth][kLoads] = {};  // weight windows in flight
+        load_x(0, xq[0]);
+        load_x(1, xq[1]);
+        static_for<kDepth>([&](auto d_tag) {
+            constexpr int d = decltype(d_tag)::value;
+            load_window(d, ring[d]);
+        });
+        store_x(0, xq[0]);
+        load_x(2, xq[0]);
+        __syncthreads();  // window 0 of x is in LDS (first pass: the table too)
+
+        for (int w0 = 0; w0 < windows; w0 += kDepth) {
+            static_for<kDepth>([&](auto d_tag) {
+                constexpr int d = decltype(d_tag)::value;
+                const int win = w0 + d;
+                // weights through LDS into the operand layout; the wavefront's LDS accesses execute in order
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int j = 0; j < kLoads; j++)
+                    if (G::kChunks % 64 == 0 || 64 * j + lane < G::kChunks) *reinterpret_cast<u32x4_t *>(stage + wstore[j]) = ring[d][j];
+                load_window(win + kDepth, ring[d]);  // the registers are free again: refill them
+                __builtin_amdgcn_wave_barrier();
+                asm volatile("" ::: "memory");
+                uint32_t codes[2][BITS];
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int p = 0; p < kPieces; p++) {
+                        const unsigned char *src = stage + wread[t][p];
+                        if constexpr (kPiece == 4) {
+                            const u32x4_t v = *reinterpret_cast<const u32x4_t *>(src);
+                            codes[t][4 * p] = v.x, codes[t][4 * p + 1] = v.y, codes[t][4 * p + 2] = v.z, codes[t][4 * p + 3] = v.w;
+                        } else if constexpr (kPiece == 2) {
+                            const u32x2_t v = *reinterpret_cast<const u32x2_t *>(src);
+                            codes[t][2 * p] = v.x, codes[t][2 * p + 1] = v.y;
+                        } else {
+                            codes[t][p] = *reinterpret_cast<const uint32_t *>(src);
+                        }
+                    }
+                asm volatile("" ::: "memory");
+                if (win < windows) {
+                    const unsigned char *xs = lds + (win & 1) * kXStageBytes;
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        if (2 * win + t < steps) {
+                            float scale, bias;
+                            load_scales(2 * win + t, scale, bias);
+                            static_for<4>([&](auto kk_tag) {
+                                constexpr int kk = decltype(kk_tag)::value;
+                                const uint4 wb = expand_piece<T, BITS, FP4, kk>(codes[t], scale, bias);
+                                acc[0] = Ops<T>::mfma(*reinterpret_cast<const uint4 *>(xs + xread[t][kk]), wb, acc[0]);
+                                if (two) acc[1] = Ops<T>::mfma(*reinterpret_cast<const uint4 *>(xs + 32 * 256 + xread[t][kk]), wb, acc[1]);
+                            });
+                        }
+                    }
+                }
+                // the next window of x goes into the other stage (last read one window ago, before the previous
+                // barrier); its registers then take the window after the next
+                store_x(win + 1, xq[(d + 1) & 1]);
+                load_x(win + 3, xq[(d + 1) & 1]);
+                __syncthreads();
+            });
+        }
+
+        // Accumulator element el of lane l is tile row 8 (el / 4) + 4 (l / 32) + el % 4 (a row of x), column l % 32.
+        const int col = n0 + 32 * wave + l32;
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int el = 0; el < 16; el++) {
+                const int m = 32 * u + 8 * (el >> 2) + 4 * h + (el & 3);
+                if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, acc[u][el]);
+            }
+    }
+}
+
+// Bytes of the LDS table of scales (and biases) for the block's rows.
+inline size_t table_bytes(const ProductArgs &a) { return qmf::table_bytes(a, kRows); }
+
+template <typename T, int BITS, bool FP4>
+int32_t run(const ProductArgs &a, hipStream_t s) {
+    using G = Geometry<BITS>;
+    static bool configured = false;
+    auto kernel = qmg_kernel<T, BITS, FP4>;
+    const size_t lds_bytes = G::kFixedLdsBytes + table_bytes(a);
+    if (!configured) {
+        NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        G::kFixedLdsBytes + kTableMaxBytes));
+        configured = true;
+    }
+    const dim3 grid((unsigned)((a.n + kRows - 1) / kRows), 1, (unsigned)a.experts);
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
+    NVQ_LAUNCH_CHECK("qmg");
+    return NVQ_OK;
+}
+
+template <int BITS, bool FP4>
+int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
+    return a.dtype == NVQ_BF16 ? run<bf16_t, BITS, FP4>(a, s) : run<f16_t, BITS, FP4>(a, s);
+}
+
+}  // namespace qmg
+}  // namespace nvq
