@@ -333,10 +333,11 @@ int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, c
     a.lhs = lhs; a.rhs = rhs;
     a.x_batches = d->x_batches; a.experts = d->experts;
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
-    // weight decoded once.  Otherwise one product per pair.
+    // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;
     if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     a.offsets = nullptr;
+    if (qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }
 

@@ -6,8 +6,8 @@ namespace nvq {
 
 // Whether the few-row matrix-core kernel takes this product: MXFP4 or affine 2, 3, 4, 6 or 8 bits, bf16 or
 // f16, whole steps of 64 values (whole windows of 128 for 3 bits, whose 16-byte chunks straddle steps),
-// a scale table that fits in LDS, and either no batch, a batch with one stride per operand, or the grouped
-// gather.
+// a scale table that fits in LDS, and either no batch, a batch with one stride per operand, gathered pairs,
+// or the grouped gather.
 bool qmf_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.k < 64 || a.k % 64 != 0) return false;
@@ -30,7 +30,7 @@ bool qmf_supported(const ProductArgs &a) {
     if (a.offsets != nullptr)  // the grouped kernel: one row of x per pair, its scale table within its LDS budget
         return a.m == 1 && a.experts <= 65535 && qmg::table_bytes(a) <= (size_t)qmg::kTableMaxBytes;
     if (lds > (size_t)qmf::kLdsLimit) return false;
-    if (a.rhs != nullptr) return false;
+    if (a.rhs != nullptr) return a.batch <= 65535 && (a.m + 31) / 32 <= 65535;  // gathered pairs, one per grid z
     return (a.batch == 1 || a.batch_ndim == 1) && a.batch <= 65535 && (a.m + 31) / 32 <= 65535;
 }
 

@@ -184,7 +184,7 @@ __device__ __forceinline__ void fill_table(unsigned char *table, const S *src, i
     }
 }
 
-// blockIdx.z is a batch with one stride per operand and blockIdx.y a pass of 32 rows.
+// blockIdx.z is a batch with one stride per operand, or a gathered pair; blockIdx.y a pass of 32 rows.
 template <typename T, int BITS, bool FP4, int RG>
 __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     using G = Geometry<BITS, RG>;
@@ -208,7 +208,14 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     int64_t xo = 0, wo = 0, so = 0, yo = 0;
     row_begin = blockIdx.y * 32;
     row_end = row_begin + 32 < (int)a.m ? row_begin + 32 : (int)a.m;
-    if (a.batch_ndim > 0) {
+    if (a.rhs != nullptr) {  // gathered pairs: pair z takes x batch lhs[z] and weight matrix rhs[z]
+        // An index outside its operand is the caller's error; it is clamped so that it cannot fault the device.
+        const int64_t l = min((int64_t)a.lhs[blockIdx.z], a.x_batches - 1), r = min((int64_t)a.rhs[blockIdx.z], a.experts - 1);
+        xo = l * a.m * K;
+        wo = r * N * row_bytes;
+        so = r * N * kgroups;
+        yo = (int64_t)blockIdx.z * a.m * N;
+    } else if (a.batch_ndim > 0) {
         xo = (int64_t)blockIdx.z * a.x_strides[0];
         wo = (int64_t)blockIdx.z * a.w_strides[0] * 4;  // the stride counts packed words
         so = (int64_t)blockIdx.z * a.s_strides[0];
