@@ -11,6 +11,8 @@
 
 #include "nvq_internal.h"
 
+#include <math.h>
+
 namespace nvq {
 
 namespace {
@@ -137,6 +139,20 @@ int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose
 }  // namespace nvq
 
 using namespace nvq;
+
+// Estimated cost of the two matrix-core routes, from their measured behaviour: the tiled kernel walks K in
+// steps of 64 at about 1.7 us per step and round of 256 x 256 tiles over the compute units; the few-row kernel
+// takes a pass per 32 rows, each bound by the expansion of every weight (0.29 us per million weights) and
+// never under 4 us.  The counterpart of the reference's device-specific `qmv_batch_limit`
+// (crates/nuvec-core/src/gpu.rs:1506-1538).
+static bool tiled_is_faster(const nvq::ProductArgs &a) {
+    const double tiles = (double)((a.m + 255) / 256) * (double)((a.n + 255) / 256) * (double)a.batch;
+    const double rounds = ceil(tiles / (double)nvq::compute_units());
+    const double tiled_us = rounds * (double)(a.k / 64) * 1.7;
+    const double pass_us = fmax(4.0, 0.29e-6 * (double)a.n * (double)a.k);
+    const double few_us = (double)((a.m + 31) / 32) * pass_us * (double)a.batch / fmax(1.0, fmin((double)a.batch, 256.0 / fmax(1.0, (double)((a.n + 63) / 64))));
+    return tiled_us < few_us;
+}
 
 extern "C" {
 
@@ -283,9 +299,10 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
         a.w_strides[i] = d->w_strides[i];
         a.s_strides[i] = d->s_strides[i];
     }
-    // Routed by one item's rows, as the reference does (gpu.rs:6975-6981).
+    // Routed by one item's rows, as the reference does (gpu.rs:6975-6981): the tiled kernel where its tiles
+    // cost less than the passes of the few-row kernel.
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
-    if (item >= kQmmMinRows && qmm_supported(a)) return launch_qmm(a, (hipStream_t)stream);
+    if (item > 32 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a))) return launch_qmm(a, (hipStream_t)stream);
     // Up to four rows of 4-bit affine weights: the decode kernel (per-row work on the vector units, which is
     // cheaper than the matrix-core kernel's full dequantization up to there).  Other few-row products share
     // one weight decode on the matrix cores where that kernel takes them.

@@ -66,10 +66,6 @@ int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
 bool qmm_supported(const ProductArgs &a);
 int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
-// Rows of x from which a product goes to the tiled kernel rather than the few-row kernels
-// (the counterpart of the reference's device-specific `qmv_batch_limit`,
-// crates/nuvec-core/src/gpu.rs:1506-1538).
-constexpr int64_t kQmmMinRows = 193;  // seven passes of the few-row kernel cost about one tile of the tiled kernel
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
 bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);

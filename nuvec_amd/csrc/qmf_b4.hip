@@ -1,10 +1,14 @@
-// The few-row and the grouped matrix-core kernels for affine 4-bit codes (qmf_kernel.h, qmg_kernel.h).
+// The few-row, grouped and tiled matrix-core kernels for affine 4-bit codes (qmf_kernel.h, qmg_kernel.h,
+// qmm_kernel.h).
 #include "qmg_kernel.h"
+#include "qmm_kernel.h"
 
 namespace nvq {
 
 int32_t launch_qmf_b4(const ProductArgs &a, hipStream_t s) {
     return a.offsets != nullptr ? qmg::run_dtype<4, false>(a, s) : qmf::run_dtype<4, false>(a, s);
 }
+
+int32_t launch_qmm_b4(const ProductArgs &a, hipStream_t s) { return qmm::run_dtype<4, false>(a, s); }
 
 }  // namespace nvq
