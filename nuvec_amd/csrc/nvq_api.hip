@@ -140,18 +140,15 @@ int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose
 
 using namespace nvq;
 
-// Estimated cost of the two matrix-core routes, from their measured behaviour: the tiled kernel walks K in
-// steps of 64 at about 1.7 us per step and round of 256 x 256 tiles over the compute units; the few-row kernel
-// takes a pass per 32 rows, each bound by the expansion of every weight (0.29 us per million weights) and
-// never under 4 us.  The counterpart of the reference's device-specific `qmv_batch_limit`
+// Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row
+// kernel takes a pass per 32 rows, each bound by the expansion of every weight (0.29 us per million weights)
+// and never under 4 us.  The counterpart of the reference's device-specific `qmv_batch_limit`
 // (crates/nuvec-core/src/gpu.rs:1506-1538).
 static bool tiled_is_faster(const nvq::ProductArgs &a) {
-    const double tiles = (double)((a.m + 255) / 256) * (double)((a.n + 255) / 256) * (double)a.batch;
-    const double rounds = ceil(tiles / (double)nvq::compute_units());
-    const double tiled_us = rounds * (double)(a.k / 64) * 1.7;
     const double pass_us = fmax(4.0, 0.29e-6 * (double)a.n * (double)a.k);
-    const double few_us = (double)((a.m + 31) / 32) * pass_us * (double)a.batch / fmax(1.0, fmin((double)a.batch, 256.0 / fmax(1.0, (double)((a.n + 63) / 64))));
-    return tiled_us < few_us;
+    const double at_once = fmax(1.0, fmin((double)a.batch, 256.0 / fmax(1.0, (double)((a.n + 63) / 64))));  // batch items side by side
+    const double few_us = (double)((a.m + 31) / 32) * pass_us * (double)a.batch / at_once;
+    return nvq::qmm_estimate_us(a) < few_us;
 }
 
 extern "C" {

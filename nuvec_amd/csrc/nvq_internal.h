@@ -66,6 +66,7 @@ int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
 bool qmm_supported(const ProductArgs &a);
 int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
+double qmm_estimate_us(const ProductArgs &a);  // estimated duration of the tiled kernel with its better tile
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
 bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);

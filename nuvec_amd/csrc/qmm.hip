@@ -18,6 +18,11 @@ bool qmm_supported(const ProductArgs &a) {
     return a.batch <= 65535 && a.k >= qmm::BK && a.k % qmm::BK == 0;
 }
 
+double qmm_estimate_us(const ProductArgs &a) {
+    const int cus = compute_units();
+    return fmin(qmm::estimate_us<qmm::BigTile>(a, cus), qmm::estimate_us<qmm::SmallTile>(a, cus));
+}
+
 int32_t launch_qmm(const ProductArgs &a, hipStream_t s) {
     if (a.mode == NVQ_MXFP4) return launch_qmm_fp4(a, s);
     switch (a.bits) {

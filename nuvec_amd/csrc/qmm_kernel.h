@@ -7,7 +7,8 @@
 // (crates/nuvec-kernels/src/metal/quantized.h:583-817, 1358-1485).
 //
 // One block of 512 threads (eight wavefronts, 2 x 4, each 128 x 64 of y) owns a BM x BN = 256 x 256 tile
-// and walks K in steps of BK = 64 through a ring of three LDS stages.  A stage holds
+// and walks K in steps of BK = 64 through a ring of three LDS stages (products whose 256 x 256 tiles would not
+// fill the chip take 128 x 128 tiles of four wavefronts, two blocks per compute unit).  A stage holds
 //   * the x tile, 256 rows x 128 B, 16-byte chunk index XOR-ed with (row & 7) so that the 16-byte
 //     fragment reads of the matrix instruction are bank-conflict free, and
 //   * the w tile still packed, 256 rows x 8 BITS bytes: lane (row, half) of the loading threads owns the BITS
@@ -26,18 +27,31 @@
 
 #include "qmf_kernel.h"
 
+#include <math.h>
+
 namespace nvq {
 namespace qmm {
 
 using namespace qmf;  // element operations and code expansion
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 512;
+constexpr int BK = 64;
 constexpr int kStages = 3;
-constexpr int kRowBytes = BK * 2;                    // 128 B per x row in LDS
-constexpr int kXBytes = BM * kRowBytes;              // 32 KB
-constexpr int kPeriod = 256;                         // values of K per scale/bias table
-constexpr int kSbBytes = (kPeriod / 32) * BN * 4;    // one table: up to 8 groups x 256 rows x (scale, bias)
+constexpr int kRowBytes = BK * 2;   // 128 B per x row in LDS
+constexpr int kPeriod = 256;        // values of K per scale/bias table
+
+// A block's tile: WM x WN wavefronts, each TI x TJ matrix tiles of 32 x 32.  The number of threads equals
+// twice the weight rows (one loading lane per row half) and the x tile takes four 16-byte pieces per thread.
+template <int WM_, int WN_, int TI_, int TJ_>
+struct Tile {
+    static constexpr int WM = WM_, WN = WN_, TI = TI_, TJ = TJ_;
+    static constexpr int BM = WM * TI * 32, BN = WN * TJ * 32;
+    static constexpr int kThreads = WM * WN * 64;
+    static constexpr int kXBytes = BM * kRowBytes;
+    static constexpr int kSbBytes = (kPeriod / 32) * BN * 4;  // one table: up to 8 groups x BN rows x (scale, bias)
+    static_assert(kThreads == 2 * BN && BM * 8 == 4 * kThreads, "the loading assignment below assumes these");
+};
+using BigTile = Tile<2, 4, 4, 2>;    // 256 x 256, 512 threads
+using SmallTile = Tile<2, 2, 2, 2>;  // 128 x 128, 256 threads: for products whose big tiles would not fill the chip
 
 // How a lane's BITS dwords travel into LDS: one or two pieces of 4, 3 or 1 dwords.
 template <int BITS> struct Pieces;
@@ -47,14 +61,14 @@ template <> struct Pieces<4> { static constexpr int count = 1, dwords = 4; };
 template <> struct Pieces<6> { static constexpr int count = 2, dwords = 3; };
 template <> struct Pieces<8> { static constexpr int count = 2, dwords = 4; };
 
-template <int BITS>
+template <int BITS, class TL>
 struct Geometry {
     // a 12-byte piece lands at 16 bytes per lane, like a 16-byte one (its fourth dword is not written)
     static constexpr int kPieceBytes = Pieces<BITS>::dwords == 1 ? 4 : 16;  // of LDS per lane and piece
-    static constexpr int kRegionBytes = kThreads * kPieceBytes;         // one piece of every loading lane
-    static constexpr int kWBytes = Pieces<BITS>::count * kRegionBytes;  // packed codes of one step: 4 KB .. 16 KB
-    static constexpr int kStageBytes = kXBytes + kWBytes;
-    static constexpr int kLdsBytes = kStages * kStageBytes + 2 * kSbBytes;  // 136 KB at 4 bits, 160 KB at 8
+    static constexpr int kRegionBytes = TL::kThreads * kPieceBytes;     // one piece of every loading lane
+    static constexpr int kWBytes = Pieces<BITS>::count * kRegionBytes;  // packed codes of one step
+    static constexpr int kStageBytes = TL::kXBytes + kWBytes;
+    static constexpr int kLdsBytes = kStages * kStageBytes + 2 * TL::kSbBytes;  // big tile: 136 KB at 4 bits, 160 KB at 8
     static constexpr int kParts = 4 + Pieces<BITS>::count;              // direct-to-LDS loads per step and lane
 };
 
@@ -87,9 +101,11 @@ __device__ __forceinline__ void dma_wait() {  // all but the N most recent vecto
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <typename T, int BITS, bool FP4, bool BATCHED>
-__global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
-    using G = Geometry<BITS>;
+template <typename T, int BITS, bool FP4, bool BATCHED, class TL>
+__global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) {
+    using G = Geometry<BITS, TL>;
+    constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kXBytes = TL::kXBytes, kSbBytes = TL::kSbBytes;
+    constexpr int TI = TL::TI, TJ = TL::TJ;
     using P = Pieces<BITS>;
     using S = std::conditional_t<FP4, uint8_t, T>;  // stored scale type
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -97,7 +113,7 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
     uint32_t *sb_table = reinterpret_cast<uint32_t *>(lds + kStages * G::kStageBytes);  // [2][group][row]: scale | bias << 16
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = (wave >> 2) & 1, wn = wave & 3;  // wavefront grid 2 x 4: 128 x 64 each
+    const int wm = wave / TL::WN, wn = wave % TL::WN;  // wavefront grid WM x WN: 32 TI x 32 TJ each
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int row_dwords = (K >> 5) * BITS, kgroups = K >> gshift;
@@ -122,7 +138,7 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
     const T *xsrc[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int slot = i * 512 + wave * 64 + lane, row = slot >> 3, chunk = (slot & 7) ^ (row & 7);
+        const int slot = i * kThreads + wave * 64 + lane, row = slot >> 3, chunk = (slot & 7) ^ (row & 7);
         const int grow = m0 + row < M ? m0 + row : M - 1;  // tail rows are computed, not stored
         xsrc[i] = x + (int64_t)grow * K + chunk * 8;
     }
@@ -135,7 +151,7 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         const int sc = step < steps ? step : steps - 1;  // past the end: a harmless reload, keeps the wait counts uniform
         const uint32_t base = lds0 + (step % kStages) * G::kStageBytes;
         if (part < 4) {
-            dma<4>(xsrc[part] + sc * BK, base + (part * 512 + wave * 64) * 16);
+            dma<4>(xsrc[part] + sc * BK, base + (part * kThreads + wave * 64) * 16);
         } else {
             const int piece = part - 4;
             dma<P::dwords>(wsrc + sc * 2 * BITS + piece * P::dwords, base + kXBytes + piece * G::kRegionBytes + wave * 64 * G::kPieceBytes);
@@ -146,12 +162,12 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         for (int part = 0; part < G::kParts; part++) issue_part(step, part);
     };
 
-    // Scale/bias tables: thread t < 256 owns tile row t.
-    const int srow = n0 + (tid & 255) < N ? n0 + (tid & 255) : N - 1;
+    // Scale/bias tables: thread t < BN owns tile row t.
+    const int srow = n0 + (tid % BN) < N ? n0 + (tid % BN) : N - 1;
     const S *sp = scales + (int64_t)srow * kgroups, *bp = biases + (int64_t)srow * kgroups;
     S sreg[8], breg[8];
     auto sb_load = [&](int period) {
-        if (tid < 256) {
+        if (tid < BN) {
 #pragma unroll
             for (int g = 0; g < 8; g++)
                 if (g < gper) {
@@ -162,7 +178,7 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         }
     };
     auto sb_store = [&](int period) {
-        if (tid < 256) {
+        if (tid < BN) {
             uint32_t *t = sb_table + (period & 1) * (kSbBytes / 4);
 #pragma unroll
             for (int g = 0; g < 8; g++)
@@ -179,11 +195,11 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         }
     };
 
-    floatx16_t acc[4][2];
+    floatx16_t acc[TI][TJ];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
@@ -202,11 +218,11 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         for (int part = 4; part < G::kParts; part++) issue_part(step + 2, part);  // the x parts are spread over the matrix work below
         const unsigned char *xs = lds + (step % kStages) * G::kStageBytes, *ws = xs + kXBytes;
         const uint32_t *sbt = sb_table + ((step >> 2) & 1) * (kSbBytes / 4) + ((((step & 3) * BK + 32 * h) >> gshift) * BN);
-        uint32_t raw[2][BITS];
-        float sc[2], bi[2];
+        uint32_t raw[TJ][BITS];
+        float sc[TJ], bi[TJ];
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int col = wn * 64 + j * 32 + l32;
+        for (int j = 0; j < TJ; j++) {
+            const int col = wn * (32 * TJ) + j * 32 + l32;
 #pragma unroll
             for (int piece = 0; piece < P::count; piece++) {
                 const unsigned char *src = ws + piece * G::kRegionBytes + (col * 2 + h) * G::kPieceBytes;
@@ -228,23 +244,23 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
             }
         }
         // x fragments are read one substep ahead of the matrix instructions that use them.
-        uint4 af[2][4];
+        uint4 af[2][TI];
 #pragma unroll
-        for (int i = 0; i < 4; i++) af[0][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + l32, 4 * h));
+        for (int i = 0; i < TI; i++) af[0][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * (32 * TI) + i * 32 + l32, 4 * h));
         static_for<4>([&](auto kk_tag) {
             constexpr int kk = decltype(kk_tag)::value;
-            uint4 bf[2];
+            uint4 bf[TJ];
             if constexpr (kk < 3) {
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    af[(kk + 1) & 1][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * 128 + i * 32 + l32, 4 * h + kk + 1));
+                for (int i = 0; i < TI; i++)
+                    af[(kk + 1) & 1][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * (32 * TI) + i * 32 + l32, 4 * h + kk + 1));
             }
 #pragma unroll
-            for (int j = 0; j < 2; j++) bf[j] = expand_piece<T, BITS, FP4, kk>(raw[j], sc[j], bi[j]);
+            for (int j = 0; j < TJ; j++) bf[j] = expand_piece<T, BITS, FP4, kk>(raw[j], sc[j], bi[j]);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = Ops<T>::mfma(af[kk & 1][i], bf[j], acc[i][j]);
+                for (int j = 0; j < TJ; j++) acc[i][j] = Ops<T>::mfma(af[kk & 1][i], bf[j], acc[i][j]);
             issue_part(step + 2, kk);
         });
         if ((step & 3) == 2 && step + 2 < steps) sb_store((step + 2) >> 2);
@@ -255,11 +271,11 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
     // The 32 lanes of a half-wavefront store 32 consecutive elements of one row.
     const bool full = m0 + BM <= M && n0 + BN <= N;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int col = n0 + wn * 64 + j * 32 + l32;
-            const int row0 = m0 + wm * 128 + i * 32 + 4 * h;
+        for (int j = 0; j < TJ; j++) {
+            const int col = n0 + wn * (32 * TJ) + j * 32 + l32;
+            const int row0 = m0 + wm * (32 * TI) + i * 32 + 4 * h;
 #pragma unroll
             for (int e = 0; e < 16; e += 2) {
                 const uint32_t pair = Ops<T>::pack(acc[i][j][e], acc[i][j][e + 1]);  // rounded to nearest even
@@ -271,20 +287,37 @@ __global__ void __launch_bounds__(kThreads) qmm_kernel(const ProductArgs a) {
         }
 }
 
-template <typename T, int BITS, bool FP4>
-int32_t run(const ProductArgs &a, hipStream_t s) {
-    using G = Geometry<BITS>;
+// Estimated microseconds of the tiled kernel with tile TL on `cus` compute units, from its measured behaviour:
+// about 1.7 us (big tile, one block per compute unit) or 1.0 us (small tile, two blocks) per step of 64 values
+// and round of tiles.
+template <class TL>
+inline double estimate_us(const ProductArgs &a, int cus) {
+    const double tiles = (double)((a.m + TL::BM - 1) / TL::BM) * (double)((a.n + TL::BN - 1) / TL::BN) * (double)a.batch;
+    const bool big = TL::BM == 256;
+    const double rounds = ceil(tiles / ((double)cus * (big ? 1.0 : 2.0)));
+    return rounds * (double)(a.k / BK) * (big ? 1.7 : 1.0);
+}
+inline bool small_tile_is_faster(const ProductArgs &a, int cus) { return estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus); }
+
+template <typename T, int BITS, bool FP4, class TL>
+int32_t run_tile(const ProductArgs &a, hipStream_t s) {
+    using G = Geometry<BITS, TL>;
     static bool configured[2] = {false, false};
     const bool batched = a.batch > 1;
-    auto kernel = batched ? qmm_kernel<T, BITS, FP4, true> : qmm_kernel<T, BITS, FP4, false>;
+    auto kernel = batched ? qmm_kernel<T, BITS, FP4, true, TL> : qmm_kernel<T, BITS, FP4, false, TL>;
     if (!configured[batched]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes));
         configured[batched] = true;
     }
-    dim3 grid((unsigned)((a.n + BN - 1) / BN), (unsigned)((a.m + BM - 1) / BM), (unsigned)a.batch);
-    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), G::kLdsBytes, s, a);
+    dim3 grid((unsigned)((a.n + TL::BN - 1) / TL::BN), (unsigned)((a.m + TL::BM - 1) / TL::BM), (unsigned)a.batch);
+    hipLaunchKernelGGL(kernel, grid, dim3(TL::kThreads), G::kLdsBytes, s, a);
     NVQ_LAUNCH_CHECK("qmm");
     return NVQ_OK;
+}
+
+template <typename T, int BITS, bool FP4>
+int32_t run(const ProductArgs &a, hipStream_t s) {
+    return small_tile_is_faster(a, compute_units()) ? run_tile<T, BITS, FP4, SmallTile>(a, s) : run_tile<T, BITS, FP4, BigTile>(a, s);
 }
 
 template <int BITS, bool FP4>
