@@ -21,7 +21,6 @@ namespace {
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
 
-constexpr int kWaves = 4;             // wavefronts per block
 constexpr int kStep = 64 * 32;        // values of K per wavefront step
 
 // Element offsets of batch `z` for x, w (in packed dwords), scales/biases and y.
@@ -53,11 +52,6 @@ __device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int6
     return o;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-    return v;
-}
 
 // v + (v moved across lanes by a DPP control); lanes the control does not feed add 0.
 template <int CTRL, int ROW_MASK>
@@ -118,76 +112,94 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&d)[BITS], int i) {
     return v & mask;
 }
 
-// ── generic kernel: any bit width, any element type, affine or MXFP4 ──────────────────────
-template <typename T, int BITS, bool FP4, int RM, int RN>
-__global__ void __launch_bounds__(kWaves * 64) qmv_generic_kernel(const ProductArgs a) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t n0 = ((int64_t)blockIdx.x * kWaves + wave) * RN;
-    if (n0 >= a.n) return;
-    const int64_t m0 = (int64_t)blockIdx.y * RM;
-    const int64_t kwords = a.k * BITS / 32, kgroups = a.k / a.group;
-    const BatchOffsets o = batch_offsets(a, blockIdx.z, kwords, kgroups);
+// ── general kernel: any bit width, any element type, affine or MXFP4 ──────────────────────
+// A block of eight wavefronts shares the x slice of one K step (2048 values) through LDS, converted to
+// float32 once and laid out [piece][lane] so that a lane's eight 16-byte reads of its 32 values are free of
+// bank conflicts, together with the sums of the 32-value slices (the bias term).  A wavefront owns one
+// weight row: per step a lane loads the BITS dwords of its 32 codes (the wavefront's loads are one
+// contiguous piece of the row), extracts them at compile-time bit positions, converts and accumulates in
+// float32.  Every load of a step is issued before the first use.
+template <typename T, int BITS, bool FP4, int RM>
+__global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
+    constexpr int kBlockWaves = 8;
+    constexpr int kPer = 4;  // values of one x row per thread and step: 2048 / 512
+    __shared__ float4 x_vals[RM][8][64];  // [row][piece][lane]: values 4 piece .. + 4 of the lane's 32
+    __shared__ float x_sums[RM][64];      // [row][lane]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
+    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int n = __builtin_amdgcn_readfirstlane(blockIdx.x * kBlockWaves + wave);
+    const int nc = n < N ? n : N - 1;  // tail rows are computed, not stored
+    const int m0 = blockIdx.y * RM;
+    const int row_dwords = (K >> 5) * BITS, kgroups = K >> gshift;
+    const BatchOffsets o = batch_offsets(a, blockIdx.z, row_dwords, kgroups);
     const T *x = (const T *)a.x + o.x;
-    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    const uint32_t *wrow = (const uint32_t *)a.w + o.w + (int64_t)nc * row_dwords;
     T *y = (T *)a.y + o.y;
 
-    float acc[RN][RM];
+    float acc[RM];
 #pragma unroll
-    for (int r = 0; r < RN; r++)
-#pragma unroll
-        for (int i = 0; i < RM; i++) acc[r][i] = 0.0f;
+    for (int i = 0; i < RM; i++) acc[i] = 0.0f;
 
-    for (int64_t k0 = 0; k0 < a.k; k0 += kStep) {
-        const int64_t kb = k0 + lane * 32;
-        if (kb >= a.k) continue;  // K is a multiple of 32: a lane's slice is whole or absent
-        float xv[RM][32], xs[RM];
+    for (int k0 = 0; k0 < K; k0 += kStep) {
+        // x first: it is needed first and arrives from the cache.
+        float xin[RM][kPer];
+        const int kx = k0 + tid * kPer;
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int j = 0; j < kPer; j++) xin[i][j] = (kx < K && m0 + i < M) ? Elem<T>::load(x, (int64_t)(m0 + i) * K + kx + j) : 0.0f;
+        const int kb = k0 + lane * 32;
+        const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
+        uint32_t d[BITS];
+        load_words<BITS>(wrow + (kc >> 5) * BITS, d);
+        float sc, bi = 0.0f;
+        if constexpr (FP4) {
+            sc = ftz(e8m0_to_f32(((const uint8_t *)a.scales)[o.s + (int64_t)nc * kgroups + (kc >> gshift)]));
+        } else {
+            sc = Elem<T>::load((const T *)a.scales + o.s, (int64_t)nc * kgroups + (kc >> gshift));
+            bi = Elem<T>::load((const T *)a.biases + o.s, (int64_t)nc * kgroups + (kc >> gshift));
+        }
+        if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
 #pragma unroll
         for (int i = 0; i < RM; i++) {
-            xs[i] = 0.0f;
-            const bool row = m0 + i < a.m;
+            // thread t holds values 4 t .. 4 t + 3 of the step: piece t % 8 of lane t / 8
+            x_vals[i][tid & 7][tid >> 3] = make_float4(xin[i][0], xin[i][1], xin[i][2], xin[i][3]);
+            float sum = (xin[i][0] + xin[i][1]) + (xin[i][2] + xin[i][3]);
+            sum += __shfl_xor(sum, 1);  // the eight pieces of a lane's slice sit in adjacent threads
+            sum += __shfl_xor(sum, 2);
+            sum += __shfl_xor(sum, 4);
+            if ((tid & 7) == 0) x_sums[i][tid >> 3] = sum;
+        }
+        __syncthreads();
+        float dot[RM];
 #pragma unroll
-            for (int j = 0; j < 32; j++) {
-                xv[i][j] = row ? Elem<T>::load(x, (m0 + i) * a.k + kb + j) : 0.0f;
-                xs[i] += xv[i][j];
+        for (int i = 0; i < RM; i++) dot[i] = 0.0f;
+#pragma unroll
+        for (int p = 0; p < 8; p++) {
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t c = code_at<BITS>(d, 4 * p + j);
+                v[j] = FP4 ? e2m1_to_f32(c) : (float)c;
+            }
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                const float4 xv = x_vals[i][p][lane];
+                dot[i] = __builtin_fmaf(xv.x, v[0], dot[i]);
+                dot[i] = __builtin_fmaf(xv.y, v[1], dot[i]);
+                dot[i] = __builtin_fmaf(xv.z, v[2], dot[i]);
+                dot[i] = __builtin_fmaf(xv.w, v[3], dot[i]);
             }
         }
 #pragma unroll
-        for (int r = 0; r < RN; r++) {
-            const int64_t n = n0 + r;
-            if (n >= a.n) break;
-            uint32_t d[BITS];
-            load_words<BITS>(w + n * kwords + kb * BITS / 32, d);
-            const int64_t g = n * kgroups + kb / a.group;
-            float dot[RM];
-#pragma unroll
-            for (int i = 0; i < RM; i++) dot[i] = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 32; j++) {
-                const uint32_t c = code_at<BITS>(d, j);
-                const float v = FP4 ? e2m1_to_f32(c) : (float)c;
-#pragma unroll
-                for (int i = 0; i < RM; i++) dot[i] = __builtin_fmaf(xv[i][j], v, dot[i]);
-            }
-            if constexpr (FP4) {
-                const float s = ftz(e8m0_to_f32(((const uint8_t *)a.scales)[o.s + g]));
-#pragma unroll
-                for (int i = 0; i < RM; i++) acc[r][i] = __builtin_fmaf(s, dot[i], acc[r][i]);
-            } else {
-                const float s = Elem<T>::load((const T *)a.scales + o.s, g);
-                const float b = Elem<T>::load((const T *)a.biases + o.s, g);
-#pragma unroll
-                for (int i = 0; i < RM; i++)
-                    acc[r][i] = __builtin_fmaf(s, dot[i], __builtin_fmaf(b, xs[i], acc[r][i]));
-            }
-        }
+        for (int i = 0; i < RM; i++) acc[i] = __builtin_fmaf(sc, dot[i], __builtin_fmaf(bi, x_sums[i][lane], acc[i]));
     }
 #pragma unroll
-    for (int r = 0; r < RN; r++)
-#pragma unroll
-        for (int i = 0; i < RM; i++) {
-            const float v = wave_sum(acc[r][i]);
-            if (lane == 0 && n0 + r < a.n && m0 + i < a.m) Elem<T>::store(y, (m0 + i) * a.n + n0 + r, v);
-        }
+    for (int i = 0; i < RM; i++) {
+        const float v = wave_sum_lane63(acc[i]);
+        if (lane == 63 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, v);
+    }
 }
 
 // ── 4-bit affine, bf16 / f16: packed-pair dot products ────────────────────────────────────
@@ -214,111 +226,6 @@ template <> struct Pair<f16_t> {
     __device__ static __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[0]; }
     __device__ static __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[1]; }
 };
-
-// One wavefront per block, RN weight rows per wavefront, KU steps of 2048 values per loop
-// iteration with every load of the iteration issued before the first use: at K = 4096 the
-// whole product of a wavefront is one round trip to memory (KU*RN 128-bit loads per lane in
-// flight), and the block count (N / RN) spreads evenly over the compute units.
-template <typename T, int RM, int RN, int KU>
-__global__ void __launch_bounds__(64) qmv4_pair_kernel(const ProductArgs a) {
-    const int lane = threadIdx.x;
-    const int64_t n0 = (int64_t)blockIdx.x * RN;
-    const int64_t m0 = (int64_t)blockIdx.y * RM;
-    const int64_t kwords = a.k / 8, kgroups = a.k / a.group;
-    const BatchOffsets o = batch_offsets(a, blockIdx.z, kwords, kgroups);
-    const T *x = (const T *)a.x + o.x;
-    const uint32_t *w = (const uint32_t *)a.w + o.w;
-    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
-    T *y = (T *)a.y + o.y;
-    constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
-
-    float acc[RN][RM];
-#pragma unroll
-    for (int r = 0; r < RN; r++)
-#pragma unroll
-        for (int i = 0; i < RM; i++) acc[r][i] = 0.0f;
-
-    for (int64_t k0 = 0; k0 < a.k; k0 += (int64_t)KU * kStep) {
-        uint4 xq[KU][RM][4], wq[KU][RN];
-        T sraw[KU][RN], braw[KU][RN];
-        bool live[KU];
-#pragma unroll
-        for (int u = 0; u < KU; u++) {
-            const int64_t kb = k0 + (int64_t)u * kStep + lane * 32;
-            live[u] = kb < a.k;  // K is a multiple of 32: a lane's slice is whole or absent
-            const int64_t kc = live[u] ? kb : 0;
-#pragma unroll
-            for (int i = 0; i < RM; i++) {
-                const int64_t row = m0 + i < a.m ? m0 + i : a.m - 1;
-                const uint4 *px = reinterpret_cast<const uint4 *>(x + row * a.k + kc);
-#pragma unroll
-                for (int j = 0; j < 4; j++) xq[u][i][j] = px[j];
-            }
-#pragma unroll
-            for (int r = 0; r < RN; r++) {
-                const int64_t n = n0 + r < a.n ? n0 + r : a.n - 1;  // clamp: tail rows are computed, not stored
-                wq[u][r] = *reinterpret_cast<const uint4 *>(w + n * kwords + kc / 8);
-                const int64_t g = n * kgroups + kc / a.group;
-                sraw[u][r] = scales[g];
-                braw[u][r] = biases[g];
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < KU; u++) {
-            // x pairs in the order the nibbles pair up: word j holds values 8j..8j+7, and
-            // (w >> 4t) & 0x000F000F picks values 8j+t (low half) and 8j+t+4 (high half).
-            uint32_t xp[RM][16];
-            float xs[RM];
-#pragma unroll
-            for (int i = 0; i < RM; i++) {
-                xs[i] = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint4 q = xq[u][i][j];  // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
-                    xp[i][4 * j + 0] = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
-                    xp[i][4 * j + 1] = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
-                    xp[i][4 * j + 2] = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
-                    xp[i][4 * j + 3] = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) xs[i] = Pair<T>::dot2(xp[i][4 * j + t], ones, xs[i]);
-                }
-                if (!live[u] || m0 + i >= a.m) {  // an absent slice or row contributes nothing
-                    xs[i] = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 16; j++) xp[i][j] = 0u;
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < RN; r++) {
-                const uint32_t d[4] = {wq[u][r].x, wq[u][r].y, wq[u][r].z, wq[u][r].w};
-                float dot[RM];
-#pragma unroll
-                for (int i = 0; i < RM; i++) dot[i] = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const uint32_t pair = ((d[j] >> (4 * t)) & 0x000F000Fu) | Pair<T>::magic;
-#pragma unroll
-                        for (int i = 0; i < RM; i++) dot[i] = Pair<T>::dot2(xp[i][4 * j + t], pair, dot[i]);
-                    }
-                // scale * (dot - B * sum x) + bias * sum x
-                const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
-                const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
-#pragma unroll
-                for (int i = 0; i < RM; i++)
-                    acc[r][i] = __builtin_fmaf(sc, dot[i], __builtin_fmaf(bb, xs[i], acc[r][i]));
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RN; r++)
-#pragma unroll
-        for (int i = 0; i < RM; i++) {
-            const float v = wave_sum(acc[r][i]);
-            if (lane == 0 && n0 + r < a.n && m0 + i < a.m) Elem<T>::store(y, (m0 + i) * a.n + n0 + r, v);
-        }
-}
 
 // ── 4-bit affine, bf16 / f16, one or two rows of x: the decode kernel ─────────────────────
 // A block of WAVES wavefronts shares the x slice of one K step (4096 values) through LDS, stored
@@ -468,25 +375,22 @@ int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int BITS, bool FP4, int RM, int RN>
-int32_t run_generic(const ProductArgs &a, hipStream_t s) {
-    dim3 grid((unsigned)((a.n + kWaves * RN - 1) / (kWaves * RN)), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
-    hipLaunchKernelGGL((qmv_generic_kernel<T, BITS, FP4, RM, RN>), grid, dim3(kWaves * 64), 0, s, a);
+template <typename T, int BITS, bool FP4>
+int32_t run_general(const ProductArgs &a, hipStream_t s) {
+    const unsigned gx = (unsigned)((a.n + 7) / 8);
+    if (a.m == 1) {
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, FP4, 1>), dim3(gx, 1, (unsigned)a.batch), dim3(512), 0, s, a);
+    } else {  // passes of four rows over grid.y
+        if ((a.m + 3) / 4 > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld rows exceed the grid limit", (long long)a.m);
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, FP4, 4>), dim3(gx, (unsigned)((a.m + 3) / 4), (unsigned)a.batch), dim3(512), 0, s, a);
+    }
     NVQ_LAUNCH_CHECK("qmv");
-    return NVQ_OK;
-}
-
-template <typename T, int RM, int RN, int KU>
-int32_t run_pair4(const ProductArgs &a, hipStream_t s) {
-    dim3 grid((unsigned)((a.n + RN - 1) / RN), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
-    hipLaunchKernelGGL((qmv4_pair_kernel<T, RM, RN, KU>), grid, dim3(64), 0, s, a);
-    NVQ_LAUNCH_CHECK("qmv4_pair");
     return NVQ_OK;
 }
 
 template <typename T>
 int32_t run_typed(const ProductArgs &a, hipStream_t s) {
-    if (a.mode == NVQ_MXFP4) return a.m == 1 ? run_generic<T, 4, true, 1, 4>(a, s) : run_generic<T, 4, true, 2, 4>(a, s);
+    if (a.mode == NVQ_MXFP4) return run_general<T, 4, true>(a, s);
     if constexpr (!std::is_same<T, float>::value) {
         if (a.bits == 4) {
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
@@ -495,7 +399,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
             return run_lds4<T, 4, 1, 8>(a, s);  // more rows: passes of four over grid.y
         }
     }
-#define NVQ_GENERIC(B) (a.m == 1 ? run_generic<T, B, false, 1, 4>(a, s) : run_generic<T, B, false, 2, 4>(a, s))
+#define NVQ_GENERIC(B) run_general<T, B, false>(a, s)
     switch (a.bits) {
     case 1: return NVQ_GENERIC(1);
     case 2: return NVQ_GENERIC(2);
