@@ -159,10 +159,22 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t chunks, int lanes, uint8
         }
     }
     if (!active) return;
+    // code = rint((v - bias) / scale) with the correctly rounded quotient.  Eight divisions per lane are the
+    // bulk of this kernel's arithmetic, and only the rounded integer is needed: (v - bias) * (1 / scale) is
+    // within 2^-23 relative of the quotient, so both round to the same integer unless they lie that close to
+    // a half; those few values (and odd scales) take the division.
+    const float inv = 1.0f / scale;
+    const float mag = fabsf(scale);
+    const bool plain = mag > 1e-30f && mag < 1e30f;  // finite, normal, with a finite normal reciprocal
     uint64_t stream = 0;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        float q = rintf((v[i] - bias) / scale);
+        const float d = v[i] - bias;
+        float t = d * inv;
+        const float u = fabsf(t);
+        const float frac = u - floorf(u);
+        if (!plain || !(fabsf(frac - 0.5f) > 4e-7f * u)) t = d / scale;  // also NaN and infinities
+        float q = rintf(t);
         q = fminf(fmaxf(q, 0.0f), n_bins);  // NaN -> 0, as Rust's clamp followed by `as u32`
         stream |= (uint64_t)(uint32_t)q << (i * BITS);
     }
