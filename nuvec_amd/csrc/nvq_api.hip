@@ -259,8 +259,7 @@ static int32_t check_qmm(const nvq_qmm_desc *d, const char *op) {
 int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
     if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
     if (!d->transpose) return 0;  // x . w (qvm / qmm_n) has no gfx950 kernel yet
-    if (d->quant.mode != NVQ_AFFINE && d->quant.mode != NVQ_MXFP4) return 0;
-    return 1;
+    return 1;  // every mode: the matrix-core kernels take affine and MXFP4, the general kernel the rest
 }
 
 size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *) { return 0; }
@@ -331,7 +330,7 @@ int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, c
     if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr || lhs == nullptr || rhs == nullptr)
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null operand");
     NVQ_TRY(require_device());
-    if (!d->transpose || (d->quant.mode != NVQ_AFFINE && d->quant.mode != NVQ_MXFP4))
+    if (!d->transpose)
         return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for mode %s, transpose=%d", mode_name(d->quant.mode), d->transpose);
     NVQ_TRY(check_aligned("gather_qmm", "x", x));
     NVQ_TRY(check_aligned("gather_qmm", "w", w));

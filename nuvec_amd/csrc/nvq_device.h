@@ -88,6 +88,32 @@ __device__ __forceinline__ float e2m1_to_f32(uint32_t code) {
     float v = m == 0u ? 0.0f : m == 1u ? 0.5f : u2f(((126u + (m >> 1)) << 23) | ((m & 1u) << 22));
     return (code & 8u) ? -v : v;
 }
+// fp8.rs:16-37: float32 -> E4M3 (FN variant: no infinities, 0x7F is NaN), round to nearest even, saturating
+// to 0x7E (448); NaN goes to 0x7E too, as everything at or above the limit does after the sign is removed.
+__device__ __forceinline__ uint32_t e4m3_from_f32(float x) {
+    constexpr uint32_t kMax = 543u << 21, kDenorm = 141u << 23;
+    uint32_t bits = f2u(x);
+    const uint32_t sign = bits & 0x80000000u;
+    bits ^= sign;
+    uint32_t code;
+    if (bits >= kMax) {
+        code = 0x7Eu;
+    } else if (bits < (121u << 23)) {
+        code = (f2u(u2f(bits) + u2f(kDenorm)) - kDenorm) & 0xFFu;
+    } else {
+        const uint32_t odd = (bits >> 20) & 1u;
+        bits += ((uint32_t)(7 - 127) << 23) + 0x7FFFFu;
+        bits += odd;
+        code = (bits >> 20) & 0xFFu;
+    }
+    return code | (sign >> 24);
+}
+// fp8.rs:39-45: the code's bits placed in a half and scaled by 256 (exact)
+__device__ __forceinline__ float e4m3_to_f32(uint32_t code) {
+    const uint32_t v = code & 127u;
+    const uint16_t u = (uint16_t)((v << 7) | (((v + 1u) >> 7) << 14) | ((code >> 7) << 15));
+    return (float)__builtin_bit_cast(_Float16, u) * 256.0f;
+}
 // fp8.rs:95-102
 __device__ __forceinline__ float e8m0_to_f32(uint32_t code) {
     return code == 0u ? u2f(0x400000u) : u2f(code << 23);

@@ -112,22 +112,26 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&d)[BITS], int i) {
     return v & mask;
 }
 
-// ── general kernel: any bit width, any element type, affine or MXFP4 ──────────────────────
+// ── general kernel: any bit width, any element type, affine or a floating-point block format ──
 // A block of eight wavefronts shares the x slice of one K step (2048 values) through LDS, converted to
 // float32 once and laid out [piece][lane] so that a lane's eight 16-byte reads of its 32 values are free of
 // bank conflicts, together with the sums of the 32-value slices (the bias term).  A wavefront owns one
 // weight row: per step a lane loads the BITS dwords of its 32 codes (the wavefront's loads are one
 // contiguous piece of the row), extracts them at compile-time bit positions, converts and accumulates in
-// float32.  Every load of a step is issued before the first use.
-template <typename T, int BITS, bool FP4, int RM>
+// float32.  Every load of a step is issued before the first use.  MODE: NVQ_AFFINE, or NVQ_MXFP4 /
+// NVQ_MXFP8 / NVQ_NVFP4 (E2M1 or E4M3 values; E8M0 scales per 32 or E4M3 scales per 16 values, a lane's
+// slice then spanning two groups).
+template <typename T, int BITS, int MODE, int RM>
 __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
     constexpr int kBlockWaves = 8;
     constexpr int kPer = 4;  // values of one x row per thread and step: 2048 / 512
+    constexpr bool kAffine = MODE == NVQ_AFFINE;
+    constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
     __shared__ float4 x_vals[RM][8][64];  // [row][piece][lane]: values 4 piece .. + 4 of the lane's 32
     __shared__ float x_sums[RM][64];      // [row][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
-    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int gshift = kAffine ? (a.group == 32 ? 5 : a.group == 64 ? 6 : 7) : (MODE == NVQ_NVFP4 ? 4 : 5);
     const int n = __builtin_amdgcn_readfirstlane(blockIdx.x * kBlockWaves + wave);
     const int nc = n < N ? n : N - 1;  // tail rows are computed, not stored
     const int m0 = blockIdx.y * RM;
@@ -153,12 +157,14 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
         const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
         uint32_t d[BITS];
         load_words<BITS>(wrow + (kc >> 5) * BITS, d);
-        float sc, bi = 0.0f;
-        if constexpr (FP4) {
-            sc = ftz(e8m0_to_f32(((const uint8_t *)a.scales)[o.s + (int64_t)nc * kgroups + (kc >> gshift)]));
-        } else {
-            sc = Elem<T>::load((const T *)a.scales + o.s, (int64_t)nc * kgroups + (kc >> gshift));
+        float sc[kHalves], bi = 0.0f;
+        if constexpr (kAffine) {
+            sc[0] = Elem<T>::load((const T *)a.scales + o.s, (int64_t)nc * kgroups + (kc >> gshift));
             bi = Elem<T>::load((const T *)a.biases + o.s, (int64_t)nc * kgroups + (kc >> gshift));
+        } else {
+            const uint8_t *sp = (const uint8_t *)a.scales + o.s + (int64_t)nc * kgroups + (kc >> gshift);
+#pragma unroll
+            for (int hf = 0; hf < kHalves; hf++) sc[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(sp[hf]) : e8m0_to_f32(sp[hf]));
         }
         if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
 #pragma unroll
@@ -172,28 +178,40 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
             if ((tid & 7) == 0) x_sums[i][tid >> 3] = sum;
         }
         __syncthreads();
-        float dot[RM];
+        float dot[RM][kHalves];
 #pragma unroll
-        for (int i = 0; i < RM; i++) dot[i] = 0.0f;
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int hf = 0; hf < kHalves; hf++) dot[i][hf] = 0.0f;
 #pragma unroll
         for (int p = 0; p < 8; p++) {
+            constexpr int kPiecesPerHalf = 8 / kHalves;
             float v[4];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t c = code_at<BITS>(d, 4 * p + j);
-                v[j] = FP4 ? e2m1_to_f32(c) : (float)c;
+                v[j] = kAffine ? (float)c : (MODE == NVQ_MXFP8 ? e4m3_to_f32(c) : e2m1_to_f32(c));
             }
 #pragma unroll
             for (int i = 0; i < RM; i++) {
                 const float4 xv = x_vals[i][p][lane];
-                dot[i] = __builtin_fmaf(xv.x, v[0], dot[i]);
-                dot[i] = __builtin_fmaf(xv.y, v[1], dot[i]);
-                dot[i] = __builtin_fmaf(xv.z, v[2], dot[i]);
-                dot[i] = __builtin_fmaf(xv.w, v[3], dot[i]);
+                float t = dot[i][p / kPiecesPerHalf];
+                t = __builtin_fmaf(xv.x, v[0], t);
+                t = __builtin_fmaf(xv.y, v[1], t);
+                t = __builtin_fmaf(xv.z, v[2], t);
+                t = __builtin_fmaf(xv.w, v[3], t);
+                dot[i][p / kPiecesPerHalf] = t;
             }
         }
 #pragma unroll
-        for (int i = 0; i < RM; i++) acc[i] = __builtin_fmaf(sc, dot[i], __builtin_fmaf(bi, x_sums[i][lane], acc[i]));
+        for (int i = 0; i < RM; i++) {
+            if constexpr (kAffine) {
+                acc[i] = __builtin_fmaf(sc[0], dot[i][0], __builtin_fmaf(bi, x_sums[i][lane], acc[i]));
+            } else {
+#pragma unroll
+                for (int hf = 0; hf < kHalves; hf++) acc[i] = __builtin_fmaf(sc[hf], dot[i][hf], acc[i]);
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < RM; i++) {
@@ -375,14 +393,14 @@ int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int BITS, bool FP4>
+template <typename T, int BITS, int MODE>
 int32_t run_general(const ProductArgs &a, hipStream_t s) {
     const unsigned gx = (unsigned)((a.n + 7) / 8);
     if (a.m == 1) {
-        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, FP4, 1>), dim3(gx, 1, (unsigned)a.batch), dim3(512), 0, s, a);
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 1>), dim3(gx, 1, (unsigned)a.batch), dim3(512), 0, s, a);
     } else {  // passes of four rows over grid.y
         if ((a.m + 3) / 4 > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld rows exceed the grid limit", (long long)a.m);
-        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, FP4, 4>), dim3(gx, (unsigned)((a.m + 3) / 4), (unsigned)a.batch), dim3(512), 0, s, a);
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 4>), dim3(gx, (unsigned)((a.m + 3) / 4), (unsigned)a.batch), dim3(512), 0, s, a);
     }
     NVQ_LAUNCH_CHECK("qmv");
     return NVQ_OK;
@@ -390,7 +408,9 @@ int32_t run_general(const ProductArgs &a, hipStream_t s) {
 
 template <typename T>
 int32_t run_typed(const ProductArgs &a, hipStream_t s) {
-    if (a.mode == NVQ_MXFP4) return run_general<T, 4, true>(a, s);
+    if (a.mode == NVQ_MXFP4) return run_general<T, 4, NVQ_MXFP4>(a, s);
+    if (a.mode == NVQ_MXFP8) return run_general<T, 8, NVQ_MXFP8>(a, s);
+    if (a.mode == NVQ_NVFP4) return run_general<T, 4, NVQ_NVFP4>(a, s);
     if constexpr (!std::is_same<T, float>::value) {
         if (a.bits == 4) {
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
@@ -399,7 +419,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
             return run_lds4<T, 4, 1, 8>(a, s);  // more rows: passes of four over grid.y
         }
     }
-#define NVQ_GENERIC(B) run_general<T, B, false>(a, s)
+#define NVQ_GENERIC(B) run_general<T, B, NVQ_AFFINE>(a, s)
     switch (a.bits) {
     case 1: return NVQ_GENERIC(1);
     case 2: return NVQ_GENERIC(2);

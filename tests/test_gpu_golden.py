@@ -61,14 +61,16 @@ def test_affine_dequantize_equals_oracle_on_device_vectors(hip, golden_gpu):
     assert not _failures(cases, check)
 
 
-def test_mxfp4_quantize_bits(hip, golden_gpu):
-    cases = [c for c in golden_gpu[1] if c.op == "quantize"]
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
+def test_fp_quantize_bits(hip, golden_gpu, mode):
+    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode]
     assert len(cases) == 18
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
 
 
-def test_mxfp4_dequantize_bits(hip, golden_gpu):
-    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == "mxfp4"]
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
+def test_fp_dequantize_bits(hip, golden_gpu, mode):
+    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode]
     assert len(cases) == 15
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
 

@@ -368,3 +368,27 @@ def test_tiled_mxfp4():
     want = ref.quantized_matmul(x, packed, scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16, threads=8)
     got = to_host(nv.quantized_matmul(to_dev(x), q))
     assert_rows_close(got, want, ref.BF16, "tiled mxfp4")
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
+def test_mxfp8_nvfp4_quantize_and_products(mode, qmode, dtype):
+    """The other two floating-point block formats (no global scale): quantize and dequantize bit for bit,
+    products (on the general kernel) within the bar.  The CPU path keeps these weights in float32, so the
+    bar holds for every output."""
+    rng = np.random.default_rng(300 + mode + dtype)
+    n, k = 200, 1152
+    w = make_w(rng, n, k, dtype)
+    packed, scales = ref.fp_quantize(w, dtype, mode)
+    q = nv.quantize(to_dev(w), getattr(nv.QuantMode, qmode))
+    assert np.array_equal(to_host(q.weight), packed) and np.array_equal(to_host(q.scales), scales)
+    for out in (ref.BF16, ref.F32, ref.F16):
+        want = ref.fp_dequantize(packed, scales, mode, out)
+        assert np.array_equal(to_host(nv.dequantize(q, TORCH[out])).view(np.uint8), want.view(np.uint8))
+    group, bits = ref.FP_PARAMS[mode]
+    for m in (1, 5, 40):
+        x = make_x(rng, m, k, dtype)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        ratio = _excess(got, want, dtype)
+        assert float(np.max(ratio)) <= 1.0, f"{qmode} M={m}: max error is {float(np.max(ratio)):.3f} x the bound"

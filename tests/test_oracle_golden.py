@@ -27,7 +27,7 @@ def test_fixture_meta(golden_cpu, golden_gpu):
     assert len(cases) == 135
     meta, cases = golden_gpu
     assert "mlx=0.32.4" in meta and "device=gpu" in meta
-    assert len(cases) == 176
+    assert len(cases) == 276
 
 
 def test_affine_quantize_bits(golden_cpu):
@@ -70,15 +70,17 @@ def test_affine_dequantize_device_vectors(golden_gpu):
     assert not _failures(cases, cpu)
 
 
-def test_mxfp4_quantize_bits(golden_gpu):
-    """18 cases incl. NaN/Inf/subnormal/signed-zero edges, transposed and reversed inputs."""
-    cases = [c for c in golden_gpu[1] if c.op == "quantize"]
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
+def test_fp_quantize_bits(golden_gpu, mode):
+    """18 cases per format incl. NaN/Inf/subnormal/signed-zero edges, transposed and reversed inputs."""
+    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode]
     assert len(cases) == 18
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
 
 
-def test_mxfp4_dequantize_bits(golden_gpu):
-    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == "mxfp4"]
+@pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
+def test_fp_dequantize_bits(golden_gpu, mode):
+    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode]
     assert len(cases) == 15
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
 
