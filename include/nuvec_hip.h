@@ -164,7 +164,8 @@ NVQ_API int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void
                        const void *biases, int64_t rows, int64_t cols, void *out, void *stream);
 
 /* Bytes of scratch nvq_quantized_matmul needs for `desc` (split-K partials; the reference
- * allocates them on its side of the boundary, gpu.rs:7562).  0 = none. */
+ * allocates them on its side of the boundary, gpu.rs:7562).  0 = none; nonzero only for
+ * transpose = 0 products whose K is split over the grid (float32 partial sums). */
 NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
 
 /* GpuEval::quantized_matmul / fp_quantized_matmul (gpu.rs:6934-7168, 6336-6577); values of

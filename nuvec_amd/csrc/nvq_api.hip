@@ -151,6 +151,22 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
     return nvq::qmm_estimate_us(a) < few_us;
 }
 
+// The kernels' view of a product descriptor.
+static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
+    nvq::ProductArgs a{};
+    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
+    a.m = d->m; a.n = d->n; a.k = d->k;
+    a.batch = batch;
+    a.batch_ndim = d->batch_ndim;
+    for (int i = 0; i < d->batch_ndim; i++) {
+        a.batch_shape[i] = d->batch_shape[i];
+        a.x_strides[i] = d->x_strides[i];
+        a.w_strides[i] = d->w_strides[i];
+        a.s_strides[i] = d->s_strides[i];
+    }
+    return a;
+}
+
 extern "C" {
 
 const char *nvq_last_error(void) { return g_error; }
@@ -258,15 +274,19 @@ static int32_t check_qmm(const nvq_qmm_desc *d, const char *op) {
 
 int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
     if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
-    if (!d->transpose) return 0;  // x . w (qvm / qmm_n) has no gfx950 kernel yet
-    return 1;  // every mode: the matrix-core kernels take affine and MXFP4, the general kernel the rest
+    return 1;  // every mode and both orientations: the matrix-core kernels take affine and MXFP4 transposed, the general kernels the rest
 }
 
-size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *) { return 0; }
+size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
+    if (check_qmm(d, "quantized_matmul") != NVQ_OK || d->transpose) return 0;
+    int64_t batch = 1;
+    for (int i = 0; i < d->batch_ndim; i++) batch *= d->batch_shape[i];
+    if (batch == 0 || d->m == 0 || d->n == 0 || d->k == 0 || require_device() != NVQ_OK) return 0;
+    return qvm_workspace_bytes(product_args(d, batch));  // float32 partial sums of the splits of K
+}
 
 int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                              void *y, void *workspace, void *stream) {
-    (void)workspace;
     NVQ_TRY(check_qmm(d, "quantized_matmul"));
     NVQ_TRY(check_groups("quantized_matmul", d->quant.mode, biases));
     int64_t batch = 1;
@@ -283,18 +303,9 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     if (d->k == 0) {  // an empty reduction is zero (crates/nuvec-cpu/src/matmul.rs:237-240)
         return launch_fill_zero(y, batch * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
     }
-    ProductArgs a{};
+    ProductArgs a = product_args(d, batch);
     a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
-    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
-    a.m = d->m; a.n = d->n; a.k = d->k;
-    a.batch = batch;
-    a.batch_ndim = d->batch_ndim;
-    for (int i = 0; i < d->batch_ndim; i++) {
-        a.batch_shape[i] = d->batch_shape[i];
-        a.x_strides[i] = d->x_strides[i];
-        a.w_strides[i] = d->w_strides[i];
-        a.s_strides[i] = d->s_strides[i];
-    }
+    if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
     // Routed by one item's rows, as the reference does (gpu.rs:6975-6981): the tiled kernel where its tiles
     // cost less than the passes of the few-row kernel.
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;

@@ -71,5 +71,9 @@ double qmm_estimate_us(const ProductArgs &a);  // estimated duration of the tile
 bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);
 int32_t launch_fill_zero(void *p, int64_t bytes, hipStream_t s);
+// Products with the weights stored [K, N] (transpose = false); K is split over the grid through a float32 workspace.
+int qvm_splits(const ProductArgs &a);
+size_t qvm_workspace_bytes(const ProductArgs &a);
+int32_t launch_qvm(const ProductArgs &a, void *workspace, hipStream_t s);
 
 }  // namespace nvq

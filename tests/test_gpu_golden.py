@@ -21,8 +21,8 @@ def hip():
 
 
 def _supported(c):
-    """transpose=0 (x . w) and bits the first kernels do not cover are refused by the backend."""
-    return c.params.get("transpose", "1") == "1"
+    """Gathered products with the weights stored [K, N] (transpose=0) are refused by the backend."""
+    return c.op != "gather_qmm" or c.params.get("transpose", "1") == "1"
 
 
 def _failures(cases, check):
@@ -93,10 +93,12 @@ def test_gathers_against_mlx_gpu(hip, golden_gpu):
     assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
 
 
-def test_untransposed_products_are_refused_not_faked(hip, golden_cpu):
-    """x . w has no gfx950 kernel yet: the backend must say so (the caller then takes its CPU
-    path) instead of answering from anywhere else."""
+def test_untransposed_gathers_are_refused_not_faked(hip, golden_gpu):
+    """gather_qmm with weights stored [K, N] has no gfx950 kernel yet: the backend must say so (the caller
+    then takes its CPU path) instead of answering from anywhere else."""
     import nuvec_amd as nv
-    case = next(c for c in golden_cpu[1] if c.name == "qmm-n")
+    cases = [c for c in golden_gpu[1] if c.op == "gather_qmm" and c.params.get("transpose", "1") == "0"]
+    if not cases:
+        pytest.skip("no untransposed gather among the committed vectors")
     with pytest.raises(nv.Unsupported):
-        replay.run_case(case, hip)
+        replay.run_case(cases[0], hip)

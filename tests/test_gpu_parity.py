@@ -392,3 +392,49 @@ def test_mxfp8_nvfp4_quantize_and_products(mode, qmode, dtype):
         got = to_host(nv.quantized_matmul(to_dev(x), q))
         ratio = _excess(got, want, dtype)
         assert float(np.max(ratio)) <= 1.0, f"{qmode} M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(64, 4), (32, 2), (128, 6), (64, 5), (128, 1), (32, 3), (64, 8)])
+def test_untransposed_products_every_width(dtype, group, bits):
+    """Weights stored [K, N] (transpose=False): one row and a few rows of x, K split over the grid or not,
+    N beyond and below one wavefront's 2048 outputs."""
+    rng = np.random.default_rng(1700 + 10 * bits + group + dtype)
+    for m, k, n in [(1, 300, 2 * 128), (5, 64, 2048 + 3 * 128), (1, 2500, 128)]:
+        w = make_w(rng, k, n, dtype)  # quantized along N
+        x = make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, transpose=False)
+        got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
+        assert got.shape == (m, n)
+        assert_rows_close(got, want, dtype, f"x.w b{bits} g{group} M={m} K={k} N={n}")
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+def test_untransposed_products_block_formats(mode, qmode):
+    rng = np.random.default_rng(1800 + mode)
+    group, bits = ref.FP_PARAMS[mode]
+    for m, k, n in [(1, 200, 256), (7, 96, 2048 + 64)]:
+        w, x = make_w(rng, k, n, ref.BF16), make_x(rng, m, k, ref.BF16)
+        packed, scales = ref.fp_quantize(w, ref.BF16, mode)
+        q = nv.quantize(to_dev(w), getattr(nv.QuantMode, qmode))
+        assert np.array_equal(to_host(q.weight), packed)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=ref.BF16, transpose=False)
+        got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
+        ratio = _excess(got, want, ref.BF16)
+        assert float(np.max(ratio)) <= 1.0, f"x.w {qmode} M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
+
+
+def test_untransposed_products_batched():
+    """x [B, M, K] against w [B, K, N/8]: one product per batch item."""
+    rng = np.random.default_rng(1900)
+    b, m, k, n = 3, 2, 160, 256
+    w = make_w(rng, b * k, n, ref.F32).reshape(b, k, n)
+    x = make_x(rng, b * m, k, ref.F32).reshape(b, m, k)
+    packed, scales, biases = ref.affine_quantize(w, ref.F32, 64, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.F32, transpose=False)
+    got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
+    assert got.shape == (b, m, n)
+    assert_rows_close(got, want, ref.F32, "batched x.w")
