@@ -163,6 +163,16 @@ NVQ_API int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *
 NVQ_API int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
                        const void *biases, int64_t rows, int64_t cols, void *out, void *stream);
 
+/* The rows of a quantized table dequantized: output row r is table row ids[r], bit for bit
+ * nvq_dequantize of the taken rows (QuantizedEmbedding::forward, crates/nuvec-nn/src/layers.rs:245-255:
+ * `take` of weight, scales and biases along axis 0, then `dequantize`).  Fused so that the taken packed
+ * rows are never materialised.
+ *   packed u32 [table_rows, cols*bits/32]; scales / biases [table_rows, cols/group]; ids u32 [count]
+ *   (an id beyond the table is the caller's error and is clamped); out dtype [count, cols]. */
+NVQ_API int32_t nvq_dequantize_rows(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
+                            const void *biases, int64_t table_rows, int64_t cols, const uint32_t *ids, int64_t count,
+                            void *out, void *stream);
+
 /* Bytes of scratch nvq_quantized_matmul needs for `desc` (split-K partials; the reference
  * allocates them on its side of the boundary, gpu.rs:7562).  0 = none; nonzero only for
  * transpose = 0 products whose K is split over the grid (float32 partial sums). */

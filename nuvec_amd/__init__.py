@@ -1,7 +1,8 @@
 """nuvec_amd — MI355X (gfx950) backend for nuvec's quantized-matmul path.
 
 `libnuvec_hip.so` (C ABI in include/nuvec_hip.h) holds the kernels; `ops` mirrors nuvec's
-public `quantize`, `dequantize`, `quantized_matmul` and `gather_qmm`.
+public `quantize`, `dequantize`, `quantized_matmul` and `gather_qmm`, and the row lookup of
+nuvec-nn's `QuantizedEmbedding` as `embedding`.
 """
-from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, gather_qmm,  # noqa: F401
-                  quantize, quantized_matmul, sorted_offsets)
+from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, embedding,  # noqa: F401
+                  gather_qmm, quantize, quantized_matmul, sorted_offsets)

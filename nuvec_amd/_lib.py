@@ -72,6 +72,8 @@ SIGNATURES = {
                                  C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_dequantize": (C.c_int32, [C.POINTER(QuantC), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                    C.c_int64, C.c_void_p, C.c_void_p]),
+    "nvq_dequantize_rows": (C.c_int32, [C.POINTER(QuantC), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                        C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]),
     "nvq_quantized_matmul_workspace_bytes": (C.c_size_t, [C.POINTER(QmmDescC)]),
     "nvq_quantized_matmul": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.c_void_p, C.c_void_p]),

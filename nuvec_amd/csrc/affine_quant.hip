@@ -186,15 +186,24 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t chunks, int lanes, uint8
     }
 }
 
-// kernels.rs:835-859: round(round(code * scale) + bias), both roundings in T.
+// kernels.rs:835-859: round(round(code * scale) + bias), both roundings in T.  With `ids`, output row r is
+// table row ids[r] (the rows of a quantized embedding, crates/nuvec-nn/src/layers.rs:245-255): `row_chunks` chunks
+// per row, ids clamped to the table's `table_rows`.
 template <typename T, int BITS>
 __global__ void __launch_bounds__(kBlock)
 affine_dequantize_kernel(const uint8_t *__restrict__ packed, const T *__restrict__ scales,
-                         const T *__restrict__ biases, int64_t chunks, int lanes, T *__restrict__ out) {
+                         const T *__restrict__ biases, int64_t chunks, int lanes, T *__restrict__ out,
+                         const uint32_t *__restrict__ ids, int64_t row_chunks, int64_t table_rows) {
     const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (chunk >= chunks) return;
-    const uint64_t stream = load_codes<BITS>(packed, chunk);
-    const int64_t g = chunk / lanes;
+    int64_t src = chunk;
+    if (ids != nullptr) {
+        const int64_t r = chunk / row_chunks;
+        const int64_t row = min((int64_t)ids[r], table_rows - 1);
+        src = row * row_chunks + (chunk - r * row_chunks);
+    }
+    const uint64_t stream = load_codes<BITS>(packed, src);
+    const int64_t g = src / lanes;
     const float s = Elem<T>::load(scales, g), b = Elem<T>::load(biases, g);
     constexpr uint32_t mask = (1u << BITS) - 1u;
     float r[8];
@@ -217,11 +226,12 @@ int32_t quantize_t(int group, const void *w, int64_t n, void *packed, void *scal
 }
 template <typename T, int BITS>
 int32_t dequantize_t(int group, const void *packed, const void *scales, const void *biases, int64_t n, void *out,
-                     hipStream_t s) {
+                     const uint32_t *ids, int64_t cols, int64_t table_rows, hipStream_t s) {
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((affine_dequantize_kernel<T, BITS>), dim3(blocks), dim3(kBlock), 0, s,
-                       (const uint8_t *)packed, (const T *)scales, (const T *)biases, chunks, group / 8, (T *)out);
+                       (const uint8_t *)packed, (const T *)scales, (const T *)biases, chunks, group / 8, (T *)out, ids, cols / 8,
+                       table_rows);
     NVQ_LAUNCH_CHECK("affine_dequantize");
     return NVQ_OK;
 }
@@ -251,10 +261,11 @@ int32_t launch_affine_quantize(int32_t dtype, int group, int bits, const void *w
 }
 
 int32_t launch_affine_dequantize(int32_t dtype, int group, int bits, const void *packed, const void *scales,
-                                 const void *biases, int64_t n, void *out, hipStream_t s) {
-#define D_F32(B) dequantize_t<float, B>(group, packed, scales, biases, n, out, s)
-#define D_BF16(B) dequantize_t<bf16_t, B>(group, packed, scales, biases, n, out, s)
-#define D_F16(B) dequantize_t<f16_t, B>(group, packed, scales, biases, n, out, s)
+                                 const void *biases, int64_t n, void *out, const uint32_t *ids, int64_t cols,
+                                 int64_t table_rows, hipStream_t s) {
+#define D_F32(B) dequantize_t<float, B>(group, packed, scales, biases, n, out, ids, cols, table_rows, s)
+#define D_BF16(B) dequantize_t<bf16_t, B>(group, packed, scales, biases, n, out, ids, cols, table_rows, s)
+#define D_F16(B) dequantize_t<f16_t, B>(group, packed, scales, biases, n, out, ids, cols, table_rows, s)
     if (dtype == NVQ_F32) { NVQ_BITS_SWITCH(bits, D_F32) }
     if (dtype == NVQ_BF16) { NVQ_BITS_SWITCH(bits, D_BF16) }
     NVQ_BITS_SWITCH(bits, D_F16)

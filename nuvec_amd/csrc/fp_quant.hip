@@ -67,26 +67,34 @@ fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict
     if (chunk % F::lanes == 0) scales[chunk / F::lanes] = (uint8_t)code;
 }
 
-// kernels.rs:976-1009 without a global scale.
+// kernels.rs:976-1009 without a global scale.  With `ids`, output row r is table row ids[r] (`row_chunks` chunks
+// per row, ids clamped to `table_rows`): the rows of a quantized embedding.
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
-fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, int64_t chunks, T *__restrict__ out) {
+fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, int64_t chunks, T *__restrict__ out,
+                     const uint32_t *__restrict__ ids, int64_t row_chunks, int64_t table_rows) {
     using F = Format<MODE>;
-    const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (chunk >= chunks) return;
+    const int64_t out_chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (out_chunk >= chunks) return;
+    int64_t chunk = out_chunk;
+    if (ids != nullptr) {
+        const int64_t r = out_chunk / row_chunks;
+        const int64_t row = min((int64_t)ids[r], table_rows - 1);
+        chunk = row * row_chunks + (out_chunk - r * row_chunks);
+    }
     const uint32_t sc = scales[chunk / F::lanes];
     const float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
     if constexpr (F::bits == 4) {
         const uint32_t word = packed[chunk];
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            Elem<T>::store(out, chunk * 8 + i, canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu))));
+            Elem<T>::store(out, out_chunk * 8 + i, canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu))));
     } else {
         const uint2 words = reinterpret_cast<const uint2 *>(packed)[chunk];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            Elem<T>::store(out, chunk * 8 + i, canonical(ftz(scale * e4m3_to_f32((words.x >> (8 * i)) & 0xFFu))));
-            Elem<T>::store(out, chunk * 8 + 4 + i, canonical(ftz(scale * e4m3_to_f32((words.y >> (8 * i)) & 0xFFu))));
+            Elem<T>::store(out, out_chunk * 8 + i, canonical(ftz(scale * e4m3_to_f32((words.x >> (8 * i)) & 0xFFu))));
+            Elem<T>::store(out, out_chunk * 8 + 4 + i, canonical(ftz(scale * e4m3_to_f32((words.y >> (8 * i)) & 0xFFu))));
         }
     }
 }
@@ -101,11 +109,12 @@ int32_t quantize_t(const void *w, int64_t n, void *packed, void *scales, hipStre
     return NVQ_OK;
 }
 template <typename T, int MODE>
-int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *out, hipStream_t s) {
+int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *out, const uint32_t *ids, int64_t cols,
+                     int64_t table_rows, hipStream_t s) {
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((fp_dequantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const uint32_t *)packed,
-                       (const uint8_t *)scales, chunks, (T *)out);
+                       (const uint8_t *)scales, chunks, (T *)out, ids, cols / 8, table_rows);
     NVQ_LAUNCH_CHECK("fp_dequantize");
     return NVQ_OK;
 }
@@ -120,11 +129,12 @@ int32_t quantize_mode(int32_t mode, const void *w, int64_t n, void *packed, void
     }
 }
 template <typename T>
-int32_t dequantize_mode(int32_t mode, const void *packed, const void *scales, int64_t n, void *out, hipStream_t s) {
+int32_t dequantize_mode(int32_t mode, const void *packed, const void *scales, int64_t n, void *out, const uint32_t *ids,
+                        int64_t cols, int64_t table_rows, hipStream_t s) {
     switch (mode) {
-    case NVQ_MXFP4: return dequantize_t<T, NVQ_MXFP4>(packed, scales, n, out, s);
-    case NVQ_MXFP8: return dequantize_t<T, NVQ_MXFP8>(packed, scales, n, out, s);
-    case NVQ_NVFP4: return dequantize_t<T, NVQ_NVFP4>(packed, scales, n, out, s);
+    case NVQ_MXFP4: return dequantize_t<T, NVQ_MXFP4>(packed, scales, n, out, ids, cols, table_rows, s);
+    case NVQ_MXFP8: return dequantize_t<T, NVQ_MXFP8>(packed, scales, n, out, ids, cols, table_rows, s);
+    case NVQ_NVFP4: return dequantize_t<T, NVQ_NVFP4>(packed, scales, n, out, ids, cols, table_rows, s);
     default: return fail(NVQ_INVALID_ARGUMENT, "dequantize: mode %s is not a floating-point block format", mode_name(mode));
     }
 }
@@ -141,11 +151,11 @@ int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n
 }
 
 int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales, int64_t n,
-                             void *out, hipStream_t s) {
+                             void *out, const uint32_t *ids, int64_t cols, int64_t table_rows, hipStream_t s) {
     switch (out_dtype) {
-    case NVQ_F32: return dequantize_mode<float>(mode, packed, scales, n, out, s);
-    case NVQ_BF16: return dequantize_mode<bf16_t>(mode, packed, scales, n, out, s);
-    default: return dequantize_mode<f16_t>(mode, packed, scales, n, out, s);
+    case NVQ_F32: return dequantize_mode<float>(mode, packed, scales, n, out, ids, cols, table_rows, s);
+    case NVQ_BF16: return dequantize_mode<bf16_t>(mode, packed, scales, n, out, ids, cols, table_rows, s);
+    default: return dequantize_mode<f16_t>(mode, packed, scales, n, out, ids, cols, table_rows, s);
     }
 }
 

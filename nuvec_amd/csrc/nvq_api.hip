@@ -237,26 +237,41 @@ int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64
     return launch_fp_quantize(quant->mode, dtype, w, n, packed, scales, (hipStream_t)stream);
 }
 
+// Shared by nvq_dequantize and nvq_dequantize_rows: `count` output rows, each table row ids[r] (or row r).
+static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
+                              const void *biases, int64_t table_rows, int64_t cols, const uint32_t *ids, int64_t count,
+                              void *out, void *stream) {
+    NVQ_TRY(check_quant(quant, op));
+    NVQ_TRY(check_groups(op, quant->mode, biases));
+    // primitive.rs:1272-1276
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "%s: unsupported dtype %s", op, dtype_name(dtype));
+    if (table_rows < 0 || count < 0 || cols < 0 || cols % quant->group_size != 0 || (cols * quant->bits) % 32 != 0)
+        return fail(NVQ_INVALID_ARGUMENT,
+                    "%s: packed weights [%lld, %lld] and scales [%lld, %lld] do not match group size %d and %d bits", op,
+                    (long long)table_rows, (long long)(cols * quant->bits / 32), (long long)table_rows,
+                    (long long)(cols / quant->group_size), quant->group_size, quant->bits);
+    if (count == 0 || cols == 0) return NVQ_OK;
+    if (table_rows == 0) return fail(NVQ_INVALID_ARGUMENT, "%s: rows of an empty table", op);
+    if (packed == nullptr || scales == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null operand", op);
+    NVQ_TRY(require_device());
+    NVQ_TRY(check_aligned(op, "packed", packed));
+    NVQ_TRY(check_aligned(op, "out", out));
+    const int64_t n = count * cols;
+    if (quant->mode == NVQ_AFFINE)
+        return launch_affine_dequantize(dtype, quant->group_size, quant->bits, packed, scales, biases, n, out, ids, cols,
+                                        table_rows, (hipStream_t)stream);
+    return launch_fp_dequantize(quant->mode, dtype, packed, scales, n, out, ids, cols, table_rows, (hipStream_t)stream);
+}
+
 int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales, const void *biases,
                        int64_t rows, int64_t cols, void *out, void *stream) {
-    NVQ_TRY(check_quant(quant, "dequantize"));
-    NVQ_TRY(check_groups("dequantize", quant->mode, biases));
-    // primitive.rs:1272-1276
-    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "dequantize: unsupported dtype %s", dtype_name(dtype));
-    if (rows < 0 || cols < 0 || cols % quant->group_size != 0 || (cols * quant->bits) % 32 != 0)
-        return fail(NVQ_INVALID_ARGUMENT,
-                    "dequantize: packed weights [%lld, %lld] and scales [%lld, %lld] do not match group size %d and %d bits",
-                    (long long)rows, (long long)(cols * quant->bits / 32), (long long)rows,
-                    (long long)(cols / quant->group_size), quant->group_size, quant->bits);
-    if (rows == 0 || cols == 0) return NVQ_OK;
-    if (packed == nullptr || scales == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "dequantize: null operand");
-    NVQ_TRY(require_device());
-    NVQ_TRY(check_aligned("dequantize", "packed", packed));
-    NVQ_TRY(check_aligned("dequantize", "out", out));
-    const int64_t n = rows * cols;
-    if (quant->mode == NVQ_AFFINE)
-        return launch_affine_dequantize(dtype, quant->group_size, quant->bits, packed, scales, biases, n, out, (hipStream_t)stream);
-    return launch_fp_dequantize(quant->mode, dtype, packed, scales, n, out, (hipStream_t)stream);
+    return dequantize_any("dequantize", quant, dtype, packed, scales, biases, rows, cols, nullptr, rows, out, stream);
+}
+
+int32_t nvq_dequantize_rows(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales, const void *biases,
+                            int64_t table_rows, int64_t cols, const uint32_t *ids, int64_t count, void *out, void *stream) {
+    if (ids == nullptr && count > 0) return fail(NVQ_INVALID_ARGUMENT, "dequantize_rows: null ids");
+    return dequantize_any("dequantize_rows", quant, dtype, packed, scales, biases, table_rows, cols, ids, count, out, stream);
 }
 
 static int32_t check_qmm(const nvq_qmm_desc *d, const char *op) {

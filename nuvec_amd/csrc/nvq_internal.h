@@ -39,12 +39,15 @@ const char *mode_name(int32_t m);
 // ── kernel launchers (each validates nothing: the entry points did) ─────────────────────
 int32_t launch_affine_quantize(int32_t dtype, int group, int bits, const void *w, int64_t n_values,
                                void *packed, void *scales, void *biases, hipStream_t s);
+// `ids` non-NULL: output row r is table row ids[r] (rows of `cols` values, ids clamped to `table_rows`).
 int32_t launch_affine_dequantize(int32_t dtype, int group, int bits, const void *packed, const void *scales,
-                                 const void *biases, int64_t n_values, void *out, hipStream_t s);
+                                 const void *biases, int64_t n_values, void *out, const uint32_t *ids, int64_t cols,
+                                 int64_t table_rows, hipStream_t s);
 int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n_values, void *packed,
                            void *scales, hipStream_t s);
 int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales,
-                             int64_t n_values, void *out, hipStream_t s);
+                             int64_t n_values, void *out, const uint32_t *ids, int64_t cols, int64_t table_rows,
+                             hipStream_t s);
 int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
                               int32_t *offsets, hipStream_t s);
 

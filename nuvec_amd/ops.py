@@ -210,6 +210,35 @@ def dequantize(q: Quantized, dtype: Optional[torch.dtype] = None) -> torch.Tenso
     return out
 
 
+def embedding(q: Quantized, ids: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """nuvec-nn layers.rs:245-255 (`QuantizedEmbedding::forward`): the rows `ids` of a quantized table,
+    dequantized; shape `ids.shape + [cols]`.  Equals `dequantize` of the taken rows bit for bit."""
+    op = "dequantize_rows"
+    quant = q.quant
+    quant.checked(op)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    if q.weight.ndim != 2:
+        raise InvalidArgument(f"{op}: the table must be two-dimensional, got {list(q.weight.shape)}")
+    if ids.dtype.is_floating_point or ids.dtype == torch.bool:
+        raise InvalidArgument(f"{op}: ids must be integers, got {_name(ids.dtype)}")
+    affine = quant.mode == QuantMode.AFFINE
+    cols = _quantized_columns(op, q.weight, q.scales, q.biases, quant)
+    compute = q.scales.dtype if affine else (dtype or torch.bfloat16)
+    if compute not in _FLOATS:
+        raise InvalidArgument(f"{op}: unsupported dtype {_name(compute)}")
+    _init(q.weight)
+    w, s = _u32(q.weight).contiguous(), q.scales.contiguous()
+    b = q.biases.contiguous() if affine else None
+    flat = ids.reshape(-1) if ids.dtype == torch.uint32 else ids.reshape(-1).to(torch.int32).view(torch.uint32)
+    flat = flat.contiguous()
+    out = torch.empty(tuple(ids.shape) + (cols,), dtype=compute, device=w.device)
+    _lib.check(_lib.load().nvq_dequantize_rows(C.byref(quant._c()), _CODE[compute], _ptr(w), _ptr(s), _ptr(b), w.shape[0], cols,
+                                               _ptr(flat), flat.numel(), _ptr(out), _stream()))
+    if affine and dtype is not None and dtype != out.dtype:
+        out = out.to(dtype)
+    return out
+
+
 def _promoted(op: str, x, scales, biases) -> torch.dtype:
     """quantized.rs:491-497: affine promotes x, scales and biases; fp modes keep x's dtype."""
     dtype = x.dtype

@@ -68,6 +68,13 @@ def test_argument_errors_come_before_the_device():
     assert lib.nvq_quantize(C.byref(q), _lib.I32, None, 2, 128, None, None, None, None) == _lib.INVALID_ARGUMENT
     assert lib.nvq_dequantize(C.byref(q), _lib.F32, None, None, None, 2, 128, None, None) == _lib.INVALID_ARGUMENT
     assert _lib.last_error() == "dequantize: biases must be provided for affine quantization"
+    one = C.c_void_p(16)
+    assert lib.nvq_dequantize_rows(C.byref(q), _lib.F32, one, one, one, 4, 100, one, 2, one, None) == _lib.INVALID_ARGUMENT
+    assert "dequantize_rows: packed weights [4, 12]" in _lib.last_error()
+    assert lib.nvq_dequantize_rows(C.byref(q), _lib.F32, one, one, one, 4, 128, None, 2, one, None) == _lib.INVALID_ARGUMENT
+    assert _lib.last_error() == "dequantize_rows: null ids"
+    assert lib.nvq_dequantize_rows(C.byref(q), _lib.F32, one, one, one, 0, 128, one, 2, one, None) == _lib.INVALID_ARGUMENT
+    assert lib.nvq_dequantize_rows(C.byref(q), _lib.F32, one, one, one, 4, 128, None, 0, one, None) == _lib.OK
     d = _lib.QmmDescC()
     d.quant, d.dtype, d.transpose, d.m, d.n, d.k = q, _lib.F32, 1, 1, 8, 100
     assert lib.nvq_quantized_matmul_supported(C.byref(d)) == 0

@@ -438,3 +438,69 @@ def test_untransposed_products_batched():
     got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
     assert got.shape == (b, m, n)
     assert_rows_close(got, want, ref.F32, "batched x.w")
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(64, 4), (32, 3), (128, 8), (64, 6), (32, 2)])
+def test_embedding_rows_bit_exact(dtype, group, bits):
+    """The lookup of a quantized embedding (nuvec-nn layers.rs:245-255: take of weight, scales and biases, then
+    dequantize): equal to the oracle's dequantize of the taken rows bit for bit; repeated, first and last ids."""
+    rng = np.random.default_rng(2100 + bits + group + dtype)
+    vocab, dim = 777, 384
+    w = make_w(rng, vocab, dim, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+    ids = rng.integers(0, vocab, size=(3, 41))
+    ids[0, :4] = [0, vocab - 1, 5, 5]
+    want = ref.affine_dequantize(packed[ids.reshape(-1)], scales[ids.reshape(-1)], biases[ids.reshape(-1)], dtype, group, bits)
+    for torch_ids in (torch.tensor(ids, dtype=torch.int64), torch.tensor(ids, dtype=torch.int32)):
+        got = nv.embedding(q, torch_ids.cuda())
+        assert tuple(got.shape) == (3, 41, dim)
+        assert np.array_equal(to_host(got).reshape(-1, dim).view(np.uint8), want.view(np.uint8))
+    assert nv.embedding(q, torch.zeros((0,), dtype=torch.int64).cuda()).shape == (0, dim)
+    with pytest.raises(nv.InvalidArgument):
+        nv.embedding(q, torch.zeros(3).cuda())
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+def test_embedding_rows_block_formats(mode, qmode):
+    rng = np.random.default_rng(2200 + mode)
+    vocab, dim = 300, 256
+    w = make_w(rng, vocab, dim, ref.BF16)
+    packed, scales = ref.fp_quantize(w, ref.BF16, mode)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+    ids = rng.integers(0, vocab, size=97)
+    for out in (ref.BF16, ref.F32, ref.F16):
+        want = ref.fp_dequantize(packed[ids], scales[ids], mode, out)
+        got = to_host(nv.embedding(q, torch.tensor(ids).cuda(), TORCH[out]))
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_layers_mirror_the_reference_callers():
+    """QuantizedLinear (layers.rs:121-162) and QuantizedEmbedding (layers.rs:221-262) over the library:
+    from_linear quantizes as the oracle, forward is product + bias, the tied embedding serves both ways."""
+    from nuvec_amd.layers import QuantizedEmbedding, QuantizedLinear
+    rng = np.random.default_rng(2300)
+    n, k, m = 320, 512, 6
+    w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+    bias = make_x(rng, 1, n, ref.BF16).reshape(n)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+    layer = QuantizedLinear.from_linear(to_dev(w), to_dev(bias))
+    assert np.array_equal(to_host(layer.weight), packed)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16)
+    plain = to_host(QuantizedLinear.from_linear(to_dev(w))(to_dev(x)))
+    assert_rows_close(plain, want, ref.BF16, "QuantizedLinear without bias")
+    # The bias is one more rounded addition on the product this library returned.
+    with_bias = to_host(layer(to_dev(x)))
+    expect = ref.from_f32(ref.to_f32(plain, ref.BF16) + ref.to_f32(bias, ref.BF16), ref.BF16)
+    assert np.array_equal(with_bias.view(np.uint8), expect.view(np.uint8))
+    assert np.array_equal(to_host(layer.dequantized_weight()).view(np.uint8),
+                          ref.affine_dequantize(packed, scales, biases, ref.BF16, 64, 4).view(np.uint8))
+    emb = QuantizedEmbedding.from_embedding(to_dev(w), nv.QuantMode.MXFP4)
+    fp_packed, fp_scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+    ids = rng.integers(0, n, size=(2, 9))
+    assert np.array_equal(to_host(emb(torch.tensor(ids).cuda())).reshape(-1, k).view(np.uint8),
+                          ref.fp_dequantize(fp_packed[ids.reshape(-1)], fp_scales[ids.reshape(-1)], ref.MXFP4, ref.BF16).view(np.uint8))
+    tied = to_host(emb.as_linear(to_dev(x)))
+    want = ref.quantized_matmul(x, fp_packed, fp_scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16)
+    assert_rows_close(tied, want, ref.BF16, "tied embedding")
