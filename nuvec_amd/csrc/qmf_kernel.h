@@ -77,14 +77,15 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// Byte B of `v` as a float (v_cvt_f32_ubyteB).  `opaque` hides how a word was masked, so that the compiler keeps
+// the byte conversions instead of re-deriving bit-field extracts from the mask.
+__device__ __forceinline__ uint32_t opaque(uint32_t v) {
+    asm("" : "+v"(v));
+    return v;
+}
 template <int B>
 __device__ __forceinline__ float ubyte_to_float(uint32_t v) {
-    float f;
-    if constexpr (B == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v));
-    else if constexpr (B == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v));
-    else if constexpr (B == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v));
-    else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v));
-    return f;
+    return (float)((v >> (8 * B)) & 0xFFu);
 }
 
 template <typename T> struct Ops;
@@ -140,7 +141,7 @@ __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float 
         r.w = Ops<T>::template fp4_pair<3>(word, s);
     } else if constexpr (BITS == 4) {
         const uint32_t word = dw[KK];
-        const uint32_t even = word & 0x0F0F0F0Fu, odd = (word >> 4) & 0x0F0F0F0Fu;
+        const uint32_t even = opaque(word & 0x0F0F0F0Fu), odd = opaque((word >> 4) & 0x0F0F0F0Fu);
         r.x = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<0>(even), s, b), __builtin_fmaf(ubyte_to_float<0>(odd), s, b));
         r.y = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<1>(even), s, b), __builtin_fmaf(ubyte_to_float<1>(odd), s, b));
         r.z = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<2>(even), s, b), __builtin_fmaf(ubyte_to_float<2>(odd), s, b));

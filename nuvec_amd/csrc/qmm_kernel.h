@@ -37,21 +37,23 @@ using namespace qmf;  // element operations and code expansion
 constexpr int BK = 64;
 constexpr int kStages = 3;
 constexpr int kRowBytes = BK * 2;   // 128 B per x row in LDS
-constexpr int kPeriod = 256;        // values of K per scale/bias table
 
-// A block's tile: WM x WN wavefronts, each TI x TJ matrix tiles of 32 x 32.  The number of threads equals
-// twice the weight rows (one loading lane per row half) and the x tile takes four 16-byte pieces per thread.
+// A block's tile: WM x WN wavefronts, each TI x TJ matrix tiles of 32 x 32.  Per step a thread brings kXParts
+// 16-byte pieces of the x tile and the codes of kWSlots weight row halves (32 codes each).
 template <int WM_, int WN_, int TI_, int TJ_>
 struct Tile {
     static constexpr int WM = WM_, WN = WN_, TI = TI_, TJ = TJ_;
     static constexpr int BM = WM * TI * 32, BN = WN * TJ * 32;
     static constexpr int kThreads = WM * WN * 64;
     static constexpr int kXBytes = BM * kRowBytes;
-    static constexpr int kSbBytes = (kPeriod / 32) * BN * 4;  // one table: up to 8 groups x BN rows x (scale, bias)
-    static_assert(kThreads == 2 * BN && BM * 8 == 4 * kThreads, "the loading assignment below assumes these");
+    static constexpr int kSbBytes = 2 * 4 * BN * 4;  // one table: (scales, biases) x 4 groups x BN rows, a dword each
+    static constexpr int kXParts = BM * 8 / kThreads, kWSlots = 2 * BN / kThreads;
+    static constexpr int kWavesPerSimd = TI * TJ >= 16 ? 1 : 2;  // by the accumulators: 256 or 128 registers of the 512
+    static_assert(kXParts % 4 == 0 && kXParts * kThreads == BM * 8 && kWSlots * kThreads == 2 * BN && BN <= kThreads,
+                  "the loading assignment below assumes these");
 };
-using BigTile = Tile<2, 4, 4, 2>;    // 256 x 256, 512 threads
-using SmallTile = Tile<2, 2, 2, 2>;  // 128 x 128, 256 threads: for products whose big tiles would not fill the chip
+using BigTile = Tile<1, 4, 8, 2>;    // 256 x 256, 256 threads: one wavefront per SIMD owns 256 x 64, no code is expanded twice
+using SmallTile = Tile<2, 2, 2, 2>;  // 128 x 128, 256 threads, two blocks per compute unit: for products whose big tiles would not fill the chip
 
 // How a lane's BITS dwords travel into LDS: one or two pieces of 4, 3 or 1 dwords.
 template <int BITS> struct Pieces;
@@ -65,15 +67,18 @@ template <int BITS, class TL>
 struct Geometry {
     // a 12-byte piece lands at 16 bytes per lane, like a 16-byte one (its fourth dword is not written)
     static constexpr int kPieceBytes = Pieces<BITS>::dwords == 1 ? 4 : 16;  // of LDS per lane and piece
-    static constexpr int kRegionBytes = TL::kThreads * kPieceBytes;     // one piece of every loading lane
+    static constexpr int kRegionBytes = 2 * TL::BN * kPieceBytes;       // one piece of every row half
     static constexpr int kWBytes = Pieces<BITS>::count * kRegionBytes;  // packed codes of one step
     static constexpr int kStageBytes = TL::kXBytes + kWBytes;
     static constexpr int kLdsBytes = kStages * kStageBytes + 2 * TL::kSbBytes;  // big tile: 136 KB at 4 bits, 160 KB at 8
-    static constexpr int kParts = 4 + Pieces<BITS>::count;              // direct-to-LDS loads per step and lane
+    static constexpr int kParts = TL::kXParts + TL::kWSlots * Pieces<BITS>::count;  // direct-to-LDS loads per step and lane
 };
 
-// Byte offset of 16-byte chunk `chunk` (0..7) of LDS row `row`.
-__device__ __forceinline__ int lds_offset(int row, int chunk) { return row * kRowBytes + ((chunk ^ (row & 7)) << 4); }
+// Byte offset of 16-byte chunk `chunk` (0..7) of LDS row `row`.  The LDS has 64 banks of 4 bytes: sixteen
+// consecutive rows reading the same chunk fall on sixteen different 16-byte bank groups (the row's parity picks
+// the half, the swizzle the group within it).
+__device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int lds_offset(int row, int chunk) { return row * kRowBytes + ((chunk ^ swizzle(row)) << 4); }
 
 // Low / high 16 bits of a table entry as element-type values.
 template <typename T> __device__ __forceinline__ float half_lo(uint32_t p);
@@ -83,26 +88,56 @@ template <> __device__ __forceinline__ float half_hi<bf16_t>(uint32_t p) { retur
 template <> __device__ __forceinline__ float half_lo<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[0]; }
 template <> __device__ __forceinline__ float half_hi<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[1]; }
 
-// DWORDS x 4 bytes per lane from global memory straight into LDS: lane l of the wavefront writes
-// lds_base + 16 l (4 l for a single dword).  Issued as assembly so that the compiler keeps no account of it: the waits are
-// placed by hand (dma_wait), which is what lets the loads of later steps stay in flight across
-// the LDS reads of the current one.
+// DWORDS x 4 bytes per lane from global memory straight into LDS: lane l of the wavefront reads base + offset
+// (a wavefront-uniform base, so the per-step address arithmetic is scalar) and writes lds_base + 16 l (4 l for
+// a single dword).  Issued as assembly so that the compiler keeps no account of it: the waits are placed by hand
+// (dma_wait), which is what lets the loads of later steps stay in flight across the LDS reads of the current one.
 template <int DWORDS>
-__device__ __forceinline__ void dma(const void *src, uint32_t lds_base) {
+__device__ __forceinline__ void dma(const void *base, uint32_t offset, uint32_t lds_base) {
     if constexpr (DWORDS == 4)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(src) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
     else if constexpr (DWORDS == 3)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx3 %1, off" : : "s"(lds_base), "v"(src) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx3 %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
     else
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_base), "v"(src) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void dma_wait() {  // all but the N most recent vector-memory loads of this lane are complete
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
+// One 16-bit (or 8-bit) element per lane, zero-extended to the dword at lds_base + 4 l.
+template <int BYTES>
+__device__ __forceinline__ void dma_element(const void *base, uint32_t offset, uint32_t lds_base) {
+    if constexpr (BYTES == 2)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ubyte %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
+}
+// Nothing moves across this point when the compiler orders the instructions: the interleaving of matrix
+// instructions, LDS reads and code expansion below is the written one.
+__device__ __forceinline__ void pin() { __builtin_amdgcn_sched_barrier(0); }
+// A use of `v` at this point: what computes it stays in this block of the loop instead of sinking into the block
+// of its first real use, where nothing would run beside it.
+__device__ __forceinline__ void keep(const uint4 &v) { asm volatile("" : : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)); }
+
+// Dword D (two elements) of piece KK of a lane's 32 codes: expand_piece, one register at a time.
+template <typename T, int BITS, bool FP4, int KK, int D>
+__device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], float s, float b) {
+    if constexpr (FP4) {
+        return Ops<T>::template fp4_pair<D>(dw[KK], s);
+    } else if constexpr (BITS == 4) {
+        const uint32_t word = dw[KK];
+        const uint32_t even = opaque(word & 0x0F0F0F0Fu), odd = opaque((word >> 4) & 0x0F0F0F0Fu);
+        return Ops<T>::pack(__builtin_fmaf(ubyte_to_float<D>(even), s, b), __builtin_fmaf(ubyte_to_float<D>(odd), s, b));
+    } else {
+        constexpr int J = 8 * KK + 2 * D;
+        return Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 1>(dw), s, b));
+    }
+}
 
 template <typename T, int BITS, bool FP4, bool BATCHED, class TL>
-__global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) {
+__global__ void __launch_bounds__(TL::kThreads) __attribute__((amdgpu_waves_per_eu(TL::kWavesPerSimd, TL::kWavesPerSimd)))
+qmm_kernel(const ProductArgs a) {
     using G = Geometry<BITS, TL>;
     constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kXBytes = TL::kXBytes, kSbBytes = TL::kSbBytes;
     constexpr int TI = TL::TI, TJ = TL::TJ;
@@ -110,14 +145,17 @@ __global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) 
     using S = std::conditional_t<FP4, uint8_t, T>;  // stored scale type
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
-    uint32_t *sb_table = reinterpret_cast<uint32_t *>(lds + kStages * G::kStageBytes);  // [2][group][row]: scale | bias << 16
+    // Scale and bias tables, two buffers of [scale | bias][group 0..3][row] dwords (the element in the low bits).
+    const uint32_t *sb_table = reinterpret_cast<const uint32_t *>(lds + kStages * G::kStageBytes);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / TL::WN, wn = wave % TL::WN;  // wavefront grid WM x WN: 32 TI x 32 TJ each
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int row_dwords = (K >> 5) * BITS, kgroups = K >> gshift;
-    const int gper = kPeriod >> gshift;  // groups per table: 8, 4 or 2
+    // A table covers a period of 4 groups (2 of 128): two steps for groups of 32, else four.
+    const int pshift = gshift == 5 ? 1 : 2, psteps = 1 << pshift;
+    const int gper = (psteps * BK) >> gshift;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     int64_t bx = 0, bw = 0, bs = 0, by = 0;
     if constexpr (BATCHED) {  // a batch with one stride per operand
@@ -132,66 +170,77 @@ __global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) 
     T *y = (T *)a.y + by;
 
     // Direct-to-LDS assignment.  x: instruction i of wavefront v fills the 64 consecutive 16-byte
-    // slots starting at slot i*512 + v*64; slot S is row S/8, position S%8, and holds chunk
-    // position ^ (row & 7) of that row.  w: loading lane v*64 + l is half l%2 of row (v*64 + l)/2 and owns the
-    // BITS dwords of that half's 32 codes.
-    const T *xsrc[4];
+    // slots starting at slot i*kThreads + v*64; slot S is row S/8, position S%8, and holds chunk
+    // position ^ (row & 7) of that row.  w: loading slot S is half S%2 of row S/2 and owns the BITS dwords of that
+    // half's 32 codes.  Addresses are a block-uniform base (advanced per step with scalar arithmetic) plus a
+    // per-lane byte offset that never changes.
+    constexpr int XP = TL::kXParts, WS = TL::kWSlots;
+    const char *xbase = reinterpret_cast<const char *>(x + (int64_t)m0 * K);
+    const char *wbase = reinterpret_cast<const char *>(w + (int64_t)n0 * row_dwords);
+    uint32_t xoff[XP], woff[WS];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int slot = i * kThreads + wave * 64 + lane, row = slot >> 3, chunk = (slot & 7) ^ (row & 7);
-        const int grow = m0 + row < M ? m0 + row : M - 1;  // tail rows are computed, not stored
-        xsrc[i] = x + (int64_t)grow * K + chunk * 8;
+    for (int i = 0; i < XP; i++) {
+        const int slot = i * kThreads + wave * 64 + lane, row = slot >> 3, chunk = (slot & 7) ^ swizzle(row);
+        const int r = m0 + row < M ? row : M - 1 - m0;  // tail rows are computed, not stored
+        xoff[i] = ((uint32_t)r * (uint32_t)K + chunk * 8) * 2;
     }
-    const int wslot = wave * 64 + lane;
-    const int wrow = n0 + (wslot >> 1) < N ? n0 + (wslot >> 1) : N - 1;
-    const uint32_t *wsrc = w + (int64_t)wrow * row_dwords + (wslot & 1) * BITS;
+#pragma unroll
+    for (int j = 0; j < WS; j++) {
+        const int slot = j * kThreads + wave * 64 + lane;
+        const int r = n0 + (slot >> 1) < N ? (slot >> 1) : N - 1 - n0;
+        woff[j] = ((uint32_t)r * (uint32_t)row_dwords + (slot & 1) * BITS) * 4;
+    }
     const int steps = K / BK;  // K is a multiple of 64 (checked on the host)
-    // Load `part` (0..3: x, 4..: the pieces of w) of `step`.
-    auto issue_part = [&](int step, int part) {
-        const int sc = step < steps ? step : steps - 1;  // past the end: a harmless reload, keeps the wait counts uniform
-        const uint32_t base = lds0 + (step % kStages) * G::kStageBytes;
-        if (part < 4) {
-            dma<4>(xsrc[part] + sc * BK, base + (part * kThreads + wave * 64) * 16);
+    // The loads of one step: its global bases (a step past the end reloads the last one, harmlessly, which keeps
+    // the wait counts uniform) and the LDS address of this wavefront's lane 0 in the step's stage.
+    struct Loads {
+        const char *x, *w[P::count];
+        uint32_t lds;
+    };
+    const uint32_t lds_wave = lds0 + wave * 64 * 16;
+    auto loads_of = [&](int step, int stage) {
+        const int sc = step < steps ? step : steps - 1;
+        Loads l;
+        l.x = xbase + sc * (BK * 2);
+#pragma unroll
+        for (int piece = 0; piece < P::count; piece++) l.w[piece] = wbase + sc * (2 * BITS * 4) + piece * (P::dwords * 4);
+        l.lds = lds_wave + stage * G::kStageBytes;
+        // computed here once, in scalar registers, not again at every load
+        asm volatile("" : "+s"(l.x), "+s"(l.lds));
+#pragma unroll
+        for (int piece = 0; piece < P::count; piece++) asm volatile("" : "+s"(l.w[piece]));
+        return l;
+    };
+    // Load `part` (0..XP-1: x, then the pieces of each weight slot).
+    auto issue_part = [&](const Loads &l, auto part_tag) {
+        constexpr int part = decltype(part_tag)::value;
+        if constexpr (part < XP) {
+            dma<4>(l.x, xoff[part], l.lds + part * kThreads * 16);
         } else {
-            const int piece = part - 4;
-            dma<P::dwords>(wsrc + sc * 2 * BITS + piece * P::dwords, base + kXBytes + piece * G::kRegionBytes + wave * 64 * G::kPieceBytes);
+            constexpr int j = (part - XP) / P::count, piece = (part - XP) % P::count;
+            // the wavefront's share of a weight region starts at wave * 64 pieces, not wave * 64 * 16 bytes
+            constexpr int off = kXBytes + piece * G::kRegionBytes + j * kThreads * G::kPieceBytes;
+            dma<P::dwords>(l.w[piece], woff[j], l.lds + off - (G::kPieceBytes == 16 ? 0 : wave * 64 * 12));
         }
     };
-    auto issue = [&](int step) {
-#pragma unroll
-        for (int part = 0; part < G::kParts; part++) issue_part(step, part);
+    auto issue_parts = [&](const Loads &l, auto first_tag, auto count_tag) {
+        static_for<decltype(count_tag)::value>([&](auto i) { issue_part(l, std::integral_constant<int, decltype(first_tag)::value + decltype(i)::value>{}); });
     };
-
-    // Scale/bias tables: thread t < BN owns tile row t.
-    const int srow = n0 + (tid % BN) < N ? n0 + (tid % BN) : N - 1;
-    const S *sp = scales + (int64_t)srow * kgroups, *bp = biases + (int64_t)srow * kgroups;
-    S sreg[8], breg[8];
-    auto sb_load = [&](int period) {
-        if (tid < BN) {
+    // The table of period `period`: every wavefront brings kTableLoads times 64 consecutive rows of one group's
+    // scales or biases (groups past the row's last one repeat it: they are never read).
+    constexpr int kKinds = FP4 ? 1 : 2, kTableLoads = kKinds * 4 * BN / kThreads;
+    const int trow = n0 + tid % BN < N ? tid % BN : N - 1 - n0;
+    const uint32_t toff = (uint32_t)trow * (uint32_t)kgroups * (uint32_t)sizeof(S);
+    const char *sbase = reinterpret_cast<const char *>(scales + (int64_t)n0 * kgroups);
+    const char *bbase = reinterpret_cast<const char *>(biases + (int64_t)n0 * kgroups);
+    auto issue_table = [&](int period) {
+        const uint32_t tbase = lds0 + kStages * G::kStageBytes + (period & 1) * kSbBytes;
 #pragma unroll
-            for (int g = 0; g < 8; g++)
-                if (g < gper) {
-                    const int gi = period * gper + g < kgroups ? period * gper + g : kgroups - 1;
-                    sreg[g] = sp[gi];
-                    if constexpr (!FP4) breg[g] = bp[gi];
-                }
-        }
-    };
-    auto sb_store = [&](int period) {
-        if (tid < BN) {
-            uint32_t *t = sb_table + (period & 1) * (kSbBytes / 4);
-#pragma unroll
-            for (int g = 0; g < 8; g++)
-                if (g < gper) {
-                    if constexpr (FP4) {
-                        t[g * BN + tid] = (uint32_t)sreg[g];
-                    } else {
-                        uint16_t sbits, bbits;
-                        __builtin_memcpy(&sbits, &sreg[g], 2);
-                        __builtin_memcpy(&bbits, &breg[g], 2);
-                        t[g * BN + tid] = (uint32_t)sbits | ((uint32_t)bbits << 16);
-                    }
-                }
+        for (int i = 0; i < kTableLoads; i++) {
+            const int entry = i * kThreads + wave * 64;  // of this wavefront's first lane: [kind][group][row]
+            const int kind = entry / (4 * BN), g = (entry / BN) % 4;
+            const int gi = period * gper + g < kgroups ? period * gper + g : kgroups - 1;
+            dma_element<sizeof(S)>((kind ? bbase : sbase) + gi * (int)sizeof(S), toff, tbase + entry * 4);
         }
     };
 
@@ -204,22 +253,13 @@ __global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) 
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     const int h = lane >> 5, l32 = lane & 31;
-    issue(0);
-    issue(1);
-    sb_load(0);
-    sb_store(0);
-    for (int step = 0; step < steps; step++) {
-        dma_wait<G::kParts>();  // this lane's loads of `step` have landed (those of step + 1 may be in flight)
-        __syncthreads();        // ... and everyone's; everyone is also done reading the stage refilled next
-        // The table of the next 256 values of K is loaded two steps ahead and written one step ahead.
-        // Its loads go before this step's direct-to-LDS loads so that the wait above never covers them.
-        if ((step & 3) == 1 && step + 3 < steps) sb_load((step + 3) >> 2);
-#pragma unroll
-        for (int part = 4; part < G::kParts; part++) issue_part(step + 2, part);  // the x parts are spread over the matrix work below
-        const unsigned char *xs = lds + (step % kStages) * G::kStageBytes, *ws = xs + kXBytes;
-        const uint32_t *sbt = sb_table + ((step >> 2) & 1) * (kSbBytes / 4) + ((((step & 3) * BK + 32 * h) >> gshift) * BN);
-        uint32_t raw[TJ][BITS];
-        float sc[TJ], bi[TJ];
+    uint32_t raw[TJ][BITS], sraw[TJ], braw[TJ];  // codes and table entries as read: converted where first used
+    float sc[TJ], bi[TJ];
+    uint4 af[2][TI], bf[2][TJ];
+    // The packed codes, scales and biases of this lane's TJ columns for `step` (its stage and table are visible).
+    auto read_codes = [&](int step, int stage) {
+        const unsigned char *ws = lds + stage * G::kStageBytes + kXBytes;
+        const uint32_t *sbt = sb_table + ((step >> pshift) & 1) * (kSbBytes / 4) + ((((step & (psteps - 1)) * BK + 32 * h) >> gshift) * BN);
 #pragma unroll
         for (int j = 0; j < TJ; j++) {
             const int col = wn * (32 * TJ) + j * 32 + l32;
@@ -234,57 +274,122 @@ __global__ void __launch_bounds__(TL::kThreads) qmm_kernel(const ProductArgs a) 
                     for (int d = 0; d < P::dwords; d++) raw[j][P::dwords * piece + d] = reinterpret_cast<const uint32_t *>(src)[d];
                 }
             }
-            const uint32_t sbv = sbt[col];
-            if constexpr (FP4) {
-                sc[j] = ftz(e8m0_to_f32((uint8_t)sbv));
-                bi[j] = 0.0f;
-            } else {
-                sc[j] = half_lo<T>(sbv);
-                bi[j] = half_hi<T>(sbv);
-            }
+            sraw[j] = sbt[col];
+            if constexpr (!FP4) braw[j] = sbt[4 * BN + col];
         }
-        // x fragments are read one substep ahead of the matrix instructions that use them.
-        uint4 af[2][TI];
-#pragma unroll
-        for (int i = 0; i < TI; i++) af[0][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * (32 * TI) + i * 32 + l32, 4 * h));
+    };
+    auto convert_scales = [&](int j) {
+        if constexpr (FP4) {
+            sc[j] = ftz(e8m0_to_f32((uint8_t)sraw[j]));
+            bi[j] = 0.0f;
+        } else {
+            sc[j] = half_lo<T>(sraw[j]);
+            bi[j] = half_lo<T>(braw[j]);
+        }
+    };
+    // x fragment i of substep kk of the step in `stage`.
+    auto read_x = [&](int stage, int kk, int i) {
+        return *reinterpret_cast<const uint4 *>(lds + stage * G::kStageBytes + lds_offset(wm * (32 * TI) + i * 32 + l32, 4 * h + kk));
+    };
+    // The side work that prepares substep (step, KK) into buffer (KK & 1), in items: first x fragment reads and
+    // expanded dwords alternate, then what is left of either.  Item t of kItems.
+    // Substep 0 of the next step takes all reads first: its codes were only just requested.
+    constexpr int kItems = TI + 4 * TJ, kPairs = TI < 4 * TJ ? TI : 4 * TJ;
+    auto side_item = [&](int stage, auto kk_tag, auto t_tag) {
+        constexpr int KK = decltype(kk_tag)::value, t = decltype(t_tag)::value;
+        constexpr bool alternate = KK != 0 && t < 2 * kPairs;
+        constexpr bool is_read = KK == 0 ? t < TI : (alternate ? t % 2 == 0 : TI > 4 * TJ);
+        constexpr int index = KK == 0 ? (t < TI ? t : t - TI) : (alternate ? t / 2 : t - kPairs);
+        if constexpr (is_read) {
+            af[KK & 1][index] = read_x(stage, KK, index);
+        } else {
+            constexpr int j = index / 4, d = index % 4;
+            if constexpr (KK == 0 && d == 0) convert_scales(j);
+            const uint32_t v = expand_dword<T, BITS, FP4, KK, d>(raw[j], sc[j], bi[j]);
+            if constexpr (d == 0) bf[KK & 1][j].x = v;
+            else if constexpr (d == 1) bf[KK & 1][j].y = v;
+            else if constexpr (d == 2) bf[KK & 1][j].z = v;
+            else bf[KK & 1][j].w = v;
+        }
+    };
+
+    // Prologue: tables, two steps of loads in flight, the first substep's operands.
+    issue_table(0);
+    if (psteps == 2) issue_table(1);
+    using c0 = std::integral_constant<int, 0>;
+    issue_parts(loads_of(0, 0), c0{}, std::integral_constant<int, G::kParts>{});
+    issue_parts(loads_of(1, 1), c0{}, std::integral_constant<int, G::kParts>{});
+    dma_wait<G::kParts>();
+    __syncthreads();
+    read_codes(0, 0);
+    static_for<kItems>([&](auto t) { side_item(0, c0{}, t); });
+
+    constexpr int kMfmas = TI * TJ;
+    int stage = 0;  // step % kStages
+    for (int step = 0; step < steps; step++) {
+        // Entering: stage `step` is visible to everyone, this lane holds its codes, and buffer 0 holds substep 0.
+        const int stage1 = stage == kStages - 1 ? 0 : stage + 1, stage2 = stage1 == kStages - 1 ? 0 : stage1 + 1;
+        const Loads next2 = loads_of(step + 2, stage2);
+        issue_parts(next2, std::integral_constant<int, XP>{}, std::integral_constant<int, G::kParts - XP>{});  // w first; x is spread below
         static_for<4>([&](auto kk_tag) {
             constexpr int kk = decltype(kk_tag)::value;
-            uint4 bf[TJ];
-            if constexpr (kk < 3) {
-#pragma unroll
-                for (int i = 0; i < TI; i++)
-                    af[(kk + 1) & 1][i] = *reinterpret_cast<const uint4 *>(xs + lds_offset(wm * (32 * TI) + i * 32 + l32, 4 * h + kk + 1));
+            constexpr int next = (kk + 1) & 3;
+            using next_tag = std::integral_constant<int, next>;
+            if constexpr (kk == 3) {
+                // The step's last substep also turns to the next step: its stage must have landed for everyone
+                // (and everyone is done reading the stage that the next loads refill), then its codes and first
+                // operands are read and expanded under this substep's matrix instructions.
+                issue_parts(next2, std::integral_constant<int, 3 * (XP / 4)>{}, std::integral_constant<int, XP - 3 * (XP / 4)>{});
+                // (a table issued after the previous step's barrier is older than those loads: it is waited for too,
+                // a step after its issue rather than two)
+                dma_wait<G::kParts>();
+                __syncthreads();
+                if (((step + 3) & (psteps - 1)) == 0 && step + 3 < steps) issue_table((step + 3) >> pshift);
+                read_codes(step + 1, stage1);
+                pin();
             }
+            static_for<kMfmas>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value, i = q % TI, j = q / TI;
+                acc[i][j] = Ops<T>::mfma(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
+                static_for<kItems>([&](auto t_tag) {
+                    constexpr int t = decltype(t_tag)::value;
+                    if constexpr (t >= q * kItems / kMfmas && t < (q + 1) * kItems / kMfmas) side_item(kk == 3 ? stage1 : stage, next_tag{}, t_tag);
+                });
+                pin();
+            });
+            if constexpr (kk < 3) issue_parts(next2, std::integral_constant<int, kk * (XP / 4)>{}, std::integral_constant<int, XP / 4>{});
+            if constexpr (kk >= 2) {  // the blocks of the loop end after substeps 2 and 3
 #pragma unroll
-            for (int j = 0; j < TJ; j++) bf[j] = expand_piece<T, BITS, FP4, kk>(raw[j], sc[j], bi[j]);
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++) acc[i][j] = Ops<T>::mfma(af[kk & 1][i], bf[j], acc[i][j]);
-            issue_part(step + 2, kk);
+                for (int j = 0; j < TJ; j++) keep(bf[next & 1][j]);
+            }
         });
-        if ((step & 3) == 2 && step + 2 < steps) sb_store((step + 2) >> 2);
+        stage = stage1;
     }
     dma_wait<0>();
 
     // Epilogue: accumulator element e of a 32 x 32 tile is row 8 (e / 4) + 4 (lane / 32) + e % 4, column lane % 32.
     // The 32 lanes of a half-wavefront store 32 consecutive elements of one row.
-    const bool full = m0 + BM <= M && n0 + BN <= N;
+    auto store_tile = [&](auto whole_tag) {
+        constexpr bool whole = decltype(whole_tag)::value;  // the tile lies inside y: no element is tested
+        uint16_t *out0 = reinterpret_cast<uint16_t *>(y) + (int64_t)(m0 + wm * (32 * TI) + 4 * h) * N + n0 + wn * (32 * TJ) + l32;
 #pragma unroll
-    for (int i = 0; i < TI; i++)
+        for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < TJ; j++) {
-            const int col = n0 + wn * (32 * TJ) + j * 32 + l32;
-            const int row0 = m0 + wm * (32 * TI) + i * 32 + 4 * h;
+            for (int j = 0; j < TJ; j++) {
+                const int col = n0 + wn * (32 * TJ) + j * 32 + l32;
+                const int row0 = m0 + wm * (32 * TI) + i * 32 + 4 * h;
 #pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-                const uint32_t pair = Ops<T>::pack(acc[i][j][e], acc[i][j][e + 1]);  // rounded to nearest even
-                const int row = row0 + 8 * (e >> 2) + (e & 3);
-                uint16_t *out = reinterpret_cast<uint16_t *>(y) + (int64_t)row * N + col;
-                if (full || (row < M && col < N)) out[0] = (uint16_t)pair;
-                if (full || (row + 1 < M && col < N)) out[N] = (uint16_t)(pair >> 16);
+                for (int e = 0; e < 16; e += 2) {
+                    const uint32_t pair = Ops<T>::pack(acc[i][j][e], acc[i][j][e + 1]);  // rounded to nearest even
+                    const int r = i * 32 + 8 * (e >> 2) + (e & 3);
+                    uint16_t *out = out0 + (int64_t)r * N + j * 32;
+                    if (whole || (row0 + r - i * 32 < M && col < N)) out[0] = (uint16_t)pair;
+                    if (whole || (row0 + r - i * 32 + 1 < M && col < N)) out[N] = (uint16_t)(pair >> 16);
+                }
             }
-        }
+    };
+    if (m0 + BM <= M && n0 + BN <= N) store_tile(std::true_type{});
+    else store_tile(std::false_type{});
 }
 
 // Estimated microseconds of the tiled kernel with tile TL on `cus` compute units, from its measured behaviour:
