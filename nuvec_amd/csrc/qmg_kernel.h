@@ -46,7 +46,9 @@ struct Geometry {
 };
 
 template <typename T, int BITS, bool FP4>
-__global__ void __launch_bounds__(kThreads) qmg_kernel(const ProductArgs a) {
+// Three blocks per compute unit (three wavefronts per SIMD): the registers are capped for that, and the LDS of a
+// block (two x stages, the weight stages, the table) fits three times.
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) qmg_kernel(const ProductArgs a) {
     using G = Geometry<BITS>;
     constexpr int kDepth = G::kDepth, kLoads = G::kLoads;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -164,13 +166,16 @@ __global__ void __launch_bounds__(kThreads) qmg_kernel(const ProductArgs a) {
         auto load_x = [&](int win, u32x4_t (&xq)[4]) {
             // a window of one step has no second half: those chunks (pieces 8..15) fetch the first half again
             const int k0 = win < windows ? win * 128 - ((2 * win + 1 >= steps && xc >= 8) ? 64 : 0) : 0;
+            // chunks 2 and 3 are rows 32..63: fetched only when the pass has a second tile (the loads are issued
+            // either way, so that the waits see the same number of them: a tile-less one reads the start of x)
 #pragma unroll
-            for (int i = 0; i < 4; i++) xq[i] = *reinterpret_cast<const u32x4_t *>(xsrc[i] + k0);
+            for (int i = 0; i < 4; i++) xq[i] = *reinterpret_cast<const u32x4_t *>(i < 2 || two ? xsrc[i] + k0 : x);
         };
         auto store_x = [&](int win, const u32x4_t (&xq)[4]) {
             unsigned char *dst = lds + (win & 1) * kXStageBytes;
 #pragma unroll
-            for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4_t *>(dst + xstore[i]) = xq[i];
+            for (int i = 0; i < 4; i++)
+                if (i < 2 || two) *reinterpret_cast<u32x4_t *>(dst + xstore[i]) = xq[i];
         };
 
         floatx16_t acc[2];
@@ -221,19 +226,43 @@ __global__ void __launch_bounds__(kThreads) qmg_kernel(const ProductArgs a) {
                     }
                 asm volatile("" ::: "memory");
                 if (win < windows) {
+                    // All x operands of a tile are requested before the first matrix instruction needs one (LDS
+                    // answers in order), so the window pays the LDS latency once, not once per instruction.  A
+                    // window of one step reads its absent second step too (stale but valid LDS) and skips its
+                    // matrix instructions.
                     const unsigned char *xs = lds + (win & 1) * kXStageBytes;
+                    const bool second_step = 2 * win + 1 < steps;
+                    uint4 xf[2][4], wb[2][4];
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+#pragma unroll
+                        for (int kk = 0; kk < 4; kk++) xf[t][kk] = *reinterpret_cast<const uint4 *>(xs + xread[t][kk]);
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        if (2 * win + t < steps) {
-                            float scale, bias;
-                            load_scales(2 * win + t, scale, bias);
-                            static_for<4>([&](auto kk_tag) {
-                                constexpr int kk = decltype(kk_tag)::value;
-                                const uint4 wb = expand_piece<T, BITS, FP4, kk>(codes[t], scale, bias);
-                                acc[0] = Ops<T>::mfma(*reinterpret_cast<const uint4 *>(xs + xread[t][kk]), wb, acc[0]);
-                                if (two) acc[1] = Ops<T>::mfma(*reinterpret_cast<const uint4 *>(xs + 32 * 256 + xread[t][kk]), wb, acc[1]);
-                            });
+                        float scale, bias;
+                        load_scales(2 * win + (t == 0 || second_step ? t : 0), scale, bias);
+                        static_for<4>([&](auto kk_tag) {
+                            constexpr int kk = decltype(kk_tag)::value;
+                            wb[t][kk] = expand_piece<T, BITS, FP4, kk>(codes[t], scale, bias);
+                        });
+                    }
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+                        if (t == 0 || second_step) {
+#pragma unroll
+                            for (int kk = 0; kk < 4; kk++) acc[0] = Ops<T>::mfma(xf[t][kk], wb[t][kk], acc[0]);
                         }
+                    if (two) {
+#pragma unroll
+                        for (int t = 0; t < 2; t++)
+#pragma unroll
+                            for (int kk = 0; kk < 4; kk++) xf[t][kk] = *reinterpret_cast<const uint4 *>(xs + 32 * 256 + xread[t][kk]);
+#pragma unroll
+                        for (int t = 0; t < 2; t++)
+                            if (t == 0 || second_step) {
+#pragma unroll
+                                for (int kk = 0; kk < 4; kk++) acc[1] = Ops<T>::mfma(xf[t][kk], wb[t][kk], acc[1]);
+                            }
                     }
                 }
                 // the next window of x goes into the other stage (last read one window ago, before the previous
