@@ -6,21 +6,25 @@
 // fma(code, scale, bias)) and the products accumulate in float32
 // (crates/nuvec-kernels/src/metal/quantized.h:583-817, 1358-1485).
 //
-// One block of 512 threads (eight wavefronts, 2 x 4, each 128 x 64 of y) owns a BM x BN = 256 x 256 tile
-// and walks K in steps of BK = 64 through a ring of three LDS stages (products whose 256 x 256 tiles would not
-// fill the chip take 128 x 128 tiles of four wavefronts, two blocks per compute unit).  A stage holds
-//   * the x tile, 256 rows x 128 B, 16-byte chunk index XOR-ed with (row & 7) so that the 16-byte
-//     fragment reads of the matrix instruction are bank-conflict free, and
-//   * the w tile still packed, 256 rows x 8 BITS bytes: lane (row, half) of the loading threads owns the BITS
-//     dwords of its 32 codes and brings them in one or two pieces (16, 12 or 4 bytes each), each piece of all
-//     lanes forming one region of the stage (16 bytes per lane, 4 for single dwords).
-// Both arrive by direct global-to-LDS loads (no registers, no copy instructions); the loads of step
-// s+2 are issued before the matrix work of step s, and there is one barrier per step.  Scales and
-// biases are staged per 256 values of K (four steps) in a small double-buffered LDS table.
-// A wavefront dequantizes its own weight fragments right before use: per step and lane the LDS reads
-// bring the 64 codes of its two columns; 8 codes -> float -> fma(code, scale, bias) -> packed element type
-// (MXFP4: scaled FP4 conversions) make one matrix operand.  With two wavefronts per
-// SIMD the conversion arithmetic of one runs under the matrix instructions of the other.
+// One block of 256 threads (four wavefronts, one per SIMD, each 256 x 64 of y in 256 accumulator registers) owns a
+// BM x BN = 256 x 256 tile and walks K in steps of BK = 64 through a ring of three LDS stages (products whose
+// 256 x 256 tiles would not fill the chip take 128 x 128 tiles of 2 x 2 wavefronts, two blocks per compute unit).
+// A wavefront covers all rows of the tile, so every weight is expanded once per block.  A stage holds
+//   * the x tile, 256 rows x 128 B, 16-byte chunk index XOR-ed with (row >> 1) & 7 so that the 16-byte
+//     fragment reads of the matrix instruction are free of conflicts on the 64 LDS banks, and
+//   * the w tile still packed, 256 rows x 8 BITS bytes: loading slot (row, half) owns the BITS dwords of its 32
+//     codes and brings them in one or two pieces (16, 12 or 4 bytes each), each piece of all slots forming one
+//     region of the stage (16 bytes per slot, 4 for single dwords).
+// Both arrive by direct global-to-LDS loads (no registers, no copy instructions) whose addresses are a scalar
+// base per step plus a constant per-lane offset; the loads of step s+2 are issued during step s, and there is one
+// barrier per step.  Scales and biases of four groups at a time (two of 128) travel the same way, one 16-bit
+// element per lane and load, into a double-buffered table.
+// The K loop is a written software pipeline.  A wavefront issues little more than one instruction per five cycles,
+// so whatever is not a matrix instruction has to fit under one: after each of a substep's sixteen matrix
+// instructions comes one item of side work for the next substep (the read of one x fragment, or two codes ->
+// float -> fma(code, scale, bias) -> packed element type; MXFP4: scaled FP4 conversions), kept in that order with
+// scheduling barriers.  The step's last substep first waits for the next stage (and everyone's), then prepares
+// the next step's first operands under its own matrix instructions.
 // The K order inside a step is permuted (fragment kk of lane half h is packed word 4 h + kk) so that
 // a lane's four weight words are one contiguous 16 bytes; x fragments follow the same order.
 #pragma once
@@ -171,7 +175,7 @@ qmm_kernel(const ProductArgs a) {
 
     // Direct-to-LDS assignment.  x: instruction i of wavefront v fills the 64 consecutive 16-byte
     // slots starting at slot i*kThreads + v*64; slot S is row S/8, position S%8, and holds chunk
-    // position ^ (row & 7) of that row.  w: loading slot S is half S%2 of row S/2 and owns the BITS dwords of that
+    // position ^ swizzle(row) of that row.  w: loading slot S is half S%2 of row S/2 and owns the BITS dwords of that
     // half's 32 codes.  Addresses are a block-uniform base (advanced per step with scalar arithmetic) plus a
     // per-lane byte offset that never changes.
     constexpr int XP = TL::kXParts, WS = TL::kWSlots;
@@ -393,14 +397,14 @@ qmm_kernel(const ProductArgs a) {
 }
 
 // Estimated microseconds of the tiled kernel with tile TL on `cus` compute units, from its measured behaviour:
-// about 1.7 us (big tile, one block per compute unit) or 1.0 us (small tile, two blocks) per step of 64 values
+// about 1.7 us (big tile, one block per compute unit) or 1.2 us (small tile, two blocks) per step of 64 values
 // and round of tiles.
 template <class TL>
 inline double estimate_us(const ProductArgs &a, int cus) {
     const double tiles = (double)((a.m + TL::BM - 1) / TL::BM) * (double)((a.n + TL::BN - 1) / TL::BN) * (double)a.batch;
     const bool big = TL::BM == 256;
     const double rounds = ceil(tiles / ((double)cus * (big ? 1.0 : 2.0)));
-    return rounds * (double)(a.k / BK) * (big ? 1.7 : 1.0);
+    return rounds * (double)(a.k / BK) * (big ? 1.7 : 1.2);
 }
 inline bool small_tile_is_faster(const ProductArgs &a, int cus) { return estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus); }
 
