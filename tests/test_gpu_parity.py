@@ -504,3 +504,29 @@ def test_layers_mirror_the_reference_callers():
     tied = to_host(emb.as_linear(to_dev(x)))
     want = ref.quantized_matmul(x, fp_packed, fp_scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16)
     assert_rows_close(tied, want, ref.BF16, "tied embedding")
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,k,n", [(64, 2048, 100), (128, 4096, 96), (64, 6144, 33), (128, 10240, 64)])
+def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
+    """Four rows of x at 4 bits, K a multiple of 2048 (the matrix-core decode kernel): N not a multiple of its 32
+    weight rows, K beyond one staging round, both group sizes it takes, and a batch of products."""
+    rng = np.random.default_rng(2400 + group + k + n + dtype)
+    w, x = make_w(rng, n, k, dtype), make_x(rng, 4, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, 4))
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=4, dtype=dtype)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, dtype, f"four rows g{group} K={k} N={n}")
+    assert_device_arithmetic(got, x, packed, scales, biases, group, 4, dtype, f"four rows g{group} K={k} N={n}")
+    if k == 2048:  # x [3, 4, K] against one weight matrix and against a matrix per item
+        xb = make_x(rng, 12, k, dtype).reshape(3, 4, k)
+        want = ref.quantized_matmul(xb, packed, scales, biases, group=group, bits=4, dtype=dtype)
+        got = to_host(nv.quantized_matmul(to_dev(xb), q))
+        assert_rows_close(got.reshape(12, n), want.reshape(12, n), dtype, "four rows, shared weights")
+        wb = make_w(rng, 3 * n, k, dtype).reshape(3, n, k)
+        pb, sb, bb = ref.affine_quantize(wb, dtype, group, 4)
+        qb = nv.Quantized(to_dev(pb), to_dev(sb), to_dev(bb), nv.Quant.affine(group, 4))
+        want = ref.quantized_matmul(xb, pb, sb, bb, group=group, bits=4, dtype=dtype)
+        got = to_host(nv.quantized_matmul(to_dev(xb), qb))
+        assert_rows_close(got.reshape(12, n), want.reshape(12, n), dtype, "four rows, a matrix per item")
