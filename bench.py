@@ -225,14 +225,14 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the M=2048 leg")
     ap.add_argument("--all-configs", action="store_true",
-                    help="also time every BASELINE configuration (C1..C5) and report them under \"configs\"")
+                    help="also time every configuration of the reference's benchmark list (C1..C5) and report them under \"configs\"")
     ap.add_argument("--only", choices=["qmv", "qmm", "copy"], default=None,
                     help="profiling aid: run just the rotating decode leg, just the prefill leg, or a plain 1 GiB "
                          "device copy (the known-size kernel the HBM counters are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N without exchange, "
-                 "see DESIGN.md)")
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N without exchange: "
+                 "each GPU would run the same kernels on its rows of the weight)")
 
     import torch
 

@@ -189,6 +189,15 @@ NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, co
 NVQ_API int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
                            int32_t *offsets, void *stream);
 
+/* The pairs of a mixture-of-experts layer ordered by expert: what SwitchGlu::forward computes with `argsort`
+ * of the flattened expert ids, `argsort` of that (the inverse) and `sorted_offsets`
+ * (crates/nuvec-lm/src/model.rs:2193-2210), as one stable counting sort.
+ *   ids u32[pairs] (an id beyond `experts` is the caller's error and is clamped);
+ *   order u32[pairs]: the pair at each sorted position, ties in pair order;  restore u32[pairs]: its inverse;
+ *   sorted_ids u32[pairs] = ids[order];  offsets i32[experts]: where each expert's pairs start. */
+NVQ_API int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
+                      uint32_t *sorted_ids, int32_t *offsets, void *stream);
+
 NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);
 
 /* GpuEval::gather_qmm / fp_gather_qmm (gpu.rs:7174-7294, 6758-6876); values of the gathered

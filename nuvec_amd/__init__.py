@@ -5,4 +5,4 @@ public `quantize`, `dequantize`, `quantized_matmul` and `gather_qmm`, and the ro
 nuvec-nn's `QuantizedEmbedding` as `embedding`.
 """
 from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, embedding,  # noqa: F401
-                  gather_qmm, quantize, quantized_matmul, sorted_offsets)
+                  gather_qmm, gather_qmm_grouped, moe_order, quantize, quantized_matmul, sorted_offsets)

@@ -23,6 +23,83 @@ __global__ void sorted_offsets_kernel(const uint32_t *__restrict__ indices, int6
     offsets[t] = (int32_t)lo;
 }
 
+// The pairs (token, choice) of a mixture-of-experts layer ordered by expert, stably: what SwitchGlu::forward gets
+// from `argsort` of the flattened expert ids, its inverse, and `sorted_offsets` of the sorted ids
+// (crates/nuvec-lm/src/model.rs:2193-2210), in one block.  A counting sort: a histogram of the ids in LDS, an
+// exclusive scan over the experts (the offsets), then the pairs placed chunk by chunk in pair order; inside a
+// chunk a pair's rank among the equal ids before it comes from wavefront ballots (lanes before it in its own
+// wavefront) plus the counts of the wavefronts before its own.
+constexpr int kOrderThreads = 1024, kOrderWaves = kOrderThreads / 64;
+
+__global__ void __launch_bounds__(kOrderThreads)
+moe_order_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t experts, uint32_t *__restrict__ order,
+                 uint32_t *__restrict__ restore, uint32_t *__restrict__ sorted_ids, int32_t *__restrict__ offsets) {
+    extern __shared__ int32_t lds_i[];
+    int32_t *next = lds_i;                       // [experts]: histogram, then where each expert's next pair goes
+    int32_t *wave_count = lds_i + experts;       // [waves][experts]: this chunk's pairs per wavefront and expert
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < experts; e += kOrderThreads) next[e] = 0;
+    __syncthreads();
+    for (int64_t p = tid; p < pairs; p += kOrderThreads) atomicAdd(&next[min(ids[p], (uint32_t)(experts - 1))], 1);
+    __syncthreads();
+    // Exclusive scan by one wavefront, 64 experts at a time.
+    if (wave == 0) {
+        int32_t carry = 0;
+        for (int base = 0; base < experts; base += 64) {
+            const int e = base + lane;
+            const int32_t count = e < experts ? next[e] : 0;
+            int32_t incl = count;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int32_t up = __shfl_up(incl, d);
+                if (lane >= d) incl += up;
+            }
+            if (e < experts) {
+                next[e] = carry + incl - count;
+                offsets[e] = carry + incl - count;
+            }
+            carry += __shfl(incl, 63);
+        }
+    }
+    __syncthreads();
+    for (int64_t chunk = 0; chunk < pairs; chunk += kOrderThreads) {
+        for (int i = tid; i < kOrderWaves * experts; i += kOrderThreads) wave_count[i] = 0;
+        __syncthreads();
+        const int64_t p = chunk + tid;
+        const bool live = p < pairs;
+        const uint32_t e = live ? min(ids[p], (uint32_t)(experts - 1)) : 0u;  // an id beyond the experts is clamped
+        // Rank among the lanes of this wavefront with the same id: one ballot per distinct id.
+        int rank = 0;
+        uint64_t todo = __ballot(live);
+        while (todo != 0) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const uint32_t e0 = __shfl(e, leader);
+            const uint64_t same = __ballot(live && e == e0);
+            if (live && e == e0) {
+                rank = __popcll(same & ((1ull << lane) - 1ull));
+                if (lane == leader) wave_count[wave * experts + e0] = __popcll(same);
+            }
+            todo &= ~same;
+        }
+        __syncthreads();
+        if (live) {
+            int before = 0;
+            for (int w = 0; w < wave; w++) before += wave_count[w * experts + e];
+            const uint32_t at = (uint32_t)(next[e] + before + rank);
+            order[at] = (uint32_t)p;
+            restore[p] = at;
+            sorted_ids[at] = e;
+        }
+        __syncthreads();
+        for (int ee = tid; ee < experts; ee += kOrderThreads) {
+            int total = 0;
+            for (int w = 0; w < kOrderWaves; w++) total += wave_count[w * experts + ee];
+            next[ee] += total;
+        }
+        __syncthreads();
+    }
+}
+
 __global__ void fill_zero_kernel(uint16_t *p, int64_t halves) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t < halves) p[t] = 0;
@@ -35,6 +112,16 @@ int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, 
     const int64_t n = rows * groups;
     hipLaunchKernelGGL(sorted_offsets_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, indices, rows, m, groups, offsets);
     NVQ_LAUNCH_CHECK("sorted_offsets");
+    return NVQ_OK;
+}
+
+size_t moe_order_lds_bytes(int32_t experts) { return (size_t)(1 + kOrderWaves) * experts * sizeof(int32_t); }
+
+int32_t launch_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
+                         uint32_t *sorted_ids, int32_t *offsets, hipStream_t s) {
+    hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(kOrderThreads), moe_order_lds_bytes(experts), s, ids, pairs, experts, order,
+                       restore, sorted_ids, offsets);
+    NVQ_LAUNCH_CHECK("moe_order");
     return NVQ_OK;
 }
 

@@ -343,6 +343,18 @@ int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int
 
 size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *) { return 0; }
 
+int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
+                      uint32_t *sorted_ids, int32_t *offsets, void *stream) {
+    if (pairs < 0 || experts <= 0) return fail(NVQ_INVALID_ARGUMENT, "moe_order: %lld pairs, %d experts", (long long)pairs, experts);
+    if (pairs > INT32_MAX) return fail(NVQ_INVALID_ARGUMENT, "moe_order: %lld pairs exceed 32-bit positions", (long long)pairs);
+    if (moe_order_lds_bytes(experts) > 64 * 1024)
+        return fail(NVQ_UNSUPPORTED, "moe_order: %d experts exceed the block's counters", experts);
+    if (offsets == nullptr || (pairs > 0 && (ids == nullptr || order == nullptr || restore == nullptr || sorted_ids == nullptr)))
+        return fail(NVQ_INVALID_ARGUMENT, "moe_order: null operand");
+    NVQ_TRY(require_device());
+    return launch_moe_order(ids, pairs, experts, order, restore, sorted_ids, offsets, (hipStream_t)stream);
+}
+
 int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                        const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
     (void)workspace;

@@ -160,7 +160,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
         for (int i = 0; i < 4; i++) {
             const int r = (tid >> 4) + 16 * i;
             int64_t g = pass + (r < rows ? r : 0);
-            g = a.lhs != nullptr ? (int64_t)a.lhs[g] : g;
+            if (a.lhs != nullptr) g = min((int64_t)a.lhs[g], a.x_batches - 1);  // an index beyond x is the caller's error: clamped
             xsrc[i] = x + (r < rows ? g * K : 0) + 8 * xc;
         }
         auto load_x = [&](int win, u32x4_t (&xq)[4]) {

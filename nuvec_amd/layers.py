@@ -1,6 +1,7 @@
-"""The two callers of the quantized path in nuvec-nn (crates/nuvec-nn/src/layers.rs:89-162 and
-207-262): a linear layer and an embedding whose weights are stored packed.  Thin host glue over
-`ops`; every product, lookup and quantization runs in the HIP library.
+"""The callers of the quantized path: nuvec-nn's linear layer and embedding with packed weights
+(crates/nuvec-nn/src/layers.rs:89-162 and 207-262) and nuvec-lm's expert projections of a mixture-of-experts
+block (crates/nuvec-lm/src/model.rs:2103-2211).  Thin host glue over `ops`; every product, lookup, ordering
+and quantization runs in the HIP library.
 """
 from __future__ import annotations
 
@@ -73,5 +74,66 @@ class QuantizedEmbedding:
     def as_linear(self, x: torch.Tensor) -> torch.Tensor:
         """layers.rs:258-261: `x W^T` with the quantized table (tied embeddings)."""
         return ops.quantized_matmul(x, self.quantized(), transpose=True)
+
+    __call__ = forward
+
+
+@dataclass
+class SwitchProjection:
+    """model.rs:2103-2146 (`SwitchProjection::Quantized`, mlx-lm's `SwitchLinear`): one packed weight
+    `[experts, output_dims, input_dims * bits / 32]` per expert, an optional bias `[experts, output_dims]`."""
+    weight: torch.Tensor
+    scales: torch.Tensor
+    biases: Optional[torch.Tensor]
+    bias: Optional[torch.Tensor] = None
+    quant: Quant = Quant()
+
+    def quantized(self) -> Quantized:
+        return Quantized(self.weight, self.scales, self.biases, self.quant)
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False) -> torch.Tensor:
+        """model.rs:2113-2146: `x` (`[..., 1, input_dims]` batches) through the experts `indices`."""
+        y = ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices))
+        return y if self.bias is None else y + self.bias[indices.long()].unsqueeze(-2)
+
+    def forward_sorted_rows(self, x: torch.Tensor, rows, sorted_ids: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+        """Rows `rows` of `x` (`[T, input_dims]`; None: its rows in order) through experts sorted by id."""
+        if rows is None:
+            rows = torch.arange(x.shape[0], dtype=torch.int32, device=x.device)
+        y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets)
+        return y if self.bias is None else y + self.bias[sorted_ids.long()]
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up in the activations' type (elementwise; not part of the quantized path)."""
+    return torch.nn.functional.silu(gate) * up
+
+
+@dataclass
+class SwitchGlu:
+    """model.rs:2149-2211 (mlx-lm's `SwitchGLU`): the experts' gated MLPs."""
+    gate_proj: SwitchProjection
+    up_proj: SwitchProjection
+    down_proj: SwitchProjection
+
+    def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+        """`x` `[B, L, D]` through each token's experts `indices` `[B, L, k]`: `[B, L, k, D]`.  With 64 pairs or
+        more they are ordered by expert (model.rs:2193-2210) so that each expert's weights are read once; here one
+        kernel orders the pairs, the products take the token rows of `x` themselves, and only the result is
+        put back in pair order."""
+        b, l, d = x.shape
+        k = indices.shape[2]
+        if indices.numel() < 64:  # model.rs:2189-2192
+            xe = x.reshape(b, l, 1, 1, d)
+            up, gate = self.up_proj.forward(xe, indices), self.gate_proj.forward(xe, indices)
+            return self.down_proj.forward(swiglu(gate, up), indices).squeeze(-2)
+        experts = self.up_proj.weight.shape[0]
+        order, restore, sorted_ids, offsets = ops.moe_order(indices, experts)
+        tokens = torch.div(order, k, rounding_mode="floor").to(torch.int32)  # pair t*k + j belongs to token t
+        xt = x.reshape(b * l, d)
+        up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+        gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+        out = self.down_proj.forward_sorted_rows(swiglu(gate, up), None, sorted_ids, offsets)
+        return out[restore.long()].reshape(b, l, k, -1)
 
     __call__ = forward

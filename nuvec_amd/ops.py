@@ -325,6 +325,56 @@ def sorted_offsets(rhs: torch.Tensor, groups: int) -> torch.Tensor:
     return out
 
 
+def moe_order(expert_ids: torch.Tensor, experts: int):
+    """nuvec-lm model.rs:2193-2210 (`SwitchGlu::forward`): the flattened pairs (token, choice) ordered by expert.
+    Returns `(order, restore, sorted_ids, offsets)`: `order = argsort(ids)` (stable), `restore = argsort(order)`,
+    `sorted_ids = ids[order]` and `offsets = sorted_offsets(sorted_ids, experts)`, from one kernel."""
+    if expert_ids.dtype.is_floating_point or expert_ids.dtype == torch.bool:
+        raise InvalidArgument("moe_order: expert ids must be integers")
+    _init(expert_ids)
+    ids = expert_ids.reshape(-1)
+    ids = (ids if ids.dtype == torch.uint32 else ids.to(torch.int32)).contiguous()
+    pairs = ids.numel()
+    order = torch.empty(pairs, dtype=torch.int32, device=ids.device)
+    restore, sorted_ids = torch.empty_like(order), torch.empty_like(order)
+    offsets = torch.empty(experts, dtype=torch.int32, device=ids.device)
+    _lib.check(_lib.load().nvq_moe_order(_ptr(ids), pairs, experts, _ptr(order), _ptr(restore), _ptr(sorted_ids), _ptr(offsets),
+                                         _stream()))
+    return order, restore, sorted_ids, offsets
+
+
+def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor,
+                       offsets: torch.Tensor) -> torch.Tensor:
+    """The grouped route of `gather_qmm` (quantized.rs:646-651, 772-782) with the rows of x taken inside the kernel:
+    output row i = x[rows[i]] . dequantize(w)[sorted_ids[i]]^T for ids sorted by expert (`offsets` from `moe_order`
+    or `sorted_offsets`).  Equal to `gather_qmm(x[rows], q, None, sorted_ids, sorted)`; the gathered copy of x is
+    never written.  x is `[T, K]`, the result `[len(rows), N]`."""
+    op = "gather_qmm"
+    quant = q.quant
+    quant.checked(op)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    affine = quant.mode == QuantMode.AFFINE
+    dtype = _promoted(op, x, q.scales, q.biases)
+    w = _u32(q.weight).contiguous()
+    if x.ndim != 2 or w.ndim != 3:
+        raise InvalidArgument(f"{op}: x must be [T, K] and w [E, N, K'], got {list(x.shape)} and {list(w.shape)}")
+    x = x.to(dtype).contiguous()
+    scales = (q.scales.to(dtype) if affine else q.scales).contiguous()
+    biases = q.biases.to(dtype).contiguous() if affine else None
+    columns = _quantized_columns(op, w, scales, biases, quant)
+    if x.shape[-1] != columns:
+        raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not match")
+    _init(x)
+    lhs, rhs = _indices(op, x, rows.reshape(-1)).contiguous(), _indices(op, w, sorted_ids.reshape(-1)).contiguous()
+    if lhs.numel() != rhs.numel() or offsets.numel() != w.shape[0] or offsets.dtype != torch.int32:
+        raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
+    out = torch.empty((rhs.numel(), w.shape[-2]), dtype=dtype, device=x.device)
+    d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 1, w.shape[-2], columns, rhs.numel(), x.shape[0], w.shape[0])
+    _lib.check(_lib.load().nvq_gather_qmm(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs),
+                                          _ptr(offsets.contiguous()), _ptr(out), _ptr(None), _stream()))
+    return out
+
+
 def _indices(op: str, a: torch.Tensor, given: Optional[torch.Tensor]) -> torch.Tensor:
     """quantized.rs:739-767: integer indices as uint32 (carried as int32 bit patterns)."""
     batch = a.shape[:-2]

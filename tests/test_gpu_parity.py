@@ -530,3 +530,55 @@ def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
         want = ref.quantized_matmul(xb, pb, sb, bb, group=group, bits=4, dtype=dtype)
         got = to_host(nv.quantized_matmul(to_dev(xb), qb))
         assert_rows_close(got.reshape(12, n), want.reshape(12, n), dtype, "four rows, a matrix per item")
+
+
+@pytest.mark.parametrize("pairs,experts", [(0, 4), (5, 3), (1024, 32), (3000, 7), (5000, 130)])
+def test_moe_order_is_the_stable_argsort(pairs, experts):
+    """The ordering of a mixture-of-experts layer's pairs (nuvec-lm model.rs:2193-2210): argsort of the expert
+    ids with ties in pair order, its inverse, the sorted ids and where each expert starts: integers, exact."""
+    rng = np.random.default_rng(2500 + pairs + experts)
+    ids = rng.integers(0, experts, size=pairs).astype(np.int32)
+    if pairs > 100:
+        ids[ids == 1] = 0  # an expert without pairs
+    order, restore, sorted_ids, offsets = nv.moe_order(torch.from_numpy(ids).cuda(), experts)
+    want = np.argsort(ids, kind="stable")
+    assert np.array_equal(order.cpu().numpy(), want)
+    assert np.array_equal(sorted_ids.cpu().numpy(), ids[want])
+    inverse = np.empty(pairs, dtype=np.int64)
+    inverse[want] = np.arange(pairs)
+    assert np.array_equal(restore.cpu().numpy(), inverse)
+    assert np.array_equal(offsets.cpu().numpy(), np.searchsorted(ids[want], np.arange(experts), side="left"))
+    if pairs:
+        assert np.array_equal(offsets.cpu().numpy(), nv.sorted_offsets(sorted_ids, experts).cpu().numpy())
+
+
+def test_switch_glu_sorts_gathers_and_restores():
+    """SwitchGlu::forward (nuvec-lm model.rs:2177-2211) over the library: pairs ordered by expert, token rows taken
+    inside the grouped products, results put back in pair order.  Each projection against the oracle's per-pair
+    product; the few-pairs route (no sorting) against the same."""
+    from nuvec_amd.layers import SwitchGlu, SwitchProjection
+    rng = np.random.default_rng(2600)
+    experts, d, inner, b, l, k = 6, 256, 320, 2, 24, 2
+    def projection(n, kk):
+        w = make_w(rng, experts * n, kk, ref.BF16).reshape(experts, n, kk)
+        packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+        return (packed, scales), SwitchProjection(to_dev(packed), to_dev(scales), None, None, nv.Quant.new(nv.QuantMode.MXFP4))
+    (gp, gate), (up_, up), (dp, down) = projection(inner, d), projection(inner, d), projection(d, inner)
+    glu = SwitchGlu(gate, up, down)
+    x = make_x(rng, b * l, d, ref.BF16).reshape(b, l, d)
+    idx = np.stack([rng.permutation(experts)[:k] for _ in range(b * l)]).reshape(b, l, k).astype(np.int32)
+    # the ordered products, one projection at a time, against the oracle on the pairs in their own order
+    order, restore, sorted_ids, offsets = nv.moe_order(torch.from_numpy(idx).cuda(), experts)
+    tokens = torch.div(order, k, rounding_mode="floor").to(torch.int32)
+    got_up = to_host(up.forward_sorted_rows(to_dev(x).reshape(b * l, d), tokens, sorted_ids, offsets)[restore.long()])
+    flat = idx.reshape(-1)
+    xrows = np.repeat(x.reshape(b * l, d), k, axis=0)
+    want_up = np.stack([ref.quantized_matmul(xrows[p:p + 1], up_[0][flat[p]], up_[1][flat[p]], None, mode=ref.MXFP4, group=32, bits=4,
+                                             dtype=ref.BF16)[0] for p in range(flat.size)])
+    assert_rows_close(got_up, want_up, ref.BF16, "up projection, ordered")
+    # the whole block both ways: ordered (96 pairs) and pair by pair (the same pairs, a few at a time)
+    whole = glu(to_dev(x), torch.from_numpy(idx).cuda())
+    assert tuple(whole.shape) == (b, l, k, d)
+    few = torch.cat([glu(to_dev(x)[:, t:t + 8], torch.from_numpy(idx).cuda()[:, t:t + 8]) for t in range(0, l, 8)], dim=1)
+    scale = float(few.float().abs().max())
+    assert float((whole.float() - few.float()).abs().max()) <= 2e-2 * scale
