@@ -189,6 +189,21 @@ NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, co
 NVQ_API int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
                            int32_t *offsets, void *stream);
 
+/* One layer of a Hugging Face AWQ / GPTQ checkpoint as nuvec's affine layout, as the loader converts it
+ * (crates/nuvec-lm/src/quant.rs:35-196, crates/nuvec-lm/src/config.rs:30-48).
+ *   qweight i32/u32 [rows, cols]: AWQ [in, out / 8] (4 bits, AWQ's nibble order), GPTQ [in * bits / 32, out];
+ *   qzeros likewise along the outputs, [groups, ceil(out * bits / 32)], or NULL (zero = 2^(bits - 1));
+ *   scales dtype [groups, out].
+ * Outputs: weight u32 [out, in * bits / 32]; scales_out, biases_out dtype [out, groups] with
+ * bias = -(zero) * scale (GPTQ v1 stores each zero minus one).  A `g_idx` must be the identity grouping: the
+ * caller checks it, as the reference does (quant.rs:104-118). */
+#define NVQ_PACKED_AWQ 0
+#define NVQ_PACKED_GPTQ_V1 1
+#define NVQ_PACKED_GPTQ_V2 2
+NVQ_API int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32_t dtype, const uint32_t *qweight,
+                           const uint32_t *qzeros, const void *scales, int64_t rows, int64_t cols, uint32_t *weight,
+                           void *scales_out, void *biases_out, void *stream);
+
 /* The pairs of a mixture-of-experts layer ordered by expert: what SwitchGlu::forward computes with `argsort`
  * of the flattened expert ids, `argsort` of that (the inverse) and `sorted_offsets`
  * (crates/nuvec-lm/src/model.rs:2193-2210), as one stable counting sort.

@@ -80,6 +80,8 @@ SIGNATURES = {
     "nvq_sorted_offsets": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
     "nvq_moe_order": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_void_p]),
+    "nvq_convert_packed": (C.c_int32, [C.c_int32, C.POINTER(QuantC), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                       C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_gather_qmm_workspace_bytes": (C.c_size_t, [C.POINTER(GatherDescC)]),
     "nvq_gather_qmm": (C.c_int32, [C.POINTER(GatherDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -343,6 +343,28 @@ int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int
 
 size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *) { return 0; }
 
+int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32_t dtype, const uint32_t *qweight, const uint32_t *qzeros,
+                           const void *scales, int64_t rows, int64_t cols, uint32_t *weight, void *scales_out, void *biases_out,
+                           void *stream) {
+    NVQ_TRY(check_quant(quant, "convert_packed"));
+    NVQ_TRY(check_float("convert_packed", dtype));
+    const int32_t bits = quant->bits;
+    if (quant->mode != NVQ_AFFINE || format < NVQ_PACKED_AWQ || format > NVQ_PACKED_GPTQ_V2 ||
+        (format == NVQ_PACKED_AWQ ? bits != 4 : (bits != 4 && bits != 8)))  // config.rs:1140-1168
+        return fail(NVQ_INVALID_ARGUMENT, "convert_packed: format %d with %d bits (AWQ loads 4 bits, GPTQ 4 and 8)", format, bits);
+    if (rows < 0 || cols < 0) return fail(NVQ_INVALID_ARGUMENT, "convert_packed: negative size");
+    const int64_t per_word = 32 / bits;
+    const int64_t inputs = format == NVQ_PACKED_AWQ ? rows : rows * per_word, outputs = format == NVQ_PACKED_AWQ ? cols * per_word : cols;
+    if (inputs % quant->group_size != 0)  // quant.rs:96-103
+        return fail(NVQ_INVALID_ARGUMENT, "convert_packed: %lld inputs do not match groups of %d", (long long)inputs, quant->group_size);
+    if (inputs == 0 || outputs == 0) return NVQ_OK;
+    if (qweight == nullptr || scales == nullptr || weight == nullptr || scales_out == nullptr || biases_out == nullptr)
+        return fail(NVQ_INVALID_ARGUMENT, "convert_packed: null operand");
+    NVQ_TRY(require_device());
+    return launch_convert_packed(format, bits, dtype, qweight, qzeros, scales, inputs, outputs, inputs / quant->group_size, weight,
+                                 scales_out, biases_out, (hipStream_t)stream);
+}
+
 int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
                       uint32_t *sorted_ids, int32_t *offsets, void *stream) {
     if (pairs < 0 || experts <= 0) return fail(NVQ_INVALID_ARGUMENT, "moe_order: %lld pairs, %d experts", (long long)pairs, experts);

@@ -50,6 +50,10 @@ int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed
                              hipStream_t s);
 int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
                               int32_t *offsets, hipStream_t s);
+// Hugging Face integer packings into the affine layout (repack.hip).  format 0: AWQ, 1: GPTQ v1, 2: GPTQ v2.
+int32_t launch_convert_packed(int32_t format, int32_t bits, int32_t dtype, const uint32_t *qweight, const uint32_t *qzeros,
+                              const void *scales, int64_t inputs, int64_t outputs, int64_t groups, uint32_t *packed,
+                              void *scales_out, void *biases_out, hipStream_t s);
 size_t moe_order_lds_bytes(int32_t experts);
 int32_t launch_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
                          uint32_t *sorted_ids, int32_t *offsets, hipStream_t s);
