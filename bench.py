@@ -65,10 +65,13 @@ class Product:
         d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = 1, m, n, k, m, 0
         self.d, self.fn = d, lib.nvq_quantized_matmul
         biases = q.biases.data_ptr() if q.biases is not None else None
+        import torch
+        need = lib.nvq_quantized_matmul_workspace_bytes(C.byref(d))  # the caller's scratch, as the boundary defines it
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
         self.args = (C.byref(d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),
                      C.c_void_p(q.scales.data_ptr()), C.c_void_p(biases), C.c_void_p(y.data_ptr()),
-                     C.c_void_p(None))
-        self.keep = (x, q, y)
+                     C.c_void_p(workspace.data_ptr() if need else None))
+        self.keep = (x, q, y, workspace)
 
     def __call__(self, stream):
         rc = self.fn(*self.args, stream)

@@ -174,13 +174,15 @@ NVQ_API int32_t nvq_dequantize_rows(const nvq_quant *quant, int32_t dtype, const
                             void *out, void *stream);
 
 /* Bytes of scratch nvq_quantized_matmul needs for `desc` (split-K partials; the reference
- * allocates them on its side of the boundary, gpu.rs:7562).  0 = none; nonzero only for
- * transpose = 0 products whose K is split over the grid (float32 partial sums). */
+ * allocates them on its side of the boundary, gpu.rs:7562).  0 = none; nonzero for products whose K is
+ * split over the grid (float32 partial sums): transpose = 0, and transpose = 1 products of many rows with few
+ * output tiles and a long K (the counterpart of the reference's qmm_t_splitk, gpu.rs:7507-7590).  A transposed
+ * product given no workspace runs unsplit. */
 NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
 
 /* GpuEval::quantized_matmul / fp_quantized_matmul (gpu.rs:6934-7168, 6336-6577); values of
  * kernels::quantized_matmul (kernels.rs:1091-1142) within the stated tolerance.
- * `workspace` may be NULL when nvq_quantized_matmul_workspace_bytes(desc) == 0. */
+ * `workspace` may be NULL when nvq_quantized_matmul_workspace_bytes(desc) == 0 (and for transposed products). */
 NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
                              const void *biases, void *y, void *workspace, void *stream);
 

@@ -141,13 +141,12 @@ int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose
 using namespace nvq;
 
 // Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row
-// kernel takes a pass per 32 rows, each bound by the expansion of every weight (0.29 us per million weights)
-// and never under 4 us.  The counterpart of the reference's device-specific `qmv_batch_limit`
+// kernel runs a block per pass of 32 rows and 64 weight rows, a round of blocks on the chip taking about 3.2 us
+// per 1024 values of K (never under 4 us).  The counterpart of the reference's device-specific `qmv_batch_limit`
 // (crates/nuvec-core/src/gpu.rs:1506-1538).
 static bool tiled_is_faster(const nvq::ProductArgs &a) {
-    const double pass_us = fmax(4.0, 0.29e-6 * (double)a.n * (double)a.k);
-    const double at_once = fmax(1.0, fmin((double)a.batch, 256.0 / fmax(1.0, (double)((a.n + 63) / 64))));  // batch items side by side
-    const double few_us = (double)((a.m + 31) / 32) * pass_us * (double)a.batch / at_once;
+    const double blocks = (double)((a.m + 31) / 32) * (double)((a.n + 63) / 64) * (double)a.batch;
+    const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * fmax(4.0, 3.2e-3 * (double)a.k);
     return nvq::qmm_estimate_us(a) < few_us;
 }
 
@@ -292,12 +291,22 @@ int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
     return 1;  // every mode and both orientations: the matrix-core kernels take affine and MXFP4 transposed, the general kernels the rest
 }
 
+// Whether a transposed product goes to the tiled kernel: routed by one item's rows, as the reference does
+// (gpu.rs:6975-6981), where its tiles cost less than the passes of the few-row kernel.
+static bool takes_tiled(const nvq_qmm_desc *d, const ProductArgs &a) {
+    const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
+    return item > 32 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a));
+}
+
 size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
-    if (check_qmm(d, "quantized_matmul") != NVQ_OK || d->transpose) return 0;
+    if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
     int64_t batch = 1;
     for (int i = 0; i < d->batch_ndim; i++) batch *= d->batch_shape[i];
     if (batch == 0 || d->m == 0 || d->n == 0 || d->k == 0 || require_device() != NVQ_OK) return 0;
-    return qvm_workspace_bytes(product_args(d, batch));  // float32 partial sums of the splits of K
+    const ProductArgs a = product_args(d, batch);
+    // float32 partial sums of the splits of K: weights stored [K, N], or few tiles of a long K
+    if (!d->transpose) return qvm_workspace_bytes(a);
+    return takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
 }
 
 int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
@@ -321,10 +330,7 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     ProductArgs a = product_args(d, batch);
     a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
-    // Routed by one item's rows, as the reference does (gpu.rs:6975-6981): the tiled kernel where its tiles
-    // cost less than the passes of the few-row kernel.
-    const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
-    if (item > 32 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a))) return launch_qmm(a, (hipStream_t)stream);
+    if (takes_tiled(d, a)) return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
     // Up to four rows of 4-bit affine weights: the decode kernel (per-row work on the vector units, which is
     // cheaper than the matrix-core kernel's full dequantization up to there).  Other few-row products share
     // one weight decode on the matrix cores where that kernel takes them.

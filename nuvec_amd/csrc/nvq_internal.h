@@ -71,11 +71,14 @@ struct ProductArgs {
     const uint32_t *lhs, *rhs;      // gather: batch z reads x batch lhs[z] and weight batch rhs[z]
     int64_t x_batches, experts;     // gather: index bounds (an index beyond them is clamped)
     const int32_t *offsets;         // grouped gather: rows of expert e are [offsets[e], offsets[e+1]) of `batch` rows
+    int32_t k_splits, k_split_steps;  // tiled kernel: K split over grid z (0 or 1: no split), steps of 64 values per split
+    float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
 bool qmm_supported(const ProductArgs &a);
-int32_t launch_qmm(const ProductArgs &a, hipStream_t s);
+size_t qmm_workspace_bytes(const ProductArgs &a);  // float32 partial sums when K is split over the grid, else 0
+int32_t launch_qmm(const ProductArgs &a, void *workspace, hipStream_t s);  // workspace NULL: no split
 double qmm_estimate_us(const ProductArgs &a);  // estimated duration of the tiled kernel with its better tile
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
 bool qmf_supported(const ProductArgs &a);

@@ -9,6 +9,6 @@ int32_t launch_qmf_b4(const ProductArgs &a, hipStream_t s) {
     return a.offsets != nullptr ? qmg::run_dtype<4, false>(a, s) : qmf::run_dtype<4, false>(a, s);
 }
 
-int32_t launch_qmm_b4(const ProductArgs &a, hipStream_t s) { return qmm::run_dtype<4, false>(a, s); }
+int32_t launch_qmm_b4(const ProductArgs &a, void *workspace, hipStream_t s) { return qmm::run_dtype<4, false>(a, workspace, s); }
 
 }  // namespace nvq

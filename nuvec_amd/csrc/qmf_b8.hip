@@ -9,6 +9,6 @@ int32_t launch_qmf_b8(const ProductArgs &a, hipStream_t s) {
     return a.offsets != nullptr ? qmg::run_dtype<8, false>(a, s) : qmf::run_dtype<8, false>(a, s);
 }
 
-int32_t launch_qmm_b8(const ProductArgs &a, hipStream_t s) { return qmm::run_dtype<8, false>(a, s); }
+int32_t launch_qmm_b8(const ProductArgs &a, void *workspace, hipStream_t s) { return qmm::run_dtype<8, false>(a, workspace, s); }
 
 }  // namespace nvq

@@ -8,6 +8,6 @@ int32_t launch_qmf_fp4(const ProductArgs &a, hipStream_t s) {
     return a.offsets != nullptr ? qmg::run_dtype<4, true>(a, s) : qmf::run_dtype<4, true>(a, s);
 }
 
-int32_t launch_qmm_fp4(const ProductArgs &a, hipStream_t s) { return qmm::run_dtype<4, true>(a, s); }
+int32_t launch_qmm_fp4(const ProductArgs &a, void *workspace, hipStream_t s) { return qmm::run_dtype<4, true>(a, workspace, s); }
 
 }  // namespace nvq

@@ -18,19 +18,27 @@ bool qmm_supported(const ProductArgs &a) {
     return a.batch <= 65535 && a.k >= qmm::BK && a.k % qmm::BK == 0;
 }
 
+// With its better tile and, for a single product, its better split of K (the caller is expected to bring the
+// workspace the size query names).
 double qmm_estimate_us(const ProductArgs &a) {
-    const int cus = compute_units();
-    return fmin(qmm::estimate_us<qmm::BigTile>(a, cus), qmm::estimate_us<qmm::SmallTile>(a, cus));
+    double us = 0.0;
+    qmm::k_splits(a, compute_units(), nullptr, &us);
+    return us;
 }
 
-int32_t launch_qmm(const ProductArgs &a, hipStream_t s) {
-    if (a.mode == NVQ_MXFP4) return launch_qmm_fp4(a, s);
+size_t qmm_workspace_bytes(const ProductArgs &a) {
+    const int splits = qmm::k_splits(a, compute_units());
+    return splits > 1 ? (size_t)splits * (size_t)a.m * (size_t)a.n * sizeof(float) : 0;
+}
+
+int32_t launch_qmm(const ProductArgs &a, void *workspace, hipStream_t s) {
+    if (a.mode == NVQ_MXFP4) return launch_qmm_fp4(a, workspace, s);
     switch (a.bits) {
-    case 2: return launch_qmm_b2(a, s);
-    case 3: return launch_qmm_b3(a, s);
-    case 4: return launch_qmm_b4(a, s);
-    case 6: return launch_qmm_b6(a, s);
-    default: return launch_qmm_b8(a, s);
+    case 2: return launch_qmm_b2(a, workspace, s);
+    case 3: return launch_qmm_b3(a, workspace, s);
+    case 4: return launch_qmm_b4(a, workspace, s);
+    case 6: return launch_qmm_b6(a, workspace, s);
+    default: return launch_qmm_b8(a, workspace, s);
     }
 }
 

@@ -161,6 +161,16 @@ qmm_kernel(const ProductArgs a) {
     const int pshift = gshift == 5 ? 1 : 2, psteps = 1 << pshift;
     const int gper = (psteps * BK) >> gshift;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // A single product may split K over grid z (few tiles, long K): this block takes the steps
+    // [step0, step0 + steps) and leaves float32 partial sums for a second kernel.
+    int step0 = 0, steps = K / BK;  // K is a multiple of 64 (checked on the host)
+    if constexpr (!BATCHED) {
+        if (a.k_splits > 1) {
+            step0 = blockIdx.z * a.k_split_steps;  // whole table periods
+            steps = steps - step0 < a.k_split_steps ? steps - step0 : a.k_split_steps;
+            if (steps <= 0) return;  // (the host sizes the grid so that every split has a step)
+        }
+    }
     int64_t bx = 0, bw = 0, bs = 0, by = 0;
     if constexpr (BATCHED) {  // a batch with one stride per operand
         bx = (int64_t)blockIdx.z * a.x_strides[0];
@@ -179,8 +189,8 @@ qmm_kernel(const ProductArgs a) {
     // half's 32 codes.  Addresses are a block-uniform base (advanced per step with scalar arithmetic) plus a
     // per-lane byte offset that never changes.
     constexpr int XP = TL::kXParts, WS = TL::kWSlots;
-    const char *xbase = reinterpret_cast<const char *>(x + (int64_t)m0 * K);
-    const char *wbase = reinterpret_cast<const char *>(w + (int64_t)n0 * row_dwords);
+    const char *xbase = reinterpret_cast<const char *>(x + (int64_t)m0 * K + (int64_t)step0 * BK);
+    const char *wbase = reinterpret_cast<const char *>(w + (int64_t)n0 * row_dwords + (int64_t)step0 * 2 * BITS);
     uint32_t xoff[XP], woff[WS];
 #pragma unroll
     for (int i = 0; i < XP; i++) {
@@ -194,7 +204,6 @@ qmm_kernel(const ProductArgs a) {
         const int r = n0 + (slot >> 1) < N ? (slot >> 1) : N - 1 - n0;
         woff[j] = ((uint32_t)r * (uint32_t)row_dwords + (slot & 1) * BITS) * 4;
     }
-    const int steps = K / BK;  // K is a multiple of 64 (checked on the host)
     // The loads of one step: its global bases (a step past the end reloads the last one, harmlessly, which keeps
     // the wait counts uniform) and the LDS address of this wavefront's lane 0 in the step's stage.
     struct Loads {
@@ -235,15 +244,16 @@ qmm_kernel(const ProductArgs a) {
     constexpr int kKinds = FP4 ? 1 : 2, kTableLoads = kKinds * 4 * BN / kThreads;
     const int trow = n0 + tid % BN < N ? tid % BN : N - 1 - n0;
     const uint32_t toff = (uint32_t)trow * (uint32_t)kgroups * (uint32_t)sizeof(S);
-    const char *sbase = reinterpret_cast<const char *>(scales + (int64_t)n0 * kgroups);
-    const char *bbase = reinterpret_cast<const char *>(biases + (int64_t)n0 * kgroups);
+    const int g0 = (step0 * BK) >> gshift, groups_left = kgroups - g0;  // this block's first group
+    const char *sbase = reinterpret_cast<const char *>(scales + (int64_t)n0 * kgroups + g0);
+    const char *bbase = reinterpret_cast<const char *>(biases + (int64_t)n0 * kgroups + g0);
     auto issue_table = [&](int period) {
         const uint32_t tbase = lds0 + kStages * G::kStageBytes + (period & 1) * kSbBytes;
 #pragma unroll
         for (int i = 0; i < kTableLoads; i++) {
             const int entry = i * kThreads + wave * 64;  // of this wavefront's first lane: [kind][group][row]
             const int kind = entry / (4 * BN), g = (entry / BN) % 4;
-            const int gi = period * gper + g < kgroups ? period * gper + g : kgroups - 1;
+            const int gi = period * gper + g < groups_left ? period * gper + g : groups_left - 1;
             dma_element<sizeof(S)>((kind ? bbase : sbase) + gi * (int)sizeof(S), toff, tbase + entry * 4);
         }
     };
@@ -392,24 +402,96 @@ qmm_kernel(const ProductArgs a) {
                 }
             }
     };
+    if constexpr (!BATCHED) {
+        if (a.k_splits > 1) {  // float32 partial sums [split][M][N]
+            float *out0 = a.partials + ((int64_t)blockIdx.z * M + m0 + wm * (32 * TI) + 4 * h) * N + n0 + wn * (32 * TJ) + l32;
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    const int col = n0 + wn * (32 * TJ) + j * 32 + l32;
+                    const int row0 = m0 + wm * (32 * TI) + i * 32 + 4 * h;
+#pragma unroll
+                    for (int e = 0; e < 16; e++) {
+                        const int r = 8 * (e >> 2) + (e & 3);
+                        if (row0 + r < M && col < N) out0[(int64_t)(i * 32 + r) * N + j * 32] = acc[i][j][e];
+                    }
+                }
+            return;
+        }
+    }
     if (m0 + BM <= M && n0 + BN <= N) store_tile(std::true_type{});
     else store_tile(std::false_type{});
 }
 
-// Estimated microseconds of the tiled kernel with tile TL on `cus` compute units, from its measured behaviour:
-// about 1.7 us (big tile, one block per compute unit) or 1.2 us (small tile, two blocks) per step of 64 values
-// and round of tiles.
+// y = the splits' partial sums added in split order, rounded once.
+template <typename T>
+__global__ void __launch_bounds__(256) qmm_reduce_kernel(const float *__restrict__ partials, T *__restrict__ y, int splits, int64_t total) {
+    const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (idx >= total) return;
+    if (idx + 4 <= total) {
+        float4 sum = *reinterpret_cast<const float4 *>(partials + idx);
+        for (int s = 1; s < splits; s++) {
+            const float4 v = *reinterpret_cast<const float4 *>(partials + s * total + idx);
+            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+        }
+        Elem<T>::store(y, idx, sum.x), Elem<T>::store(y, idx + 1, sum.y), Elem<T>::store(y, idx + 2, sum.z), Elem<T>::store(y, idx + 3, sum.w);
+    } else {
+        for (int64_t i = idx; i < total; i++) {
+            float sum = 0.0f;
+            for (int s = 0; s < splits; s++) sum += partials[s * total + i];
+            Elem<T>::store(y, i, sum);
+        }
+    }
+}
+
+// Estimated microseconds of `tiles` tiles of TL walking `steps` steps of 64 values on `cus` compute units, from
+// the kernel's measured behaviour: about 1.7 us per step for the big tile (one block per compute unit); the small
+// tile takes 0.8 us per step alone on a compute unit and 1.2 us when two share it.
+template <class TL>
+inline double tiles_us(double tiles, double steps, int cus) {
+    if (TL::BM == 256) return ceil(tiles / cus) * steps * 1.7;
+    if (tiles <= cus) return steps * 0.8;
+    return ceil(tiles / (2.0 * cus)) * steps * 1.2;
+}
 template <class TL>
 inline double estimate_us(const ProductArgs &a, int cus) {
     const double tiles = (double)((a.m + TL::BM - 1) / TL::BM) * (double)((a.n + TL::BN - 1) / TL::BN) * (double)a.batch;
-    const bool big = TL::BM == 256;
-    const double rounds = ceil(tiles / ((double)cus * (big ? 1.0 : 2.0)));
-    return rounds * (double)(a.k / BK) * (big ? 1.7 : 1.2);
+    return tiles_us<TL>(tiles, (double)(a.k / BK), cus);
 }
 inline bool small_tile_is_faster(const ProductArgs &a, int cus) { return estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus); }
 
+// How many ways a single product splits K over the grid, by estimate: the splits fill the chip's block slots
+// with its (few) tiles, and cost a second kernel that reads their float32 partial sums (about 3 us to launch and
+// 4 bytes per microsecond and compute unit... in all: 4 TB/s).  Each split has at least eight steps, in whole table
+// periods; at most eight splits.  1: no split.
+inline int k_splits(const ProductArgs &a, int cus, int *steps_per_split = nullptr, double *estimate = nullptr) {
+    const int64_t steps = a.k / BK;
+    if (steps_per_split != nullptr) *steps_per_split = (int)steps;
+    const bool small = small_tile_is_faster(a, cus);
+    if (estimate != nullptr) *estimate = small ? estimate_us<SmallTile>(a, cus) : estimate_us<BigTile>(a, cus);
+    if (a.batch != 1) return 1;
+    const int64_t bm = small ? SmallTile::BM : BigTile::BM, bn = small ? SmallTile::BN : BigTile::BN;
+    const double tiles = (double)(((a.m + bm - 1) / bm) * ((a.n + bn - 1) / bn));
+    auto walk_us = [&](double t, double st) { return small ? tiles_us<SmallTile>(t, st, cus) : tiles_us<BigTile>(t, st, cus); };
+    double best_us = walk_us(tiles, (double)steps);
+    int best = 1;
+    int64_t best_per = steps;
+    for (int want = 2; want <= 8 && want <= steps / 8; want++) {
+        const int64_t per = (((steps + want - 1) / want) + 3) & ~(int64_t)3;  // whole table periods
+        const int splits = (int)((steps + per - 1) / per);                    // every split has a step
+        if (splits < 2) continue;
+        const double reduce_us = 3.0 + ((double)splits * 4.0 + 2.0) * (double)a.m * (double)a.n * 2.0 / 4.0e6;  // written, then read
+        const double us = walk_us(tiles * splits, (double)per) + reduce_us;
+        if (us < 0.9 * best_us) best_us = us, best = splits, best_per = per;
+    }
+    if (steps_per_split != nullptr) *steps_per_split = (int)best_per;
+    if (estimate != nullptr) *estimate = best_us;
+    return best;
+}
+
 template <typename T, int BITS, bool FP4, class TL>
-int32_t run_tile(const ProductArgs &a, hipStream_t s) {
+int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     using G = Geometry<BITS, TL>;
     static bool configured[2] = {false, false};
     const bool batched = a.batch > 1;
@@ -418,30 +500,41 @@ int32_t run_tile(const ProductArgs &a, hipStream_t s) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes));
         configured[batched] = true;
     }
-    dim3 grid((unsigned)((a.n + TL::BN - 1) / TL::BN), (unsigned)((a.m + TL::BM - 1) / TL::BM), (unsigned)a.batch);
+    int per = 0;
+    const int splits = workspace != nullptr ? k_splits(a, compute_units(), &per) : 1;
+    a.k_splits = splits;
+    a.k_split_steps = per;
+    a.partials = splits > 1 ? static_cast<float *>(workspace) : nullptr;
+    dim3 grid((unsigned)((a.n + TL::BN - 1) / TL::BN), (unsigned)((a.m + TL::BM - 1) / TL::BM), (unsigned)(batched ? a.batch : splits));
     hipLaunchKernelGGL(kernel, grid, dim3(TL::kThreads), G::kLdsBytes, s, a);
     NVQ_LAUNCH_CHECK("qmm");
+    if (splits > 1) {
+        const int64_t total = a.m * a.n;
+        hipLaunchKernelGGL((qmm_reduce_kernel<T>), dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s, a.partials, (T *)a.y, splits, total);
+        NVQ_LAUNCH_CHECK("qmm_reduce");
+    }
     return NVQ_OK;
 }
 
 template <typename T, int BITS, bool FP4>
-int32_t run(const ProductArgs &a, hipStream_t s) {
-    return small_tile_is_faster(a, compute_units()) ? run_tile<T, BITS, FP4, SmallTile>(a, s) : run_tile<T, BITS, FP4, BigTile>(a, s);
+int32_t run(const ProductArgs &a, void *workspace, hipStream_t s) {
+    return small_tile_is_faster(a, compute_units()) ? run_tile<T, BITS, FP4, SmallTile>(a, workspace, s)
+                                                    : run_tile<T, BITS, FP4, BigTile>(a, workspace, s);
 }
 
 template <int BITS, bool FP4>
-int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
-    return a.dtype == NVQ_BF16 ? run<bf16_t, BITS, FP4>(a, s) : run<f16_t, BITS, FP4>(a, s);
+int32_t run_dtype(const ProductArgs &a, void *workspace, hipStream_t s) {
+    return a.dtype == NVQ_BF16 ? run<bf16_t, BITS, FP4>(a, workspace, s) : run<f16_t, BITS, FP4>(a, workspace, s);
 }
 
 }  // namespace qmm
 
 // One per code width, each in its own translation unit.
-int32_t launch_qmm_b2(const ProductArgs &a, hipStream_t s);
-int32_t launch_qmm_b3(const ProductArgs &a, hipStream_t s);
-int32_t launch_qmm_b4(const ProductArgs &a, hipStream_t s);
-int32_t launch_qmm_b6(const ProductArgs &a, hipStream_t s);
-int32_t launch_qmm_b8(const ProductArgs &a, hipStream_t s);
-int32_t launch_qmm_fp4(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmm_b2(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b3(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b4(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b6(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b8(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_fp4(const ProductArgs &a, void *workspace, hipStream_t s);
 
 }  // namespace nvq
