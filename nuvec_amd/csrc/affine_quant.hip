@@ -60,7 +60,7 @@ __device__ __forceinline__ void store8<bf16_t>(bf16_t *out, int64_t base, const 
     uint32_t r[4];
 #pragma unroll
     for (int i = 0; i < 4; i++)
-        r[i] = (uint32_t)f32_to_bf16_bits(v[2 * i]) | ((uint32_t)f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        r[i] = f32_to_bf16_pair(v[2 * i], v[2 * i + 1]);
     *reinterpret_cast<uint4 *>(out + base) = make_uint4(r[0], r[1], r[2], r[3]);
 }
 template <>
@@ -114,40 +114,135 @@ __device__ __forceinline__ uint64_t load_codes(const uint8_t *bytes, int64_t chu
     }
 }
 
-// kernels.rs:774-831.  `chunks` = n_values / 8; `lanes` = group / 8 (4, 8 or 16).
-template <typename T, int BITS>
-__global__ void __launch_bounds__(kBlock)
-affine_quantize_kernel(const T *__restrict__ w, int64_t chunks, int lanes, uint8_t *__restrict__ packed,
-                       T *__restrict__ scales, T *__restrict__ biases) {
-    const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    // chunks is a multiple of `lanes` and the block size is a multiple of 16: a group's lanes
-    // are all in range or all out of range, so the shuffles below never mix the two.
-    const bool active = chunk < chunks;
-    float v[8];
-    if (active) {
-        load8<T>(w, chunk * 8, v);
+// ---- quantize ----
+//
+// A lane owns 32 consecutive values (a whole group of 32, half a group of 64, a quarter of a group of 128), so
+// the group's extremes need at most two lane exchanges and the scale arithmetic (four divisions) is done once per
+// 32 values.  A wavefront fetches its 64 x 32 values with coalesced 16-byte loads and turns them through a private
+// LDS stage into one row per lane; the swizzle keeps both the 16-byte writes and the 16-byte reads free of bank
+// conflicts on the 64 banks (a row is 4 or 8 pieces; 16 consecutive lanes must touch 16 different piece slots).
+template <int P> __device__ __forceinline__ int stage_slot(int row, int piece) {
+    if constexpr (P == 4) return row * 4 + (piece ^ ((row >> 2) & 3));
+    else return row * 8 + (piece ^ ((row >> 1) & 7));
+}
+
+// The lane's 32 values as float32.  A signalling NaN is quieted (hardware min/max would return it, a quiet one
+// they skip, as the reference's f32::min/max skip every NaN).
+template <typename T> __device__ __forceinline__ void widen(const uint4 *in, float (&v)[32]);
+template <> __device__ __forceinline__ void widen<float>(const uint4 *in, float (&v)[32]) {
+#pragma unroll
+    for (int p = 0; p < 8; p++) {
+        v[4 * p] = u2f(in[p].x); v[4 * p + 1] = u2f(in[p].y); v[4 * p + 2] = u2f(in[p].z); v[4 * p + 3] = u2f(in[p].w);
+    }
+}
+template <> __device__ __forceinline__ void widen<bf16_t>(const uint4 *in, float (&v)[32]) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const uint32_t r[4] = {in[p].x, in[p].y, in[p].z, in[p].w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            v[8 * p + 2 * i] = u2f(r[i] << 16);
+            v[8 * p + 2 * i + 1] = u2f(r[i] & 0xFFFF0000u);
+        }
+    }
+}
+template <> __device__ __forceinline__ void widen<f16_t>(const uint4 *in, float (&v)[32]) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        f16_t h[8];
+        __builtin_memcpy(h, &in[p], 16);
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[8 * p + i] = (float)h[i];
+    }
+}
+
+// The value of the lane `lane ^ 1` (kSwap1) or `lane ^ 2` (kSwap2): a move inside the quad, no LDS.
+constexpr int kSwap1 = 0xB1, kSwap2 = 0x4E;
+template <int CTRL> __device__ __forceinline__ float quad_swap(float x) {
+    return u2f((uint32_t)__builtin_amdgcn_mov_dpp((int)f2u(x), CTRL, 0xF, 0xF, true));
+}
+
+// Packs 32 codes into BITS words of the little-endian bit stream.  `raw[i]` is the code plus JUNK (the bits of
+// the float 1.5 * 2^23 when the code sits in a float's low mantissa bits); where a word holds whole codes the junk
+// is summed along and taken off once per word, so a code costs one shift-and-add.
+template <int BITS, uint32_t JUNK>
+__device__ __forceinline__ void pack_words(const uint32_t (&raw)[32], uint32_t (&words)[BITS]) {
+    if constexpr (32 % BITS == 0) {
+        constexpr int kPer = 32 / BITS;
+        uint64_t ones = 0;
+        for (int i = 0; i < kPer; i++) ones += (uint64_t)1 << (BITS * i);
+        const uint32_t junk = (uint32_t)((uint64_t)JUNK * ones);
+#pragma unroll
+        for (int k = 0; k < BITS; k++) {
+            uint32_t acc = raw[k * kPer + kPer - 1];
+#pragma unroll
+            for (int i = kPer - 2; i >= 0; i--) acc = (acc << BITS) + raw[k * kPer + i];
+            words[k] = acc - junk;
+        }
     } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.0f;
+        for (int k = 0; k < BITS; k++) words[k] = 0u;
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            const uint32_t code = raw[i] - JUNK;
+            const int k = (i * BITS) / 32, shift = (i * BITS) % 32;
+            words[k] |= code << shift;
+            if (shift + BITS > 32) words[k + 1] |= code >> (32 - shift);
+        }
     }
-    // f32 extremes of the group: min/max ignore NaN and order -0 below +0, so the fold's
-    // order does not matter (the reference folds from +Inf / -Inf in index order).
+}
+
+// kernels.rs:774-831.  `rows` = n_values / 32; a group is `1 << lanes_log2` adjacent lanes (1, 2 or 4).
+template <typename T, int BITS>
+__global__ void __launch_bounds__(kBlock)
+affine_quantize_kernel(const T *__restrict__ w, int64_t rows, int lanes_log2, uint32_t *__restrict__ packed,
+                       T *__restrict__ scales, T *__restrict__ biases) {
+    constexpr int P = 32 * (int)sizeof(T) / 16;  // 16-byte pieces of a lane's row
+    __shared__ uint4 stages[kBlock / 64][64 * P];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row0 = ((int64_t)blockIdx.x * (kBlock / 64) + wave) * 64;
+    if (row0 >= rows) return;  // the whole wavefront; nothing below synchronizes across wavefronts
+    uint4 *stage = stages[wave];
+    const uint4 *src = reinterpret_cast<const uint4 *>(w) + row0 * P;
+    const int64_t last = (rows - row0) * P - 1;  // beyond the end the last piece is read again and never used
+    uint4 in[P];
+#pragma unroll
+    for (int j = 0; j < P; j++) in[j] = src[min((int64_t)(j * 64 + lane), last)];
+#pragma unroll
+    for (int j = 0; j < P; j++) {
+        const int c = j * 64 + lane;
+        stage[stage_slot<P>(c / P, c % P)] = in[j];
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int p = 0; p < P; p++) in[p] = stage[stage_slot<P>(lane, p)];
+    float v[32];
+    widen<T>(in, v);
+#pragma unroll
+    for (int i = 0; i < 32; i++) v[i] = __builtin_canonicalizef(v[i]);
+
+    // f32 extremes of the group: the hardware's min/max skip NaN and order -0 below +0, as the reference's fold
+    // from +Inf / -Inf does on its hosts, so the order of the fold does not matter.
     float lo = INFINITY, hi = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 8; i++) { lo = rs_min(lo, v[i]); hi = rs_max(hi, v[i]); }
-    for (int d = 1; d < lanes; d <<= 1) {
-        lo = rs_min(lo, __shfl_xor(lo, d));
-        hi = rs_max(hi, __shfl_xor(hi, d));
+    for (int i = 0; i < 32; i++) { lo = __builtin_fminf(lo, v[i]); hi = __builtin_fmaxf(hi, v[i]); }
+    if (lanes_log2 >= 1) {
+        lo = __builtin_fminf(lo, quad_swap<kSwap1>(lo));
+        hi = __builtin_fmaxf(hi, quad_swap<kSwap1>(hi));
     }
-    const float n_bins = (float)((1u << BITS) - 1u);
+    if (lanes_log2 >= 2) {
+        lo = __builtin_fminf(lo, quad_swap<kSwap2>(lo));
+        hi = __builtin_fmaxf(hi, quad_swap<kSwap2>(hi));
+    }
+    constexpr float n_bins = (float)((1u << BITS) - 1u);
     const float eps = 1e-7f;
     float scale, bias;
     if constexpr (BITS == 1) {
-        scale = rs_max(hi - lo, eps);
+        scale = __builtin_fmaxf(hi - lo, eps);
         bias = lo;
     } else {
         const bool wide = fabsf(lo) > fabsf(hi);
-        scale = rs_max((hi - lo) / n_bins, eps);
+        scale = __builtin_fmaxf((hi - lo) / n_bins, eps);
         scale = wide ? scale : -scale;
         const float edge = wide ? lo : hi;
         const float q0 = rintf(edge / scale);
@@ -158,29 +253,44 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t chunks, int lanes, uint8
             bias = edge;
         }
     }
-    if (!active) return;
-    // code = rint((v - bias) / scale) with the correctly rounded quotient.  Eight divisions per lane are the
-    // bulk of this kernel's arithmetic, and only the rounded integer is needed: (v - bias) * (1 / scale) is
-    // within 2^-23 relative of the quotient, so both round to the same integer unless they lie that close to
-    // a half; those few values (and odd scales) take the division.
-    const float inv = 1.0f / scale;
+    // code = clamp(rint((v - bias) / scale)) with the correctly rounded quotient.  Thirty-two divisions would be the
+    // bulk of the kernel; with y = 1 / scale (correctly rounded, once per lane) the quotient of d by scale is
+    // t0 = d * y, then twice t <- fma(fma(-scale, t, d), y, t): the first step leaves t within a rounding of the
+    // quotient and the second is then the correctly rounded quotient itself (Markstein's theorem, the same
+    // scheme the compiler's own division expands to, with a better reciprocal).  It needs scale, y and the
+    // remainders in the normal range: other groups (tiny or huge scales, infinite values) take the divisions.
+    // Adding 1.5 * 2^23 rounds to the nearest integer, ties to even, and leaves it in the low mantissa bits.
+    constexpr float kMagic = 12582912.0f;
+    const float y = 1.0f / scale;
     const float mag = fabsf(scale);
-    const bool plain = mag > 1e-30f && mag < 1e30f;  // finite, normal, with a finite normal reciprocal
-    uint64_t stream = 0;
+    const bool plain = mag > 1e-20f && mag < 1e20f && (hi - lo) * fabsf(y) < 1024.0f;
+    uint32_t raw[32], words[BITS];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < 32; i++) {
         const float d = v[i] - bias;
-        float t = d * inv;
-        const float u = fabsf(t);
-        const float frac = u - floorf(u);
-        if (!plain || !(fabsf(frac - 0.5f) > 4e-7f * u)) t = d / scale;  // also NaN and infinities
-        float q = rintf(t);
-        q = fminf(fmaxf(q, 0.0f), n_bins);  // NaN -> 0, as Rust's clamp followed by `as u32`
-        stream |= (uint64_t)(uint32_t)q << (i * BITS);
+        float t = d * y;
+        t = __builtin_fmaf(__builtin_fmaf(-scale, t, d), y, t);
+        t = __builtin_fmaf(__builtin_fmaf(-scale, t, d), y, t);
+        raw[i] = f2u(__builtin_amdgcn_fmed3f(t + kMagic, kMagic, kMagic + n_bins));  // NaN -> the smallest: code 0
     }
-    store_codes<BITS>(packed, chunk, stream);
-    if (chunk % lanes == 0) {
-        const int64_t g = chunk / lanes;
+    pack_words<BITS, 0x4B400000u>(raw, words);
+    if (!plain) {
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            float q = rintf((v[i] - bias) / scale);
+            q = fminf(fmaxf(q, 0.0f), n_bins);  // NaN -> 0, as Rust's clamp followed by `as u32`
+            raw[i] = (uint32_t)q;
+        }
+        pack_words<BITS, 0u>(raw, words);
+    }
+    const int64_t row = row0 + lane;
+    if (row >= rows) return;
+    struct Words { uint32_t w[BITS]; } out;
+#pragma unroll
+    for (int k = 0; k < BITS; k++) out.w[k] = words[k];
+    *reinterpret_cast<Words *>(packed + row * BITS) = out;
+    if ((lane & ((1 << lanes_log2) - 1)) == 0) {
+        const int64_t g = row >> lanes_log2;
         Elem<T>::store(scales, g, scale);
         Elem<T>::store(biases, g, bias);
     }
@@ -192,35 +302,46 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t chunks, int lanes, uint8
 template <typename T, int BITS>
 __global__ void __launch_bounds__(kBlock)
 affine_dequantize_kernel(const uint8_t *__restrict__ packed, const T *__restrict__ scales,
-                         const T *__restrict__ biases, int64_t chunks, int lanes, T *__restrict__ out,
-                         const uint32_t *__restrict__ ids, int64_t row_chunks, int64_t table_rows) {
-    const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+                         const T *__restrict__ biases, uint32_t chunks, int lanes_log2, T *__restrict__ out,
+                         const uint32_t *__restrict__ ids, uint32_t row_chunks, int64_t table_rows) {
+    const uint32_t chunk = blockIdx.x * kBlock + threadIdx.x;  // fewer than 2^29: an operand has fewer than 2^32 elements
     if (chunk >= chunks) return;
     int64_t src = chunk;
     if (ids != nullptr) {
-        const int64_t r = chunk / row_chunks;
+        const uint32_t r = chunk / row_chunks;
         const int64_t row = min((int64_t)ids[r], table_rows - 1);
         src = row * row_chunks + (chunk - r * row_chunks);
     }
     const uint64_t stream = load_codes<BITS>(packed, src);
-    const int64_t g = src / lanes;
+    const int64_t g = src >> lanes_log2;
     const float s = Elem<T>::load(scales, g), b = Elem<T>::load(biases, g);
     constexpr uint32_t mask = (1u << BITS) - 1u;
-    float r[8];
+    float c[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const float c = (float)((uint32_t)(stream >> (i * BITS)) & mask);
-        r[i] = Elem<T>::add(Elem<T>::mul(c, s), b);
+    for (int i = 0; i < 8; i++) c[i] = (float)((uint32_t)(stream >> (i * BITS)) & mask);
+    if constexpr (sizeof(T) == 2 && Elem<T>::code == 10) {
+        // bfloat16: the two roundings of a pair of values are one conversion instruction each.
+        uint32_t r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t p = f32_to_bf16_pair(c[2 * i] * s, c[2 * i + 1] * s);
+            r[i] = f32_to_bf16_pair(u2f(p << 16) + b, u2f(p & 0xFFFF0000u) + b);
+        }
+        *reinterpret_cast<uint4 *>(out + (int64_t)chunk * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+    } else {
+        float r[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) r[i] = Elem<T>::add(Elem<T>::mul(c[i], s), b);
+        store8<T>(out, (int64_t)chunk * 8, r);
     }
-    store8<T>(out, chunk * 8, r);
 }
 
 template <typename T, int BITS>
 int32_t quantize_t(int group, const void *w, int64_t n, void *packed, void *scales, void *biases, hipStream_t s) {
-    const int64_t chunks = n / 8;
-    const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL((affine_quantize_kernel<T, BITS>), dim3(blocks), dim3(kBlock), 0, s, (const T *)w, chunks,
-                       group / 8, (uint8_t *)packed, (T *)scales, (T *)biases);
+    const int64_t rows = n / 32;  // a lane's 32 values; the group is 1, 2 or 4 of them
+    const unsigned blocks = (unsigned)((rows + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL((affine_quantize_kernel<T, BITS>), dim3(blocks), dim3(kBlock), 0, s, (const T *)w, rows,
+                       group == 32 ? 0 : group == 64 ? 1 : 2, (uint32_t *)packed, (T *)scales, (T *)biases);
     NVQ_LAUNCH_CHECK("affine_quantize");
     return NVQ_OK;
 }
@@ -230,8 +351,8 @@ int32_t dequantize_t(int group, const void *packed, const void *scales, const vo
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((affine_dequantize_kernel<T, BITS>), dim3(blocks), dim3(kBlock), 0, s,
-                       (const uint8_t *)packed, (const T *)scales, (const T *)biases, chunks, group / 8, (T *)out, ids, cols / 8,
-                       table_rows);
+                       (const uint8_t *)packed, (const T *)scales, (const T *)biases, (uint32_t)chunks,
+                       group == 32 ? 2 : group == 64 ? 3 : 4, (T *)out, ids, (uint32_t)(cols / 8), table_rows);
     NVQ_LAUNCH_CHECK("affine_dequantize");
     return NVQ_OK;
 }

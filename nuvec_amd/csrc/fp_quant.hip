@@ -5,8 +5,8 @@
 //   NVFP4: E2M1 values, groups of 16, E4M3 scales (the maximum over 6, rounded to nearest).
 //
 // A lane owns 8 consecutive values = one (4-bit) or two (8-bit) uint32 of packed codes, value i in bits
-// i*bits of the stream; a group is 4 (2 for NVFP4) adjacent lanes.  The reference flushes float32
-// subnormals explicitly at every step (it reproduces a device that flushes them); gfx950 keeps
+// i*bits of the stream; a group is 4 (2 for NVFP4) adjacent lanes, a quad or half a quad.  The reference flushes
+// float32 subnormals explicitly at every step (it reproduces a device that flushes them); gfx950 keeps
 // subnormals, so the same explicit flushes are applied here.
 #include "nvq_device.h"
 #include "nvq_internal.h"
@@ -21,23 +21,168 @@ template <> struct Format<NVQ_MXFP4> { static constexpr int lanes = 4, bits = 4;
 template <> struct Format<NVQ_MXFP8> { static constexpr int lanes = 4, bits = 8; static constexpr float max_element = 448.0f; static constexpr bool mx = true; };
 template <> struct Format<NVQ_NVFP4> { static constexpr int lanes = 2, bits = 4; static constexpr float max_element = 6.0f; static constexpr bool mx = false; };
 
+// ---- the formats' conversion instructions ----
+//
+// gfx950 converts pairs of float32 / bfloat16 / half values to E2M1 or E4M3 codes divided by a power-of-two scale
+// (v_cvt_scalef32_pk_fp4_*, v_cvt_scalef32_pk_fp8_*), and pairs of E2M1 codes back, in one instruction.  Compared
+// with the integer formulation of the reference's arithmetic (flush, multiply by the reciprocal, flush, encode)
+// on every float32, bfloat16 and half input, they give the same codes whenever
+//   - the value is not a NaN (the instruction keeps a NaN's sign, the reference encodes the canonical NaN),
+//   - the E8M0 scale code is in [4, 253] for E2M1 and [12, 253] for E4M3 (below, a subnormal input that the reference
+//     flushes still rounds to a nonzero code; 254 has a subnormal reciprocal, which the reference flushes),
+//   - the quotient does not exceed the format's largest value (E4M3 only: the instruction then gives the NaN code,
+//     the reference saturates), which a group's own scale guarantees;
+// and the decoding instructions give the reference's products for scale codes in [2, 254] (below, the reference
+// flushes subnormal products; 255 is an infinite scale).  Groups outside these conditions take the integer
+// formulation, so every input gives the reference's bits.
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kSwap1 = 0xB1, kSwap2 = 0x4E;  // quad permutations: the lane `lane ^ 1`, `lane ^ 2`
+template <int CTRL> __device__ __forceinline__ uint32_t quad_swap(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, CTRL, 0xF, 0xF, true);
+}
+
+// A lane's 8 values as loaded: 4 words of pairs (16-bit types) or 8 words (float32).
+template <typename T> struct Raw { uint32_t w[sizeof(T) * 2]; };
+
+template <typename T> __device__ __forceinline__ Raw<T> load_raw(const T *w, int64_t chunk) {
+    Raw<T> r;
+    const uint4 *p = reinterpret_cast<const uint4 *>(w + chunk * 8);
+    const uint4 a = p[0];
+    r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
+    if constexpr (sizeof(T) == 4) {
+        const uint4 b = p[1];
+        r.w[4] = b.x; r.w[5] = b.y; r.w[6] = b.z; r.w[7] = b.w;
+    }
+    return r;
+}
+template <typename T> __device__ __forceinline__ void widen_raw(const Raw<T> &r, float (&v)[8]) {
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = u2f(r.w[i]);
+    } else if constexpr (Elem<T>::code == 10) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) { v[2 * i] = u2f(r.w[i] << 16); v[2 * i + 1] = u2f(r.w[i] & 0xFFFF0000u); }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const f16x2_t h = __builtin_bit_cast(f16x2_t, r.w[i]);
+            v[2 * i] = (float)h.x; v[2 * i + 1] = (float)h.y;
+        }
+    }
+}
+// The float32 bits of the largest magnitude among the lane's values, by integer comparison of the magnitude bits:
+// a NaN compares above infinity, so the result says whether the lane holds one.
+template <typename T> __device__ __forceinline__ uint32_t magnitude_bits(const Raw<T> &r) {
+    if constexpr (sizeof(T) == 4) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) m = max(m, r.w[i] & 0x7FFFFFFFu);
+        return m;
+    } else {
+        u16x2_t m = {0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; i++) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2_t, r.w[i] & 0x7FFF7FFFu));
+        const uint32_t top = max((uint32_t)m.x, (uint32_t)m.y);
+        if constexpr (Elem<T>::code == 10) return top << 16;
+        else return f2u((float)__builtin_bit_cast(_Float16, (uint16_t)top));  // exact; a half NaN stays a NaN
+    }
+}
+// Codes of the pair `pair` of the lane's values, divided by the scale whose exponent field `scale` carries.
+template <typename T> __device__ __forceinline__ uint32_t fp4_pair(uint32_t word, const Raw<T> &r, int pair, float scale, int byte) {
+    // `byte` must be a constant in the callers' unrolled loops
+    if constexpr (sizeof(T) == 4) {
+        switch (byte) {
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, 3);
+        }
+    } else if constexpr (Elem<T>::code == 10) {
+        const bf16x2_t v = __builtin_bit_cast(bf16x2_t, r.w[pair]);
+        switch (byte) {
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(word, v, scale, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(word, v, scale, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(word, v, scale, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_bf16(word, v, scale, 3);
+        }
+    } else {
+        const f16x2_t v = __builtin_bit_cast(f16x2_t, r.w[pair]);
+        switch (byte) {
+        case 0: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(word, v, scale, 0);
+        case 1: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(word, v, scale, 1);
+        case 2: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(word, v, scale, 2);
+        default: return __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(word, v, scale, 3);
+        }
+    }
+}
+template <typename T> __device__ __forceinline__ s16x2_t fp8_pair(s16x2_t word, const Raw<T> &r, int pair, float scale, bool high) {
+    if constexpr (sizeof(T) == 4) {
+        return high ? __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, true)
+                    : __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(word, u2f(r.w[2 * pair]), u2f(r.w[2 * pair + 1]), scale, false);
+    } else if constexpr (Elem<T>::code == 10) {
+        const bf16x2_t v = __builtin_bit_cast(bf16x2_t, r.w[pair]);
+        return high ? __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(word, v, scale, true) : __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(word, v, scale, false);
+    } else {
+        const f16x2_t v = __builtin_bit_cast(f16x2_t, r.w[pair]);
+        return high ? __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(word, v, scale, true) : __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(word, v, scale, false);
+    }
+}
+
 // kernels.rs:914-971 without a global scale.
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
 fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict__ packed, uint8_t *__restrict__ scales) {
     using F = Format<MODE>;
     const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const bool active = chunk < chunks;  // chunks is a multiple of the lanes per group: a group is wholly in or out of range
+    // chunks is a multiple of the lanes per group and so is the block: a group is wholly in or out of range
+    if (chunk >= chunks) return;
+    const Raw<T> raw = load_raw<T>(w, chunk);
+    if constexpr (F::mx) {
+        // The group's scale code straight from the bits of its largest magnitude m * 2^e: the reference's
+        // round_up(ftz(amax / max_element)) has the exponent of the quotient plus one unless the quotient is a
+        // power of two, i.e. e - 2 + (m > 1.5) for 6 = 1.5 * 2^2 and e - 8 + (m > 1.75) for 448 = 1.75 * 2^8.
+        constexpr uint32_t kCarry = F::bits == 4 ? 0x3FFFFFu : 0x1FFFFFu, kShift = F::bits == 4 ? 2u : 8u;
+        constexpr uint32_t kLowest = F::bits == 4 ? 4u : 12u;
+        uint32_t top = magnitude_bits<T>(raw);
+        top = max(top, quad_swap<kSwap1>(top));
+        top = max(top, quad_swap<kSwap2>(top));
+        const uint32_t code = ((top + kCarry) >> 23) - kShift;
+        if (top < 0x7F800000u && code - kLowest <= 253u - kLowest) {
+            const float scale = u2f(code << 23);
+            if constexpr (F::bits == 4) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) word = fp4_pair<T>(word, raw, i, scale, i);
+                packed[chunk] = word;
+            } else {
+                s16x2_t lo = {0, 0}, hi = {0, 0};
+                lo = fp8_pair<T>(lo, raw, 0, scale, false); lo = fp8_pair<T>(lo, raw, 1, scale, true);
+                hi = fp8_pair<T>(hi, raw, 2, scale, false); hi = fp8_pair<T>(hi, raw, 3, scale, true);
+                reinterpret_cast<uint2 *>(packed)[chunk] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+            }
+            if ((chunk & 3) == 0) scales[chunk >> 2] = (uint8_t)code;
+            return;
+        }
+    }
+    // The reference's arithmetic step by step: every group of NVFP4 (its scale is no power of two), and the groups
+    // of the MX formats with a NaN, an infinity, or a scale at either end of the range.  The lanes of a group are
+    // all here or none is.
     float v[8];
+    widen_raw<T>(raw, v);
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        v[i] = active ? ftz(Elem<T>::load(w, chunk * 8 + i)) : 0.0f;
+        v[i] = ftz(v[i]);
         amax = fmaxf(amax, fabsf(v[i]));  // NaN is ignored, as Rust's f32::max
     }
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    if constexpr (F::lanes == 4) amax = fmaxf(amax, __shfl_xor(amax, 2));
-    if (!active) return;
+    amax = fmaxf(amax, u2f(quad_swap<kSwap1>(f2u(amax))));
+    if constexpr (F::lanes == 4) amax = fmaxf(amax, u2f(quad_swap<kSwap2>(f2u(amax))));
     const float scale = ftz(amax / F::max_element);
     uint32_t code;
     float decoded;
@@ -67,36 +212,83 @@ fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict
     if (chunk % F::lanes == 0) scales[chunk / F::lanes] = (uint8_t)code;
 }
 
+// Eight decoded values of a lane, stored with 16-byte stores.
+template <typename T> __device__ __forceinline__ void store_values(T *out, int64_t base, const float (&v)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        float4 *p = reinterpret_cast<float4 *>(out + base);
+        p[0] = make_float4(v[0], v[1], v[2], v[3]);
+        p[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint32_t r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if constexpr (Elem<T>::code == 10) {
+                r[i] = f32_to_bf16_pair(v[2 * i], v[2 * i + 1]);
+            } else {
+                const f16x2_t h = {(_Float16)v[2 * i], (_Float16)v[2 * i + 1]};
+                r[i] = __builtin_bit_cast(uint32_t, h);
+            }
+        }
+        *reinterpret_cast<uint4 *>(out + base) = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+}
+
 // kernels.rs:976-1009 without a global scale.  With `ids`, output row r is table row ids[r] (`row_chunks` chunks
 // per row, ids clamped to `table_rows`): the rows of a quantized embedding.
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
-fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, int64_t chunks, T *__restrict__ out,
-                     const uint32_t *__restrict__ ids, int64_t row_chunks, int64_t table_rows) {
+fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, uint32_t chunks, T *__restrict__ out,
+                     const uint32_t *__restrict__ ids, uint32_t row_chunks, int64_t table_rows) {
     using F = Format<MODE>;
-    const int64_t out_chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t out_chunk = blockIdx.x * kBlock + threadIdx.x;  // fewer than 2^29: an operand has fewer than 2^32 elements
     if (out_chunk >= chunks) return;
     int64_t chunk = out_chunk;
     if (ids != nullptr) {
-        const int64_t r = out_chunk / row_chunks;
+        const uint32_t r = out_chunk / row_chunks;
         const int64_t row = min((int64_t)ids[r], table_rows - 1);
         chunk = row * row_chunks + (out_chunk - r * row_chunks);
     }
     const uint32_t sc = scales[chunk / F::lanes];
+    const int64_t base = (int64_t)out_chunk * 8;
+    if constexpr (MODE == NVQ_MXFP4) {
+        const uint32_t word = packed[chunk];
+        if (sc - 2u <= 252u) {  // one instruction per pair of codes
+            const float scale = u2f(sc << 23);
+            if constexpr (sizeof(T) == 4) {
+                const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 1),
+                              c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 3);
+                float4 *p = reinterpret_cast<float4 *>(out + base);
+                p[0] = make_float4(a.x, a.y, b.x, b.y);
+                p[1] = make_float4(c.x, c.y, d.x, d.y);
+            } else if constexpr (Elem<T>::code == 10) {
+                const bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 1),
+                               c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3);
+                *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                    __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+            } else {
+                const f16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 1),
+                              c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 3);
+                *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                    __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+            }
+            return;
+        }
+    }
     const float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
+    float v[8];
     if constexpr (F::bits == 4) {
         const uint32_t word = packed[chunk];
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            Elem<T>::store(out, out_chunk * 8 + i, canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu))));
+        for (int i = 0; i < 8; i++) v[i] = canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu)));
     } else {
         const uint2 words = reinterpret_cast<const uint2 *>(packed)[chunk];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            Elem<T>::store(out, out_chunk * 8 + i, canonical(ftz(scale * e4m3_to_f32((words.x >> (8 * i)) & 0xFFu))));
-            Elem<T>::store(out, out_chunk * 8 + 4 + i, canonical(ftz(scale * e4m3_to_f32((words.y >> (8 * i)) & 0xFFu))));
+            v[i] = canonical(ftz(scale * e4m3_to_f32((words.x >> (8 * i)) & 0xFFu)));
+            v[4 + i] = canonical(ftz(scale * e4m3_to_f32((words.y >> (8 * i)) & 0xFFu)));
         }
     }
+    store_values<T>(out, base, v);
 }
 
 template <typename T, int MODE>
@@ -114,7 +306,7 @@ int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *ou
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((fp_dequantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const uint32_t *)packed,
-                       (const uint8_t *)scales, chunks, (T *)out, ids, cols / 8, table_rows);
+                       (const uint8_t *)scales, (uint32_t)chunks, (T *)out, ids, (uint32_t)(cols / 8), table_rows);
     NVQ_LAUNCH_CHECK("fp_dequantize");
     return NVQ_OK;
 }

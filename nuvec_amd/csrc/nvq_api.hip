@@ -231,6 +231,7 @@ int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64
     NVQ_TRY(check_aligned("quantize", "w", w));
     NVQ_TRY(check_aligned("quantize", "packed", packed));
     const int64_t n = rows * cols;
+    if (n >= (1LL << 32)) return fail(NVQ_INVALID_ARGUMENT, "quantize: %lld elements; an operand holds fewer than 2^32", (long long)n);
     if (quant->mode == NVQ_AFFINE)
         return launch_affine_quantize(dtype, quant->group_size, quant->bits, w, n, packed, scales, biases, (hipStream_t)stream);
     return launch_fp_quantize(quant->mode, dtype, w, n, packed, scales, (hipStream_t)stream);
@@ -256,6 +257,8 @@ static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dt
     NVQ_TRY(check_aligned(op, "packed", packed));
     NVQ_TRY(check_aligned(op, "out", out));
     const int64_t n = count * cols;
+    if (n >= (1LL << 32) || table_rows * cols >= (1LL << 32))  // gpu.rs:1582-1590
+        return fail(NVQ_INVALID_ARGUMENT, "%s: %lld elements; an operand holds fewer than 2^32", op, (long long)n);
     if (quant->mode == NVQ_AFFINE)
         return launch_affine_dequantize(dtype, quant->group_size, quant->bits, packed, scales, biases, n, out, ids, cols,
                                         table_rows, (hipStream_t)stream);

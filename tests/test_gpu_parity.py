@@ -88,6 +88,50 @@ def test_affine_quantize_dequantize_bit_exact(dtype, group, bits):
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
+@pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(32, 4), (64, 4), (128, 4), (64, 3), (32, 8), (64, 2), (128, 6), (32, 5), (64, 1)])
+def test_affine_quantize_ties_specials_and_tails(dtype, group, bits):
+    """Groups whose quotients are exact halves or one unit in the last place from a half (the rounding the kernel
+    must take from the true division), zeros of both signs, NaN (quiet and signalling), infinities, a constant
+    group and tiny ranges; a number of rows that fills neither a wavefront nor a group of lanes."""
+    rng = np.random.default_rng(31 * bits + group)
+    n_bins, groups = (1 << bits) - 1, 37
+    w = np.zeros((groups, group), np.float32)
+    for g in range(groups):
+        top = float(2.0 ** int(rng.integers(-3, 4))) * n_bins
+        codes = rng.integers(0, n_bins + 1, group).astype(np.float32)
+        half = rng.integers(0, 2, group).astype(np.float32) * 0.5
+        v = np.minimum(codes + half, n_bins) * (top / n_bins)
+        v[:2] = (0.0, top)
+        w[g] = v if g % 2 else -v
+    w = ref.to_f32(ref.from_f32(w, dtype), dtype)
+    near = w.view(np.uint32).copy()
+    if dtype == ref.F32:
+        near[5::3, 7::5] += 1  # one unit in the last place beside the ties
+        near[6::3, 9::5] -= 1
+    w = near.view(np.float32)
+    w[3, :] = 0.0
+    w[3, ::3] = -0.0
+    w[4, :] = -0.0
+    w[7, :] = 1.25
+    w[8, 3] = np.nan
+    w[9, 5] = np.inf
+    w[10, 6] = -np.inf
+    w[11, :] = np.float32(1.0) + np.arange(group, dtype=np.float32) * np.float32(2.0 ** -20 if dtype == ref.F32 else 2.0 ** -7)
+    bits_w = w.view(np.uint32)
+    bits_w[12, 4] = 0x7F810000  # a signalling NaN in every element type's range
+    bits_w[13, :] = 0x00010000 * (1 + np.arange(group, dtype=np.uint32) % 5)  # float32 subnormals
+    stored = ref.from_f32(w, dtype)
+    if dtype != ref.F32:  # the conversion above quiets the signalling NaN: put its bits back
+        raw = stored.view(np.uint16)
+        raw[12, 4] = 0x7F81 if dtype == ref.BF16 else 0x7D01
+    packed, scales, biases = ref.affine_quantize(stored, dtype, group, bits)
+    q = nv.quantize(to_dev(stored), nv.Quant.affine(group, bits))
+    assert np.array_equal(to_host(q.weight), packed)
+    assert np.array_equal(to_host(q.scales).view(np.uint8), scales.view(np.uint8))
+    assert np.array_equal(to_host(q.biases).view(np.uint8), biases.view(np.uint8))
+
+
 def test_config1_fp32_4bit_g64():
     """BASELINE config 1: W f32 [4096,4096] ~ N(0,0.02), x f32 [1,4096], 4-bit g64."""
     rng = np.random.default_rng(20260101)
