@@ -215,6 +215,23 @@ NVQ_API int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32
 NVQ_API int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
                       uint32_t *sorted_ids, int32_t *offsets, void *stream);
 
+/* fast::moe_route (crates/nuvec-core/src/fast.rs:740-746, fast/imp.rs:2652-2673; kernel
+ * crates/nuvec-kernels/src/metal/moe.metal:33-88): per row of `experts` router probabilities the k largest in the
+ * stable ascending order of the sort (NaN last for float32 and half), i.e. the last k of `argsort`, their values
+ * and, with `normalize`, those divided by their sum (summed in `dtype`, in order).
+ *   probs dtype[rows, experts] (contiguous);  indices u32[rows, k];  scores dtype[rows, k].
+ * Up to 1024 experts and, with `normalize`, k <= 64 (beyond, the reference composes argpartition / take / sum /
+ * divide itself: NVQ_UNSUPPORTED). */
+NVQ_API int32_t nvq_moe_route(int32_t dtype, const void *probs, int64_t rows, int32_t experts, int32_t k, int32_t normalize,
+                      uint32_t *indices, void *scores, void *stream);
+
+/* fast::weighted_sum (fast/imp.rs:2731-2747; kernel moe.metal:90-118): out[r, c] = sum_j x[r, j, c] * w[r, j], the
+ * experts' outputs weighted by the router's scores, every product and addition rounded to `dtype` in the kernel's
+ * order (min(k, 8) interleaved partial sums, added in order).
+ *   x dtype[rows, k, d];  w dtype[rows, k];  out dtype[rows, d];  1 <= k < 32 (beyond: NVQ_UNSUPPORTED). */
+NVQ_API int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out,
+                         void *stream);
+
 NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);
 
 /* GpuEval::gather_qmm / fp_gather_qmm (gpu.rs:7174-7294, 6758-6876); values of the gathered

@@ -100,6 +100,88 @@ moe_order_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t expert
     }
 }
 
+// round(a / b) in the element type.  The float32 quotient is correctly rounded and float32 carries more than twice
+// the element types' digits, so rounding it again gives the correctly rounded quotient of the element type.
+template <typename T> __device__ __forceinline__ float elem_div(float a, float b) {
+    if constexpr (sizeof(T) == 4) return a / b;
+    else if constexpr (Elem<T>::code == 10) return bf16_bits_to_f32(f32_to_bf16_bits(a / b));
+    else return (float)(f16_t)(a / b);
+}
+
+// The order of the reference's sort: NaN last for float32 and half; bfloat16 compares plainly, as its sort does
+// (crates/nuvec-kernels/src/metal/moe.metal:19-31).
+template <typename T> __device__ __forceinline__ bool route_less(float a, float b) {
+    if constexpr (Elem<T>::code != 10) {
+        const bool an = a != a, bn = b != b;
+        if (an | bn) return (!an) & bn;
+    }
+    return a < b;
+}
+
+// fast::moe_route (crates/nuvec-kernels/src/metal/moe.metal:33-88): per row of `n` probabilities the k largest in
+// the stable ascending order, their values and, with `normalize`, those divided by their sum (summed in the
+// element type, in order).  One block per row, one thread per expert: an expert's position in the sorted row is
+// the number of experts sorting before it.
+template <typename T>
+__global__ void __launch_bounds__(1024) moe_route_kernel(const T *__restrict__ probs, uint32_t *__restrict__ indices,
+                                                         T *__restrict__ scores, int n, int k, int normalize) {
+    __shared__ float p[1024], top[1024];
+    __shared__ float total;
+    const int e = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    probs += row * n;
+    indices += row * k;
+    scores += row * k;
+    if (e < n) p[e] = Elem<T>::load(probs, e);
+    __syncthreads();
+    if (e < n) {
+        const float v = p[e];
+        int rank = 0;
+        for (int j = 0; j < n; j++) {
+            const float u = p[j];
+            rank += (route_less<T>(u, v) || (!route_less<T>(v, u) && j < e)) ? 1 : 0;
+        }
+        const int slot = rank - (n - k);
+        if (slot >= 0) {
+            indices[slot] = (uint32_t)e;
+            top[slot] = v;
+        }
+    }
+    __syncthreads();
+    if (normalize) {
+        if (e == 0) {
+            float sum = 0.0f;
+            for (int j = 0; j < k; j++) sum = Elem<T>::add(top[j], sum);
+            total = sum;
+        }
+        __syncthreads();
+        if (e < k) Elem<T>::store(scores, e, elem_div<T>(top[e], total));
+    } else if (e < k) {
+        Elem<T>::store(scores, e, top[e]);
+    }
+}
+
+// fast::weighted_sum (moe.metal:90-118): out[r, c] = sum over j of x[r, j, c] * w[r, j], every product and every
+// addition rounded to the element type: min(k, 8) partial sums of every min(k, 8)-th product (one partial sum when
+// D = 1), added in order.  One thread per output element.
+template <typename T>
+__global__ void __launch_bounds__(256) weighted_sum_kernel(const T *__restrict__ x, const T *__restrict__ w, T *__restrict__ out,
+                                                           int64_t rows, int k, int64_t d) {
+    const int64_t at = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= rows * d) return;
+    const int64_t r = at / d, c = at - r * d;
+    x += r * k * d + c;
+    w += r * k;
+    const int lanes = d == 1 ? 1 : (k < 8 ? k : 8);
+    float sum = 0.0f;
+    for (int y = 0; y < lanes; y++) {
+        float t = 0.0f;
+        for (int j = y; j < k; j += lanes) t = Elem<T>::add(Elem<T>::mul(Elem<T>::load(x, (int64_t)j * d), Elem<T>::load(w, j)), t);
+        sum = y == 0 ? t : Elem<T>::add(t, sum);
+    }
+    Elem<T>::store(out, at, sum);
+}
+
 __global__ void fill_zero_kernel(uint16_t *p, int64_t halves) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t < halves) p[t] = 0;
@@ -122,6 +204,31 @@ int32_t launch_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, ui
     hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(kOrderThreads), moe_order_lds_bytes(experts), s, ids, pairs, experts, order,
                        restore, sorted_ids, offsets);
     NVQ_LAUNCH_CHECK("moe_order");
+    return NVQ_OK;
+}
+
+int32_t launch_moe_route(int32_t dtype, const void *probs, int64_t rows, int32_t experts, int32_t k, int32_t normalize,
+                         uint32_t *indices, void *scores, hipStream_t s) {
+    const dim3 grid((unsigned)rows), block((unsigned)((experts + 63) / 64 * 64));
+    if (dtype == NVQ_F32)
+        hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, 0, s, (const float *)probs, indices, (float *)scores, experts, k, normalize);
+    else if (dtype == NVQ_BF16)
+        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, 0, s, (const bf16_t *)probs, indices, (bf16_t *)scores, experts, k, normalize);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<f16_t>, grid, block, 0, s, (const f16_t *)probs, indices, (f16_t *)scores, experts, k, normalize);
+    NVQ_LAUNCH_CHECK("moe_route");
+    return NVQ_OK;
+}
+
+int32_t launch_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out, hipStream_t s) {
+    const dim3 grid((unsigned)((rows * d + 255) / 256)), block(256);
+    if (dtype == NVQ_F32)
+        hipLaunchKernelGGL(weighted_sum_kernel<float>, grid, block, 0, s, (const float *)x, (const float *)w, (float *)out, rows, k, d);
+    else if (dtype == NVQ_BF16)
+        hipLaunchKernelGGL(weighted_sum_kernel<bf16_t>, grid, block, 0, s, (const bf16_t *)x, (const bf16_t *)w, (bf16_t *)out, rows, k, d);
+    else
+        hipLaunchKernelGGL(weighted_sum_kernel<f16_t>, grid, block, 0, s, (const f16_t *)x, (const f16_t *)w, (f16_t *)out, rows, k, d);
+    NVQ_LAUNCH_CHECK("weighted_sum");
     return NVQ_OK;
 }
 

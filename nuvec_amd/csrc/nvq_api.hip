@@ -388,6 +388,33 @@ int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint3
     return launch_moe_order(ids, pairs, experts, order, restore, sorted_ids, offsets, (hipStream_t)stream);
 }
 
+int32_t nvq_moe_route(int32_t dtype, const void *probs, int64_t rows, int32_t experts, int32_t k, int32_t normalize,
+                      uint32_t *indices, void *scores, void *stream) {
+    // fast/imp.rs:2652-2673
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "moe_route: unsupported dtype %s", dtype_name(dtype));
+    if (rows < 0 || experts < 0 || k < 1 || k > experts)
+        return fail(NVQ_INVALID_ARGUMENT, "moe_route: k must be in 1..=%d for probabilities of shape [%lld, %d]", experts, (long long)rows, experts);
+    if (experts > 1024 || (normalize && k > 64))
+        return fail(NVQ_UNSUPPORTED, "moe_route: %d experts, k = %d: the kernel takes up to 1024 experts and sums up to 64 scores", experts, k);
+    if (rows == 0) return NVQ_OK;
+    if (rows > INT32_MAX) return fail(NVQ_INVALID_ARGUMENT, "moe_route: %lld rows", (long long)rows);
+    if (probs == nullptr || indices == nullptr || scores == nullptr) return fail(NVQ_INVALID_ARGUMENT, "moe_route: null operand");
+    NVQ_TRY(require_device());
+    return launch_moe_route(dtype, probs, rows, experts, k, normalize != 0, indices, scores, (hipStream_t)stream);
+}
+
+int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out, void *stream) {
+    // fast/imp.rs:2731-2747
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "weighted_sum: unsupported dtype %s", dtype_name(dtype));
+    if (rows < 0 || k < 0 || d < 0) return fail(NVQ_INVALID_ARGUMENT, "weighted_sum: x must be [..., k, D] and w [..., k]");
+    if (k < 1 || k >= 32) return fail(NVQ_UNSUPPORTED, "weighted_sum: k = %d: the kernel sums 1 to 31 weighted rows", k);
+    if (rows == 0 || d == 0) return NVQ_OK;
+    if (rows * d >= (1LL << 32) || rows * k * d >= (1LL << 32)) return fail(NVQ_INVALID_ARGUMENT, "weighted_sum: an operand holds fewer than 2^32 elements");
+    if (x == nullptr || w == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "weighted_sum: null operand");
+    NVQ_TRY(require_device());
+    return launch_weighted_sum(dtype, x, w, rows, k, d, out, (hipStream_t)stream);
+}
+
 int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                        const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
     (void)workspace;

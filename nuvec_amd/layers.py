@@ -137,3 +137,29 @@ class SwitchGlu:
         return out[restore.long()].reshape(b, l, k, -1)
 
     __call__ = forward
+
+
+@dataclass
+class MoeMlp:
+    """model.rs:2218-2272 (`MoeMlp`, mlx-lm's sparse MoE blocks): the router's probabilities (a softmax in the
+    activations' type), each token's best `k` experts (`moe_route`), the experts' gated MLPs (`SwitchGlu`) and their
+    outputs weighted by the (renormalised) scores and summed (`weighted_sum`).  `gate` is the router's dense weight
+    `[experts, D]`; the shared expert of some models is a dense MLP outside this path and is left to the caller."""
+    gate: torch.Tensor
+    switch_mlp: SwitchGlu
+    experts_per_token: int
+    norm_topk_prob: bool = True
+
+    def route(self, x: torch.Tensor):
+        """The router: `(top, scores)` of `moe_route` over `softmax(x gate^T)`."""
+        logits = torch.nn.functional.linear(x, self.gate.to(x.dtype))
+        probs = torch.softmax(logits.float(), dim=-1).to(x.dtype)  # softmax_precise: float32 inside, one rounding
+        return ops.moe_route(probs, self.experts_per_token, self.norm_topk_prob)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """`x` `[B, L, D]` -> `[B, L, D]`."""
+        top, scores = self.route(x)
+        experts = self.switch_mlp.forward(x, top)  # [B, L, k, D]
+        return ops.weighted_sum(experts, scores)
+
+    __call__ = forward

@@ -343,6 +343,40 @@ def moe_order(expert_ids: torch.Tensor, experts: int):
     return order, restore, sorted_ids, offsets
 
 
+def moe_route(probs: torch.Tensor, k: int, normalize: bool):
+    """fast.rs:740-746 (`fast::moe_route`): per row of router probabilities `[..., E]` the `k` largest in the stable
+    ascending order of the sort (the last `k` of `argsort`; NaN last for float32 and half), as int32 `[..., k]`, and
+    their values (divided by their sum in the probabilities' type, in order, with `normalize`) `[..., k]`."""
+    if probs.dtype not in _CODE:
+        raise InvalidArgument(f"moe_route: probabilities must be floating point, got {probs.dtype}")
+    e = probs.shape[-1] if probs.ndim else 0
+    if not isinstance(k, int) or not 1 <= k <= e:
+        raise InvalidArgument(f"moe_route: k must be in 1..={e} for probabilities of shape {list(probs.shape)}")
+    _init(probs)
+    p = probs.contiguous()
+    rows = p.numel() // e
+    top = torch.empty(p.shape[:-1] + (k,), dtype=torch.int32, device=p.device)
+    scores = torch.empty(p.shape[:-1] + (k,), dtype=p.dtype, device=p.device)
+    _lib.check(_lib.load().nvq_moe_route(_CODE[p.dtype], _ptr(p), rows, e, k, int(bool(normalize)), _ptr(top), _ptr(scores), _stream()))
+    return top, scores
+
+
+def weighted_sum(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """fast.rs (`fast::weighted_sum`, fast/imp.rs:2731-2747): `sum(x * w[..., None], -2)` over `x [..., k, D]` and
+    `w [..., k]` of one floating-point type, every product and addition rounded to that type in the kernel's order."""
+    if x.ndim < 2 or tuple(w.shape) != tuple(x.shape[:-1]):
+        raise InvalidArgument(f"weighted_sum: x must be [..., k, D] and w [..., k], got {list(x.shape)} and {list(w.shape)}")
+    if x.dtype not in _CODE or w.dtype != x.dtype:
+        raise Unsupported(f"weighted_sum: x and w must share a floating-point type, got {x.dtype} and {w.dtype}")
+    _init(x)
+    x, w = x.contiguous(), w.contiguous()
+    k, d = x.shape[-2], x.shape[-1]
+    rows = w.numel() // k if k else 0
+    out = torch.empty(x.shape[:-2] + (d,), dtype=x.dtype, device=x.device)
+    _lib.check(_lib.load().nvq_weighted_sum(_CODE[x.dtype], _ptr(x), _ptr(w), rows, k, d, _ptr(out), _stream()))
+    return out
+
+
 def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor,
                        offsets: torch.Tensor) -> torch.Tensor:
     """The grouped route of `gather_qmm` (quantized.rs:646-651, 772-782) with the rows of x taken inside the kernel:

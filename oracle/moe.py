@@ -1,0 +1,73 @@
+"""TEST INFRASTRUCTURE ONLY: a CPU restatement of nuvec's mixture-of-experts glue kernels, for the parity tests.
+
+`moe_route` and `weighted_sum` follow crates/nuvec-kernels/src/metal/moe.metal line by line (33-88 and 90-118): the
+reference defines both by that kernel's arithmetic, in the element type, in that order.  What pins them beyond the
+source: the indices are the last k of a stable ascending sort with NaN last (numpy's stable argsort, a library routine,
+in tests/test_oracle_math.py), the documented example of crates/nuvec-core/src/fast.rs:733-737 and the NaN case of
+crates/nuvec-core/tests/fast.rs:900-911; the scores and sums are checked against float64 within the rounding of the
+element type.  Nothing here is imported by the product.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import ref
+
+
+def _round(a: np.ndarray, dtype: int) -> np.ndarray:
+    """float32 values rounded to the element type and widened again."""
+    return ref.to_f32(ref.from_f32(np.asarray(a, np.float32), dtype), dtype)
+
+
+def _less(a: float, b: float, dtype: int) -> bool:
+    """moe.metal:19-31: NaN sorts last where the sort compares NaN (float32 and half, not bfloat16)."""
+    if dtype != ref.BF16:
+        an, bn = np.isnan(a), np.isnan(b)
+        if an or bn:
+            return (not an) and bn
+    return bool(a < b)
+
+
+def moe_route(probs: np.ndarray, dtype: int, k: int, normalize: bool):
+    """probs: element-type array [rows, E] (as stored).  Returns (indices u32 [rows, k], scores as stored [rows, k])."""
+    p = ref.to_f32(probs, dtype)
+    rows, n = p.shape
+    indices = np.zeros((rows, k), np.uint32)
+    top = np.zeros((rows, k), np.float32)
+    for r in range(rows):
+        for e in range(n):
+            v = p[r, e]
+            rank = 0
+            for j in range(n):
+                u = p[r, j]
+                rank += 1 if (_less(u, v, dtype) or (not _less(v, u, dtype) and j < e)) else 0
+            slot = rank - (n - k)
+            if slot >= 0:
+                indices[r, slot] = e
+                top[r, slot] = v
+    if normalize:
+        scores = np.zeros_like(top)
+        for r in range(rows):
+            total = np.float32(0)
+            for j in range(k):
+                total = _round(top[r, j] + total, dtype)
+            with np.errstate(divide="ignore", invalid="ignore"):
+                scores[r] = _round(top[r] / total, dtype)
+    else:
+        scores = top
+    return indices, ref.from_f32(scores, dtype)
+
+
+def weighted_sum(x: np.ndarray, w: np.ndarray, dtype: int) -> np.ndarray:
+    """x [rows, k, D], w [rows, k] as stored; returns [rows, D] as stored."""
+    xf, wf = ref.to_f32(x, dtype), ref.to_f32(w, dtype)
+    rows, k, d = xf.shape
+    lanes = 1 if d == 1 else min(k, 8)
+    total = None
+    for y in range(lanes):
+        t = np.zeros((rows, d), np.float32)
+        for j in range(y, k, lanes):
+            product = _round(xf[:, j, :] * wf[:, j, None], dtype)
+            t = _round(product + t, dtype)
+        total = t if y == 0 else _round(t + total, dtype)
+    return ref.from_f32(total, dtype)

@@ -626,3 +626,77 @@ def test_switch_glu_sorts_gathers_and_restores():
     few = torch.cat([glu(to_dev(x)[:, t:t + 8], torch.from_numpy(idx).cuda()[:, t:t + 8]) for t in range(0, l, 8)], dim=1)
     scale = float(few.float().abs().max())
     assert float((whole.float() - few.float()).abs().max()) <= 2e-2 * scale
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+def test_moe_route_and_weighted_sum_bit_exact(dtype):
+    """fast::moe_route and fast::weighted_sum over the shapes of the reference's tests
+    (crates/nuvec-core/tests/fast.rs:841-987), bit for bit the restated kernels."""
+    from oracle import moe
+    rng = np.random.default_rng(7200 + dtype)
+    for rows, e, ks in [(3, 8, (1, 2, 8)), (5, 60, (4, 8)), (4, 128, (1, 8, 10, 128)), (2, 512, (8, 22))]:
+        logits = rng.standard_normal((rows, e)).astype(np.float32)
+        p = np.exp(logits) / np.exp(logits).sum(-1, keepdims=True)
+        ties = (np.floor(p * 4 * e) + 1) / (4 * e)
+        for name, probs in (("probs", p), ("ties", ties)):
+            stored = ref.from_f32(probs.astype(np.float32), dtype)
+            for k in ks:
+                for normalize in (False, True):
+                    if normalize and k > 64:  # beyond 64 summed scores the reference composes sum and divide itself
+                        with pytest.raises(nv.Unsupported):
+                            nv.moe_route(to_dev(stored), k, normalize)
+                        continue
+                    want_top, want_scores = moe.moe_route(stored, dtype, k, normalize)
+                    top, scores = nv.moe_route(to_dev(stored), k, normalize)
+                    case = f"{name} rows {rows} E {e} k {k} norm {normalize}"
+                    assert np.array_equal(to_host(top).astype(np.uint32), want_top), case
+                    assert np.array_equal(to_host(scores).view(np.uint8), want_scores.view(np.uint8)), case
+    if dtype != ref.BF16:  # NaN sorts last where the sort compares it
+        nan_row = ref.from_f32(np.array([[0.1, np.nan, 0.3, 0.2]], np.float32), dtype)
+        assert to_host(nv.moe_route(to_dev(nan_row), 2, False)[0]).tolist() == [[2, 1]]
+    batched = ref.from_f32(rng.random((2, 3, 16)).astype(np.float32), dtype)
+    top, scores = nv.moe_route(to_dev(batched), 4, True)
+    want_top, want_scores = moe.moe_route(batched.reshape(6, 16), dtype, 4, True)
+    assert tuple(top.shape) == (2, 3, 4) and np.array_equal(to_host(top).reshape(6, 4).astype(np.uint32), want_top)
+    assert np.array_equal(to_host(scores).reshape(6, 4).view(np.uint8), want_scores.view(np.uint8))
+    for k in (0, 17, -1):
+        with pytest.raises(nv.InvalidArgument):
+            nv.moe_route(to_dev(batched), k, False)
+    with pytest.raises(nv.InvalidArgument):
+        nv.moe_route(torch.ones(2, 8, dtype=torch.int32, device="cuda"), 2, False)
+    for rows, k, d in [(3, 1, 64), (2, 4, 7), (4, 8, 2048), (3, 10, 64), (2, 16, 1), (1, 31, 96)]:
+        x = ref.from_f32(rng.standard_normal((rows, k, d)).astype(np.float32), dtype)
+        w = ref.from_f32(rng.standard_normal((rows, k)).astype(np.float32), dtype)
+        got = to_host(nv.weighted_sum(to_dev(x), to_dev(w)))
+        assert np.array_equal(got.view(np.uint8), moe.weighted_sum(x, w, dtype).view(np.uint8)), (rows, k, d)
+    with pytest.raises(nv.Unsupported):  # 32 weighted rows and more: the reference composes multiply and sum itself
+        nv.weighted_sum(torch.ones(2, 32, 8, device="cuda"), torch.ones(2, 32, device="cuda"))
+    with pytest.raises(nv.InvalidArgument):
+        nv.weighted_sum(torch.ones(2, 4, 8, device="cuda"), torch.ones(2, 5, device="cuda"))
+
+
+def test_moe_block_routes_multiplies_and_sums():
+    """MoeMlp::forward (nuvec-lm model.rs:2251-2272) over the library: router, moe_route, the experts' gated MLPs on
+    the ordered pairs, weighted_sum; against the same steps restated on the host from the library's own routing."""
+    from oracle import moe
+    from nuvec_amd.layers import MoeMlp, SwitchGlu, SwitchProjection
+    rng = np.random.default_rng(2700)
+    experts, d, inner, b, l, k = 8, 256, 320, 2, 40, 2
+    def projection(n, kk):
+        w = make_w(rng, experts * n, kk, ref.BF16).reshape(experts, n, kk)
+        packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+        return SwitchProjection(to_dev(packed), to_dev(scales), None, None, nv.Quant.new(nv.QuantMode.MXFP4))
+    glu = SwitchGlu(projection(inner, d), projection(inner, d), projection(d, inner))
+    gate = torch.randn(experts, d, device="cuda", dtype=torch.bfloat16)
+    block = MoeMlp(gate, glu, k, True)
+    x = to_dev(make_x(rng, b * l, d, ref.BF16).reshape(b, l, d))
+    top, scores = block.route(x)
+    probs = torch.softmax(torch.nn.functional.linear(x, gate).float(), -1).to(torch.bfloat16)
+    want_top, want_scores = moe.moe_route(to_host(probs).reshape(b * l, experts), ref.BF16, k, True)
+    assert np.array_equal(to_host(top).reshape(b * l, k).astype(np.uint32), want_top)
+    assert np.array_equal(to_host(scores).reshape(b * l, k).view(np.uint8), want_scores.view(np.uint8))
+    y = block(x)
+    assert tuple(y.shape) == (b, l, d) and y.dtype == torch.bfloat16
+    outputs = glu(x, top)  # [B, L, k, D]
+    want = moe.weighted_sum(to_host(outputs).reshape(b * l, k, d), to_host(scores).reshape(b * l, k), ref.BF16)
+    assert np.array_equal(to_host(y).reshape(b * l, d).view(np.uint8), want.view(np.uint8))

@@ -172,3 +172,62 @@ def test_gather_equals_per_pair_products():
     for i in range(4):
         one = ref.quantized_matmul(x[lhs[i]], p[rhs[i]], s[rhs[i]], None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.F32)
         assert np.array_equal(y[i], one)
+
+
+# ── the mixture-of-experts glue (oracle/moe.py) ─────────────────────────────────────────
+
+def test_moe_route_documented_examples():
+    """crates/nuvec-core/src/fast.rs:733-737 and crates/nuvec-core/tests/fast.rs:900-911."""
+    from oracle import moe
+    top, scores = moe.moe_route(np.array([[0.1, 0.4, 0.2, 0.3]], np.float32), ref.F32, 2, True)
+    assert top.tolist() == [[3, 1]]
+    assert abs(scores[0, 0] - 0.3 / 0.7) < 1e-6 and abs(scores[0, 1] - 0.4 / 0.7) < 1e-6
+    nan_row = np.array([[0.1, np.nan, 0.3, 0.2]], np.float32)
+    assert moe.moe_route(nan_row, ref.F32, 2, False)[0].tolist() == [[2, 1]]
+    assert moe.moe_route(ref.from_f32(nan_row, ref.F16), ref.F16, 2, False)[0].tolist() == [[2, 1]]
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+def test_moe_route_is_the_tail_of_a_stable_sort(dtype):
+    """The indices are the last k of numpy's stable ascending argsort (ties in index order), the scores the taken
+    values, normalized ones within a rounding of the float64 quotient (crates/nuvec-core/tests/fast.rs:831-839)."""
+    from oracle import moe
+    rng = np.random.default_rng(72)
+    for rows, e, ks in [(3, 8, (1, 2, 8)), (5, 60, (4, 8)), (2, 128, (1, 10, 128))]:
+        logits = rng.standard_normal((rows, e)).astype(np.float32)
+        p = np.exp(logits) / np.exp(logits).sum(-1, keepdims=True)
+        ties = (np.floor(p * 4 * e) + 1) / (4 * e)  # a few values repeated across experts
+        for probs in (p, ties):
+            stored = ref.from_f32(probs.astype(np.float32), dtype)
+            wide = ref.to_f32(stored, dtype).astype(np.float64)
+            for k in ks:
+                want = np.argsort(wide, axis=-1, kind="stable")[:, -k:]
+                top, scores = moe.moe_route(stored, dtype, k, False)
+                assert np.array_equal(top, want)
+                assert np.array_equal(ref.to_f32(scores, dtype), np.take_along_axis(wide, want, -1).astype(np.float32))
+                _, normalized = moe.moe_route(stored, dtype, k, True)
+                taken = np.take_along_axis(wide, want, -1)
+                exact = taken / taken.sum(-1, keepdims=True)
+                eps = {ref.F32: 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+                assert np.all(np.abs(ref.to_f32(normalized, dtype) - exact) <= (k + 2) * eps * np.abs(exact) + 1e-30)
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+def test_weighted_sum_equals_multiply_and_sum(dtype):
+    """crates/nuvec-core/tests/fast.rs:955-987: sum(x * w[..., None], -2) within the rounding of k products and sums."""
+    from oracle import moe
+    rng = np.random.default_rng(73)
+    eps = {ref.F32: 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+    for rows, k, d in [(3, 1, 64), (2, 4, 7), (3, 10, 64), (2, 16, 1), (1, 31, 96)]:
+        x = ref.from_f32(rng.standard_normal((rows, k, d)).astype(np.float32), dtype)
+        w = ref.from_f32(rng.standard_normal((rows, k)).astype(np.float32), dtype)
+        got = ref.to_f32(moe.weighted_sum(x, w, dtype), dtype).astype(np.float64)
+        xf, wf = ref.to_f32(x, dtype).astype(np.float64), ref.to_f32(w, dtype).astype(np.float64)
+        exact = (xf * wf[..., None]).sum(-2)
+        bound = (k + 1) * eps * (np.abs(xf) * np.abs(wf[..., None])).sum(-2)
+        assert np.all(np.abs(got - exact) <= bound + 1e-30)
+    # one weighted row is the rounded product itself
+    x = ref.from_f32(rng.standard_normal((2, 1, 5)).astype(np.float32), dtype)
+    w = ref.from_f32(rng.standard_normal((2, 1)).astype(np.float32), dtype)
+    want = ref.from_f32((ref.to_f32(x, dtype)[:, 0] * ref.to_f32(w, dtype)).astype(np.float32), dtype)
+    assert np.array_equal(moe.weighted_sum(x, w, dtype).view(np.uint8), want.view(np.uint8))
