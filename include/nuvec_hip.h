@@ -215,6 +215,22 @@ NVQ_API int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32
 NVQ_API int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
                       uint32_t *sorted_ids, int32_t *offsets, void *stream);
 
+/* NVFP4 with a global scale (MLX's `quantize(..., global_scale=)`; ops.rs `quantize_scaled`, quantized.rs:972-1005,
+ * kernels.rs:914-1009 with `g`; validated as primitive.rs:1378-1395: NVFP4 only): `global_scale` points at one
+ * float32 value on the device; the group scales are relative to it, g / (448 * 6).  No biases in this mode. */
+NVQ_API int32_t nvq_quantize_scaled(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols,
+                            const float *global_scale, void *packed, void *scales, void *stream);
+NVQ_API int32_t nvq_dequantize_scaled(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
+                              const float *global_scale, int64_t rows, int64_t cols, void *out, void *stream);
+/* quantized.rs:469-491: x [M, K] times transposed w [N, K'] (no batch); any other shape the reference itself
+ * dequantizes and multiplies densely (NVQ_UNSUPPORTED here). */
+NVQ_API int32_t nvq_quantized_matmul_scaled(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
+                                    const float *global_scale, void *y, void *workspace, void *stream);
+/* quantized.rs:620-636, 677-719: one global scale per expert, float32 [experts]. */
+NVQ_API int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
+                              const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                              void *y, void *workspace, void *stream);
+
 /* fast::moe_route (crates/nuvec-core/src/fast.rs:740-746, fast/imp.rs:2652-2673; kernel
  * crates/nuvec-kernels/src/metal/moe.metal:33-88): per row of `experts` router probabilities the k largest in the
  * stable ascending order of the sort (NaN last for float32 and half), i.e. the last k of `argsort`, their values

@@ -137,7 +137,8 @@ template <typename T> __device__ __forceinline__ s16x2_t fp8_pair(s16x2_t word, 
 // kernels.rs:914-971 without a global scale.
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
-fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict__ packed, uint8_t *__restrict__ scales) {
+fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict__ packed, uint8_t *__restrict__ scales,
+                   const float *__restrict__ global_scale) {
     using F = Format<MODE>;
     const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     // chunks is a multiple of the lanes per group and so is the block: a group is wholly in or out of range
@@ -183,7 +184,15 @@ fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict
     }
     amax = fmaxf(amax, u2f(quad_swap<kSwap1>(f2u(amax))));
     if constexpr (F::lanes == 4) amax = fmaxf(amax, u2f(quad_swap<kSwap2>(f2u(amax))));
-    const float scale = ftz(amax / F::max_element);
+    float scale = ftz(amax / F::max_element);
+    // NVFP4's global scale g (kernels.rs:933, 941-943, 957-961): the group scales are relative to g / (448 * 6).
+    float scale_enc = 1.0f;
+    if constexpr (!F::mx) {
+        if (global_scale != nullptr) {
+            scale_enc = ftz(448.0f * 6.0f / *global_scale);
+            scale = ftz(scale * scale_enc);
+        }
+    }
     uint32_t code;
     float decoded;
     if constexpr (F::mx) {
@@ -194,7 +203,7 @@ fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict
         decoded = e4m3_to_f32(code);
     }
     decoded = ftz(decoded);
-    const float inverse = decoded == 0.0f ? 0.0f : ftz(1.0f / decoded);
+    const float inverse = decoded == 0.0f ? 0.0f : ftz(scale_enc / decoded);
     if constexpr (F::bits == 4) {
         uint32_t word = 0;
 #pragma unroll
@@ -238,7 +247,7 @@ template <typename T> __device__ __forceinline__ void store_values(T *out, int64
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
 fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, uint32_t chunks, T *__restrict__ out,
-                     const uint32_t *__restrict__ ids, uint32_t row_chunks, int64_t table_rows) {
+                     const uint32_t *__restrict__ ids, uint32_t row_chunks, int64_t table_rows, const float *__restrict__ global_scale) {
     using F = Format<MODE>;
     const uint32_t out_chunk = blockIdx.x * kBlock + threadIdx.x;  // fewer than 2^29: an operand has fewer than 2^32 elements
     if (out_chunk >= chunks) return;
@@ -274,7 +283,10 @@ fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restr
             return;
         }
     }
-    const float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
+    float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
+    if constexpr (!F::mx) {  // NVFP4's global scale (kernels.rs:992, 996-998)
+        if (global_scale != nullptr) scale = ftz(scale * ftz(*global_scale / (448.0f * 6.0f)));
+    }
     float v[8];
     if constexpr (F::bits == 4) {
         const uint32_t word = packed[chunk];
@@ -292,41 +304,41 @@ fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restr
 }
 
 template <typename T, int MODE>
-int32_t quantize_t(const void *w, int64_t n, void *packed, void *scales, hipStream_t s) {
+int32_t quantize_t(const void *w, int64_t n, void *packed, void *scales, const float *global_scale, hipStream_t s) {
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((fp_quantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const T *)w, chunks,
-                       (uint32_t *)packed, (uint8_t *)scales);
+                       (uint32_t *)packed, (uint8_t *)scales, global_scale);
     NVQ_LAUNCH_CHECK("fp_quantize");
     return NVQ_OK;
 }
 template <typename T, int MODE>
 int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *out, const uint32_t *ids, int64_t cols,
-                     int64_t table_rows, hipStream_t s) {
+                     int64_t table_rows, const float *global_scale, hipStream_t s) {
     const int64_t chunks = n / 8;
     const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((fp_dequantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const uint32_t *)packed,
-                       (const uint8_t *)scales, (uint32_t)chunks, (T *)out, ids, (uint32_t)(cols / 8), table_rows);
+                       (const uint8_t *)scales, (uint32_t)chunks, (T *)out, ids, (uint32_t)(cols / 8), table_rows, global_scale);
     NVQ_LAUNCH_CHECK("fp_dequantize");
     return NVQ_OK;
 }
 
 template <typename T>
-int32_t quantize_mode(int32_t mode, const void *w, int64_t n, void *packed, void *scales, hipStream_t s) {
+int32_t quantize_mode(int32_t mode, const void *w, int64_t n, void *packed, void *scales, const float *g, hipStream_t s) {
     switch (mode) {
-    case NVQ_MXFP4: return quantize_t<T, NVQ_MXFP4>(w, n, packed, scales, s);
-    case NVQ_MXFP8: return quantize_t<T, NVQ_MXFP8>(w, n, packed, scales, s);
-    case NVQ_NVFP4: return quantize_t<T, NVQ_NVFP4>(w, n, packed, scales, s);
+    case NVQ_MXFP4: return quantize_t<T, NVQ_MXFP4>(w, n, packed, scales, g, s);
+    case NVQ_MXFP8: return quantize_t<T, NVQ_MXFP8>(w, n, packed, scales, g, s);
+    case NVQ_NVFP4: return quantize_t<T, NVQ_NVFP4>(w, n, packed, scales, g, s);
     default: return fail(NVQ_INVALID_ARGUMENT, "quantize: mode %s is not a floating-point block format", mode_name(mode));
     }
 }
 template <typename T>
 int32_t dequantize_mode(int32_t mode, const void *packed, const void *scales, int64_t n, void *out, const uint32_t *ids,
-                        int64_t cols, int64_t table_rows, hipStream_t s) {
+                        int64_t cols, int64_t table_rows, const float *g, hipStream_t s) {
     switch (mode) {
-    case NVQ_MXFP4: return dequantize_t<T, NVQ_MXFP4>(packed, scales, n, out, ids, cols, table_rows, s);
-    case NVQ_MXFP8: return dequantize_t<T, NVQ_MXFP8>(packed, scales, n, out, ids, cols, table_rows, s);
-    case NVQ_NVFP4: return dequantize_t<T, NVQ_NVFP4>(packed, scales, n, out, ids, cols, table_rows, s);
+    case NVQ_MXFP4: return dequantize_t<T, NVQ_MXFP4>(packed, scales, n, out, ids, cols, table_rows, g, s);
+    case NVQ_MXFP8: return dequantize_t<T, NVQ_MXFP8>(packed, scales, n, out, ids, cols, table_rows, g, s);
+    case NVQ_NVFP4: return dequantize_t<T, NVQ_NVFP4>(packed, scales, n, out, ids, cols, table_rows, g, s);
     default: return fail(NVQ_INVALID_ARGUMENT, "dequantize: mode %s is not a floating-point block format", mode_name(mode));
     }
 }
@@ -334,20 +346,20 @@ int32_t dequantize_mode(int32_t mode, const void *packed, const void *scales, in
 }  // namespace
 
 int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n, void *packed, void *scales,
-                           hipStream_t s) {
+                           const float *g, hipStream_t s) {
     switch (dtype) {
-    case NVQ_F32: return quantize_mode<float>(mode, w, n, packed, scales, s);
-    case NVQ_BF16: return quantize_mode<bf16_t>(mode, w, n, packed, scales, s);
-    default: return quantize_mode<f16_t>(mode, w, n, packed, scales, s);
+    case NVQ_F32: return quantize_mode<float>(mode, w, n, packed, scales, g, s);
+    case NVQ_BF16: return quantize_mode<bf16_t>(mode, w, n, packed, scales, g, s);
+    default: return quantize_mode<f16_t>(mode, w, n, packed, scales, g, s);
     }
 }
 
 int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales, int64_t n,
-                             void *out, const uint32_t *ids, int64_t cols, int64_t table_rows, hipStream_t s) {
+                             void *out, const uint32_t *ids, int64_t cols, int64_t table_rows, const float *g, hipStream_t s) {
     switch (out_dtype) {
-    case NVQ_F32: return dequantize_mode<float>(mode, packed, scales, n, out, ids, cols, table_rows, s);
-    case NVQ_BF16: return dequantize_mode<bf16_t>(mode, packed, scales, n, out, ids, cols, table_rows, s);
-    default: return dequantize_mode<f16_t>(mode, packed, scales, n, out, ids, cols, table_rows, s);
+    case NVQ_F32: return dequantize_mode<float>(mode, packed, scales, n, out, ids, cols, table_rows, g, s);
+    case NVQ_BF16: return dequantize_mode<bf16_t>(mode, packed, scales, n, out, ids, cols, table_rows, g, s);
+    default: return dequantize_mode<f16_t>(mode, packed, scales, n, out, ids, cols, table_rows, g, s);
     }
 }
 

@@ -213,8 +213,16 @@ int32_t nvq_gather_grouped(int64_t rows, int64_t experts, int32_t row_exact) {
     return rows >= least && rows / (experts > 1 ? experts : 1) >= 4;
 }
 
-int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols, void *packed,
-                     void *scales, void *biases, void *stream) {
+// primitive.rs:1378-1395 (MLX's validate_global_scale): NVFP4 only.
+static int32_t check_global_scale(const char *op, const nvq_quant *quant, const float *global_scale) {
+    if (global_scale == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null global scale", op);
+    if (quant->mode != NVQ_NVFP4)
+        return fail(NVQ_INVALID_ARGUMENT, "%s: a global scale is only supported for nvfp4, got %s", op, mode_name(quant->mode));
+    return NVQ_OK;
+}
+
+static int32_t quantize_any(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols, void *packed,
+                            void *scales, void *biases, const float *global_scale, void *stream) {
     NVQ_TRY(check_quant(quant, "quantize"));
     // primitive.rs:1234-1243
     if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "quantize: unsupported dtype %s", dtype_name(dtype));
@@ -234,13 +242,25 @@ int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64
     if (n >= (1LL << 32)) return fail(NVQ_INVALID_ARGUMENT, "quantize: %lld elements; an operand holds fewer than 2^32", (long long)n);
     if (quant->mode == NVQ_AFFINE)
         return launch_affine_quantize(dtype, quant->group_size, quant->bits, w, n, packed, scales, biases, (hipStream_t)stream);
-    return launch_fp_quantize(quant->mode, dtype, w, n, packed, scales, (hipStream_t)stream);
+    return launch_fp_quantize(quant->mode, dtype, w, n, packed, scales, global_scale, (hipStream_t)stream);
+}
+
+int32_t nvq_quantize(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols, void *packed,
+                     void *scales, void *biases, void *stream) {
+    return quantize_any(quant, dtype, w, rows, cols, packed, scales, biases, nullptr, stream);
+}
+
+int32_t nvq_quantize_scaled(const nvq_quant *quant, int32_t dtype, const void *w, int64_t rows, int64_t cols,
+                            const float *global_scale, void *packed, void *scales, void *stream) {
+    NVQ_TRY(check_quant(quant, "quantize"));
+    NVQ_TRY(check_global_scale("quantize", quant, global_scale));
+    return quantize_any(quant, dtype, w, rows, cols, packed, scales, nullptr, global_scale, stream);
 }
 
 // Shared by nvq_dequantize and nvq_dequantize_rows: `count` output rows, each table row ids[r] (or row r).
 static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
                               const void *biases, int64_t table_rows, int64_t cols, const uint32_t *ids, int64_t count,
-                              void *out, void *stream) {
+                              void *out, void *stream, const float *global_scale = nullptr) {
     NVQ_TRY(check_quant(quant, op));
     NVQ_TRY(check_groups(op, quant->mode, biases));
     // primitive.rs:1272-1276
@@ -262,12 +282,19 @@ static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dt
     if (quant->mode == NVQ_AFFINE)
         return launch_affine_dequantize(dtype, quant->group_size, quant->bits, packed, scales, biases, n, out, ids, cols,
                                         table_rows, (hipStream_t)stream);
-    return launch_fp_dequantize(quant->mode, dtype, packed, scales, n, out, ids, cols, table_rows, (hipStream_t)stream);
+    return launch_fp_dequantize(quant->mode, dtype, packed, scales, n, out, ids, cols, table_rows, global_scale, (hipStream_t)stream);
 }
 
 int32_t nvq_dequantize(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales, const void *biases,
                        int64_t rows, int64_t cols, void *out, void *stream) {
     return dequantize_any("dequantize", quant, dtype, packed, scales, biases, rows, cols, nullptr, rows, out, stream);
+}
+
+int32_t nvq_dequantize_scaled(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
+                              const float *global_scale, int64_t rows, int64_t cols, void *out, void *stream) {
+    NVQ_TRY(check_quant(quant, "dequantize"));
+    NVQ_TRY(check_global_scale("dequantize", quant, global_scale));
+    return dequantize_any("dequantize", quant, dtype, packed, scales, nullptr, rows, cols, nullptr, rows, out, stream, global_scale);
 }
 
 int32_t nvq_dequantize_rows(const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales, const void *biases,
@@ -312,8 +339,8 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
     return takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
 }
 
-int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
-                             void *y, void *workspace, void *stream) {
+static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                                    const float *global_scale, void *y, void *workspace, void *stream) {
     NVQ_TRY(check_qmm(d, "quantized_matmul"));
     NVQ_TRY(check_groups("quantized_matmul", d->quant.mode, biases));
     int64_t batch = 1;
@@ -332,6 +359,8 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     }
     ProductArgs a = product_args(d, batch);
     a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
+    a.global_scale = global_scale;
+    if (global_scale != nullptr) return launch_qmv(a, (hipStream_t)stream);  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
     if (takes_tiled(d, a)) return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
     // Up to four rows of 4-bit affine weights: the decode kernel (per-row work on the vector units, which is
@@ -342,6 +371,22 @@ int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w
     const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 : a.bits >= 3 && a.m == 1);
     if (!decode && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
+}
+
+int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                             void *y, void *workspace, void *stream) {
+    return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream);
+}
+
+int32_t nvq_quantized_matmul_scaled(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales,
+                                    const float *global_scale, void *y, void *workspace, void *stream) {
+    NVQ_TRY(check_qmm(d, "quantized_matmul"));
+    NVQ_TRY(check_global_scale("quantized_matmul", &d->quant, global_scale));
+    // quantized.rs:481-491: with a global scale only a transposed product of two matrices reaches a kernel; the
+    // reference dequantizes and multiplies densely otherwise.
+    if (!d->transpose || d->batch_ndim != 0)
+        return fail(NVQ_UNSUPPORTED, "quantized_matmul: with a global scale only x [M, K] times transposed w [N, K'] has a kernel");
+    return quantized_matmul_any(d, x, w, scales, nullptr, global_scale, y, workspace, stream);
 }
 
 int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups, int32_t *offsets, void *stream) {
@@ -415,8 +460,9 @@ int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t ro
     return launch_weighted_sum(dtype, x, w, rows, k, d, out, (hipStream_t)stream);
 }
 
-int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
-                       const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
+static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                              const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y,
+                              void *workspace, void *stream) {
     (void)workspace;
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
     NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
@@ -443,6 +489,7 @@ int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, c
     a.batch = d->pairs;
     a.lhs = lhs; a.rhs = rhs;
     a.x_batches = d->x_batches; a.experts = d->experts;
+    a.global_scale = global_scale;
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;
@@ -450,6 +497,22 @@ int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, c
     a.offsets = nullptr;
     if (qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
+}
+
+int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                       const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
+    return gather_qmm_any(d, x, w, scales, biases, nullptr, lhs, rhs, offsets, y, workspace, stream);
+}
+
+int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *d, const void *x, const void *w, const void *scales,
+                              const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                              void *y, void *workspace, void *stream) {
+    if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
+    NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
+    if (global_scales == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null global scale");
+    if (d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
+        return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
+    return gather_qmm_any(d, x, w, scales, nullptr, global_scales, lhs, rhs, offsets, y, workspace, stream);
 }
 
 }  // extern "C"

@@ -43,11 +43,12 @@ int32_t launch_affine_quantize(int32_t dtype, int group, int bits, const void *w
 int32_t launch_affine_dequantize(int32_t dtype, int group, int bits, const void *packed, const void *scales,
                                  const void *biases, int64_t n_values, void *out, const uint32_t *ids, int64_t cols,
                                  int64_t table_rows, hipStream_t s);
+// `global_scale`: NULL, or NVFP4's one float32 value on the device
 int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n_values, void *packed,
-                           void *scales, hipStream_t s);
+                           void *scales, const float *global_scale, hipStream_t s);
 int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales,
                              int64_t n_values, void *out, const uint32_t *ids, int64_t cols, int64_t table_rows,
-                             hipStream_t s);
+                             const float *global_scale, hipStream_t s);
 int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,
                               int32_t *offsets, hipStream_t s);
 // Hugging Face integer packings into the affine layout (repack.hip).  format 0: AWQ, 1: GPTQ v1, 2: GPTQ v2.
@@ -76,6 +77,7 @@ struct ProductArgs {
     const int32_t *offsets;         // grouped gather: rows of expert e are [offsets[e], offsets[e+1]) of `batch` rows
     int32_t k_splits, k_split_steps;  // tiled kernel: K split over grid z (0 or 1: no split), steps of 64 values per split
     float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
+    const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (general kernel only)
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.

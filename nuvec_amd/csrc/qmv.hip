@@ -166,6 +166,16 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
             const uint8_t *sp = (const uint8_t *)a.scales + o.s + (int64_t)nc * kgroups + (kc >> gshift);
 #pragma unroll
             for (int hf = 0; hf < kHalves; hf++) sc[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(sp[hf]) : e8m0_to_f32(sp[hf]));
+            if constexpr (MODE == NVQ_NVFP4) {
+                // kernels.rs:992-998: a global scale g turns every group scale into ftz(scale * ftz(g / (448 * 6)));
+                // a gather has one g per expert (quantized.rs:620-636)
+                if (a.global_scale != nullptr) {
+                    const float g = a.global_scale[a.rhs != nullptr ? min((int64_t)a.rhs[blockIdx.z], a.experts - 1) : 0];
+                    const float inv_enc = ftz(g / (448.0f * 6.0f));
+#pragma unroll
+                    for (int hf = 0; hf < kHalves; hf++) sc[hf] = ftz(sc[hf] * inv_enc);
+                }
+            }
         }
         if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
 #pragma unroll

@@ -77,6 +77,11 @@ class Quantized:
     scales: torch.Tensor
     biases: Optional[torch.Tensor]
     quant: Quant
+    global_scale: Optional[torch.Tensor] = None  # NVFP4: one float32 value, or one per expert (`[E]`) of stacked experts
+
+    def with_global_scale(self, global_scale: torch.Tensor) -> "Quantized":
+        """quantized.rs:248-253."""
+        return Quantized(self.weight, self.scales, self.biases, self.quant, global_scale)
 
     @staticmethod
     def affine(weight, scales, biases, group_size, bits) -> "Quantized":
@@ -163,8 +168,20 @@ def _quantized_columns(op: str, w, scales, biases, quant: Quant) -> int:
     return groups
 
 
-def quantize(w: torch.Tensor, quant: Quant | QuantMode = Quant()) -> Quantized:
-    """ops.rs:965-1008, primitive.rs:1223-1259: quantizes the last axis of `w`."""
+def _global_scale(op: str, quant: Quant, g: Optional[torch.Tensor], device) -> Optional[torch.Tensor]:
+    """primitive.rs:1378-1395 (MLX's `validate_global_scale`): NVFP4 only, one float32 value."""
+    if g is None:
+        return None
+    if quant.mode != QuantMode.NVFP4:
+        raise InvalidArgument(f"{op}: a global scale is only supported for nvfp4, got {quant.mode.mlx_name}")
+    if g.numel() != 1 or g.dtype != torch.float32:
+        raise InvalidArgument(f"{op}: the global scale must be one float32 value, got {_name(g.dtype)} {list(g.shape)}")
+    return g.to(device).contiguous()
+
+
+def quantize(w: torch.Tensor, quant: Quant | QuantMode = Quant(), global_scale: Optional[torch.Tensor] = None) -> Quantized:
+    """ops.rs:965-1008 (`quantize`, `quantize_scaled`), primitive.rs:1223-1259: quantizes the last axis of `w`; with
+    NVFP4's `global_scale` the group scales are relative to it, g / (448 * 6), and the result carries it."""
     quant = Quant.new(quant) if isinstance(quant, QuantMode) else quant
     group, bits = quant.checked("quantize")
     if w.dtype not in _FLOATS:
@@ -180,6 +197,11 @@ def quantize(w: torch.Tensor, quant: Quant | QuantMode = Quant()) -> Quantized:
     affine = quant.mode == QuantMode.AFFINE
     scales = torch.empty(w.shape[:-1] + (last // group,), dtype=w.dtype if affine else torch.uint8, device=w.device)
     biases = torch.empty_like(scales) if affine else None
+    g = _global_scale("quantize", quant, global_scale, w.device)
+    if g is not None:
+        _lib.check(_lib.load().nvq_quantize_scaled(C.byref(quant._c()), _CODE[w.dtype], _ptr(w), rows, last, _ptr(g), _ptr(packed),
+                                                   _ptr(scales), _stream()))
+        return Quantized(packed, scales, None, quant, global_scale)
     _lib.check(_lib.load().nvq_quantize(C.byref(quant._c()), _CODE[w.dtype], _ptr(w), rows, last, _ptr(packed),
                                         _ptr(scales), _ptr(biases), _stream()))
     return Quantized(packed, scales, biases, quant)
@@ -203,6 +225,11 @@ def dequantize(q: Quantized, dtype: Optional[torch.dtype] = None) -> torch.Tenso
     b = q.biases.contiguous() if affine else None
     out = torch.empty(w.shape[:-1] + (cols,), dtype=compute, device=w.device)
     rows = out.numel() // cols if cols else 0
+    g = _global_scale("dequantize", quant, q.global_scale, w.device)
+    if g is not None:
+        _lib.check(_lib.load().nvq_dequantize_scaled(C.byref(quant._c()), _CODE[compute], _ptr(w), _ptr(s), _ptr(g), rows, cols,
+                                                     _ptr(out), _stream()))
+        return out
     _lib.check(_lib.load().nvq_dequantize(C.byref(quant._c()), _CODE[compute], _ptr(w), _ptr(s), _ptr(b), rows, cols,
                                           _ptr(out), _stream()))
     if affine and dtype is not None and dtype != out.dtype:
@@ -259,6 +286,12 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     quant = q.quant
     group, bits = quant.checked(op)
     _check_groups(op, quant.mode, q.scales, q.biases)
+    g = _global_scale(op, quant, q.global_scale, x.device)
+    if g is not None and (q.weight.ndim > 2 or x.ndim > 2 or not transpose):
+        # quantized.rs:481-491: only x [M, K] times transposed w [N, K'] reaches a kernel with a global scale; the
+        # reference dequantizes in x's type and multiplies densely otherwise.
+        dense = dequantize(q, x.dtype)
+        return x.matmul(dense.transpose(-1, -2) if transpose else dense)
     affine = quant.mode == QuantMode.AFFINE
     dtype = _promoted(op, x, q.scales, q.biases)
     x = x.to(dtype)
@@ -309,8 +342,12 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     lib = _lib.load()
     need = lib.nvq_quantized_matmul_workspace_bytes(C.byref(d))
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
-    _lib.check(lib.nvq_quantized_matmul(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
-                                        _ptr(workspace), _stream()))
+    if g is not None:
+        _lib.check(lib.nvq_quantized_matmul_scaled(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(g), _ptr(out),
+                                                   _ptr(workspace), _stream()))
+    else:
+        _lib.check(lib.nvq_quantized_matmul(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
+                                            _ptr(workspace), _stream()))
     return out.squeeze(-2) if vector else out
 
 
@@ -467,6 +504,18 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
     lib = _lib.load()
     need = lib.nvq_gather_qmm_workspace_bytes(C.byref(d))
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    gs = q.global_scale
+    if gs is not None:  # quantized.rs:620-636: one float32 value per expert
+        if quant.mode != QuantMode.NVFP4:
+            raise InvalidArgument(f"{op}: global scale is only supported for 'nvfp4' quantization mode")
+        if gs.dtype != torch.float32:
+            raise InvalidArgument(f"{op}: global scale must have dtype float32 but got {_name(gs.dtype)}")
+        if tuple(gs.shape) != tuple(w.shape[:-2]):
+            raise InvalidArgument(f"{op}: global scale must have one entry per expert with shape {list(w.shape[:-2])} but got {list(gs.shape)}")
+        gs = gs.to(x.device).contiguous()
+        _lib.check(lib.nvq_gather_qmm_scaled(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(gs), _ptr(lhs), _ptr(rhs),
+                                             _ptr(offsets), _ptr(out), _ptr(workspace), _stream()))
+        return out
     _lib.check(lib.nvq_gather_qmm(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs),
                                   _ptr(offsets), _ptr(out), _ptr(workspace), _stream()))
     return out

@@ -327,34 +327,36 @@ static int fp_mode_ok(int mode, int *group, int *bits) { /* quantized.rs:48-56 *
     }
 }
 
-/* kernels.rs:914-971 with no global scale (`g = None`).  Outputs: packed u32[n*bits/32],
- * scales u8[n/group]. */
-NVQ_EXPORT int nvq_ref_fp_quantize(const void *w, int dtype, int64_t n, int mode,
-                                   uint32_t *packed, uint8_t *scales) {
+/* kernels.rs:914-971.  `g` NULL = no global scale; otherwise the NVFP4 global scale: group scales are
+ * relative to g / (448 * 6).  Outputs: packed u32[n*bits/32], scales u8[n/group]. */
+static int fp_quantize_impl(const void *w, int dtype, int64_t n, int mode, const float *g,
+                            uint32_t *packed, uint8_t *scales) {
     int group, bits;
     if (!dtype_ok(dtype) || !fp_mode_ok(mode, &group, &bits) || n % group) return 1;
     uint8_t *bytes = (uint8_t *)packed;
     const int mx = group == 32;
     const float max_element = bits == 4 ? E2M1_MAX : E4M3_MAX;
-    for (int64_t g = 0; g < n / group; g++) {
+    const float scale_enc = g ? nvq_ref_ftz(E4M3_MAX * E2M1_MAX / *g) : 1.0f;
+    for (int64_t gi = 0; gi < n / group; gi++) {
         float amax = 0.0f;
         for (int j = 0; j < group; j++)
-            amax = rs_max(amax, fabsf(nvq_ref_ftz(load_f32(w, g * group + j, dtype))));
+            amax = rs_max(amax, fabsf(nvq_ref_ftz(load_f32(w, gi * group + j, dtype))));
         float scale = nvq_ref_ftz(amax / max_element);
+        if (g) scale = nvq_ref_ftz(scale * scale_enc);
         uint8_t code;
         float decoded;
-        if (mx) {
+        if (mx && !g) {
             code = nvq_ref_e8m0_from_f32(nvq_ref_mx_scale_round_up(scale));
             decoded = nvq_ref_e8m0_to_f32(code);
         } else {
             code = nvq_ref_e4m3_from_f32(scale);
             decoded = nvq_ref_e4m3_to_f32(code);
         }
-        scales[g] = code;
+        scales[gi] = code;
         decoded = nvq_ref_ftz(decoded);
-        float inverse = decoded == 0.0f ? 0.0f : nvq_ref_ftz(1.0f / decoded);
+        float inverse = decoded == 0.0f ? 0.0f : nvq_ref_ftz(scale_enc / decoded);
         for (int j = 0; j < group; j++) {
-            int64_t i = g * group + j;
+            int64_t i = gi * group + j;
             float v = nvq_ref_ftz(load_f32(w, i, dtype));
             float scaled = nvq_ref_canonical(nvq_ref_ftz(v * inverse));
             if (bits == 8) {
@@ -368,25 +370,43 @@ NVQ_EXPORT int nvq_ref_fp_quantize(const void *w, int dtype, int64_t n, int mode
     }
     return 0;
 }
+NVQ_EXPORT int nvq_ref_fp_quantize(const void *w, int dtype, int64_t n, int mode,
+                                   uint32_t *packed, uint8_t *scales) {
+    return fp_quantize_impl(w, dtype, n, mode, NULL, packed, scales);
+}
+NVQ_EXPORT int nvq_ref_fp_quantize_scaled(const void *w, int dtype, int64_t n, int mode, float g,
+                                          uint32_t *packed, uint8_t *scales) {
+    return fp_quantize_impl(w, dtype, n, mode, &g, packed, scales);
+}
 
-static inline float fp_value(const uint8_t *codes, const uint8_t *s, int64_t i, int group, int bits) {
-    /* kernels.rs:994-1005 without a global scale */
+static inline float fp_value(const uint8_t *codes, const uint8_t *s, int64_t i, int group, int bits, const float *inv_enc) {
+    /* kernels.rs:994-1005; `inv_enc` NULL = no global scale, else ftz(g / (448 * 6)) */
     uint8_t sc = s[i / group];
     float scale = nvq_ref_ftz(group == 32 ? nvq_ref_e8m0_to_f32(sc) : nvq_ref_e4m3_to_f32(sc));
+    if (inv_enc) scale = nvq_ref_ftz(scale * *inv_enc);
     float value = bits == 8 ? nvq_ref_e4m3_to_f32(codes[i])
                             : nvq_ref_e2m1_to_f32((uint8_t)((codes[i / 2] >> (4 * (i % 2))) & 0xF));
     return nvq_ref_canonical(nvq_ref_ftz(scale * value));
 }
 
-/* kernels.rs:976-1009 with no global scale. */
-NVQ_EXPORT int nvq_ref_fp_dequantize(const uint32_t *packed, const uint8_t *scales, int64_t n, int mode,
-                                     int out_dtype, void *out) {
+/* kernels.rs:976-1009. */
+static int fp_dequantize_impl(const uint32_t *packed, const uint8_t *scales, int64_t n, int mode,
+                              int out_dtype, const float *g, void *out) {
     int group, bits;
     if (!dtype_ok(out_dtype) || !fp_mode_ok(mode, &group, &bits) || n % group) return 1;
     const uint8_t *codes = (const uint8_t *)packed;
+    float inv = g ? nvq_ref_ftz(*g / (E4M3_MAX * E2M1_MAX)) : 0.0f;
     for (int64_t i = 0; i < n; i++)
-        store_rounded(out, i, out_dtype, (double)fp_value(codes, scales, i, group, bits));
+        store_rounded(out, i, out_dtype, (double)fp_value(codes, scales, i, group, bits, g ? &inv : NULL));
     return 0;
+}
+NVQ_EXPORT int nvq_ref_fp_dequantize(const uint32_t *packed, const uint8_t *scales, int64_t n, int mode,
+                                     int out_dtype, void *out) {
+    return fp_dequantize_impl(packed, scales, n, mode, out_dtype, NULL, out);
+}
+NVQ_EXPORT int nvq_ref_fp_dequantize_scaled(const uint32_t *packed, const uint8_t *scales, int64_t n, int mode,
+                                            int out_dtype, float g, void *out) {
+    return fp_dequantize_impl(packed, scales, n, mode, out_dtype, &g, out);
 }
 
 /* ── sorted offsets (kernels.rs:873-892) ─────────────────────────────────────────── */
@@ -481,6 +501,19 @@ static void product_rows(int dtype, int transpose, int64_t M, int64_t N, int64_t
  * `batch`.  scales/biases: `dtype` for affine, uint8 / NULL for the fp modes.  Each batch is
  * its own M-row product (kernels.rs:1145-1149 loops the batches).  K == 0 gives zeros
  * (matmul.rs:237-240). */
+/* x[M,K] times an already dequantized float32 matrix (`dense` [N,K] if transpose else [K,N]), rounded once to
+ * `dtype`: the product step of kernels.rs:1112-1142 on its own, for weights dequantized with a global scale. */
+NVQ_EXPORT int nvq_ref_dense_matmul(int dtype, int transpose, int64_t M, int64_t N, int64_t K, const void *x,
+                                    const float *dense, void *y, int threads) {
+    if (!dtype_ok(dtype)) return 1;
+    float *x32 = (float *)malloc((size_t)(M * K) * 4 + 4);
+    if (!x32) return 2;
+    for (int64_t i = 0; i < M * K; i++) x32[i] = load_f32(x, i, dtype);
+    product_rows(dtype, transpose, M, N, K, x32, dense, y, threads < 1 ? 1 : threads);
+    free(x32);
+    return 0;
+}
+
 NVQ_EXPORT int nvq_ref_quantized_matmul(int mode, int group, int bits, int dtype, int transpose,
                                         int64_t batch, int64_t M, int64_t N, int64_t K, int64_t w_batch,
                                         const void *x, const uint32_t *w, const void *scales,

@@ -118,25 +118,53 @@ def affine_dequantize(packed, scales, biases, dtype: int, group: int, bits: int,
     return out
 
 
-def fp_quantize(w: np.ndarray, dtype: int, mode: int):
+def fp_quantize(w: np.ndarray, dtype: int, mode: int, global_scale=None):
+    """kernels.rs:914-971; `global_scale`: NVFP4's one float32 value (scales relative to g / (448 * 6))."""
     w = _c(w)
     group, bits = FP_PARAMS[mode]
     last = w.shape[-1]
     packed = np.zeros(w.shape[:-1] + (last * bits // 32,), np.uint32)
     scales = np.zeros(w.shape[:-1] + (last // group,), np.uint8)
-    _check(lib().nvq_ref_fp_quantize(_p(w), dtype, C.c_int64(w.size), mode, _p(packed), _p(scales)),
-           "fp_quantize")
+    if global_scale is None:
+        rc = lib().nvq_ref_fp_quantize(_p(w), dtype, C.c_int64(w.size), mode, _p(packed), _p(scales))
+    else:
+        rc = lib().nvq_ref_fp_quantize_scaled(_p(w), dtype, C.c_int64(w.size), mode, C.c_float(float(global_scale)),
+                                              _p(packed), _p(scales))
+    _check(rc, "fp_quantize")
     return packed, scales
 
 
-def fp_dequantize(packed, scales, mode: int, out_dtype: int):
+def fp_dequantize(packed, scales, mode: int, out_dtype: int, global_scale=None):
+    """kernels.rs:976-1009; `global_scale`: NVFP4's one float32 value."""
     packed, scales = _c(packed, np.uint32), _c(scales, np.uint8)
     _, bits = FP_PARAMS[mode]
     last = packed.shape[-1] * 32 // bits
     out = np.zeros(packed.shape[:-1] + (last,), NP_OF[out_dtype])
-    _check(lib().nvq_ref_fp_dequantize(_p(packed), _p(scales), C.c_int64(out.size), mode, out_dtype, _p(out)),
-           "fp_dequantize")
+    if global_scale is None:
+        rc = lib().nvq_ref_fp_dequantize(_p(packed), _p(scales), C.c_int64(out.size), mode, out_dtype, _p(out))
+    else:
+        rc = lib().nvq_ref_fp_dequantize_scaled(_p(packed), _p(scales), C.c_int64(out.size), mode, out_dtype,
+                                                C.c_float(float(global_scale)), _p(out))
+    _check(rc, "fp_dequantize")
     return out
+
+
+def dense_matmul(x, dense, dtype: int, transpose: bool = True, threads: int = 1):
+    """x [M, K] times an already dequantized float32 matrix ([N, K] if transpose else [K, N]), rounded once to
+    `dtype`: the product step of kernels.rs:1112-1142 (weights dequantized with a global scale go this way)."""
+    x, dense = _c(x), _c(dense, np.float32)
+    M, K = x.shape
+    N = dense.shape[0] if transpose else dense.shape[1]
+    y = np.zeros((M, N), NP_OF[dtype])
+    _check(lib().nvq_ref_dense_matmul(dtype, int(transpose), C.c_int64(M), C.c_int64(N), C.c_int64(K), _p(x), _p(dense),
+                                      _p(y), threads), "dense_matmul")
+    return y
+
+
+def fp_quantized_matmul_scaled(x, packed, scales, mode: int, dtype: int, global_scale, transpose: bool = True):
+    """quantized.rs:469-491 with a global scale: x . dequantize(w, float32, g)^T (or x . dequantize(w)), one rounding."""
+    dense = fp_dequantize(packed, scales, mode, F32, global_scale)
+    return dense_matmul(x, dense, dtype, transpose)
 
 
 def sorted_offsets(indices: np.ndarray, groups: int) -> np.ndarray:

@@ -3,7 +3,7 @@
 Reads (as bytes, nothing is imported or executed) the two data files the reference's own
 tests replay — crates/nuvec-core/tests/fixtures/mlx.bin (MLX 0.32.4 on the CPU) and
 mlx_gpu.bin (MLX 0.32.4 on the GPU) — keeps the cases of the quantized-matmul path
-(affine, MXFP4, MXFP8 and NVFP4 without a global scale) and re-serialises them unchanged in the same
+(affine, MXFP4, MXFP8 and NVFP4, the latter also with its global scale) and re-serialises them unchanged in the same
 BSMXFIX1 container:
 
     golden_cpu.bin   every affine quantize / dequantize / quantized_matmul case of mlx.bin
@@ -27,7 +27,7 @@ PATH_OPS = ("quantize", "dequantize", "quantized_matmul", "gather_qmm")
 
 def in_scope(case) -> bool:
     mode = case.params.get("mode", "affine")
-    return case.op in PATH_OPS and mode in ("affine", "mxfp4", "mxfp8", "nvfp4") and case.params.get("gs") != "1"
+    return case.op in PATH_OPS and mode in ("affine", "mxfp4", "mxfp8", "nvfp4")
 
 
 def keep_gpu(case) -> bool:
@@ -39,6 +39,8 @@ def keep_gpu(case) -> bool:
     # to keep the file near 3 MiB; the MoE-shaped grouped gather (K = 2880) is kept whole.
     if "-float16" in case.name:
         return False
+    if case.params.get("gs") == "1":  # gathers with one global scale per expert: the transposed ones that reach a kernel
+        return case.params.get("transpose", "1") == "1" and case.nbytes() <= 160_000
     if case.params.get("mode", "affine") in ("mxfp8", "nvfp4"):
         return case.nbytes() <= 40_000
     if case.name.endswith("oss-grouped"):

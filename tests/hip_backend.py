@@ -41,12 +41,13 @@ def quant(mode, group, bits):
 class HipBackend:
     name = "hip"
 
-    def quantize(self, w, dtype, mode, group, bits):
-        q = nv.quantize(to_dev(w), quant(mode, group, bits))
+    def quantize(self, w, dtype, mode, group, bits, global_scale=None):
+        q = nv.quantize(to_dev(w), quant(mode, group, bits), None if global_scale is None else to_dev(np.asarray(global_scale)))
         return to_host(q.weight), to_host(q.scales), None if q.biases is None else to_host(q.biases)
 
-    def dequantize(self, w, scales, biases, mode, group, bits, scales_dtype, out_dtype=None):
-        q = nv.Quantized(to_dev(w), to_dev(scales), to_dev(biases), quant(mode, group, bits))
+    def dequantize(self, w, scales, biases, mode, group, bits, scales_dtype, out_dtype=None, global_scale=None):
+        q = nv.Quantized(to_dev(w), to_dev(scales), to_dev(biases), quant(mode, group, bits),
+                         None if global_scale is None else to_dev(np.asarray(global_scale)))
         out = nv.dequantize(q, None if out_dtype is None else TORCH[out_dtype])
         code = {torch.float16: ref.F16, torch.bfloat16: ref.BF16, torch.float32: ref.F32}[out.dtype]
         return to_host(out), code
@@ -55,8 +56,9 @@ class HipBackend:
         q = nv.Quantized(to_dev(w), to_dev(scales), to_dev(biases), quant(mode, group, bits))
         return to_host(nv.quantized_matmul(to_dev(x), q, transpose))
 
-    def gather_qmm(self, x, w, scales, biases, lhs, rhs, mode, group, bits, dtype, transpose, sorted_indices):
-        q = nv.Quantized(to_dev(w), to_dev(scales), to_dev(biases), quant(mode, group, bits))
+    def gather_qmm(self, x, w, scales, biases, lhs, rhs, mode, group, bits, dtype, transpose, sorted_indices,
+                   global_scales=None):
+        q = nv.Quantized(to_dev(w), to_dev(scales), to_dev(biases), quant(mode, group, bits), to_dev(global_scales))
         idx = lambda i: None if i is None else torch.from_numpy(np.ascontiguousarray(i).astype(np.int64)).cuda()
         y = nv.gather_qmm(to_dev(x), q, idx(lhs), idx(rhs), nv.GatherQmm(transpose, sorted_indices))
         return to_host(y)

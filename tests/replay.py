@@ -30,20 +30,20 @@ class OracleBackend:
 
     name = "oracle"
 
-    def quantize(self, w, dtype, mode, group, bits):
+    def quantize(self, w, dtype, mode, group, bits, global_scale=None):
         if mode == ref.AFFINE:
             return ref.affine_quantize(w, dtype, group, bits)
-        packed, scales = ref.fp_quantize(w, dtype, mode)
+        packed, scales = ref.fp_quantize(w, dtype, mode, global_scale)
         return packed, scales, None
 
-    def dequantize(self, w, scales, biases, mode, group, bits, scales_dtype, out_dtype=None):
+    def dequantize(self, w, scales, biases, mode, group, bits, scales_dtype, out_dtype=None, global_scale=None):
         if mode == ref.AFFINE:
             out = ref.affine_dequantize(w, scales, biases, scales_dtype, group, bits)
             if out_dtype is not None and out_dtype != scales_dtype:
                 out = ref.from_f32(ref.to_f32(out, scales_dtype), out_dtype)
             return out, (out_dtype or scales_dtype)
         out_dtype = out_dtype or ref.BF16
-        return ref.fp_dequantize(w, scales, mode, out_dtype), out_dtype
+        return ref.fp_dequantize(w, scales, mode, out_dtype, global_scale), out_dtype
 
     def quantized_matmul(self, x, w, scales, biases, mode, group, bits, dtype, transpose):
         vector = x.ndim == 1
@@ -58,12 +58,18 @@ class OracleBackend:
                                  transpose=transpose)
         return y[..., 0, :] if vector else y
 
-    def gather_qmm(self, x, w, scales, biases, lhs, rhs, mode, group, bits, dtype, transpose, sorted_indices):
+    def gather_qmm(self, x, w, scales, biases, lhs, rhs, mode, group, bits, dtype, transpose, sorted_indices,
+                   global_scales=None):
         xb = int(np.prod(x.shape[:-2], dtype=np.int64))
         eb = int(np.prod(w.shape[:-2], dtype=np.int64))
         lhs = np.arange(xb, dtype=np.uint32).reshape(x.shape[:-2]) if lhs is None else lhs
         rhs = np.arange(eb, dtype=np.uint32).reshape(w.shape[:-2]) if rhs is None else rhs
         lhs, rhs = np.broadcast_arrays(lhs, rhs)
+        if global_scales is not None:  # quantized.rs:677-719: each pair against its expert's weights and scale
+            xf, wf, sf = (a.reshape((-1,) + a.shape[-2:]) for a in (x, w, scales))
+            outs = [ref.fp_quantized_matmul_scaled(xf[l], wf[r], sf[r], mode, dtype, float(global_scales.reshape(-1)[r]), transpose)
+                    for l, r in zip(lhs.reshape(-1), rhs.reshape(-1))]
+            return np.stack(outs).reshape(rhs.shape + outs[0].shape)
         return ref.gather_qmm(x, w, scales, biases, lhs, rhs, mode=mode, group=group, bits=bits, dtype=dtype,
                               transpose=transpose)
 
@@ -81,15 +87,21 @@ def run_case(case, backend):
             w = np.ascontiguousarray(np.swapaxes(w, -1, -2))
         elif p.get("pre") == "r":
             w = np.ascontiguousarray(w[..., ::-1])
-        packed, scales, biases = backend.quantize(w, DT[names[0]], mode, group, bits)
+        if p.get("gs") == "1":
+            packed, scales, biases = backend.quantize(w, DT[names[0]], mode, group, bits, global_scale=xs[1])
+        else:
+            packed, scales, biases = backend.quantize(w, DT[names[0]], mode, group, bits)
         out = [(packed, "u32"), (scales, names[0] if mode == ref.AFFINE else "u8")]
         if biases is not None:
             out.append((biases, names[0]))
         return out
     if case.op == "dequantize":
         out_dtype = int(p["dtype"]) if "dtype" in p else None
-        biases = xs[2] if len(xs) > 2 else None
         sdt = DT.get(names[1])
+        if p.get("gs") == "1":
+            out, code = backend.dequantize(xs[0], xs[1], None, mode, group, bits, sdt, out_dtype, global_scale=xs[2])
+            return [(out, ref_name(code))]
+        biases = xs[2] if len(xs) > 2 else None
         out, code = backend.dequantize(xs[0], xs[1], biases, mode, group, bits, sdt, out_dtype)
         return [(out, ref_name(code))]
     if case.op == "quantized_matmul":
@@ -98,11 +110,12 @@ def run_case(case, backend):
         return [(y, names[0])]
     if case.op == "gather_qmm":
         rest = list(xs[3:])
+        extra = {"global_scales": rest.pop(0)} if p.get("gs") == "1" else {}
         idx = p.get("idx", "")
         lhs = rest.pop(0) if "l" in idx else None
         rhs = rest.pop(0) if "r" in idx else None
         y = backend.gather_qmm(xs[0], xs[1], xs[2], None, lhs, rhs, mode, group, bits, DT[names[0]], transpose,
-                               p.get("sorted") == "1")
+                               p.get("sorted") == "1", **extra)
         return [(y, names[0])]
     raise KeyError(case.op)
 

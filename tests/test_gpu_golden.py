@@ -63,16 +63,26 @@ def test_affine_dequantize_equals_oracle_on_device_vectors(hip, golden_gpu):
 
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
 def test_fp_quantize_bits(hip, golden_gpu, mode):
-    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode]
+    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode and c.params.get("gs") != "1"]
     assert len(cases) == 18
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
 
 
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
 def test_fp_dequantize_bits(hip, golden_gpu, mode):
-    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode]
+    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode and c.params.get("gs") != "1"]
     assert len(cases) == 15
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+
+
+def test_nvfp4_global_scale(hip, golden_gpu):
+    """NVFP4 with a global scale: quantize and dequantize bit for bit, the gathers (one scale per expert) within FR-008."""
+    scaled = [c for c in golden_gpu[1] if c.params.get("gs") == "1"]
+    exact = [c for c in scaled if c.op in ("quantize", "dequantize")]
+    gathers = [c for c in scaled if c.op == "gather_qmm"]
+    assert len(exact) == 12 and len(gathers) >= 10
+    assert not _failures(exact, lambda c: replay.exact_bits(replay.run_case(c, hip), c.outputs))
+    assert not _failures(gathers, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
 
 
 def test_products_against_mlx_cpu(hip, golden_cpu):

@@ -438,6 +438,52 @@ def test_mxfp8_nvfp4_quantize_and_products(mode, qmode, dtype):
         assert float(np.max(ratio)) <= 1.0, f"{qmode} M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
+def test_nvfp4_global_scale(dtype):
+    """NVFP4 with a global scale (MLX's `quantize(..., global_scale=)`): codes, scales and dequantized values bit for
+    bit; the product of two matrices on the kernel and the shapes the reference multiplies densely, within the bar;
+    a gather with one scale per expert; the mode check."""
+    rng = np.random.default_rng(3300 + dtype)
+    n, k, g = 160, 1152, 3.25
+    w = make_w(rng, n, k, dtype)
+    gs = torch.tensor(g, dtype=torch.float32, device="cuda")
+    packed, scales = ref.fp_quantize(w, dtype, ref.NVFP4, g)
+    q = nv.quantize(to_dev(w), nv.QuantMode.NVFP4, gs)
+    assert q.global_scale is gs and q.biases is None
+    assert np.array_equal(to_host(q.weight), packed) and np.array_equal(to_host(q.scales), scales)
+    assert not np.array_equal(scales, ref.fp_quantize(w, dtype, ref.NVFP4)[1])  # the scale does change the codes
+    for out in (ref.BF16, ref.F32, ref.F16):
+        want = ref.fp_dequantize(packed, scales, ref.NVFP4, out, g)
+        assert np.array_equal(to_host(nv.dequantize(q, TORCH[out])).view(np.uint8), want.view(np.uint8))
+    for m in (1, 5, 40):
+        x = make_x(rng, m, k, dtype)
+        want = ref.fp_quantized_matmul_scaled(x, packed, scales, ref.NVFP4, dtype, g)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        ratio = _excess(got, want, dtype)
+        assert float(np.max(ratio)) <= 1.0, f"M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
+    # a batch of x: the reference dequantizes in x's type and multiplies densely (quantized.rs:481-491); so does the mirror
+    xb = make_x(rng, 6, k, dtype).reshape(2, 3, k)
+    got = to_host(nv.quantized_matmul(to_dev(xb), q)).reshape(6, n)
+    want = ref.fp_quantized_matmul_scaled(xb.reshape(6, k), packed, scales, ref.NVFP4, dtype, g)
+    assert float(np.max(_excess(got, want, dtype))) <= 2.0
+    # stacked experts, one scale each
+    experts, pairs = 3, 7
+    we = make_w(rng, experts * 64, 256, dtype).reshape(experts, 64, 256)
+    ge = np.array([0.5, 2.0, 7.5], np.float32)
+    pe, se = zip(*(ref.fp_quantize(we[e], dtype, ref.NVFP4, float(ge[e])) for e in range(experts)))
+    qe = nv.Quantized(to_dev(np.stack(pe)), to_dev(np.stack(se)), None, nv.Quant.new(nv.QuantMode.NVFP4), to_dev(ge))
+    xe = make_x(rng, pairs, 256, dtype).reshape(pairs, 1, 256)
+    rhs = rng.integers(0, experts, pairs)
+    got = to_host(nv.gather_qmm(to_dev(xe), qe, None, torch.from_numpy(rhs).cuda()))
+    for i in range(pairs):
+        want = ref.fp_quantized_matmul_scaled(xe[i], pe[rhs[i]], se[rhs[i]], ref.NVFP4, dtype, float(ge[rhs[i]]))
+        assert float(np.max(_excess(got[i], want, dtype))) <= 1.0, f"pair {i}"
+    with pytest.raises(nv.InvalidArgument):
+        nv.quantize(to_dev(w), nv.QuantMode.MXFP4, gs)
+    with pytest.raises(nv.InvalidArgument):
+        nv.quantize(to_dev(w), nv.QuantMode.NVFP4, torch.ones(2, device="cuda"))
+
+
 @pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
 @pytest.mark.parametrize("group,bits", [(64, 4), (32, 2), (128, 6), (64, 5), (128, 1), (32, 3), (64, 8)])
 def test_untransposed_products_every_width(dtype, group, bits):

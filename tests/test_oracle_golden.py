@@ -27,7 +27,7 @@ def test_fixture_meta(golden_cpu, golden_gpu):
     assert len(cases) == 135
     meta, cases = golden_gpu
     assert "mlx=0.32.4" in meta and "device=gpu" in meta
-    assert len(cases) == 276
+    assert len(cases) == 303
 
 
 def test_affine_quantize_bits(golden_cpu):
@@ -73,16 +73,27 @@ def test_affine_dequantize_device_vectors(golden_gpu):
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
 def test_fp_quantize_bits(golden_gpu, mode):
     """18 cases per format incl. NaN/Inf/subnormal/signed-zero edges, transposed and reversed inputs."""
-    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode]
+    cases = [c for c in golden_gpu[1] if c.op == "quantize" and c.params.get("mode") == mode and c.params.get("gs") != "1"]
     assert len(cases) == 18
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
 
 
 @pytest.mark.parametrize("mode", ["mxfp4", "mxfp8", "nvfp4"])
 def test_fp_dequantize_bits(golden_gpu, mode):
-    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode]
+    cases = [c for c in golden_gpu[1] if c.op == "dequantize" and c.params.get("mode") == mode and c.params.get("gs") != "1"]
     assert len(cases) == 15
     assert not _failures(cases, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
+
+
+def test_nvfp4_global_scale(golden_gpu):
+    """NVFP4 with a global scale (kernels.rs:914-1009 with `g`): 6 quantize and 6 dequantize cases bit for bit, the
+    gathers with one scale per expert within FR-008."""
+    scaled = [c for c in golden_gpu[1] if c.params.get("gs") == "1"]
+    exact = [c for c in scaled if c.op in ("quantize", "dequantize")]
+    gathers = [c for c in scaled if c.op == "gather_qmm"]
+    assert len(exact) == 12 and len(gathers) >= 10
+    assert not _failures(exact, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
+    assert not _failures(gathers, lambda c: replay.within_fr008(replay.run_case(c, ORACLE), c.outputs))
 
 
 def test_products_against_mlx_cpu(golden_cpu):
