@@ -248,11 +248,13 @@ NVQ_API int32_t nvq_moe_route(int32_t dtype, const void *probs, int64_t rows, in
 NVQ_API int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out,
                          void *stream);
 
+/* Bytes of float32 partial sums nvq_gather_qmm wants in `workspace`: with the weights stored [K, N] (transpose = 0) K is
+ * split over the grid (the reference's split-K scratch, gpu.rs:7562); 0 for transposed weights. */
 NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);
 
 /* GpuEval::gather_qmm / fp_gather_qmm (gpu.rs:7174-7294, 6758-6876); values of the gathered
- * products of quantized::gather_qmm_graph (quantized.rs:679-719).
- * `offsets` NULL = one product per pair; non-NULL = grouped route (see nvq_gather_desc). */
+ * products of quantized::gather_qmm_graph (quantized.rs:679-719), both weight orientations.
+ * `offsets` NULL = one product per pair; non-NULL = grouped route (see nvq_gather_desc; transposed weights only). */
 NVQ_API int32_t nvq_gather_qmm(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
                        const void *biases, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
                        void *y, void *workspace, void *stream);

@@ -397,7 +397,16 @@ int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int
     return launch_sorted_offsets(indices, rows, m, groups, offsets, (hipStream_t)stream);
 }
 
-size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *) { return 0; }
+// float32 partial sums when the weights are stored [K, N] and K is split over the grid; nothing otherwise.
+size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *d) {
+    if (d == nullptr || d->transpose || check_quant(&d->quant, "gather_qmm") != NVQ_OK) return 0;
+    if (d->pairs <= 0 || d->m <= 0 || d->n <= 0 || d->k <= 0 || require_device() != NVQ_OK) return 0;
+    ProductArgs a{};
+    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
+    a.m = d->m; a.n = d->n; a.k = d->k;
+    a.batch = d->pairs;
+    return qvm_workspace_bytes(a);
+}
 
 int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32_t dtype, const uint32_t *qweight, const uint32_t *qzeros,
                            const void *scales, int64_t rows, int64_t cols, uint32_t *weight, void *scales_out, void *biases_out,
@@ -463,7 +472,6 @@ int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t ro
 static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                               const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y,
                               void *workspace, void *stream) {
-    (void)workspace;
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
     NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
     NVQ_TRY(check_groups("gather_qmm", d->quant.mode, biases));
@@ -474,8 +482,8 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr || lhs == nullptr || rhs == nullptr)
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null operand");
     NVQ_TRY(require_device());
-    if (!d->transpose)
-        return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for mode %s, transpose=%d", mode_name(d->quant.mode), d->transpose);
+    if (!d->transpose && global_scale != nullptr)
+        return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for untransposed weights with a global scale");
     NVQ_TRY(check_aligned("gather_qmm", "x", x));
     NVQ_TRY(check_aligned("gather_qmm", "w", w));
     NVQ_TRY(check_aligned("gather_qmm", "y", y));
@@ -490,6 +498,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.lhs = lhs; a.rhs = rhs;
     a.x_batches = d->x_batches; a.experts = d->experts;
     a.global_scale = global_scale;
+    if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;

@@ -48,6 +48,13 @@ struct Offsets { int64_t x, w, s, y; };
 // Element offsets of batch `z` for x, w (packed dwords), scales/biases and y (in units of M*N).
 __device__ __forceinline__ Offsets batch_offsets(const ProductArgs &a, int64_t z) {
     Offsets o{0, 0, 0, z};
+    if (a.rhs != nullptr) {  // gathered pairs; an index outside its operand is the caller's error and is clamped
+        const int64_t l = min((int64_t)a.lhs[z], a.x_batches - 1), r = min((int64_t)a.rhs[z], a.experts - 1);
+        o.x = l * a.m * a.k;
+        o.w = r * a.k * (a.n * a.bits / 32);
+        o.s = r * a.k * (a.n / a.group);
+        return o;
+    }
     if (a.batch_ndim == 0) return o;
     int64_t rest = z;
 #pragma unroll

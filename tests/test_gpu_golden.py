@@ -21,8 +21,8 @@ def hip():
 
 
 def _supported(c):
-    """Gathered products with the weights stored [K, N] (transpose=0) are refused by the backend."""
-    return c.op != "gather_qmm" or c.params.get("transpose", "1") == "1"
+    """Every recorded case of the path has a kernel (gathers with the weights stored [K, N] included)."""
+    return True
 
 
 def _failures(cases, check):
@@ -101,14 +101,3 @@ def test_gathers_against_mlx_gpu(hip, golden_gpu):
     cases = [c for c in golden_gpu[1] if c.op == "gather_qmm" and _supported(c)]
     assert len(cases) >= 12
     assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
-
-
-def test_untransposed_gathers_are_refused_not_faked(hip, golden_gpu):
-    """gather_qmm with weights stored [K, N] has no gfx950 kernel yet: the backend must say so (the caller
-    then takes its CPU path) instead of answering from anywhere else."""
-    import nuvec_amd as nv
-    cases = [c for c in golden_gpu[1] if c.op == "gather_qmm" and c.params.get("transpose", "1") == "0"]
-    if not cases:
-        pytest.skip("no untransposed gather among the committed vectors")
-    with pytest.raises(nv.Unsupported):
-        replay.run_case(cases[0], hip)

@@ -478,6 +478,8 @@ def test_nvfp4_global_scale(dtype):
     for i in range(pairs):
         want = ref.fp_quantized_matmul_scaled(xe[i], pe[rhs[i]], se[rhs[i]], ref.NVFP4, dtype, float(ge[rhs[i]]))
         assert float(np.max(_excess(got[i], want, dtype))) <= 1.0, f"pair {i}"
+    with pytest.raises(nv.Unsupported):  # untransposed weights with a global scale: no kernel, and nothing else answers
+        nv.gather_qmm(to_dev(xe[:, :, :64]), qe, None, torch.from_numpy(rhs).cuda(), nv.GatherQmm(transpose=False))
     with pytest.raises(nv.InvalidArgument):
         nv.quantize(to_dev(w), nv.QuantMode.MXFP4, gs)
     with pytest.raises(nv.InvalidArgument):
@@ -746,3 +748,30 @@ def test_moe_block_routes_multiplies_and_sums():
     outputs = glu(x, top)  # [B, L, k, D]
     want = moe.weighted_sum(to_host(outputs).reshape(b * l, k, d), to_host(scores).reshape(b * l, k), ref.BF16)
     assert np.array_equal(to_host(y).reshape(b * l, d).view(np.uint8), want.view(np.uint8))
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.AFFINE, None), (ref.MXFP4, "MXFP4"), (ref.NVFP4, "NVFP4")])
+def test_untransposed_gathers(mode, qmode):
+    """gather_qmm with the weights stored [K, N] (transpose=False): one product per pair, K split over the grid or not,
+    one row and a few rows of x per pair, against the oracle's per-pair products."""
+    rng = np.random.default_rng(5100 + mode)
+    dtype = ref.BF16
+    experts, pairs = 4, 9
+    for m, k, n in [(1, 320, 256), (3, 2048, 384)]:
+        w = make_w(rng, experts * k, n, dtype).reshape(experts, k, n)  # quantized along N
+        if mode == ref.AFFINE:
+            group, bits = 64, 4
+            packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+            q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+        else:
+            group, bits = ref.FP_PARAMS[mode]
+            packed, scales = ref.fp_quantize(w, dtype, mode)
+            biases = None
+            q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+        x = make_x(rng, pairs * m, k, dtype).reshape(pairs, m, k)
+        lhs, rhs = rng.permutation(pairs), rng.integers(0, experts, pairs)
+        got = to_host(nv.gather_qmm(to_dev(x), q, torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), nv.GatherQmm(transpose=False)))
+        assert got.shape == (pairs, m, n)
+        want = ref.gather_qmm(x, packed, scales, biases, lhs.astype(np.uint32), rhs.astype(np.uint32), mode=mode, group=group, bits=bits,
+                              dtype=dtype, transpose=False)
+        assert_rows_close(got.reshape(pairs * m, n), want.reshape(pairs * m, n), dtype, f"untransposed gather mode {mode} M={m} K={k} N={n}")
