@@ -231,6 +231,13 @@ NVQ_API int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *desc, const void *x
                               const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
                               void *y, void *workspace, void *stream);
 
+/* FastOp::QuantizeDequantize (crates/nuvec-core/src/products.rs:307-315, kernels.rs:1011-1065; MLX's
+ * fp_quantize_dequantize): x through its quantization in a floating-point mode, i.e. the values the codes represent,
+ * in x's dtype: the activations of `qqmm` / `gather_qqmm` (products.rs:333-470), which then take
+ * nvq_quantized_matmul(_scaled) / nvq_gather_qmm(_scaled).  `global_scale`: NULL, or NVFP4's one float32 value. */
+NVQ_API int32_t nvq_quantize_dequantize(const nvq_quant *quant, int32_t dtype, const void *x, int64_t rows, int64_t cols,
+                                const float *global_scale, void *out, void *stream);
+
 /* fast::moe_route (crates/nuvec-core/src/fast.rs:740-746, fast/imp.rs:2652-2673; kernel
  * crates/nuvec-kernels/src/metal/moe.metal:33-88): per row of `experts` router probabilities the k largest in the
  * stable ascending order of the sort (NaN last for float32 and half), i.e. the last k of `argsort`, their values

@@ -6,5 +6,5 @@ nuvec-nn's `QuantizedEmbedding` as `embedding`; `moe_order`, `moe_route` and `we
 nuvec-lm's mixture-of-experts blocks around the gathered products.
 """
 from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, embedding,  # noqa: F401
-                  gather_qmm, gather_qmm_grouped, moe_order, moe_route, quantize, quantized_matmul, sorted_offsets,
-                  weighted_sum)
+                  gather_qmm, gather_qmm_grouped, gather_qqmm, moe_order, moe_route, qqmm, quantize, quantize_dequantize,
+                  quantized_matmul, sorted_offsets, weighted_sum)

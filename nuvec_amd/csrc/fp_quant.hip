@@ -242,6 +242,47 @@ template <typename T> __device__ __forceinline__ void store_values(T *out, int64
     }
 }
 
+// kernels.rs:1011-1065 (MLX's fp_quantize_dequantize, the activations of `qqmm`): per group the scale as the quantizer
+// encodes it, each value (scale / scale_enc) * float(code) in float32 and one rounding to the input's type.  The
+// reference's arithmetic step by step (the scaled conversions would need the same edge handling as the quantizer for
+// what is a small operand: the activations of one product).
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock)
+fp_quantize_dequantize_kernel(const T *__restrict__ w, int64_t chunks, T *__restrict__ out, const float *__restrict__ global_scale) {
+    using F = Format<MODE>;
+    const int64_t chunk = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (chunk >= chunks) return;  // a group is wholly in or out of range
+    const Raw<T> raw = load_raw<T>(w, chunk);
+    float v[8];
+    widen_raw<T>(raw, v);
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        v[i] = ftz(v[i]);
+        amax = fmaxf(amax, fabsf(v[i]));
+    }
+    amax = fmaxf(amax, u2f(quad_swap<kSwap1>(f2u(amax))));
+    if constexpr (F::lanes == 4) amax = fmaxf(amax, u2f(quad_swap<kSwap2>(f2u(amax))));
+    float scale = ftz(amax / F::max_element);
+    const bool scaled = global_scale != nullptr;
+    const float scale_enc = scaled ? ftz(448.0f * 6.0f / *global_scale) : 1.0f;
+    if (scaled) scale = ftz(scale * scale_enc);
+    float decoded;
+    if (F::mx && !scaled) decoded = e8m0_to_f32(e8m0_round_up_code(scale));
+    else decoded = e4m3_to_f32(e4m3_from_f32(scale));
+    decoded = ftz(decoded);
+    const float enc_b = decoded == 0.0f ? 0.0f : ftz(scale_enc / decoded);
+    const float dec = ftz(decoded / scale_enc);
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float t = canonical(ftz(v[i] * enc_b));
+        const float value = F::bits == 8 ? e4m3_to_f32(e4m3_from_f32(t)) : e2m1_to_f32(e2m1_from_f32(t));
+        r[i] = canonical(ftz(dec * value));
+    }
+    store_values<T>(out, chunk * 8, r);
+}
+
 // kernels.rs:976-1009 without a global scale.  With `ids`, output row r is table row ids[r] (`row_chunks` chunks
 // per row, ids clamped to `table_rows`): the rows of a quantized embedding.
 template <typename T, int MODE>
@@ -323,6 +364,23 @@ int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *ou
     return NVQ_OK;
 }
 
+template <typename T, int MODE>
+int32_t quantize_dequantize_t(const void *w, int64_t n, void *out, const float *g, hipStream_t s) {
+    const int64_t chunks = n / 8;
+    const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL((fp_quantize_dequantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const T *)w, chunks, (T *)out, g);
+    NVQ_LAUNCH_CHECK("fp_quantize_dequantize");
+    return NVQ_OK;
+}
+template <typename T>
+int32_t quantize_dequantize_mode(int32_t mode, const void *w, int64_t n, void *out, const float *g, hipStream_t s) {
+    switch (mode) {
+    case NVQ_MXFP4: return quantize_dequantize_t<T, NVQ_MXFP4>(w, n, out, g, s);
+    case NVQ_MXFP8: return quantize_dequantize_t<T, NVQ_MXFP8>(w, n, out, g, s);
+    case NVQ_NVFP4: return quantize_dequantize_t<T, NVQ_NVFP4>(w, n, out, g, s);
+    default: return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: mode %s is not a floating-point block format", mode_name(mode));
+    }
+}
 template <typename T>
 int32_t quantize_mode(int32_t mode, const void *w, int64_t n, void *packed, void *scales, const float *g, hipStream_t s) {
     switch (mode) {
@@ -351,6 +409,14 @@ int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n
     case NVQ_F32: return quantize_mode<float>(mode, w, n, packed, scales, g, s);
     case NVQ_BF16: return quantize_mode<bf16_t>(mode, w, n, packed, scales, g, s);
     default: return quantize_mode<f16_t>(mode, w, n, packed, scales, g, s);
+    }
+}
+
+int32_t launch_fp_quantize_dequantize(int32_t mode, int32_t dtype, const void *w, int64_t n, void *out, const float *g, hipStream_t s) {
+    switch (dtype) {
+    case NVQ_F32: return quantize_dequantize_mode<float>(mode, w, n, out, g, s);
+    case NVQ_BF16: return quantize_dequantize_mode<bf16_t>(mode, w, n, out, g, s);
+    default: return quantize_dequantize_mode<f16_t>(mode, w, n, out, g, s);
     }
 }
 

@@ -257,6 +257,25 @@ int32_t nvq_quantize_scaled(const nvq_quant *quant, int32_t dtype, const void *w
     return quantize_any(quant, dtype, w, rows, cols, packed, scales, nullptr, global_scale, stream);
 }
 
+int32_t nvq_quantize_dequantize(const nvq_quant *quant, int32_t dtype, const void *x, int64_t rows, int64_t cols,
+                                const float *global_scale, void *out, void *stream) {
+    NVQ_TRY(check_quant(quant, "quantize_dequantize"));
+    if (quant->mode == NVQ_AFFINE)  // products.rs:263-289: qqmm quantizes in a floating-point mode
+        return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: mode affine is not a floating-point block format");
+    if (global_scale != nullptr) NVQ_TRY(check_global_scale("quantize_dequantize", quant, global_scale));
+    if (!float_dtype(dtype)) return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: unsupported dtype %s", dtype_name(dtype));
+    if (rows < 0 || cols < 0 || cols % quant->group_size != 0)
+        return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: the last dimension %lld is not whole groups of %d", (long long)cols,
+                    quant->group_size);
+    if (rows == 0 || cols == 0) return NVQ_OK;
+    if (x == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: null operand");
+    if (rows * cols >= (1LL << 32)) return fail(NVQ_INVALID_ARGUMENT, "quantize_dequantize: an operand holds fewer than 2^32 elements");
+    NVQ_TRY(require_device());
+    NVQ_TRY(check_aligned("quantize_dequantize", "x", x));
+    NVQ_TRY(check_aligned("quantize_dequantize", "out", out));
+    return launch_fp_quantize_dequantize(quant->mode, dtype, x, rows * cols, out, global_scale, (hipStream_t)stream);
+}
+
 // Shared by nvq_dequantize and nvq_dequantize_rows: `count` output rows, each table row ids[r] (or row r).
 static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dtype, const void *packed, const void *scales,
                               const void *biases, int64_t table_rows, int64_t cols, const uint32_t *ids, int64_t count,

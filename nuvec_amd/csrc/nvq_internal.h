@@ -46,6 +46,8 @@ int32_t launch_affine_dequantize(int32_t dtype, int group, int bits, const void 
 // `global_scale`: NULL, or NVFP4's one float32 value on the device
 int32_t launch_fp_quantize(int32_t mode, int32_t dtype, const void *w, int64_t n_values, void *packed,
                            void *scales, const float *global_scale, hipStream_t s);
+int32_t launch_fp_quantize_dequantize(int32_t mode, int32_t dtype, const void *w, int64_t n_values, void *out,
+                                      const float *global_scale, hipStream_t s);
 int32_t launch_fp_dequantize(int32_t mode, int32_t out_dtype, const void *packed, const void *scales,
                              int64_t n_values, void *out, const uint32_t *ids, int64_t cols, int64_t table_rows,
                              const float *global_scale, hipStream_t s);

@@ -237,6 +237,67 @@ def dequantize(q: Quantized, dtype: Optional[torch.dtype] = None) -> torch.Tenso
     return out
 
 
+def quantize_dequantize(x: torch.Tensor, quant: Quant | QuantMode, global_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """products.rs:307-315 (`fake_quant`, MLX's `fp_quantize_dequantize`): `x` through its quantization in a
+    floating-point mode, in x's dtype."""
+    quant = Quant.new(quant) if isinstance(quant, QuantMode) else quant
+    group, _ = quant.checked("quantize_dequantize")
+    if quant.mode == QuantMode.AFFINE:
+        raise InvalidArgument("quantize_dequantize: mode affine is not a floating-point block format")
+    if x.dtype not in _FLOATS:
+        raise InvalidArgument(f"quantize_dequantize: unsupported dtype {_name(x.dtype)}")
+    if x.ndim < 1 or x.shape[-1] % group != 0:
+        raise InvalidArgument(f"quantize_dequantize: the last dimension of {list(x.shape)} is not whole groups of {group}")
+    _init(x)
+    x = x.contiguous()
+    g = _global_scale("quantize_dequantize", quant, global_scale, x.device)
+    out = torch.empty_like(x)
+    last = x.shape[-1]
+    _lib.check(_lib.load().nvq_quantize_dequantize(C.byref(quant._c()), _CODE[x.dtype], _ptr(x), x.numel() // last if last else 0, last,
+                                                   _ptr(g), _ptr(out), _stream()))
+    return out
+
+
+def _qq_weight(op: str, w, quant, global_scale_x):
+    """products.rs:317-330, 431-462: the weight of `qqmm` / `gather_qqmm` as a `Quantized` in a floating-point mode (a
+    dense weight is quantized for the product), and MLX's rule: NVFP4 global scales for both operands or neither."""
+    if isinstance(w, Quantized):
+        q = w
+    else:
+        quant = Quant.new(quant) if isinstance(quant, QuantMode) else quant
+        if quant is None:
+            raise InvalidArgument(f"{op}: a dense weight needs the mode to quantize it in")
+        q = quantize(w, quant)
+    if q.quant.mode == QuantMode.AFFINE:
+        raise InvalidArgument(f"{op}: both operands are quantized in a floating-point mode, got affine")
+    if (global_scale_x is None) != (q.global_scale is None):
+        raise InvalidArgument(f"{op}: for nvfp4, give global scales for both the activations and the weight, or neither")
+    return q
+
+
+def qqmm(x: torch.Tensor, w, quant=None, global_scale_x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """products.rs:333-429 (MLX's `qqmm`, forward): `x` (`[..., K]`) times `w^T` (`[N, K]`) with both quantized in a
+    floating-point mode.  `w` is a `Quantized` or a dense weight (quantized here in `quant`; with NVFP4 global scales
+    pass `quantize(w, NVFP4, gw)`)."""
+    q = _qq_weight("qqmm", w, quant, global_scale_x)
+    if x.ndim == 0:
+        raise InvalidArgument("qqmm: the activation needs at least one dimension")
+    x2 = x.reshape(-1, x.shape[-1])
+    y = quantized_matmul(quantize_dequantize(x2, q.quant, global_scale_x), q, True)
+    return y.reshape(x.shape[:-1] + (y.shape[-1],))
+
+
+def gather_qqmm(x: torch.Tensor, w, lhs_indices=None, rhs_indices=None, sorted_indices: bool = False, quant=None,
+                global_scale_x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """products.rs:431-470 (MLX's `gather_qqmm`): `gather_qmm` of the quantized activations with quantized experts
+    (`w [E, N, K]`), transposed; the weight's one global scale serves every expert."""
+    q = _qq_weight("gather_qqmm", w, quant, global_scale_x)
+    if q.global_scale is not None and q.global_scale.numel() == 1:
+        q = q.with_global_scale(q.global_scale.reshape(()).expand(q.weight.shape[:-2]).contiguous())
+    xq = quantize_dequantize(x, q.quant, global_scale_x)
+    return gather_qmm(xq, q, lhs_indices, rhs_indices, GatherQmm(True, sorted_indices))
+
+
 def embedding(q: Quantized, ids: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """nuvec-nn layers.rs:245-255 (`QuantizedEmbedding::forward`): the rows `ids` of a quantized table,
     dequantized; shape `ids.shape + [cols]`.  Equals `dequantize` of the taken rows bit for bit."""

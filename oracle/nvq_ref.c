@@ -409,6 +409,42 @@ NVQ_EXPORT int nvq_ref_fp_dequantize_scaled(const uint32_t *packed, const uint8_
     return fp_dequantize_impl(packed, scales, n, mode, out_dtype, &g, out);
 }
 
+/* kernels.rs:1011-1065 (MLX's fp_quantize_dequantize, qqmm's activations): per group the scale as the quantizer
+ * encodes it, the values (scale / scale_enc) * float(code) in float32, one rounding to the input's dtype.
+ * `g` NULL = no global scale. */
+static int fp_quantize_dequantize_impl(const void *w, int dtype, int64_t n, int mode, const float *g, void *out) {
+    int group, bits;
+    if (!dtype_ok(dtype) || !fp_mode_ok(mode, &group, &bits) || n % group) return 1;
+    const int mx = group == 32;
+    const float max_element = bits == 4 ? E2M1_MAX : E4M3_MAX;
+    const float scale_enc = g ? nvq_ref_ftz(E4M3_MAX * E2M1_MAX / *g) : 1.0f;
+    for (int64_t gi = 0; gi < n / group; gi++) {
+        float amax = 0.0f;
+        for (int j = 0; j < group; j++)
+            amax = rs_max(amax, fabsf(nvq_ref_ftz(load_f32(w, gi * group + j, dtype))));
+        float scale = nvq_ref_ftz(amax / max_element);
+        if (g) scale = nvq_ref_ftz(scale * scale_enc);
+        float decoded = nvq_ref_ftz(mx && !g ? nvq_ref_e8m0_to_f32(nvq_ref_e8m0_from_f32(nvq_ref_mx_scale_round_up(scale)))
+                                              : nvq_ref_e4m3_to_f32(nvq_ref_e4m3_from_f32(scale)));
+        float enc_b = decoded == 0.0f ? 0.0f : nvq_ref_ftz(scale_enc / decoded);
+        float dec = nvq_ref_ftz(decoded / scale_enc);
+        for (int j = 0; j < group; j++) {
+            int64_t i = gi * group + j;
+            float scaled = nvq_ref_canonical(nvq_ref_ftz(nvq_ref_ftz(load_f32(w, i, dtype)) * enc_b));
+            float value = bits == 8 ? nvq_ref_e4m3_to_f32(nvq_ref_e4m3_from_f32(scaled))
+                                    : nvq_ref_e2m1_to_f32(nvq_ref_e2m1_from_f32(scaled));
+            store_rounded(out, i, dtype, (double)nvq_ref_canonical(nvq_ref_ftz(dec * value)));
+        }
+    }
+    return 0;
+}
+NVQ_EXPORT int nvq_ref_fp_quantize_dequantize(const void *w, int dtype, int64_t n, int mode, void *out) {
+    return fp_quantize_dequantize_impl(w, dtype, n, mode, NULL, out);
+}
+NVQ_EXPORT int nvq_ref_fp_quantize_dequantize_scaled(const void *w, int dtype, int64_t n, int mode, float g, void *out) {
+    return fp_quantize_dequantize_impl(w, dtype, n, mode, &g, out);
+}
+
 /* ── sorted offsets (kernels.rs:873-892) ─────────────────────────────────────────── */
 
 NVQ_EXPORT int nvq_ref_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups,

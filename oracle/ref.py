@@ -149,6 +149,44 @@ def fp_dequantize(packed, scales, mode: int, out_dtype: int, global_scale=None):
     return out
 
 
+def fp_quantize_dequantize(x, dtype: int, mode: int, global_scale=None):
+    """kernels.rs:1011-1065: the values the quantization of `x` represents, in x's dtype (`qqmm`'s activations)."""
+    x = _c(x)
+    out = np.zeros(x.shape, NP_OF[dtype])
+    if global_scale is None:
+        rc = lib().nvq_ref_fp_quantize_dequantize(_p(x), dtype, C.c_int64(x.size), mode, _p(out))
+    else:
+        rc = lib().nvq_ref_fp_quantize_dequantize_scaled(_p(x), dtype, C.c_int64(x.size), mode, C.c_float(float(global_scale)), _p(out))
+    _check(rc, "fp_quantize_dequantize")
+    return out
+
+
+def qqmm(x, w, dtype: int, mode: int, gx=None, gw=None):
+    """products.rs:333-345, 354-367 (`qqmm` of a 2-D activation, forward): x through its quantization times the
+    quantized weight, transposed.  `w` is the dense weight [N, K]; `gx`, `gw` NVFP4's global scales (both or neither)."""
+    packed, scales = fp_quantize(w, dtype, mode, gw)
+    xq = fp_quantize_dequantize(x, dtype, mode, gx)
+    group, bits = FP_PARAMS[mode]
+    if gw is None:
+        return quantized_matmul(xq, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype)
+    return fp_quantized_matmul_scaled(xq, packed, scales, mode, dtype, gw)
+
+
+def gather_qqmm(x, w, rhs, dtype: int, mode: int, gx=None, gw=None):
+    """products.rs:431-470: `gather_qmm` of the quantized activations x [B, M, K] with the quantized experts w [E, N, K],
+    pair i against expert rhs[i]; the weight's one global scale serves every expert."""
+    xq = fp_quantize_dequantize(x, dtype, mode, gx)
+    return np.stack([qqmm_pair(xq[i], w[int(r)], dtype, mode, gw) for i, r in enumerate(np.asarray(rhs).reshape(-1))])
+
+
+def qqmm_pair(xq, w, dtype: int, mode: int, gw=None):
+    packed, scales = fp_quantize(w, dtype, mode, gw)
+    group, bits = FP_PARAMS[mode]
+    if gw is None:
+        return quantized_matmul(xq, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype)
+    return fp_quantized_matmul_scaled(xq, packed, scales, mode, dtype, gw)
+
+
 def dense_matmul(x, dense, dtype: int, transpose: bool = True, threads: int = 1):
     """x [M, K] times an already dequantized float32 matrix ([N, K] if transpose else [K, N]), rounded once to
     `dtype`: the product step of kernels.rs:1112-1142 (weights dequantized with a global scale go this way)."""

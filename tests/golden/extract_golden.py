@@ -22,7 +22,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(HERE, "..", ".."))
 from oracle import bsmxfix  # noqa: E402
 
-PATH_OPS = ("quantize", "dequantize", "quantized_matmul", "gather_qmm")
+PATH_OPS = ("quantize", "dequantize", "quantized_matmul", "gather_qmm", "qqmm", "gather_qqmm")
 
 
 def in_scope(case) -> bool:

@@ -62,3 +62,18 @@ class HipBackend:
         idx = lambda i: None if i is None else torch.from_numpy(np.ascontiguousarray(i).astype(np.int64)).cuda()
         y = nv.gather_qmm(to_dev(x), q, idx(lhs), idx(rhs), nv.GatherQmm(transpose, sorted_indices))
         return to_host(y)
+
+    def _qq_weight(self, w, mode, gw, prequantized):
+        qm = nv.Quant.new(nv.QuantMode(mode))
+        if prequantized or gw is not None:  # a dense weight with a global scale is quantized with it for the product
+            return nv.quantize(to_dev(w), qm, None if gw is None else to_dev(np.asarray(gw))), None
+        return to_dev(w), qm
+
+    def qqmm(self, x, w, dtype, mode, gx, gw, prequantized):
+        weight, qm = self._qq_weight(w, mode, gw, prequantized)
+        return to_host(nv.qqmm(to_dev(x), weight, qm, None if gx is None else to_dev(np.asarray(gx))))
+
+    def gather_qqmm(self, x, w, rhs, dtype, mode, gx, gw, prequantized):
+        weight, qm = self._qq_weight(w, mode, gw, prequantized)
+        idx = torch.from_numpy(np.ascontiguousarray(rhs).astype(np.int64)).cuda()
+        return to_host(nv.gather_qqmm(to_dev(x), weight, None, idx, False, qm, None if gx is None else to_dev(np.asarray(gx))))

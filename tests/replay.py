@@ -58,6 +58,14 @@ class OracleBackend:
                                  transpose=transpose)
         return y[..., 0, :] if vector else y
 
+    def qqmm(self, x, w, dtype, mode, gx, gw, prequantized):
+        f = lambda g: None if g is None else float(g)
+        return ref.qqmm(x, w, dtype, mode, f(gx), f(gw))
+
+    def gather_qqmm(self, x, w, rhs, dtype, mode, gx, gw, prequantized):
+        f = lambda g: None if g is None else float(g)
+        return ref.gather_qqmm(x, w, rhs, dtype, mode, f(gx), f(gw))
+
     def gather_qmm(self, x, w, scales, biases, lhs, rhs, mode, group, bits, dtype, transpose, sorted_indices,
                    global_scales=None):
         xb = int(np.prod(x.shape[:-2], dtype=np.int64))
@@ -74,6 +82,19 @@ class OracleBackend:
                               transpose=transpose)
 
 
+def _run_qq(case, backend, xs, names, mode):
+    """fixture.rs:789-819: with `gs=1` the last two inputs are the activations' and the weight's global scales;
+    `q=1` hands the weight over quantized, `q=0` dense (quantized for the product): the same values."""
+    gx = gw = None
+    if case.params.get("gs") == "1":
+        gx, gw = xs[-2], xs[-1]
+        xs = xs[:-2]
+    dtype = DT[names[0]]
+    if case.op == "qqmm":
+        return [(backend.qqmm(xs[0], xs[1], dtype, mode, gx, gw, case.params.get("q") == "1"), names[0])]
+    return [(backend.gather_qqmm(xs[0], xs[1], xs[2], dtype, mode, gx, gw, case.params.get("q") == "1"), names[0])]
+
+
 def run_case(case, backend):
     """The case's outputs from `backend`: a list of (array, dtype_name)."""
     p = case.params
@@ -81,6 +102,8 @@ def run_case(case, backend):
     names = [t.dtype for t in case.inputs]
     mode, group, bits = quant_of(case)
     transpose = p.get("transpose", "1") == "1"
+    if case.op in ("qqmm", "gather_qqmm"):
+        return _run_qq(case, backend, xs, names, mode)
     if case.op == "quantize":
         w = xs[0]
         if p.get("pre") == "t":

@@ -85,6 +85,13 @@ def test_nvfp4_global_scale(hip, golden_gpu):
     assert not _failures(gathers, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
 
 
+def test_qqmm_against_mlx_gpu(hip, golden_gpu):
+    """`qqmm` and `gather_qqmm`: the activations through nvq_quantize_dequantize, then the quantized products."""
+    cases = [c for c in golden_gpu[1] if c.op in ("qqmm", "gather_qqmm")]
+    assert len(cases) == 64
+    assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, hip), c.outputs))
+
+
 def test_products_against_mlx_cpu(hip, golden_cpu):
     cases = [c for c in golden_cpu[1] if c.op == "quantized_matmul" and _supported(c)]
     assert len(cases) >= 20

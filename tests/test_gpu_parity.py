@@ -775,3 +775,37 @@ def test_untransposed_gathers(mode, qmode):
         want = ref.gather_qmm(x, packed, scales, biases, lhs.astype(np.uint32), rhs.astype(np.uint32), mode=mode, group=group, bits=bits,
                               dtype=dtype, transpose=False)
         assert_rows_close(got.reshape(pairs * m, n), want.reshape(pairs * m, n), dtype, f"untransposed gather mode {mode} M={m} K={k} N={n}")
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
+def test_quantize_dequantize_bit_exact(mode, qmode, dtype):
+    """`fp_quantize_dequantize` (kernels.rs:1011-1065), qqmm's activations: bit for bit the oracle, special values
+    included, with and without NVFP4's global scale; it equals dequantize(quantize(x)) in x's type where no global scale
+    is involved."""
+    rng = np.random.default_rng(6100 + mode + dtype)
+    x = make_x(rng, 37, 320, dtype)
+    wide = ref.to_f32(x, dtype)
+    wide[3, :] = 0.0
+    wide[4, 5], wide[5, 6], wide[6, 7] = np.nan, np.inf, -np.inf
+    wide[7, :] = wide[7, :] * 1e-30
+    x = ref.from_f32(wide, dtype)
+    qm = getattr(nv.QuantMode, qmode)
+    want = ref.fp_quantize_dequantize(x, dtype, mode)
+    got = to_host(nv.quantize_dequantize(to_dev(x), qm))
+    nan = lambda a: np.isnan(ref.to_f32(a, dtype))
+    same = (got.view(np.uint8).reshape(got.shape + (-1,)) == want.view(np.uint8).reshape(want.shape + (-1,))).all(-1)
+    assert np.all(same | (nan(got) & nan(want)))
+    packed, scales = ref.fp_quantize(x, dtype, mode)
+    round_trip = ref.fp_dequantize(packed, scales, mode, dtype)
+    assert np.array_equal(ref.to_f32(want, dtype)[:3], ref.to_f32(round_trip, dtype)[:3])
+    if mode == ref.NVFP4:
+        g = torch.tensor(2.75, dtype=torch.float32, device="cuda")
+        want = ref.fp_quantize_dequantize(x[:3], dtype, mode, 2.75)
+        got = to_host(nv.quantize_dequantize(to_dev(x[:3]), qm, g))
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    else:
+        with pytest.raises(nv.InvalidArgument):
+            nv.quantize_dequantize(to_dev(x), qm, torch.tensor(1.0, device="cuda"))
+    with pytest.raises(nv.InvalidArgument):
+        nv.quantize_dequantize(to_dev(x), nv.Quant.affine(64, 4))

@@ -27,7 +27,7 @@ def test_fixture_meta(golden_cpu, golden_gpu):
     assert len(cases) == 135
     meta, cases = golden_gpu
     assert "mlx=0.32.4" in meta and "device=gpu" in meta
-    assert len(cases) == 303
+    assert len(cases) == 367
 
 
 def test_affine_quantize_bits(golden_cpu):
@@ -94,6 +94,14 @@ def test_nvfp4_global_scale(golden_gpu):
     assert len(exact) == 12 and len(gathers) >= 10
     assert not _failures(exact, lambda c: replay.exact_bits(replay.run_case(c, ORACLE), c.outputs))
     assert not _failures(gathers, lambda c: replay.within_fr008(replay.run_case(c, ORACLE), c.outputs))
+
+
+def test_qqmm_against_mlx_gpu(golden_gpu):
+    """`qqmm` and `gather_qqmm` (activations through their quantization, products.rs:307-470) in the three
+    floating-point modes, dense and quantized weights, with and without NVFP4 global scales: FR-008's bound."""
+    cases = [c for c in golden_gpu[1] if c.op in ("qqmm", "gather_qqmm")]
+    assert len(cases) == 64
+    assert not _failures(cases, lambda c: replay.within_fr008(replay.run_case(c, ORACLE), c.outputs))
 
 
 def test_products_against_mlx_cpu(golden_cpu):
