@@ -33,8 +33,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_214_723   # read 32,380 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
-QMM_TRAFFIC_BYTES = 275_928_611  # read 212,115 KiB + written 57,346 KiB (profiles/qmm_kernel__prefill_c3_m2048.txt)
+QMV_TRAFFIC_BYTES = 33_202_434   # read 32,368 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
+QMM_TRAFFIC_BYTES = 275_814_747  # read 212,004 KiB + written 57,347 KiB (profiles/qmm_kernel__prefill_c3_m2048.txt)
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -215,6 +215,37 @@ def all_configs(lib, device, qs):
     out.append({"config": "C5 MXFP4 gather_qmm 32 experts W[2880,2880], 1024 sorted rows", "m": tokens * top,
                 "us_per_launch": ms * 1e3, "weight_gbps": 141_004_800 / (ms * 1e-3) / 1e9,
                 "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12})
+    del weights, calls
+
+    # The weights' own kernels at the same shapes: quantize (dense in, packed out) and dequantize (packed in, dense out),
+    # inputs rotated beyond the last-level cache, outputs preallocated; GB/s counts every byte read and written.
+    def quantizers(label, shape, tdtype, code, quant, copies):
+        dense = [(torch.randn(shape, device=device) * 0.02).to(tdtype) for _ in range(copies)]
+        q = nv.quantize(dense[0], quant)
+        rows, cols = dense[0].numel() // shape[-1], shape[-1]
+        qc = q.quant._c()
+        ptr = lambda t: C.c_void_p(None if t is None else t.data_ptr())
+        packed_bytes = q.weight.numel() * 4 + q.scales.numel() * q.scales.element_size() * (2 if q.biases is not None else 1)
+        dense_bytes = dense[0].numel() * dense[0].element_size()
+
+        def quantize_call(w):
+            return lambda stream: _lib.check(lib.nvq_quantize(C.byref(qc), code, ptr(w), rows, cols, ptr(q.weight), ptr(q.scales),
+                                                              ptr(q.biases), stream))
+        ms = best_of([quantize_call(w) for w in dense], 60)
+        out.append({"config": f"quantize {label}", "m": 0, "us_per_launch": ms * 1e3,
+                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0})
+        qs_ = [nv.quantize(w, quant) for w in dense]
+
+        def dequantize_call(qq, o):
+            return lambda stream: _lib.check(lib.nvq_dequantize(C.byref(qc), code, ptr(qq.weight), ptr(qq.scales), ptr(qq.biases), rows,
+                                                                cols, ptr(o), stream))
+        ms = best_of([dequantize_call(qq, w) for qq, w in zip(qs_, dense)], 60)
+        out.append({"config": f"dequantize {label}", "m": 0, "us_per_launch": ms * 1e3,
+                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0})
+
+    quantizers("C2 W[14336,4096] bf16 <-> 4-bit g64", (N, K), torch.bfloat16, _lib.BF16, nv.Quant.affine(GROUP, BITS), 4)
+    quantizers("C1 W[4096,4096] f32 <-> 4-bit g64", (4096, 4096), torch.float32, _lib.F32, nv.Quant.affine(64, 4), 8)
+    quantizers("C5 W[32,2880,2880] bf16 <-> MXFP4", (32, 2880, 2880), torch.bfloat16, _lib.BF16, nv.Quant.new(nv.QuantMode.MXFP4), 2)
     return out
 
 
