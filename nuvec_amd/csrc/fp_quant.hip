@@ -283,65 +283,84 @@ fp_quantize_dequantize_kernel(const T *__restrict__ w, int64_t chunks, T *__rest
     store_values<T>(out, chunk * 8, r);
 }
 
-// kernels.rs:976-1009 without a global scale.  With `ids`, output row r is table row ids[r] (`row_chunks` chunks
-// per row, ids clamped to `table_rows`): the rows of a quantized embedding.
+// kernels.rs:976-1009.  With `ids`, output row r is table row ids[r] (`row_chunks` chunks per row, ids clamped to
+// `table_rows`): the rows of a quantized embedding.  A thread owns kUnroll chunks a block apart and requests the
+// codes and scales of all of them before it converts the first: a wavefront that moved one chunk per lane had too
+// few bytes in flight to cover the memory latency (4.1 TB/s at C5's weights).
+constexpr int kUnroll = 4;
 template <typename T, int MODE>
 __global__ void __launch_bounds__(kBlock)
 fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restrict__ scales, uint32_t chunks, T *__restrict__ out,
                      const uint32_t *__restrict__ ids, uint32_t row_chunks, int64_t table_rows, const float *__restrict__ global_scale) {
     using F = Format<MODE>;
-    const uint32_t out_chunk = blockIdx.x * kBlock + threadIdx.x;  // fewer than 2^29: an operand has fewer than 2^32 elements
-    if (out_chunk >= chunks) return;
-    int64_t chunk = out_chunk;
-    if (ids != nullptr) {
-        const uint32_t r = out_chunk / row_chunks;
-        const int64_t row = min((int64_t)ids[r], table_rows - 1);
-        chunk = row * row_chunks + (out_chunk - r * row_chunks);
+    const uint32_t first = blockIdx.x * (kBlock * kUnroll) + threadIdx.x;  // fewer than 2^29: an operand has fewer than 2^32 elements
+    uint32_t code_lo[kUnroll], code_hi[kUnroll], sc_[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        const uint32_t at = first + u * kBlock;
+        const uint32_t oc = at < chunks ? at : chunks - 1;  // past the end: the last chunk again, never stored
+        int64_t chunk = oc;
+        if (ids != nullptr) {
+            const uint32_t r = oc / row_chunks;
+            const int64_t row = min((int64_t)ids[r], table_rows - 1);
+            chunk = row * row_chunks + (oc - r * row_chunks);
+        }
+        sc_[u] = scales[chunk / F::lanes];
+        if constexpr (F::bits == 4) {
+            code_lo[u] = packed[chunk];
+            code_hi[u] = 0u;
+        } else {
+            const uint2 words = reinterpret_cast<const uint2 *>(packed)[chunk];
+            code_lo[u] = words.x;
+            code_hi[u] = words.y;
+        }
     }
-    const uint32_t sc = scales[chunk / F::lanes];
-    const int64_t base = (int64_t)out_chunk * 8;
-    if constexpr (MODE == NVQ_MXFP4) {
-        const uint32_t word = packed[chunk];
-        if (sc - 2u <= 252u) {  // one instruction per pair of codes
-            const float scale = u2f(sc << 23);
-            if constexpr (sizeof(T) == 4) {
-                const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 1),
-                              c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 3);
-                float4 *p = reinterpret_cast<float4 *>(out + base);
-                p[0] = make_float4(a.x, a.y, b.x, b.y);
-                p[1] = make_float4(c.x, c.y, d.x, d.y);
-            } else if constexpr (Elem<T>::code == 10) {
-                const bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 1),
-                               c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3);
-                *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
-                                                                    __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
-            } else {
-                const f16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 1),
-                              c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 3);
-                *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
-                                                                    __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        const uint32_t out_chunk = first + u * kBlock;
+        if (out_chunk >= chunks) continue;
+        const uint32_t sc = sc_[u], word = code_lo[u];
+        const int64_t base = (int64_t)out_chunk * 8;
+        if constexpr (MODE == NVQ_MXFP4) {
+            if (sc - 2u <= 252u) {  // one instruction per pair of codes
+                const float scale = u2f(sc << 23);
+                if constexpr (sizeof(T) == 4) {
+                    const f32x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 1),
+                                  c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, scale, 3);
+                    float4 *p = reinterpret_cast<float4 *>(out + base);
+                    p[0] = make_float4(a.x, a.y, b.x, b.y);
+                    p[1] = make_float4(c.x, c.y, d.x, d.y);
+                } else if constexpr (Elem<T>::code == 10) {
+                    const bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 1),
+                                   c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3);
+                    *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                        __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+                } else {
+                    const f16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 1),
+                                  c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 3);
+                    *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                        __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+                }
+                continue;
             }
-            return;
         }
-    }
-    float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
-    if constexpr (!F::mx) {  // NVFP4's global scale (kernels.rs:992, 996-998)
-        if (global_scale != nullptr) scale = ftz(scale * ftz(*global_scale / (448.0f * 6.0f)));
-    }
-    float v[8];
-    if constexpr (F::bits == 4) {
-        const uint32_t word = packed[chunk];
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu)));
-    } else {
-        const uint2 words = reinterpret_cast<const uint2 *>(packed)[chunk];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            v[i] = canonical(ftz(scale * e4m3_to_f32((words.x >> (8 * i)) & 0xFFu)));
-            v[4 + i] = canonical(ftz(scale * e4m3_to_f32((words.y >> (8 * i)) & 0xFFu)));
+        float scale = ftz(F::mx ? e8m0_to_f32(sc) : e4m3_to_f32(sc));
+        if constexpr (!F::mx) {  // NVFP4's global scale (kernels.rs:992, 996-998)
+            if (global_scale != nullptr) scale = ftz(scale * ftz(*global_scale / (448.0f * 6.0f)));
         }
+        float v[8];
+        if constexpr (F::bits == 4) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = canonical(ftz(scale * e2m1_to_f32((word >> (4 * i)) & 0xFu)));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                v[i] = canonical(ftz(scale * e4m3_to_f32((code_lo[u] >> (8 * i)) & 0xFFu)));
+                v[4 + i] = canonical(ftz(scale * e4m3_to_f32((code_hi[u] >> (8 * i)) & 0xFFu)));
+            }
+        }
+        store_values<T>(out, base, v);
     }
-    store_values<T>(out, base, v);
 }
 
 template <typename T, int MODE>
@@ -357,7 +376,7 @@ template <typename T, int MODE>
 int32_t dequantize_t(const void *packed, const void *scales, int64_t n, void *out, const uint32_t *ids, int64_t cols,
                      int64_t table_rows, const float *global_scale, hipStream_t s) {
     const int64_t chunks = n / 8;
-    const unsigned blocks = (unsigned)((chunks + kBlock - 1) / kBlock);
+    const unsigned blocks = (unsigned)((chunks + kBlock * kUnroll - 1) / (kBlock * kUnroll));
     hipLaunchKernelGGL((fp_dequantize_kernel<T, MODE>), dim3(blocks), dim3(kBlock), 0, s, (const uint32_t *)packed,
                        (const uint8_t *)scales, (uint32_t)chunks, (T *)out, ids, (uint32_t)(cols / 8), table_rows, global_scale);
     NVQ_LAUNCH_CHECK("fp_dequantize");
