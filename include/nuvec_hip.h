@@ -213,7 +213,10 @@ NVQ_API int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32
  *   order u32[pairs]: the pair at each sorted position, ties in pair order;  restore u32[pairs]: its inverse;
  *   sorted_ids u32[pairs] = ids[order];  offsets i32[experts]: where each expert's pairs start. */
 NVQ_API int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
-                      uint32_t *sorted_ids, int32_t *offsets, void *stream);
+                      uint32_t *sorted_ids, int32_t *offsets, void *workspace, void *stream);
+/* Bytes of `workspace` (per-chunk counters) with which the ordering of many pairs runs over the whole chip in three
+ * launches; 0 for few pairs, and with a NULL workspace one block orders them all. */
+NVQ_API size_t nvq_moe_order_workspace_bytes(int64_t pairs, int32_t experts);
 
 /* NVFP4 with a global scale (MLX's `quantize(..., global_scale=)`; ops.rs `quantize_scaled`, quantized.rs:972-1005,
  * kernels.rs:914-1009 with `g`; validated as primitive.rs:1378-1395: NVFP4 only): `global_scale` points at one

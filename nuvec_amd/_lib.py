@@ -87,7 +87,8 @@ SIGNATURES = {
     "nvq_moe_route": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_weighted_sum": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
     "nvq_moe_order": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-                                  C.c_void_p]),
+                                  C.c_void_p, C.c_void_p]),
+    "nvq_moe_order_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int32]),
     "nvq_convert_packed": (C.c_int32, [C.c_int32, C.POINTER(QuantC), C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                        C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_gather_qmm_workspace_bytes": (C.c_size_t, [C.POINTER(GatherDescC)]),

@@ -31,6 +31,50 @@ __global__ void sorted_offsets_kernel(const uint32_t *__restrict__ indices, int6
 // wavefront) plus the counts of the wavefronts before its own.
 constexpr int kOrderThreads = 1024, kOrderWaves = kOrderThreads / 64;
 
+// Places the pairs [chunk, chunk + 1024) of the block stably: `next[e]` is where expert e's next pair goes (advanced by
+// the chunk's count); `wave_count` is scratch [wavefronts][experts].  A pair's rank among the equal ids before it in
+// the chunk comes from wavefront ballots (lanes before it in its own wavefront) plus the counts of the wavefronts
+// before its own.
+__device__ __forceinline__ void place_chunk(const uint32_t *__restrict__ ids, int64_t pairs, int32_t experts, int64_t chunk,
+                                            int32_t *next, int32_t *wave_count, uint32_t *__restrict__ order,
+                                            uint32_t *__restrict__ restore, uint32_t *__restrict__ sorted_ids) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int i = tid; i < kOrderWaves * experts; i += kOrderThreads) wave_count[i] = 0;
+    __syncthreads();
+    const int64_t p = chunk + tid;
+    const bool live = p < pairs;
+    const uint32_t e = live ? min(ids[p], (uint32_t)(experts - 1)) : 0u;  // an id beyond the experts is clamped
+    // Rank among the lanes of this wavefront with the same id: one ballot per distinct id.
+    int rank = 0;
+    uint64_t todo = __ballot(live);
+    while (todo != 0) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const uint32_t e0 = __shfl(e, leader);
+        const uint64_t same = __ballot(live && e == e0);
+        if (live && e == e0) {
+            rank = __popcll(same & ((1ull << lane) - 1ull));
+            if (lane == leader) wave_count[wave * experts + e0] = __popcll(same);
+        }
+        todo &= ~same;
+    }
+    __syncthreads();
+    if (live) {
+        int before = 0;
+        for (int w = 0; w < wave; w++) before += wave_count[w * experts + e];
+        const uint32_t at = (uint32_t)(next[e] + before + rank);
+        order[at] = (uint32_t)p;
+        restore[p] = at;
+        sorted_ids[at] = e;
+    }
+    __syncthreads();
+    for (int ee = tid; ee < experts; ee += kOrderThreads) {
+        int total = 0;
+        for (int w = 0; w < kOrderWaves; w++) total += wave_count[w * experts + ee];
+        next[ee] += total;
+    }
+    __syncthreads();
+}
+
 __global__ void __launch_bounds__(kOrderThreads)
 moe_order_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t experts, uint32_t *__restrict__ order,
                  uint32_t *__restrict__ restore, uint32_t *__restrict__ sorted_ids, int32_t *__restrict__ offsets) {
@@ -62,42 +106,71 @@ moe_order_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t expert
         }
     }
     __syncthreads();
-    for (int64_t chunk = 0; chunk < pairs; chunk += kOrderThreads) {
-        for (int i = tid; i < kOrderWaves * experts; i += kOrderThreads) wave_count[i] = 0;
-        __syncthreads();
-        const int64_t p = chunk + tid;
-        const bool live = p < pairs;
-        const uint32_t e = live ? min(ids[p], (uint32_t)(experts - 1)) : 0u;  // an id beyond the experts is clamped
-        // Rank among the lanes of this wavefront with the same id: one ballot per distinct id.
-        int rank = 0;
-        uint64_t todo = __ballot(live);
-        while (todo != 0) {
-            const int leader = __ffsll((long long)todo) - 1;
-            const uint32_t e0 = __shfl(e, leader);
-            const uint64_t same = __ballot(live && e == e0);
-            if (live && e == e0) {
-                rank = __popcll(same & ((1ull << lane) - 1ull));
-                if (lane == leader) wave_count[wave * experts + e0] = __popcll(same);
-            }
-            todo &= ~same;
-        }
-        __syncthreads();
-        if (live) {
-            int before = 0;
-            for (int w = 0; w < wave; w++) before += wave_count[w * experts + e];
-            const uint32_t at = (uint32_t)(next[e] + before + rank);
-            order[at] = (uint32_t)p;
-            restore[p] = at;
-            sorted_ids[at] = e;
-        }
-        __syncthreads();
-        for (int ee = tid; ee < experts; ee += kOrderThreads) {
-            int total = 0;
-            for (int w = 0; w < kOrderWaves; w++) total += wave_count[w * experts + ee];
-            next[ee] += total;
-        }
-        __syncthreads();
+    for (int64_t chunk = 0; chunk < pairs; chunk += kOrderThreads) place_chunk(ids, pairs, experts, chunk, next, wave_count, order, restore, sorted_ids);
+}
+
+// The same ordering for many pairs, over the whole chip in three steps: every block counts the ids of its chunk of
+// 1024 pairs; one block turns the counts into the experts' offsets and, per chunk and expert, the position of the
+// chunk's first such pair (chunks in order: the sort stays stable); every block places its chunk.
+__global__ void __launch_bounds__(kOrderThreads)
+moe_count_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t experts, int32_t *__restrict__ counts) {
+    extern __shared__ int32_t lds_i[];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < experts; e += kOrderThreads) lds_i[e] = 0;
+    __syncthreads();
+    const int64_t p = (int64_t)blockIdx.x * kOrderThreads + tid;
+    if (p < pairs) atomicAdd(&lds_i[min(ids[p], (uint32_t)(experts - 1))], 1);
+    __syncthreads();
+    for (int e = tid; e < experts; e += kOrderThreads) counts[(int64_t)blockIdx.x * experts + e] = lds_i[e];
+}
+
+__global__ void __launch_bounds__(kOrderThreads)
+moe_scan_kernel(int32_t *__restrict__ counts, int32_t chunks, int32_t experts, int32_t *__restrict__ offsets) {
+    extern __shared__ int32_t lds_i[];  // [experts]: totals, then offsets
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < experts; e += kOrderThreads) {
+        int32_t total = 0;
+        for (int c = 0; c < chunks; c++) total += counts[(int64_t)c * experts + e];
+        lds_i[e] = total;
     }
+    __syncthreads();
+    if (wave == 0) {  // exclusive scan over the experts, 64 at a time
+        int32_t carry = 0;
+        for (int base = 0; base < experts; base += 64) {
+            const int e = base + lane;
+            const int32_t count = e < experts ? lds_i[e] : 0;
+            int32_t incl = count;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int32_t up = __shfl_up(incl, d);
+                if (lane >= d) incl += up;
+            }
+            if (e < experts) {
+                lds_i[e] = carry + incl - count;
+                offsets[e] = carry + incl - count;
+            }
+            carry += __shfl(incl, 63);
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < experts; e += kOrderThreads) {
+        int32_t at = lds_i[e];
+        for (int c = 0; c < chunks; c++) {
+            const int32_t n = counts[(int64_t)c * experts + e];
+            counts[(int64_t)c * experts + e] = at;
+            at += n;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(kOrderThreads)
+moe_place_kernel(const uint32_t *__restrict__ ids, int64_t pairs, int32_t experts, const int32_t *__restrict__ starts,
+                 uint32_t *__restrict__ order, uint32_t *__restrict__ restore, uint32_t *__restrict__ sorted_ids) {
+    extern __shared__ int32_t lds_i[];
+    int32_t *next = lds_i, *wave_count = lds_i + experts;
+    for (int e = threadIdx.x; e < experts; e += kOrderThreads) next[e] = starts[(int64_t)blockIdx.x * experts + e];
+    __syncthreads();
+    place_chunk(ids, pairs, experts, (int64_t)blockIdx.x * kOrderThreads, next, wave_count, order, restore, sorted_ids);
 }
 
 // round(a / b) in the element type.  The float32 quotient is correctly rounded and float32 carries more than twice
@@ -199,11 +272,30 @@ int32_t launch_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, 
 
 size_t moe_order_lds_bytes(int32_t experts) { return (size_t)(1 + kOrderWaves) * experts * sizeof(int32_t); }
 
+// Above this many pairs the ordering runs over the whole chip (three launches) when the caller gave the workspace.
+constexpr int64_t kOrderOneBlock = 2048;
+size_t moe_order_workspace_bytes(int64_t pairs, int32_t experts) {
+    if (pairs <= kOrderOneBlock) return 0;
+    return (size_t)((pairs + kOrderThreads - 1) / kOrderThreads) * (size_t)experts * sizeof(int32_t);
+}
+
 int32_t launch_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
-                         uint32_t *sorted_ids, int32_t *offsets, hipStream_t s) {
-    hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(kOrderThreads), moe_order_lds_bytes(experts), s, ids, pairs, experts, order,
-                       restore, sorted_ids, offsets);
-    NVQ_LAUNCH_CHECK("moe_order");
+                         uint32_t *sorted_ids, int32_t *offsets, void *workspace, hipStream_t s) {
+    if (workspace == nullptr || pairs <= kOrderOneBlock) {
+        hipLaunchKernelGGL(moe_order_kernel, dim3(1), dim3(kOrderThreads), moe_order_lds_bytes(experts), s, ids, pairs, experts, order,
+                           restore, sorted_ids, offsets);
+        NVQ_LAUNCH_CHECK("moe_order");
+        return NVQ_OK;
+    }
+    const unsigned chunks = (unsigned)((pairs + kOrderThreads - 1) / kOrderThreads);
+    int32_t *counts = (int32_t *)workspace;
+    hipLaunchKernelGGL(moe_count_kernel, dim3(chunks), dim3(kOrderThreads), (size_t)experts * sizeof(int32_t), s, ids, pairs, experts, counts);
+    NVQ_LAUNCH_CHECK("moe_order (count)");
+    hipLaunchKernelGGL(moe_scan_kernel, dim3(1), dim3(kOrderThreads), (size_t)experts * sizeof(int32_t), s, counts, (int32_t)chunks, experts, offsets);
+    NVQ_LAUNCH_CHECK("moe_order (scan)");
+    hipLaunchKernelGGL(moe_place_kernel, dim3(chunks), dim3(kOrderThreads), moe_order_lds_bytes(experts), s, ids, pairs, experts, counts, order,
+                       restore, sorted_ids);
+    NVQ_LAUNCH_CHECK("moe_order (place)");
     return NVQ_OK;
 }
 

@@ -449,8 +449,13 @@ int32_t nvq_convert_packed(int32_t format, const nvq_quant *quant, int32_t dtype
                                  scales_out, biases_out, (hipStream_t)stream);
 }
 
+size_t nvq_moe_order_workspace_bytes(int64_t pairs, int32_t experts) {
+    if (pairs <= 0 || experts <= 0) return 0;
+    return moe_order_workspace_bytes(pairs, experts);
+}
+
 int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,
-                      uint32_t *sorted_ids, int32_t *offsets, void *stream) {
+                      uint32_t *sorted_ids, int32_t *offsets, void *workspace, void *stream) {
     if (pairs < 0 || experts <= 0) return fail(NVQ_INVALID_ARGUMENT, "moe_order: %lld pairs, %d experts", (long long)pairs, experts);
     if (pairs > INT32_MAX) return fail(NVQ_INVALID_ARGUMENT, "moe_order: %lld pairs exceed 32-bit positions", (long long)pairs);
     if (moe_order_lds_bytes(experts) > 64 * 1024)
@@ -458,7 +463,7 @@ int32_t nvq_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint3
     if (offsets == nullptr || (pairs > 0 && (ids == nullptr || order == nullptr || restore == nullptr || sorted_ids == nullptr)))
         return fail(NVQ_INVALID_ARGUMENT, "moe_order: null operand");
     NVQ_TRY(require_device());
-    return launch_moe_order(ids, pairs, experts, order, restore, sorted_ids, offsets, (hipStream_t)stream);
+    return launch_moe_order(ids, pairs, experts, order, restore, sorted_ids, offsets, workspace, (hipStream_t)stream);
 }
 
 int32_t nvq_moe_route(int32_t dtype, const void *probs, int64_t rows, int32_t experts, int32_t k, int32_t normalize,

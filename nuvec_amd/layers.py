@@ -163,3 +163,33 @@ class MoeMlp:
         return ops.weighted_sum(experts, scores)
 
     __call__ = forward
+
+
+def quantized_attention(q: torch.Tensor, k: ops.Quantized, v: ops.Quantized, scale: float,
+                        sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fast.rs:694-718, fast/imp.rs:3992-4035 (`quantized_attention`, mlx-lm's quantized KV cache): attention of the
+    queries `q [B, Hq, L, D]` over affine-quantized keys and values (codes `[B, Hkv, S, D * bits / 32]`, scales and
+    biases `[B, Hkv, S, D / group]`), grouped query heads, no mask, optional per-head `sinks [Hq]`:
+    `softmax(scale * q k^T [, sinks]) v`.  This is the reference's composition (the one it runs wherever its fused
+    kernel does not fit): both products are the library's quantized products, transposed for the keys and
+    untransposed for the values; the softmax (float32 inside, one rounding) is an elementwise step outside the path."""
+    if k.quant != v.quant or k.quant.mode != ops.QuantMode.AFFINE:
+        raise ops.InvalidArgument("quantized_attention: keys and values need one affine quantization")
+    if k.biases is None or v.biases is None:
+        raise ops.InvalidArgument("quantized_attention: affine biases missing")
+    b, hq, l, d = q.shape
+    hkv = k.weight.shape[1]
+    if hq % hkv != 0:
+        raise ops.InvalidArgument(f"quantized_attention: {hq} query heads over {hkv} key heads")
+    rep = hq // hkv
+    qs = (q * scale).reshape(b, hkv, rep, l, d)
+    expand = lambda t: ops.Quantized(t.weight.unsqueeze(-3), t.scales.unsqueeze(-3), t.biases.unsqueeze(-3), t.quant)
+    scores = ops.quantized_matmul(qs, expand(k), True)  # [B, Hkv, rep, L, S]
+    s = scores.shape[-1]
+    if sinks is not None:
+        column = sinks.to(scores.dtype).reshape(1, hkv, rep, 1, 1).expand(b, hkv, rep, l, 1)
+        probs = torch.softmax(torch.cat([scores, column], dim=-1).float(), dim=-1).to(scores.dtype)[..., :s]
+    else:
+        probs = torch.softmax(scores.float(), dim=-1).to(scores.dtype)
+    out = ops.quantized_matmul(probs.contiguous(), expand(v), False)  # [B, Hkv, rep, L, D]
+    return out.reshape(b, hq, l, d)

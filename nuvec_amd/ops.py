@@ -436,8 +436,11 @@ def moe_order(expert_ids: torch.Tensor, experts: int):
     order = torch.empty(pairs, dtype=torch.int32, device=ids.device)
     restore, sorted_ids = torch.empty_like(order), torch.empty_like(order)
     offsets = torch.empty(experts, dtype=torch.int32, device=ids.device)
-    _lib.check(_lib.load().nvq_moe_order(_ptr(ids), pairs, experts, _ptr(order), _ptr(restore), _ptr(sorted_ids), _ptr(offsets),
-                                         _stream()))
+    lib = _lib.load()
+    need = lib.nvq_moe_order_workspace_bytes(pairs, experts)
+    workspace = torch.empty(need, dtype=torch.uint8, device=ids.device) if need else None
+    _lib.check(lib.nvq_moe_order(_ptr(ids), pairs, experts, _ptr(order), _ptr(restore), _ptr(sorted_ids), _ptr(offsets),
+                                 _ptr(workspace), _stream()))
     return order, restore, sorted_ids, offsets
 
 

@@ -624,7 +624,7 @@ def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
         assert_rows_close(got.reshape(12, n), want.reshape(12, n), dtype, "four rows, a matrix per item")
 
 
-@pytest.mark.parametrize("pairs,experts", [(0, 4), (5, 3), (1024, 32), (3000, 7), (5000, 130)])
+@pytest.mark.parametrize("pairs,experts", [(0, 4), (5, 3), (1024, 32), (3000, 7), (5000, 130), (2049, 32), (5000, 8), (65536, 32), (100001, 200)])
 def test_moe_order_is_the_stable_argsort(pairs, experts):
     """The ordering of a mixture-of-experts layer's pairs (nuvec-lm model.rs:2193-2210): argsort of the expert
     ids with ties in pair order, its inverse, the sorted ids and where each expert starts: integers, exact."""
@@ -809,3 +809,41 @@ def test_quantize_dequantize_bit_exact(mode, qmode, dtype):
             nv.quantize_dequantize(to_dev(x), qm, torch.tensor(1.0, device="cuda"))
     with pytest.raises(nv.InvalidArgument):
         nv.quantize_dequantize(to_dev(x), nv.Quant.affine(64, 4))
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32])
+@pytest.mark.parametrize("group,bits,d", [(64, 4, 128), (32, 8, 64), (64, 3, 128)])
+def test_quantized_attention_composition(dtype, group, bits, d):
+    """`quantized_attention` (fast.rs:694-718) as the reference composes it over the library's products: one query row
+    per head over quantized keys and values, grouped heads, with and without sinks, against attention over the
+    oracle's dequantized cache in float64 (the bound the reference states for it: that of the dequantized attention)."""
+    from nuvec_amd.layers import quantized_attention
+    rng = np.random.default_rng(8100 + bits + dtype)
+    b, hkv, rep, s = 2, 2, 4, 192
+    hq = hkv * rep
+    kd, vd = make_x(rng, b * hkv * s, d, dtype).reshape(b, hkv, s, d), make_x(rng, b * hkv * s, d, dtype).reshape(b, hkv, s, d)
+    kq, vq = ref.affine_quantize(kd, dtype, group, bits), ref.affine_quantize(vd, dtype, group, bits)
+    q = make_x(rng, b * hq, d, dtype).reshape(b, hq, 1, d)
+    sinks = ref.from_f32(rng.standard_normal(hq).astype(np.float32), dtype)
+    quant = nv.Quant.affine(group, bits)
+    K = nv.Quantized(to_dev(kq[0]), to_dev(kq[1]), to_dev(kq[2]), quant)
+    V = nv.Quantized(to_dev(vq[0]), to_dev(vq[1]), to_dev(vq[2]), quant)
+    scale = 1.0 / np.sqrt(d)
+    kf = ref.to_f32(ref.affine_dequantize(*kq, dtype, group, bits), dtype).astype(np.float64)
+    vf = ref.to_f32(ref.affine_dequantize(*vq, dtype, group, bits), dtype).astype(np.float64)
+    qf = ref.to_f32(q, dtype).astype(np.float64).reshape(b, hkv, rep, d)
+    logits = scale * np.einsum("bhrd,bhsd->bhrs", qf, kf)
+    tol = {ref.BF16: 2e-2, ref.F32: 2e-5}[dtype]
+    for use_sinks in (False, True):
+        full = logits
+        if use_sinks:
+            full = np.concatenate([logits, np.broadcast_to(ref.to_f32(sinks, dtype).astype(np.float64).reshape(1, hkv, rep, 1), (b, hkv, rep, 1))], -1)
+        p = np.exp(full - full.max(-1, keepdims=True))
+        p = (p / p.sum(-1, keepdims=True))[..., :s]
+        want = np.einsum("bhrs,bhsd->bhrd", p, vf).reshape(b, hq, 1, d)
+        got = quantized_attention(to_dev(q), K, V, scale, to_dev(sinks) if use_sinks else None)
+        assert tuple(got.shape) == (b, hq, 1, d)
+        err = np.abs(ref.to_f32(to_host(got), dtype).astype(np.float64) - want).max()
+        assert err <= tol * max(1.0, np.abs(want).max()), f"sinks={use_sinks}: {err}"
+    with pytest.raises(nv.InvalidArgument):
+        quantized_attention(to_dev(q), K, nv.Quantized(V.weight, V.scales, V.biases, nv.Quant.affine(group, 2 if bits != 2 else 4)), scale)
