@@ -146,35 +146,75 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 #pragma unroll
     for (int i = 0; i < RM; i++) acc[i] = 0.0f;
 
-    for (int k0 = 0; k0 < K; k0 += kStep) {
-        // x first: it is needed first and arrives from the cache.
+    // Everything a step reads from memory: the thread's four values of each x row (one vector load), the lane's codes
+    // and its group's scale and bias as stored.  The next step's are requested before the current step is computed, so
+    // a product of two steps (K = 4096) pays the memory latency once.
+    using S = std::conditional_t<kAffine, T, uint8_t>;
+    struct Step {
         float xin[RM][kPer];
+        uint32_t d[BITS];
+        S sc[kHalves], bi;
+    };
+    auto fetch = [&](int k0) {
+        Step st;
         const int kx = k0 + tid * kPer;
 #pragma unroll
-        for (int i = 0; i < RM; i++)
+        for (int i = 0; i < RM; i++) {
+            const bool have = kx < K && m0 + i < M;
+            const T *px = x + (have ? (int64_t)(m0 + i) * K + kx : 0);  // K is a multiple of 16 and x 16-byte aligned
+            if constexpr (sizeof(T) == 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(px);
+                st.xin[i][0] = have ? v.x : 0.0f; st.xin[i][1] = have ? v.y : 0.0f;
+                st.xin[i][2] = have ? v.z : 0.0f; st.xin[i][3] = have ? v.w : 0.0f;
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2 *>(px);
+                T e[4];
+                __builtin_memcpy(e, &v, 8);
 #pragma unroll
-            for (int j = 0; j < kPer; j++) xin[i][j] = (kx < K && m0 + i < M) ? Elem<T>::load(x, (int64_t)(m0 + i) * K + kx + j) : 0.0f;
+                for (int j = 0; j < kPer; j++) st.xin[i][j] = have ? Elem<T>::load(e, j) : 0.0f;
+            }
+        }
         const int kb = k0 + lane * 32;
         const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
-        uint32_t d[BITS];
-        load_words<BITS>(wrow + (kc >> 5) * BITS, d);
+        load_words<BITS>(wrow + (kc >> 5) * BITS, st.d);
+        const int64_t g = (int64_t)nc * kgroups + (kc >> gshift);
+        if constexpr (kAffine) {
+            st.sc[0] = ((const T *)a.scales + o.s)[g];
+            st.bi = ((const T *)a.biases + o.s)[g];
+        } else {
+            const uint8_t *sp = (const uint8_t *)a.scales + o.s + g;
+#pragma unroll
+            for (int hf = 0; hf < kHalves; hf++) st.sc[hf] = sp[hf];
+            st.bi = 0;
+        }
+        return st;
+    };
+    float inv_enc = 1.0f;
+    bool scaled = false;
+    if constexpr (MODE == NVQ_NVFP4) {
+        // kernels.rs:992-998: a global scale g turns every group scale into ftz(scale * ftz(g / (448 * 6)));
+        // a gather has one g per expert (quantized.rs:620-636)
+        if (a.global_scale != nullptr) {
+            const float g = a.global_scale[a.rhs != nullptr ? min((int64_t)a.rhs[blockIdx.z], a.experts - 1) : 0];
+            inv_enc = ftz(g / (448.0f * 6.0f));
+            scaled = true;
+        }
+    }
+
+    Step cur = fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kStep) {
+        const Step nxt = fetch(k0 + kStep);  // past the end: valid addresses, nothing of it is used
+        const auto &xin = cur.xin;
+        const auto &d = cur.d;
         float sc[kHalves], bi = 0.0f;
         if constexpr (kAffine) {
-            sc[0] = Elem<T>::load((const T *)a.scales + o.s, (int64_t)nc * kgroups + (kc >> gshift));
-            bi = Elem<T>::load((const T *)a.biases + o.s, (int64_t)nc * kgroups + (kc >> gshift));
+            sc[0] = Elem<T>::load(&cur.sc[0], 0);
+            bi = Elem<T>::load(&cur.bi, 0);
         } else {
-            const uint8_t *sp = (const uint8_t *)a.scales + o.s + (int64_t)nc * kgroups + (kc >> gshift);
 #pragma unroll
-            for (int hf = 0; hf < kHalves; hf++) sc[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(sp[hf]) : e8m0_to_f32(sp[hf]));
-            if constexpr (MODE == NVQ_NVFP4) {
-                // kernels.rs:992-998: a global scale g turns every group scale into ftz(scale * ftz(g / (448 * 6)));
-                // a gather has one g per expert (quantized.rs:620-636)
-                if (a.global_scale != nullptr) {
-                    const float g = a.global_scale[a.rhs != nullptr ? min((int64_t)a.rhs[blockIdx.z], a.experts - 1) : 0];
-                    const float inv_enc = ftz(g / (448.0f * 6.0f));
-#pragma unroll
-                    for (int hf = 0; hf < kHalves; hf++) sc[hf] = ftz(sc[hf] * inv_enc);
-                }
+            for (int hf = 0; hf < kHalves; hf++) {
+                sc[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(cur.sc[hf]) : e8m0_to_f32(cur.sc[hf]));
+                if (scaled) sc[hf] = ftz(sc[hf] * inv_enc);
             }
         }
         if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
@@ -223,6 +263,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
                 for (int hf = 0; hf < kHalves; hf++) acc[i] = __builtin_fmaf(sc[hf], dot[i][hf], acc[i]);
             }
         }
+        cur = nxt;
     }
 #pragma unroll
     for (int i = 0; i < RM; i++) {
