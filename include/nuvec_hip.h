@@ -233,6 +233,15 @@ NVQ_API int32_t nvq_quantized_matmul_scaled(const nvq_qmm_desc *desc, const void
 NVQ_API int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
                               const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
                               void *y, void *workspace, void *stream);
+/* The gathered product with its result rows put where the caller wants them: pair z (sorted position z of a grouped
+ * product) writes block out_rows[z] of y [pairs, M, N] (u32[pairs], a permutation; an index beyond `pairs` is the
+ * caller's error and is clamped).  With out_rows = the `order` of nvq_moe_order the ordered down projection of
+ * SwitchGlu::forward lands in pair order and the inverse permutation `take(out, inverse)` of
+ * crates/nuvec-lm/src/model.rs:2205-2210 is never run.  `biases` / `global_scales` as the mode needs them (either
+ * may be NULL).  Weights stored [N, K] only (transpose = 1); else NVQ_UNSUPPORTED. */
+NVQ_API int32_t nvq_gather_qmm_scatter(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
+                               const void *biases, const float *global_scales, const uint32_t *lhs, const uint32_t *rhs,
+                               const int32_t *offsets, const uint32_t *out_rows, void *y, void *workspace, void *stream);
 
 /* FastOp::QuantizeDequantize (crates/nuvec-core/src/products.rs:307-315, kernels.rs:1011-1065; MLX's
  * fp_quantize_dequantize): x through its quantization in a floating-point mode, i.e. the values the codes represent,

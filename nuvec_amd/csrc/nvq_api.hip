@@ -494,8 +494,8 @@ int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t ro
 }
 
 static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
-                              const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y,
-                              void *workspace, void *stream) {
+                              const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                              const uint32_t *out_rows, void *y, void *workspace, void *stream) {
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
     NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
     NVQ_TRY(check_groups("gather_qmm", d->quant.mode, biases));
@@ -508,6 +508,8 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(require_device());
     if (!d->transpose && global_scale != nullptr)
         return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for untransposed weights with a global scale");
+    if (!d->transpose && out_rows != nullptr)
+        return fail(NVQ_UNSUPPORTED, "gather_qmm: no gfx950 kernel for untransposed weights with scattered output rows");
     NVQ_TRY(check_aligned("gather_qmm", "x", x));
     NVQ_TRY(check_aligned("gather_qmm", "w", w));
     NVQ_TRY(check_aligned("gather_qmm", "y", y));
@@ -522,6 +524,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.lhs = lhs; a.rhs = rhs;
     a.x_batches = d->x_batches; a.experts = d->experts;
     a.global_scale = global_scale;
+    a.out_rows = out_rows;
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
@@ -534,7 +537,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
 
 int32_t nvq_gather_qmm(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                        const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets, void *y, void *workspace, void *stream) {
-    return gather_qmm_any(d, x, w, scales, biases, nullptr, lhs, rhs, offsets, y, workspace, stream);
+    return gather_qmm_any(d, x, w, scales, biases, nullptr, lhs, rhs, offsets, nullptr, y, workspace, stream);
 }
 
 int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *d, const void *x, const void *w, const void *scales,
@@ -545,7 +548,16 @@ int32_t nvq_gather_qmm_scaled(const nvq_gather_desc *d, const void *x, const voi
     if (global_scales == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null global scale");
     if (d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
-    return gather_qmm_any(d, x, w, scales, nullptr, global_scales, lhs, rhs, offsets, y, workspace, stream);
+    return gather_qmm_any(d, x, w, scales, nullptr, global_scales, lhs, rhs, offsets, nullptr, y, workspace, stream);
+}
+
+int32_t nvq_gather_qmm_scatter(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                               const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                               const uint32_t *out_rows, void *y, void *workspace, void *stream) {
+    if (out_rows == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null output rows");
+    if (global_scales != nullptr && d != nullptr && d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
+        return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
+    return gather_qmm_any(d, x, w, scales, biases, global_scales, lhs, rhs, offsets, out_rows, y, workspace, stream);
 }
 
 }  // extern "C"

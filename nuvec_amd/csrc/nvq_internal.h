@@ -81,6 +81,7 @@ struct ProductArgs {
     int32_t k_splits, k_split_steps;  // tiled kernel: K split over grid z (0 or 1: no split), steps of 64 values per split
     float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
     const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (general kernel only)
+    const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.

@@ -215,7 +215,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         xo = l * a.m * K;
         wo = r * N * row_bytes;
         so = r * N * kgroups;
-        yo = (int64_t)blockIdx.z * a.m * N;
+        yo = (a.out_rows != nullptr ? min((int64_t)a.out_rows[blockIdx.z], a.batch - 1) : (int64_t)blockIdx.z) * a.m * N;
     } else if (a.batch_ndim > 0) {
         xo = (int64_t)blockIdx.z * a.x_strides[0];
         wo = (int64_t)blockIdx.z * a.w_strides[0] * 4;  // the stride counts packed words

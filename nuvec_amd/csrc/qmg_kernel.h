@@ -275,12 +275,17 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
 
         // Accumulator element el of lane l is tile row 8 (el / 4) + 4 (l / 32) + el % 4 (a row of x), column l % 32.
         const int col = n0 + 32 * wave + l32;
+        // A scattered product writes sorted row r where the caller wants it (its pair's place): lane l fetches the
+        // place of the pass's row l (one load per wavefront) and the stores read it across lanes.
+        uint32_t place = pass + lane;
+        if (a.out_rows != nullptr) place = (uint32_t)min((int64_t)a.out_rows[pass + (lane < rows ? lane : 0)], a.batch - 1);
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
             for (int el = 0; el < 16; el++) {
-                const int m = 32 * u + 8 * (el >> 2) + 4 * h + (el & 3);
-                if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, acc[u][el]);
+                const int m0 = 32 * u + 8 * (el >> 2) + (el & 3), m = m0 + 4 * h;
+                const uint32_t lo = __builtin_amdgcn_readlane(place, m0), hi = __builtin_amdgcn_readlane(place, m0 + 4);
+                if (m < rows && col < N) Elem<T>::store(y, (int64_t)(h ? hi : lo) * N + col, acc[u][el]);
             }
     }
 }

@@ -36,6 +36,7 @@ __device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int6
         o.x = l * a.m * a.k;
         o.w = r * a.n * kwords;
         o.s = r * a.n * kgroups;
+        if (a.out_rows != nullptr) o.y = min((int64_t)a.out_rows[z], a.batch - 1) * a.m * a.n;
         return o;
     }
     if (a.batch_ndim == 0) return o;

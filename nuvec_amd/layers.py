@@ -96,12 +96,20 @@ class SwitchProjection:
         y = ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices))
         return y if self.bias is None else y + self.bias[indices.long()].unsqueeze(-2)
 
-    def forward_sorted_rows(self, x: torch.Tensor, rows, sorted_ids: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
-        """Rows `rows` of `x` (`[T, input_dims]`; None: its rows in order) through experts sorted by id."""
+    def forward_sorted_rows(self, x: torch.Tensor, rows, sorted_ids: torch.Tensor, offsets: torch.Tensor,
+                            out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Rows `rows` of `x` (`[T, input_dims]`; None: its rows in order) through experts sorted by id.  With
+        `out_rows` (a permutation) result row i is written at row `out_rows[i]`."""
         if rows is None:
             rows = torch.arange(x.shape[0], dtype=torch.int32, device=x.device)
-        y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets)
-        return y if self.bias is None else y + self.bias[sorted_ids.long()]
+        y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows)
+        if self.bias is None:
+            return y
+        if out_rows is None:
+            return y + self.bias[sorted_ids.long()]
+        ids = torch.empty_like(sorted_ids)
+        ids[out_rows.long()] = sorted_ids  # the expert of each output row
+        return y + self.bias[ids.long()]
 
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -119,8 +127,8 @@ class SwitchGlu:
     def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
         """`x` `[B, L, D]` through each token's experts `indices` `[B, L, k]`: `[B, L, k, D]`.  With 64 pairs or
         more they are ordered by expert (model.rs:2193-2210) so that each expert's weights are read once; here one
-        kernel orders the pairs, the products take the token rows of `x` themselves, and only the result is
-        put back in pair order."""
+        kernel orders the pairs, the products take the token rows of `x` themselves, and the last product writes
+        each row at its pair's place (`out_rows`), so the inverse permutation of model.rs:2210 is never run."""
         b, l, d = x.shape
         k = indices.shape[2]
         if indices.numel() < 64:  # model.rs:2189-2192
@@ -133,8 +141,8 @@ class SwitchGlu:
         xt = x.reshape(b * l, d)
         up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
         gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
-        out = self.down_proj.forward_sorted_rows(swiglu(gate, up), None, sorted_ids, offsets)
-        return out[restore.long()].reshape(b, l, k, -1)
+        out = self.down_proj.forward_sorted_rows(swiglu(gate, up), None, sorted_ids, offsets, out_rows=order)
+        return out.reshape(b, l, k, -1)
 
     __call__ = forward
 

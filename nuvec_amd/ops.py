@@ -478,12 +478,26 @@ def weighted_sum(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _out_rows(op: str, given: Optional[torch.Tensor], pairs: int, device) -> Optional[torch.Tensor]:
+    """Where each pair's result goes (`nvq_gather_qmm_scatter`): one integer per pair, a permutation of the pairs."""
+    if given is None:
+        return None
+    if given.dtype.is_floating_point or given.dtype == torch.bool:
+        raise InvalidArgument(f"{op}: output rows must be integers")
+    if given.numel() != pairs:
+        raise InvalidArgument(f"{op}: {given.numel()} output rows for {pairs} pairs")
+    given = given.to(device).reshape(-1)
+    return (given.to(torch.int32) if given.dtype != torch.uint32 else given.view(torch.int32)).contiguous()
+
+
 def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor,
-                       offsets: torch.Tensor) -> torch.Tensor:
+                       offsets: torch.Tensor, out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The grouped route of `gather_qmm` (quantized.rs:646-651, 772-782) with the rows of x taken inside the kernel:
     output row i = x[rows[i]] . dequantize(w)[sorted_ids[i]]^T for ids sorted by expert (`offsets` from `moe_order`
     or `sorted_offsets`).  Equal to `gather_qmm(x[rows], q, None, sorted_ids, sorted)`; the gathered copy of x is
-    never written.  x is `[T, K]`, the result `[len(rows), N]`."""
+    never written.  x is `[T, K]`, the result `[len(rows), N]`.  With `out_rows` (a permutation, e.g. the `order` of
+    `moe_order`) result row i is written at row `out_rows[i]`: the ordered product lands in pair order and
+    model.rs:2205-2210's `take(out, inverse)` is not needed."""
     op = "gather_qmm"
     quant = q.quant
     quant.checked(op)
@@ -505,6 +519,12 @@ def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted
         raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
     out = torch.empty((rhs.numel(), w.shape[-2]), dtype=dtype, device=x.device)
     d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 1, w.shape[-2], columns, rhs.numel(), x.shape[0], w.shape[0])
+    scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
+    if scatter is not None:
+        _lib.check(_lib.load().nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(None),
+                                                      _ptr(lhs), _ptr(rhs), _ptr(offsets.contiguous()), _ptr(scatter),
+                                                      _ptr(out), _ptr(None), _stream()))
+        return out
     _lib.check(_lib.load().nvq_gather_qmm(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs),
                                           _ptr(offsets.contiguous()), _ptr(out), _ptr(None), _stream()))
     return out
@@ -525,8 +545,10 @@ def _indices(op: str, a: torch.Tensor, given: Optional[torch.Tensor]) -> torch.T
 
 def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor] = None,
                rhs_indices: Optional[torch.Tensor] = None, options: GatherQmm = GatherQmm(), *,
-               row_exact: bool = False) -> torch.Tensor:
-    """ops.rs:1050-1074, quantized.rs:589-673: output batch i = x[lhs[i]] . dequantize(w)[rhs[i]]^T."""
+               row_exact: bool = False, out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """ops.rs:1050-1074, quantized.rs:589-673: output batch i = x[lhs[i]] . dequantize(w)[rhs[i]]^T.  `out_rows` (not in
+    the reference; one integer per pair, a permutation) writes batch i at position `out_rows[i]` of the flattened
+    batches instead."""
     op = "gather_qmm"
     quant = q.quant
     quant.checked(op)
@@ -569,6 +591,9 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
     need = lib.nvq_gather_qmm_workspace_bytes(C.byref(d))
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
     gs = q.global_scale
+    scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
+    if scatter is not None and lhs_indices is None and rhs_indices is None:
+        raise InvalidArgument(f"{op}: output rows need indices")
     if gs is not None:  # quantized.rs:620-636: one float32 value per expert
         if quant.mode != QuantMode.NVFP4:
             raise InvalidArgument(f"{op}: global scale is only supported for 'nvfp4' quantization mode")
@@ -577,6 +602,11 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
         if tuple(gs.shape) != tuple(w.shape[:-2]):
             raise InvalidArgument(f"{op}: global scale must have one entry per expert with shape {list(w.shape[:-2])} but got {list(gs.shape)}")
         gs = gs.to(x.device).contiguous()
+    if scatter is not None:
+        _lib.check(lib.nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs), _ptr(lhs),
+                                              _ptr(rhs), _ptr(offsets), _ptr(scatter), _ptr(out), _ptr(workspace), _stream()))
+        return out
+    if gs is not None:
         _lib.check(lib.nvq_gather_qmm_scaled(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(gs), _ptr(lhs), _ptr(rhs),
                                              _ptr(offsets), _ptr(out), _ptr(workspace), _stream()))
         return out

@@ -777,6 +777,55 @@ def test_untransposed_gathers(mode, qmode):
         assert_rows_close(got.reshape(pairs * m, n), want.reshape(pairs * m, n), dtype, f"untransposed gather mode {mode} M={m} K={k} N={n}")
 
 
+@pytest.mark.parametrize("route", ["grouped-mxfp4", "grouped-affine4", "pairs-affine4-decode", "pairs-affine8-few", "pairs-mxfp8-general",
+                                   "pairs-affine3-rows"])
+def test_gather_scatter_rows(route):
+    """`nvq_gather_qmm_scatter`: every transposed route of the gathered product writes pair i at `out_rows[i]`; the
+    result is the plain gathered product permuted, bit for bit.  The untransposed route refuses it."""
+    rng = np.random.default_rng(7300 + len(route))
+    dtype = ref.BF16
+    experts, k, n = 6, 512, 192
+    mode = {"mxfp4": ref.MXFP4, "mxfp8": ref.MXFP8}.get(route.split("-")[1], ref.AFFINE)
+    w = make_w(rng, experts * n, k, dtype).reshape(experts, n, k)
+    if mode == ref.AFFINE:
+        bits = int(route.split("-")[1][len("affine"):])
+        group = 64
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+    else:
+        packed, scales = ref.fp_quantize(w, dtype, mode)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(nv.QuantMode.MXFP4 if mode == ref.MXFP4 else nv.QuantMode.MXFP8))
+    if route.startswith("grouped"):
+        pairs, tokens = 300, 75
+        ids = torch.from_numpy(rng.integers(0, experts, pairs).astype(np.int32)).cuda()
+        order, restore, sorted_ids, offsets = nv.moe_order(ids, experts)
+        x = to_dev(make_x(rng, tokens, k, dtype))
+        rows = torch.div(order, pairs // tokens, rounding_mode="floor").to(torch.int32)
+        plain = nv.ops.gather_qmm_grouped(x, q, rows, sorted_ids, offsets)
+        got = nv.ops.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, out_rows=order)
+        assert torch.equal(got.view(torch.int16), plain[restore.long()].view(torch.int16)), route
+        with pytest.raises(nv.InvalidArgument):
+            nv.ops.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, out_rows=order[:-1])
+        return
+    m = 3 if route.endswith("rows") else 1
+    pairs = 11
+    x = to_dev(make_x(rng, pairs * m, k, dtype).reshape(pairs, m, k))
+    lhs = torch.from_numpy(rng.permutation(pairs).astype(np.int32)).cuda()
+    rhs = torch.from_numpy(rng.integers(0, experts, pairs).astype(np.int32)).cuda()
+    perm = torch.from_numpy(rng.permutation(pairs).astype(np.int32)).cuda()
+    plain = nv.gather_qmm(x, q, lhs, rhs)
+    got = nv.gather_qmm(x, q, lhs, rhs, out_rows=perm)
+    want = torch.empty_like(plain)
+    want[perm.long()] = plain
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16)), route
+    if route == "pairs-affine4-decode":  # the untransposed route has no scattered form
+        wt = make_w(rng, experts * k, n, dtype).reshape(experts, k, n)
+        pt, st, bt = ref.affine_quantize(wt, dtype, 64, 4)
+        qt = nv.Quantized(to_dev(pt), to_dev(st), to_dev(bt), nv.Quant.affine(64, 4))
+        with pytest.raises(nv.Unsupported):
+            nv.gather_qmm(x, qt, lhs, rhs, nv.GatherQmm(transpose=False), out_rows=perm)
+
+
 @pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
 def test_quantize_dequantize_bit_exact(mode, qmode, dtype):
