@@ -1,0 +1,17 @@
+"""Copies the small quantized checkpoints the reference's own tests hold (crates/nuvec-lm/tests/fixtures/<name>/
+config.json and model.safetensors: data files, a few hundred KB together) into tests/golden/checkpoints/, where the
+loader's tests read them.  Run once in a container that has the reference: python tests/golden/copy_checkpoints.py"""
+import os
+import shutil
+
+SOURCE = "/root/reference/crates/nuvec-lm/tests/fixtures"
+NAMES = ["qwen2_q4", "gpt_oss_mxfp4", "qwen3_moe_nvfp4_gs", "llama_mxfp8", "llama_gptq", "qwen3_awq", "qwen3_gptq8_v2"]
+
+if __name__ == "__main__":
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "checkpoints")
+    for name in NAMES:
+        os.makedirs(os.path.join(here, name), exist_ok=True)
+        for part in ("config.json", "model.safetensors"):
+            shutil.copyfile(os.path.join(SOURCE, name, part), os.path.join(here, name, part))
+            os.chmod(os.path.join(here, name, part), 0o644)
+        print(name, os.path.getsize(os.path.join(here, name, "model.safetensors")), "bytes")
