@@ -174,10 +174,11 @@ class MoeMlp:
 
 
 def quantized_attention(q: torch.Tensor, k: ops.Quantized, v: ops.Quantized, scale: float,
-                        sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        sinks: Optional[torch.Tensor] = None, causal: bool = False) -> torch.Tensor:
     """fast.rs:694-718, fast/imp.rs:3992-4035 (`quantized_attention`, mlx-lm's quantized KV cache): attention of the
     queries `q [B, Hq, L, D]` over affine-quantized keys and values (codes `[B, Hkv, S, D * bits / 32]`, scales and
-    biases `[B, Hkv, S, D / group]`), grouped query heads, no mask, optional per-head `sinks [Hq]`:
+    biases `[B, Hkv, S, D / group]`), grouped query heads, optional per-head `sinks [Hq]`, optionally causal (query i
+    of L sees keys up to S - L + i, nuvec-lm's `quantized_attention`, model.rs:3646-3700):
     `softmax(scale * q k^T [, sinks]) v`.  This is the reference's composition (the one it runs wherever its fused
     kernel does not fit): both products are the library's quantized products, transposed for the keys and
     untransposed for the values; the softmax (float32 inside, one rounding) is an elementwise step outside the path."""
@@ -194,6 +195,9 @@ def quantized_attention(q: torch.Tensor, k: ops.Quantized, v: ops.Quantized, sca
     expand = lambda t: ops.Quantized(t.weight.unsqueeze(-3), t.scales.unsqueeze(-3), t.biases.unsqueeze(-3), t.quant)
     scores = ops.quantized_matmul(qs, expand(k), True)  # [B, Hkv, rep, L, S]
     s = scores.shape[-1]
+    if causal and l > 1:
+        hidden = torch.arange(s, device=q.device)[None, :] > (s - l + torch.arange(l, device=q.device))[:, None]
+        scores = scores.masked_fill(hidden, float("-inf"))
     if sinks is not None:
         column = sinks.to(scores.dtype).reshape(1, hkv, rep, 1, 1).expand(b, hkv, rep, l, 1)
         probs = torch.softmax(torch.cat([scores, column], dim=-1).float(), dim=-1).to(scores.dtype)[..., :s]

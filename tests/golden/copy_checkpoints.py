@@ -1,6 +1,7 @@
 """Copies the small quantized checkpoints the reference's own tests hold (crates/nuvec-lm/tests/fixtures/<name>/
 config.json and model.safetensors: data files, a few hundred KB together) into tests/golden/checkpoints/, where the
-loader's tests read them.  Run once in a container that has the reference: python tests/golden/copy_checkpoints.py"""
+loader's tests read them, and the recorded quantized-attention cases (tests/fixtures/kv_quant_attention.safetensors:
+queries, quantized keys and values, mlx-lm's outputs) into tests/golden/.  Run once in a container that has the reference: python tests/golden/copy_checkpoints.py"""
 import os
 import shutil
 
@@ -15,3 +16,7 @@ if __name__ == "__main__":
             shutil.copyfile(os.path.join(SOURCE, name, part), os.path.join(here, name, part))
             os.chmod(os.path.join(here, name, part), 0o644)
         print(name, os.path.getsize(os.path.join(here, name, "model.safetensors")), "bytes")
+    recorded = os.path.join(os.path.dirname(here), "kv_quant_attention.safetensors")
+    shutil.copyfile(os.path.join(SOURCE, "kv_quant_attention.safetensors"), recorded)
+    os.chmod(recorded, 0o644)
+    print("kv_quant_attention", os.path.getsize(recorded), "bytes")
