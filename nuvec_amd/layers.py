@@ -123,6 +123,19 @@ class SwitchGlu:
     gate_proj: SwitchProjection
     up_proj: SwitchProjection
     down_proj: SwitchProjection
+    gate_up_proj: Optional[SwitchProjection] = None  # `fuse_gate_up`: both projections' rows, gate first
+
+    def fuse_gate_up(self) -> "SwitchGlu":
+        """Stores the gate and up projections as one weight `[experts, 2 * hidden, ...]` (rows of the gate, then rows of
+        the up projection; a copy made once, at load time), so that the ordered pairs take one product that reads x and
+        walks the experts once instead of two.  Every output column is computed as before: the results are bit-identical."""
+        g, u = self.gate_proj, self.up_proj
+        if g.quant != u.quant or g.weight.shape != u.weight.shape or (g.bias is None) != (u.bias is None):
+            raise ops.InvalidArgument("fuse_gate_up: the gate and up projections differ in shape or quantization")
+        cat = lambda a, b: None if a is None else torch.cat([a, b], dim=1).contiguous()
+        self.gate_up_proj = SwitchProjection(cat(g.weight, u.weight), cat(g.scales, u.scales), cat(g.biases, u.biases),
+                                             cat(g.bias, u.bias), g.quant)
+        return self
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
         """`x` `[B, L, D]` through each token's experts `indices` `[B, L, k]`: `[B, L, k, D]`.  With 64 pairs or
@@ -139,8 +152,13 @@ class SwitchGlu:
         order, restore, sorted_ids, offsets = ops.moe_order(indices, experts)
         tokens = torch.div(order, k, rounding_mode="floor").to(torch.int32)  # pair t*k + j belongs to token t
         xt = x.reshape(b * l, d)
-        up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
-        gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+        if self.gate_up_proj is not None:
+            both = self.gate_up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+            hidden = both.shape[-1] // 2
+            gate, up = both[:, :hidden], both[:, hidden:]
+        else:
+            up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+            gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
         out = self.down_proj.forward_sorted_rows(swiglu(gate, up), None, sorted_ids, offsets, out_rows=order)
         return out.reshape(b, l, k, -1)
 

@@ -748,6 +748,10 @@ def test_moe_block_routes_multiplies_and_sums():
     outputs = glu(x, top)  # [B, L, k, D]
     want = moe.weighted_sum(to_host(outputs).reshape(b * l, k, d), to_host(scores).reshape(b * l, k), ref.BF16)
     assert np.array_equal(to_host(y).reshape(b * l, d).view(np.uint8), want.view(np.uint8))
+    # gate and up projections stored as one weight: one product instead of two, the same bits
+    glu.fuse_gate_up()
+    assert glu.gate_up_proj.weight.shape == (experts, 2 * inner, d // 8)
+    assert torch.equal(glu(x, top).view(torch.int16), outputs.view(torch.int16))
 
 
 @pytest.mark.parametrize("mode,qmode", [(ref.AFFINE, None), (ref.MXFP4, "MXFP4"), (ref.NVFP4, "NVFP4")])
