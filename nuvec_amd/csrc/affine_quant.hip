@@ -61,7 +61,7 @@ __device__ __forceinline__ void store8<bf16_t>(bf16_t *out, int64_t base, const 
 #pragma unroll
     for (int i = 0; i < 4; i++)
         r[i] = f32_to_bf16_pair(v[2 * i], v[2 * i + 1]);
-    *reinterpret_cast<uint4 *>(out + base) = make_uint4(r[0], r[1], r[2], r[3]);
+    stream_store(reinterpret_cast<uint4 *>(out + base), make_uint4(r[0], r[1], r[2], r[3]));
 }
 template <>
 __device__ __forceinline__ void store8<f16_t>(f16_t *out, int64_t base, const float (&v)[8]) {
@@ -70,7 +70,7 @@ __device__ __forceinline__ void store8<f16_t>(f16_t *out, int64_t base, const fl
     for (int i = 0; i < 8; i++) h[i] = (f16_t)v[i];
     uint4 q;
     __builtin_memcpy(&q, h, 16);
-    *reinterpret_cast<uint4 *>(out + base) = q;
+    stream_store(reinterpret_cast<uint4 *>(out + base), q);
 }
 
 // Stores the low `BITS` bytes of `stream` at `bytes + BITS*chunk` with the widest stores the
@@ -97,10 +97,10 @@ template <int BITS>
 __device__ __forceinline__ uint64_t load_codes(const uint8_t *bytes, int64_t chunk) {
     const uint8_t *p = bytes + chunk * BITS;
     if constexpr (BITS == 8) {
-        uint2 q = *reinterpret_cast<const uint2 *>(p);
+        uint2 q = stream_load(reinterpret_cast<const uint2 *>(p));
         return (uint64_t)q.x | ((uint64_t)q.y << 32);
     } else if constexpr (BITS == 4) {
-        return *reinterpret_cast<const uint32_t *>(p);
+        return stream_load(reinterpret_cast<const uint32_t *>(p));
     } else if constexpr (BITS == 2) {
         return *reinterpret_cast<const uint16_t *>(p);
     } else if constexpr (BITS == 6) {
@@ -207,7 +207,7 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t rows, int lanes_log2, ui
     const int64_t last = (rows - row0) * P - 1;  // beyond the end the last piece is read again and never used
     uint4 in[P];
 #pragma unroll
-    for (int j = 0; j < P; j++) in[j] = src[min((int64_t)(j * 64 + lane), last)];
+    for (int j = 0; j < P; j++) in[j] = stream_load(src + min((int64_t)(j * 64 + lane), last));
 #pragma unroll
     for (int j = 0; j < P; j++) {
         const int c = j * 64 + lane;
@@ -285,10 +285,17 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t rows, int lanes_log2, ui
     }
     const int64_t row = row0 + lane;
     if (row >= rows) return;
-    struct Words { uint32_t w[BITS]; } out;
+    if constexpr (BITS == 4) {
+        stream_store(reinterpret_cast<uint4 *>(packed + row * 4), make_uint4(words[0], words[1], words[2], words[3]));
+    } else if constexpr (BITS == 8) {
+        stream_store(reinterpret_cast<uint4 *>(packed + row * 8), make_uint4(words[0], words[1], words[2], words[3]));
+        stream_store(reinterpret_cast<uint4 *>(packed + row * 8) + 1, make_uint4(words[4], words[5], words[6], words[7]));
+    } else {
+        struct Words { uint32_t w[BITS]; } out;
 #pragma unroll
-    for (int k = 0; k < BITS; k++) out.w[k] = words[k];
-    *reinterpret_cast<Words *>(packed + row * BITS) = out;
+        for (int k = 0; k < BITS; k++) out.w[k] = words[k];
+        *reinterpret_cast<Words *>(packed + row * BITS) = out;
+    }
     if ((lane & ((1 << lanes_log2) - 1)) == 0) {
         const int64_t g = row >> lanes_log2;
         Elem<T>::store(scales, g, scale);
@@ -344,7 +351,7 @@ affine_dequantize_kernel(const uint8_t *__restrict__ packed, const T *__restrict
                 const uint32_t p = f32_to_bf16_pair(c[2 * i] * s, c[2 * i + 1] * s);
                 r[i] = f32_to_bf16_pair(u2f(p << 16) + b, u2f(p & 0xFFFF0000u) + b);
             }
-            *reinterpret_cast<uint4 *>(out + (int64_t)chunk * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+            stream_store(reinterpret_cast<uint4 *>(out + (int64_t)chunk * 8), make_uint4(r[0], r[1], r[2], r[3]));
         } else {
             float r[8];
 #pragma unroll

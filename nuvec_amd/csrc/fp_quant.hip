@@ -53,10 +53,10 @@ template <typename T> struct Raw { uint32_t w[sizeof(T) * 2]; };
 template <typename T> __device__ __forceinline__ Raw<T> load_raw(const T *w, int64_t chunk) {
     Raw<T> r;
     const uint4 *p = reinterpret_cast<const uint4 *>(w + chunk * 8);
-    const uint4 a = p[0];
+    const uint4 a = stream_load(p);
     r.w[0] = a.x; r.w[1] = a.y; r.w[2] = a.z; r.w[3] = a.w;
     if constexpr (sizeof(T) == 4) {
-        const uint4 b = p[1];
+        const uint4 b = stream_load(p + 1);
         r.w[4] = b.x; r.w[5] = b.y; r.w[6] = b.z; r.w[7] = b.w;
     }
     return r;
@@ -160,12 +160,12 @@ fp_quantize_kernel(const T *__restrict__ w, int64_t chunks, uint32_t *__restrict
                 uint32_t word = 0;
 #pragma unroll
                 for (int i = 0; i < 4; i++) word = fp4_pair<T>(word, raw, i, scale, i);
-                packed[chunk] = word;
+                __builtin_nontemporal_store(word, packed + chunk);
             } else {
                 s16x2_t lo = {0, 0}, hi = {0, 0};
                 lo = fp8_pair<T>(lo, raw, 0, scale, false); lo = fp8_pair<T>(lo, raw, 1, scale, true);
                 hi = fp8_pair<T>(hi, raw, 2, scale, false); hi = fp8_pair<T>(hi, raw, 3, scale, true);
-                reinterpret_cast<uint2 *>(packed)[chunk] = make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+                stream_store(reinterpret_cast<uint2 *>(packed) + chunk, make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi)));
             }
             if ((chunk & 3) == 0) scales[chunk >> 2] = (uint8_t)code;
             return;
@@ -238,7 +238,7 @@ template <typename T> __device__ __forceinline__ void store_values(T *out, int64
                 r[i] = __builtin_bit_cast(uint32_t, h);
             }
         }
-        *reinterpret_cast<uint4 *>(out + base) = make_uint4(r[0], r[1], r[2], r[3]);
+        stream_store(reinterpret_cast<uint4 *>(out + base), make_uint4(r[0], r[1], r[2], r[3]));
     }
 }
 
@@ -307,10 +307,10 @@ fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restr
         }
         sc_[u] = scales[chunk / F::lanes];
         if constexpr (F::bits == 4) {
-            code_lo[u] = packed[chunk];
+            code_lo[u] = stream_load(packed + chunk);
             code_hi[u] = 0u;
         } else {
-            const uint2 words = reinterpret_cast<const uint2 *>(packed)[chunk];
+            const uint2 words = stream_load(reinterpret_cast<const uint2 *>(packed) + chunk);
             code_lo[u] = words.x;
             code_hi[u] = words.y;
         }
@@ -333,13 +333,13 @@ fp_dequantize_kernel(const uint32_t *__restrict__ packed, const uint8_t *__restr
                 } else if constexpr (Elem<T>::code == 10) {
                     const bf16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 1),
                                    c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, 3);
-                    *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
-                                                                        __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+                    stream_store(reinterpret_cast<uint4 *>(out + base), make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                                   __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d)));
                 } else {
                     const f16x2_t a = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 1),
                                   c = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, 3);
-                    *reinterpret_cast<uint4 *>(out + base) = make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
-                                                                        __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d));
+                    stream_store(reinterpret_cast<uint4 *>(out + base), make_uint4(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b),
+                                                                                   __builtin_bit_cast(uint32_t, c), __builtin_bit_cast(uint32_t, d)));
                 }
                 continue;
             }

@@ -30,6 +30,28 @@ __device__ __forceinline__ uint32_t f32_to_bf16_pair(float lo, float hi) {
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
 
+// Data that is read or written once (weights of a product, the streams of quantize and dequantize): non-temporal
+// accesses keep it from displacing what is reused (x, scales, tables) in the caches.
+typedef uint32_t stream_u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t stream_u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 stream_load(const uint4 *p) {
+    const stream_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const stream_u32x4_t *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 stream_load(const uint2 *p) {
+    const stream_u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const stream_u32x2_t *>(p));
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t stream_load(const uint32_t *p) { return __builtin_nontemporal_load(p); }
+__device__ __forceinline__ void stream_store(uint4 *p, uint4 v) {
+    const stream_u32x4_t q = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(q, reinterpret_cast<stream_u32x4_t *>(p));
+}
+__device__ __forceinline__ void stream_store(uint2 *p, uint2 v) {
+    const stream_u32x2_t q = {v.x, v.y};
+    __builtin_nontemporal_store(q, reinterpret_cast<stream_u32x2_t *>(p));
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static constexpr int code = 11;

@@ -88,18 +88,18 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_sgpr, uint3
 template <int BITS>
 __device__ __forceinline__ void load_words(const uint32_t *p, uint32_t (&d)[BITS]) {
     if constexpr (BITS == 4) {
-        const uint4 q = *reinterpret_cast<const uint4 *>(p);
+        const uint4 q = stream_load(reinterpret_cast<const uint4 *>(p));
         d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
     } else if constexpr (BITS == 8) {
-        const uint4 q0 = reinterpret_cast<const uint4 *>(p)[0], q1 = reinterpret_cast<const uint4 *>(p)[1];
+        const uint4 q0 = stream_load(reinterpret_cast<const uint4 *>(p)), q1 = stream_load(reinterpret_cast<const uint4 *>(p) + 1);
         d[0] = q0.x; d[1] = q0.y; d[2] = q0.z; d[3] = q0.w;
         d[4] = q1.x; d[5] = q1.y; d[6] = q1.z; d[7] = q1.w;
     } else if constexpr (BITS == 2) {
-        const uint2 q = *reinterpret_cast<const uint2 *>(p);
+        const uint2 q = stream_load(reinterpret_cast<const uint2 *>(p));
         d[0] = q.x; d[1] = q.y;
     } else {
 #pragma unroll
-        for (int i = 0; i < BITS; i++) d[i] = p[i];
+        for (int i = 0; i < BITS; i++) d[i] = stream_load(p + i);
     }
 }
 
@@ -356,7 +356,9 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
 #pragma unroll
             for (int r = 0; r < RN; r++) {
                 const int n = n0 + r < N ? n0 + r : N - 1;  // tail rows are computed, not stored
-                wq[u][r] = *reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 3));
+                // the codes are read once: a non-temporal load keeps them from displacing x and the scales in the caches
+                // (8.1 -> 7.8 us at W[14336,4096]; the scales, shared by neighbouring lanes and rows, lose by it)
+                wq[u][r] = stream_load(reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 3)));
                 const T *ps = scales + (int64_t)n * kgroups, *pb = biases + (int64_t)n * kgroups;
                 sraw[u][r] = ps[kc >> gshift];
                 braw[u][r] = pb[kc >> gshift];
