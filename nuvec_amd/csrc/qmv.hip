@@ -507,7 +507,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
     auto load_chunk = [&](int q, Chunk &ch) {
         const int qc = q < chunks ? q : 0;
 #pragma unroll
-        for (int t = 0; t < 4; t++) ch.w[t] = *reinterpret_cast<const u32x4_t *>(wl[t] + 8 * qc);
+        for (int t = 0; t < 4; t++) ch.w[t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(wl[t] + 8 * qc));
     };
     const int tstride = mm_table_stride(K >> 6);
     unsigned char *table_s = reinterpret_cast<unsigned char *>(partial + kMmWaves * RM * kMmRows), *table_b = table_s + kMmRows * tstride;
