@@ -716,7 +716,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
     if constexpr (!std::is_same<T, float>::value) {
         if (a.bits == 4) {
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
-            // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (8.3 against
+            // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
             // 10.4 us at one row).
             if (a.m >= 4 && mfma_decode_takes<4>(a)) return run_mfma4<T, 4>(a, s);  // more rows: passes of four over grid.y
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
