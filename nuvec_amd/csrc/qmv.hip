@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
     const int n = __builtin_amdgcn_readfirstlane(blockIdx.x * kBlockWaves + wave);
     const int nc = n < N ? n : N - 1;  // tail rows are computed, not stored
     const int m0 = blockIdx.y * RM;
-    const int row_dwords = (K >> 5) * BITS, kgroups = K >> gshift;
+    const int row_dwords = (K * BITS) >> 5, kgroups = K >> gshift;  // NVFP4 rows may end in half a slice (K % 32 == 16)
     const BatchOffsets o = batch_offsets(a, blockIdx.z, row_dwords, kgroups);
     const T *x = (const T *)a.x + o.x;
     const uint32_t *wrow = (const uint32_t *)a.w + o.w + (int64_t)nc * row_dwords;
@@ -177,7 +177,16 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
         }
         const int kb = k0 + lane * 32;
         const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
-        load_words<BITS>(wrow + (kc >> 5) * BITS, st.d);
+        // NVFP4: a row of K % 32 == 16 values ends in a slice of one group; its absent half reads the present one
+        // again (codes and scale) and meets x = 0
+        const bool second = MODE != NVQ_NVFP4 || kc + 16 < K;
+        if constexpr (MODE == NVQ_NVFP4) {
+            const uint2 *p = reinterpret_cast<const uint2 *>(wrow + (kc >> 3));
+            const uint2 lo = stream_load(p), hi = stream_load(p + (second ? 1 : 0));
+            st.d[0] = lo.x; st.d[1] = lo.y; st.d[2] = hi.x; st.d[3] = hi.y;
+        } else {
+            load_words<BITS>(wrow + (kc >> 5) * BITS, st.d);
+        }
         const int64_t g = (int64_t)nc * kgroups + (kc >> gshift);
         if constexpr (kAffine) {
             st.sc[0] = ((const T *)a.scales + o.s)[g];
@@ -185,7 +194,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
         } else {
             const uint8_t *sp = (const uint8_t *)a.scales + o.s + g;
 #pragma unroll
-            for (int hf = 0; hf < kHalves; hf++) st.sc[hf] = sp[hf];
+            for (int hf = 0; hf < kHalves; hf++) st.sc[hf] = sp[second ? hf : 0];
             st.bi = 0;
         }
         return st;

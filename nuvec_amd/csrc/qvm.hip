@@ -81,9 +81,10 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
     const int passes = (M + RM - 1) / RM;
     const int bz = blockIdx.z / passes, m0 = (blockIdx.z % passes) * RM;
     const int n0 = (blockIdx.x * 64 + lane) * 32;
-    const bool live = n0 < N;  // N is a multiple of 32: a lane's outputs are all there or all absent
+    const bool live = n0 < N;  // a lane's 32 outputs are all there or all absent, but for NVFP4's N % 32 == 16:
+    const bool whole = MODE != NVQ_NVFP4 || n0 + 32 <= N;  // the last lane then owns one group of 16
     const int nc = live ? n0 : 0;
-    const int row_dwords = (N >> 5) * BITS, ngroups = N >> gshift;
+    const int row_dwords = (N * BITS) >> 5, ngroups = N >> gshift;
     const Offsets o = batch_offsets(a, bz);
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w + (nc >> 5) * BITS;
@@ -106,7 +107,13 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
     };
     auto load_row = [&](int k, Row &r) {
         const int kc = k < k_end ? k : k_end - 1;  // past the range: a harmless reload
-        load_words<BITS>(w + (int64_t)kc * row_dwords, r.d);
+        if constexpr (MODE == NVQ_NVFP4) {  // an absent second group reads the first again; its outputs are not stored
+            const uint2 *p = reinterpret_cast<const uint2 *>(w + (int64_t)kc * row_dwords);
+            const uint2 lo = p[0], hi = p[whole ? 1 : 0];
+            r.d[0] = lo.x; r.d[1] = lo.y; r.d[2] = hi.x; r.d[3] = hi.y;
+        } else {
+            load_words<BITS>(w + (int64_t)kc * row_dwords, r.d);
+        }
         r.b = 0.0f;
         if constexpr (kAffine) {
             r.s[0] = Elem<T>::load((const T *)a.scales, s_at + (int64_t)kc * ngroups);
@@ -114,7 +121,7 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
         } else {
             const uint8_t *sp = (const uint8_t *)a.scales + s_at + (int64_t)kc * ngroups;
 #pragma unroll
-            for (int hf = 0; hf < kHalves; hf++) r.s[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(sp[hf]) : e8m0_to_f32(sp[hf]));
+            for (int hf = 0; hf < kHalves; hf++) r.s[hf] = ftz(MODE == NVQ_NVFP4 ? e4m3_to_f32(sp[whole ? hf : 0]) : e8m0_to_f32(sp[hf]));
         }
 #pragma unroll
         for (int i = 0; i < RM; i++) r.x[i] = m0 + i < M ? Elem<T>::load(x, (int64_t)(m0 + i) * K + kc) : 0.0f;
@@ -154,11 +161,13 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
         if (splits == 1) {
             T *out = (T *)a.y + (o.y * M + m0 + i) * N + n0;
 #pragma unroll
-            for (int j = 0; j < 32; j++) Elem<T>::store(out, j, acc[i][j] + accb[i]);
+            for (int j = 0; j < 32; j++)
+                if (j < 16 || whole) Elem<T>::store(out, j, acc[i][j] + accb[i]);
         } else {
             float *out = partial + (((int64_t)bz * splits + blockIdx.y) * M + m0 + i) * N + n0;
 #pragma unroll
-            for (int j = 0; j < 32; j++) out[j] = acc[i][j] + accb[i];
+            for (int j = 0; j < 32; j++)
+                if (j < 16 || whole) out[j] = acc[i][j] + accb[i];
         }
     }
 }
