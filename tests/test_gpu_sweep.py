@@ -101,3 +101,21 @@ def test_gathers_sweep(seed):
     got = to_host(got)
     assert got.shape == want.shape, what
     assert_rows_close(got.reshape(-1, n), want.reshape(-1, n), dtype, what)
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32])
+def test_nvfp4_rows_ending_in_half_a_slice(dtype):
+    """NVFP4 groups hold 16 values, so a packed row may end in half of a lane's slice of 32 (K % 32 == 16 with the
+    weights stored [N, K], N % 32 == 16 with [K, N]): row strides, the absent group's codes and scale, the stores."""
+    rng = np.random.default_rng(9900 + dtype)
+    for transpose, m, k, n in [(True, 1, 16, 40), (True, 3, 112, 33), (True, 15, 1232, 96), (False, 1, 64, 16), (False, 5, 96, 48),
+                               (False, 2, 160, 2064)]:
+        inner = k if transpose else n
+        (packed, scales, _), q = quantized(rng, ref.NVFP4, dtype, 16, 4, (), n if transpose else k, inner)
+        x = make_x(rng, m, k, dtype)
+        got = to_host(nv.quantized_matmul(to_dev(x), q, transpose))
+        want = ref.quantized_matmul(x, packed, scales, None, mode=ref.NVFP4, group=16, bits=4, dtype=dtype, transpose=transpose)
+        assert got.shape == want.shape == (m, n)
+        # few outputs per row: the bar is taken against the largest output of the product, not of the row
+        g, w = ref.to_f32(got, dtype).astype(np.float64), ref.to_f32(want, dtype).astype(np.float64)
+        assert np.abs(g - w).max() <= {ref.BF16: 1e-2, ref.F32: 1e-4}[dtype] * np.abs(w).max(), (transpose, m, k, n)
