@@ -382,12 +382,12 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     if (global_scale != nullptr) return launch_qmv(a, (hipStream_t)stream);  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
     if (takes_tiled(d, a)) return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
-    // Up to four rows of 4-bit affine weights: the decode kernel (per-row work on the vector units, which is
+    // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the decode kernel (per-row work on the vector units, which is
     // cheaper than the matrix-core kernel's full dequantization up to there).  A single row of the other affine
     // widths from 3 bits: the general vector kernel (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against
     // 11.7 us with 8 bits in groups of 32; from two rows on the matrix-core kernel is ahead).  Other few-row
     // products share one weight decode on the matrix cores where that kernel takes them.
-    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 : a.bits >= 3 && a.m == 1);
+    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || (a.m <= 8 && qmv_d16_takes(a)) : a.bits >= 3 && a.m == 1);
     if (!decode && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }

@@ -84,6 +84,8 @@ struct ProductArgs {
     const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
+// Whether the 16x16x32 matrix-core decode kernel takes the product (4-bit affine, groups of 64, K = 4096).
+bool qmv_d16_takes(const ProductArgs &a);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
 bool qmm_supported(const ProductArgs &a);
 size_t qmm_workspace_bytes(const ProductArgs &a);  // float32 partial sums when K is split over the grid, else 0

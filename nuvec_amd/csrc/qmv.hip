@@ -668,6 +668,237 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
     }
 }
 
+// ── 4-bit affine, bf16 / f16, up to eight rows of x, groups of 64, K = 4096: decode on the 16x16x32 matrix instruction ──
+// The vector units only turn nibbles into elements (the magic-number form above: three shifts and four
+// v_and_or_b32 per packed word); v_mfma_f32_16x16x32 multiplies and sums.  A block of eight wavefronts owns
+// 16 RT weight rows; wavefront v owns the K slice [v K/8, (v+1) K/8) of them, NW windows of 128 values.  Lane
+// (column n = lane % 16, quarter q = lane / 16) loads the 16 bytes [32 q, 32 q + 32) of each window of its row,
+// straight into the B operand layout: word j of the load feeds matrix instruction j of the window, whose 32
+// values of K are {32 q + 8 j .. + 7}, q = 0..3, so no weight passes through the LDS.  The 16 tile rows carry
+// rows of x times groups: tile row kGpt m + g holds row m of x restricted to group g of the phase (half s = g % 2
+// of window g / 2: the operand is zero in the lanes of the other half and in the other windows), so an
+// accumulator collects the plain sums P of kGpt groups for 16 / kGpt rows of x separately and is read once per
+// phase:   y += scale * (P - B * X) + bias * X,   X = sum of the group's x,  B = 128 (bf16) or 1024 (f16).
+// One row of x: all eight groups of the slice in one accumulator; eight rows: one window (two groups) per phase.
+// X comes from the same operands of x against a weight operand of ones, once per wavefront.
+// x is staged once per block in LDS in the pair order of the nibbles; dead tile rows read a zero piece (one
+// address: a broadcast).  The wavefronts' partial rows are added in a fixed order.
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+constexpr int kD16Waves = 8, kD16Rows = 16;
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<bf16_t> {
+    __device__ static __forceinline__ floatx4_t run(uint4 a, uint4 b, floatx4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(qmf::bf16x8_t, a), __builtin_bit_cast(qmf::bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+template <> struct Mfma16<f16_t> {
+    __device__ static __forceinline__ floatx4_t run(uint4 a, uint4 b, floatx4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(qmf::f16x8_t, a), __builtin_bit_cast(qmf::f16x8_t, b), c, 0, 0, 0);
+    }
+};
+
+// Rows of x a tile carries (RM rounded up to a power of two), the groups of the slice it carries for each
+// (kGpt), and the rows of x one lane's four accumulator elements belong to.
+template <int RM> constexpr int d16_rows_pow2() { return RM <= 1 ? 1 : RM <= 2 ? 2 : RM <= 4 ? 4 : 8; }
+template <int RM, int NW> constexpr int d16_gpt() { return 16 / d16_rows_pow2<RM>() < 2 * NW ? 16 / d16_rows_pow2<RM>() : 2 * NW; }
+template <int RM, int NW> constexpr int d16_mpl() { return d16_gpt<RM, NW>() >= 4 ? 1 : 4 / d16_gpt<RM, NW>(); }
+
+// LDS of a block: x in pair order, 64 bytes of zeros, the wavefronts' partial rows.
+template <int RM, int NW, int RT>
+__host__ __device__ constexpr size_t d16_lds_bytes() {
+    return (size_t)RM * (1024 * NW * 2 + 16) + 64 + (size_t)RT * kD16Waves * d16_mpl<RM, NW>() * 64 * 4;
+}
+
+template <typename T, int RM, int NW, int RT, bool BATCHED>
+__global__ void __launch_bounds__(kD16Waves * 64) qmv4_mm16_kernel(const ProductArgs a) {
+    constexpr int K = 1024 * NW, kPieces = K / 8, kGroups = K / 64, kSlice = 128 * NW, kSliceGroups = 2 * NW;
+    constexpr int kGpt = d16_gpt<RM, NW>();          // groups per tile and row of x: 2, 4, 8 or 16
+    constexpr int kPhases = kSliceGroups / kGpt;     // accumulators a slice goes through, one after the other
+    constexpr int kMpl = d16_mpl<RM, NW>();          // rows of x per lane of the accumulator
+    static_assert(RM <= 8 && kSliceGroups % kGpt == 0 && kSliceGroups <= 8, "the slice must split into whole tiles");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    // Rows of x lie one 16-byte piece more than their length apart: the lanes of an operand read take the same piece
+    // of up to eight rows, which then fall on different banks.
+    constexpr int kRowPieces = kPieces + 1;
+    uint4 *xs = reinterpret_cast<uint4 *>(lds);                                       // [RM][kRowPieces] + 4 pieces of zeros
+    float *partial = reinterpret_cast<float *>(lds + (size_t)RM * kRowPieces * 16 + 64);                                       // [RT][waves][kMpl][64]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nl = lane & 15, kq = lane >> 4;
+    const int N = (int)a.n, M = (int)a.m;
+    constexpr int kwords = K >> 3;
+    const int n0 = blockIdx.x * kD16Rows * RT, m0 = blockIdx.y * RM;
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kGroups) : BatchOffsets{0, 0, 0, 0};
+    const T *x = (const T *)a.x + o.x;
+    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
+    T *y = (T *)a.y + o.y;
+    constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
+    uint32_t mask, magic;
+    asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
+
+    constexpr int kThreads = kD16Waves * 64, kXPer = (kPieces + kThreads - 1) / kThreads;
+    uint4 xq[RM][kXPer];
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+#pragma unroll
+        for (int p = 0; p < kXPer; p++) {
+            const int idx = tid + p * kThreads;
+            xq[i][p] = (idx < kPieces && m0 + i < M) ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * idx) : make_uint4(0, 0, 0, 0);
+        }
+    if (tid < 4) xs[RM * kRowPieces + tid] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+#pragma unroll
+        for (int p = 0; p < kXPer; p++) {
+            const int idx = tid + p * kThreads;
+            const uint4 q = xq[i][p];
+            uint4 pr;
+            pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+            pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+            pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+            pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+            if (idx < kPieces) xs[i * kRowPieces + idx] = pr;
+        }
+    // The weights are asked for once x is on its way into the LDS: requests return in the order they were made, and
+    // x queued behind the weights of every wavefront of the compute unit would arrive last.
+    uint4 wq[RT][NW];
+    int rows[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        rows[rt] = n0 + 16 * rt + nl < N ? n0 + 16 * rt + nl : N - 1;  // tail rows are computed, not stored
+        const uint4 *wp = reinterpret_cast<const uint4 *>(w + (int64_t)rows[rt] * kwords) + ((wave * kSlice + 32 * kq) >> 5);
+#pragma unroll
+        for (int d = 0; d < NW; d++) wq[rt][d] = wp[4 * d];
+    }
+    // Accumulator element j of this lane is tile row t = 4 q + j: row t / kGpt of x, group t % kGpt of the phase.
+    // The lane's scales and biases: the slice's groups (tiles of up to four groups: every lane uses them all), or
+    // the four groups of the lane's half of a tile of eight.
+    constexpr int kScaleWords = kGpt >= 8 ? 2 : kSliceGroups / 2;  // dwords of scales a lane holds
+    const int gl0 = kGpt >= 8 ? (4 * kq) % kGpt : 0;
+    uint32_t sraw[RT][kScaleWords], braw[RT][kScaleWords];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        const T *sp = scales + (int64_t)rows[rt] * kGroups + wave * kSliceGroups + gl0, *bp = biases + (int64_t)rows[rt] * kGroups + wave * kSliceGroups + gl0;
+        if constexpr (kScaleWords == 4) {
+            const uint4 sv = *reinterpret_cast<const uint4 *>(sp), bv = *reinterpret_cast<const uint4 *>(bp);
+            sraw[rt][0] = sv.x; sraw[rt][1] = sv.y; sraw[rt][2] = sv.z; sraw[rt][3] = sv.w;
+            braw[rt][0] = bv.x; braw[rt][1] = bv.y; braw[rt][2] = bv.z; braw[rt][3] = bv.w;
+        } else {
+            const uint2 sv = *reinterpret_cast<const uint2 *>(sp), bv = *reinterpret_cast<const uint2 *>(bp);
+            sraw[rt][0] = sv.x; sraw[rt][1] = sv.y;
+            braw[rt][0] = bv.x; braw[rt][1] = bv.y;
+        }
+    }
+
+    __syncthreads();
+
+    // A operands: tile row nl = row nl / kGpt of x, group nl % kGpt of the phase: window (nl % kGpt) / 2 of the
+    // phase, from the lanes of half nl % 2 only.
+    const int ma = nl / kGpt, da = (nl % kGpt) >> 1, sa = nl & 1;
+    const bool alive = (kq >> 1) == sa && ma < RM;
+    const int a_live = ma * kRowPieces + ((wave * kSlice) >> 3) + 4 * kq, a_zero = RM * kRowPieces;
+    const int me = (4 * kq) / kGpt;  // the first row of x among this lane's accumulator elements
+    // The sums X of the groups come from the matrix cores as well: the same x operands against a weight operand of
+    // ones, once per wavefront, land in the accumulator layout of P.
+    const uint4 b_ones = make_uint4(ones, ones, ones, ones);
+    floatx4_t accx[kPhases];
+#pragma unroll
+    for (int ph = 0; ph < kPhases; ph++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) accx[ph][e] = 0.0f;
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+    float part[kMpl];
+#pragma unroll
+    for (int u = 0; u < kMpl; u++) part[u] = 0.0f;
+#pragma unroll
+    for (int ph = 0; ph < kPhases; ph++) {
+        floatx4_t acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[u][e] = 0.0f;
+#pragma unroll
+        for (int dd = 0; dd < kGpt / 2; dd++) {
+            const int d = ph * (kGpt / 2) + dd;
+            const uint4 *xa = xs + ((alive && da == dd) ? a_live + 16 * d : a_zero);
+            const uint32_t dws[4] = {wq[rt][d].x, wq[rt][d].y, wq[rt][d].z, wq[rt][d].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t dw = dws[j];
+                uint4 b;
+                // written in C (the constants sit in registers, so each line is one v_and_or_b32): the compiler
+                // must see these writes to keep the matrix instruction's operand hazards
+                b.x = (dw & mask) | magic;
+                b.y = ((dw >> 4) & mask) | magic;
+                b.z = ((dw >> 8) & mask) | magic;
+                b.w = ((dw >> 12) & mask) | magic;
+                acc[j & 1] = Mfma16<T>::run(xa[j], b, acc[j & 1]);
+                if (rt == 0) accx[ph] = Mfma16<T>::run(xa[j], b_ones, accx[ph]);
+            }
+        }
+        // y += scale * (P - B X) + bias * X for the lane's four (row of x, group) pairs
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int u = kGpt >= 4 ? 0 : j / kGpt;                  // which of the lane's rows of x
+            const int gi = kGpt >= 8 ? j : ph * kGpt + j % kGpt;     // index among the lane's scales
+            const uint32_t sw = sraw[rt][gi >> 1], bw = braw[rt][gi >> 1];
+            const float sc = (gi & 1) ? Pair<T>::hi(sw) : Pair<T>::lo(sw), bi = (gi & 1) ? Pair<T>::hi(bw) : Pair<T>::lo(bw);
+            const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+            part[u] = __builtin_fmaf(sc, acc[0][j] + acc[1][j], __builtin_fmaf(bb, accx[ph][j], part[u]));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kMpl; u++) partial[((rt * kD16Waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[u] : 0.0f;
+    }
+    __syncthreads();
+    for (int out = tid; out < RT * RM * 16; out += kThreads) {
+        const int rt = out / (RM * 16), m = (out >> 4) % RM, n = out & 15;
+        float v = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < kD16Waves; wv++)
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+#pragma unroll
+                for (int u = 0; u < kMpl; u++)
+                    if ((4 * q) / kGpt + u == m) v += partial[((rt * kD16Waves + wv) * kMpl + u) * 64 + 16 * q + n];
+        if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, v);
+    }
+}
+
+// Whether the 16x16x32 decode kernel takes the product: groups of 64, K = 4096, 16-byte aligned scale and bias rows.
+inline bool d16_takes(const ProductArgs &a) {
+    if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64 || a.k != 4096) return false;
+    return ((uintptr_t)a.scales | (uintptr_t)a.biases) % 16 == 0;
+}
+
+template <typename T, int RM, int NW, int RT>
+int32_t run_d16_sized(const ProductArgs &a, hipStream_t s) {
+    constexpr size_t lds_bytes = d16_lds_bytes<RM, NW, RT>();
+    dim3 grid((unsigned)((a.n + kD16Rows * RT - 1) / (kD16Rows * RT)), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
+    const bool batched = !(a.batch == 1 && a.rhs == nullptr);
+    void (*kernel)(const ProductArgs) = batched ? qmv4_mm16_kernel<T, RM, NW, RT, true> : qmv4_mm16_kernel<T, RM, NW, RT, false>;
+    static bool configured[2] = {false, false};
+    if (lds_bytes > 64 * 1024 && !configured[batched]) {
+        NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        configured[batched] = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(kD16Waves * 64), lds_bytes, s, a);
+    NVQ_LAUNCH_CHECK("qmv4_mm16");
+    return NVQ_OK;
+}
+
+template <typename T>
+int32_t run_d16(const ProductArgs &a, hipStream_t s) {
+    if (a.m == 1) return run_d16_sized<T, 1, 4, 1>(a, s);
+    if (a.m == 2) return run_d16_sized<T, 2, 4, 1>(a, s);
+    if (a.m <= 4) return run_d16_sized<T, 4, 4, 2>(a, s);
+    return run_d16_sized<T, 8, 4, 2>(a, s);  // more rows: passes of eight over grid.y
+}
+
 // Whether the matrix-core decode kernel takes the product: groups of 64 or 128, K in whole chunks per wavefront,
 // the staged x within the LDS.
 template <int RM>
@@ -727,6 +958,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
             // 10.4 us at one row).
+            if (a.m >= 2 && d16_takes(a)) return run_d16<T>(a, s);  // 9.8 / 10.6 / 12.1 us at 2 / 4 / 8 rows of W[14336,4096] (vector and 32x32x16 kernels: 10.0 / 12.7 / 17.3)
             if (a.m >= 4 && mfma_decode_takes<4>(a)) return run_mfma4<T, 4>(a, s);  // more rows: passes of four over grid.y
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
             if (a.m == 2) return run_lds4<T, 2, 1, 8>(a, s);
@@ -749,6 +981,8 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 }
 
 }  // namespace
+
+bool qmv_d16_takes(const ProductArgs &a) { return d16_takes(a); }
 
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s) {
     if (a.batch > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld batches exceed the grid limit", (long long)a.batch);

@@ -624,6 +624,30 @@ def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
         assert_rows_close(got.reshape(12, n), want.reshape(12, n), dtype, "four rows, a matrix per item")
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("m,n", [(2, 100), (3, 33), (4, 64), (5, 47), (8, 130)])
+def test_decode_rows_on_16x16x32(dtype, m, n):
+    """Two to eight rows of x at 4 bits, groups of 64, K = 4096 (the 16x16x32 matrix-core decode kernel): every
+    tile-row layout (rows of x times groups), N not a multiple of a block's weight rows, and a matrix per item."""
+    k, group = 4096, 64
+    rng = np.random.default_rng(5100 + 16 * m + n + dtype)
+    w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, 4))
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=4, dtype=dtype)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    assert_rows_close(got, want, dtype, f"{m} rows N={n}")
+    assert_device_arithmetic(got, x, packed, scales, biases, group, 4, dtype, f"{m} rows N={n}")
+    if n == 33:  # x [2, m, K] against a matrix per item
+        xb = make_x(rng, 2 * m, k, dtype).reshape(2, m, k)
+        wb = make_w(rng, 2 * n, k, dtype).reshape(2, n, k)
+        pb, sb, bb = ref.affine_quantize(wb, dtype, group, 4)
+        qb = nv.Quantized(to_dev(pb), to_dev(sb), to_dev(bb), nv.Quant.affine(group, 4))
+        want = ref.quantized_matmul(xb, pb, sb, bb, group=group, bits=4, dtype=dtype)
+        got = to_host(nv.quantized_matmul(to_dev(xb), qb))
+        assert_rows_close(got.reshape(2 * m, n), want.reshape(2 * m, n), dtype, f"{m} rows, a matrix per item")
+
+
 @pytest.mark.parametrize("pairs,experts", [(0, 4), (5, 3), (1024, 32), (3000, 7), (5000, 130), (2049, 32), (5000, 8), (65536, 32), (100001, 200)])
 def test_moe_order_is_the_stable_argsort(pairs, experts):
     """The ordering of a mixture-of-experts layer's pairs (nuvec-lm model.rs:2193-2210): argsort of the expert
