@@ -387,7 +387,7 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     // widths from 3 bits: the general vector kernel (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against
     // 11.7 us with 8 bits in groups of 32; from two rows on the matrix-core kernel is ahead).  Other few-row
     // products share one weight decode on the matrix cores where that kernel takes them.
-    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || (a.m <= 8 && qmv_d16_takes(a)) : a.bits >= 3 && a.m == 1);
+    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || qmv_d16_takes(a) : a.bits >= 3 && a.m == 1);
     if (!decode && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }

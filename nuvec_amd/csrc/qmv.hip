@@ -668,10 +668,10 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
     }
 }
 
-// ── 4-bit affine, bf16 / f16, up to eight rows of x, groups of 64, K = 4096: decode on the 16x16x32 matrix instruction ──
+// ── 4-bit affine, bf16 / f16, up to eight rows of x, groups of 64, K = 512 W <= 8192: decode on the 16x16x32 matrix instruction ──
 // The vector units only turn nibbles into elements (the magic-number form above: three shifts and four
-// v_and_or_b32 per packed word); v_mfma_f32_16x16x32 multiplies and sums.  A block of eight wavefronts owns
-// 16 RT weight rows; wavefront v owns the K slice [v K/8, (v+1) K/8) of them, NW windows of 128 values.  Lane
+// v_and_or_b32 per packed word); v_mfma_f32_16x16x32 multiplies and sums.  A block of W = K / 512 wavefronts owns
+// 16 RT weight rows; wavefront v owns the K slice [512 v, 512 v + 512) of them, NW = 4 windows of 128 values.  Lane
 // (column n = lane % 16, quarter q = lane / 16) loads the 16 bytes [32 q, 32 q + 32) of each window of its row,
 // straight into the B operand layout: word j of the load feeds matrix instruction j of the window, whose 32
 // values of K are {32 q + 8 j .. + 7}, q = 0..3, so no weight passes through the LDS.  The 16 tile rows carry
@@ -684,7 +684,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
 // x is staged once per block in LDS in the pair order of the nibbles; dead tile rows read a zero piece (one
 // address: a broadcast).  The wavefronts' partial rows are added in a fixed order.
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
-constexpr int kD16Waves = 8, kD16Rows = 16;
+constexpr int kD16Rows = 16, kD16Slice = 512;  // weight rows of a tile; values of K per wavefront (a block has K / 512 wavefronts)
 
 template <typename T> struct Mfma16;
 template <> struct Mfma16<bf16_t> {
@@ -706,13 +706,16 @@ template <int RM, int NW> constexpr int d16_mpl() { return d16_gpt<RM, NW>() >= 
 
 // LDS of a block: x in pair order, 64 bytes of zeros, the wavefronts' partial rows.
 template <int RM, int NW, int RT>
-__host__ __device__ constexpr size_t d16_lds_bytes() {
-    return (size_t)RM * (1024 * NW * 2 + 16) + 64 + (size_t)RT * kD16Waves * d16_mpl<RM, NW>() * 64 * 4;
+__host__ __device__ constexpr size_t d16_lds_bytes(int waves) {
+    return (size_t)RM * (waves * 128 * NW * 2 + 16) + 64 + (size_t)RT * waves * d16_mpl<RM, NW>() * 64 * 4;
 }
 
 template <typename T, int RM, int NW, int RT, bool BATCHED>
-__global__ void __launch_bounds__(kD16Waves * 64) qmv4_mm16_kernel(const ProductArgs a) {
-    constexpr int K = 1024 * NW, kPieces = K / 8, kGroups = K / 64, kSlice = 128 * NW, kSliceGroups = 2 * NW;
+__global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
+    constexpr int kSlice = 128 * NW, kSliceGroups = 2 * NW;
+    static_assert(kSlice == kD16Slice, "the host sizes the block by the slice");
+    const int waves = __builtin_amdgcn_readfirstlane(blockDim.x >> 6);  // K / kSlice
+    const int K = waves * kSlice, kPieces = K >> 3, kGroups = K >> 6;
     constexpr int kGpt = d16_gpt<RM, NW>();          // groups per tile and row of x: 2, 4, 8 or 16
     constexpr int kPhases = kSliceGroups / kGpt;     // accumulators a slice goes through, one after the other
     constexpr int kMpl = d16_mpl<RM, NW>();          // rows of x per lane of the accumulator
@@ -720,14 +723,14 @@ __global__ void __launch_bounds__(kD16Waves * 64) qmv4_mm16_kernel(const Product
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     // Rows of x lie one 16-byte piece more than their length apart: the lanes of an operand read take the same piece
     // of up to eight rows, which then fall on different banks.
-    constexpr int kRowPieces = kPieces + 1;
+    const int kRowPieces = kPieces + 1;
     uint4 *xs = reinterpret_cast<uint4 *>(lds);                                       // [RM][kRowPieces] + 4 pieces of zeros
     float *partial = reinterpret_cast<float *>(lds + (size_t)RM * kRowPieces * 16 + 64);                                       // [RT][waves][kMpl][64]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
     const int N = (int)a.n, M = (int)a.m;
-    constexpr int kwords = K >> 3;
+    const int kwords = K >> 3;
     const int n0 = blockIdx.x * kD16Rows * RT, m0 = blockIdx.y * RM;
     const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kGroups) : BatchOffsets{0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
@@ -739,28 +742,21 @@ __global__ void __launch_bounds__(kD16Waves * 64) qmv4_mm16_kernel(const Product
     asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
 
-    constexpr int kThreads = kD16Waves * 64, kXPer = (kPieces + kThreads - 1) / kThreads;
-    uint4 xq[RM][kXPer];
+    // x first: a row is one 16-byte piece per thread (K / 8 pieces, K / 8 threads).
+    uint4 xq[RM];
 #pragma unroll
     for (int i = 0; i < RM; i++)
-#pragma unroll
-        for (int p = 0; p < kXPer; p++) {
-            const int idx = tid + p * kThreads;
-            xq[i][p] = (idx < kPieces && m0 + i < M) ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * idx) : make_uint4(0, 0, 0, 0);
-        }
+        xq[i] = m0 + i < M ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * tid) : make_uint4(0, 0, 0, 0);
     if (tid < 4) xs[RM * kRowPieces + tid] = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < RM; i++)
-#pragma unroll
-        for (int p = 0; p < kXPer; p++) {
-            const int idx = tid + p * kThreads;
-            const uint4 q = xq[i][p];
+    for (int i = 0; i < RM; i++) {
+            const uint4 q = xq[i];
             uint4 pr;
             pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
             pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
             pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
             pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
-            if (idx < kPieces) xs[i * kRowPieces + idx] = pr;
+            xs[i * kRowPieces + tid] = pr;
         }
     // The weights are asked for once x is on its way into the LDS: requests return in the order they were made, and
     // x queued behind the weights of every wavefront of the compute unit would arrive last.
@@ -852,51 +848,61 @@ __global__ void __launch_bounds__(kD16Waves * 64) qmv4_mm16_kernel(const Product
         }
     }
 #pragma unroll
-    for (int u = 0; u < kMpl; u++) partial[((rt * kD16Waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[u] : 0.0f;
+    for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[u] : 0.0f;
     }
     __syncthreads();
-    for (int out = tid; out < RT * RM * 16; out += kThreads) {
+    for (int out = tid; out < RT * RM * 16; out += (int)blockDim.x) {
         const int rt = out / (RM * 16), m = (out >> 4) % RM, n = out & 15;
         float v = 0.0f;
-#pragma unroll
-        for (int wv = 0; wv < kD16Waves; wv++)
+        for (int wv = 0; wv < waves; wv++)
 #pragma unroll
             for (int q = 0; q < 4; q++)
 #pragma unroll
                 for (int u = 0; u < kMpl; u++)
-                    if ((4 * q) / kGpt + u == m) v += partial[((rt * kD16Waves + wv) * kMpl + u) * 64 + 16 * q + n];
+                    if ((4 * q) / kGpt + u == m) v += partial[((rt * waves + wv) * kMpl + u) * 64 + 16 * q + n];
         if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, v);
     }
 }
 
-// Whether the 16x16x32 decode kernel takes the product: groups of 64, K = 4096, 16-byte aligned scale and bias rows.
+// Whether the 16x16x32 decode kernel takes the product: two to eight rows of x, groups of 64, K a multiple of 512
+// (a wavefront per 512 values) up to 7168, 16-byte aligned scale and bias rows.  Measured against the vector kernel
+// and the 32x32x16 kernels (us per launch at 2 / 4 / 8 rows, old -> new): W[8192,1024] 5.6 / 8.7 / 7.0 -> 3.7 / 3.9 /
+// 5.1; W[18944,3584] 11.8 / 18.4 / 30.1 -> 10.9 / 13.4 / 15.6; W[14336,4096] 9.8 / 14.2 / 17.3 -> 10.6 / 11.1 / 12.3;
+// W[13824,5120] 15.8 / 25.7 / 22.0 -> 13.3 / 15.8 / 19.1; W[28672,8192] 32.0 / 46.0 / 52.7 -> 34.9 / 42.0 / 55.7.
+// Two rows with K in (2048, 4096] stay on the vector kernel, whose single step of 4096 values is ahead there
+// (W[6144,3072]: 5.2 against 6.3 us); K = 8192 stays where it was.
 inline bool d16_takes(const ProductArgs &a) {
-    if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64 || a.k != 4096) return false;
+    if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64) return false;
+    if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || a.k > 14 * kD16Slice) return false;
+    if (a.m < 2 || a.m > 8 || (a.m == 2 && a.k > 2048 && a.k <= 4096)) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases) % 16 == 0;
 }
 
 template <typename T, int RM, int NW, int RT>
 int32_t run_d16_sized(const ProductArgs &a, hipStream_t s) {
-    constexpr size_t lds_bytes = d16_lds_bytes<RM, NW, RT>();
+    const int waves = (int)(a.k / kD16Slice);
+    const size_t lds_bytes = d16_lds_bytes<RM, NW, RT>(waves);
     dim3 grid((unsigned)((a.n + kD16Rows * RT - 1) / (kD16Rows * RT)), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
     const bool batched = !(a.batch == 1 && a.rhs == nullptr);
     void (*kernel)(const ProductArgs) = batched ? qmv4_mm16_kernel<T, RM, NW, RT, true> : qmv4_mm16_kernel<T, RM, NW, RT, false>;
     static bool configured[2] = {false, false};
     if (lds_bytes > 64 * 1024 && !configured[batched]) {
-        NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         configured[batched] = true;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(kD16Waves * 64), lds_bytes, s, a);
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmv4_mm16");
     return NVQ_OK;
 }
 
 template <typename T>
 int32_t run_d16(const ProductArgs &a, hipStream_t s) {
-    if (a.m == 1) return run_d16_sized<T, 1, 4, 1>(a, s);
     if (a.m == 2) return run_d16_sized<T, 2, 4, 1>(a, s);
-    if (a.m <= 4) return run_d16_sized<T, 4, 4, 2>(a, s);
-    return run_d16_sized<T, 8, 4, 2>(a, s);  // more rows: passes of eight over grid.y
+    // Two tiles of weight rows per block halve the staging of x; with fewer than 8192 weight rows the blocks of one
+    // tile are needed to fill the chip.
+    const bool two = a.n >= 8192;
+    if (a.m <= 4) return two ? run_d16_sized<T, 4, 4, 2>(a, s) : run_d16_sized<T, 4, 4, 1>(a, s);
+    return two ? run_d16_sized<T, 8, 4, 2>(a, s) : run_d16_sized<T, 8, 4, 1>(a, s);
 }
 
 // Whether the matrix-core decode kernel takes the product: groups of 64 or 128, K in whole chunks per wavefront,
@@ -958,7 +964,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
             // 10.4 us at one row).
-            if (a.m >= 2 && d16_takes(a)) return run_d16<T>(a, s);  // 9.8 / 10.6 / 12.1 us at 2 / 4 / 8 rows of W[14336,4096] (vector and 32x32x16 kernels: 10.0 / 12.7 / 17.3)
+            if (d16_takes(a)) return run_d16<T>(a, s);  // 9.8 / 10.6 / 12.1 us at 2 / 4 / 8 rows of W[14336,4096] (vector and 32x32x16 kernels: 10.0 / 12.7 / 17.3)
             if (a.m >= 4 && mfma_decode_takes<4>(a)) return run_mfma4<T, 4>(a, s);  // more rows: passes of four over grid.y
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
             if (a.m == 2) return run_lds4<T, 2, 1, 8>(a, s);
