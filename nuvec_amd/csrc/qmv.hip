@@ -704,10 +704,10 @@ template <int RM> constexpr int d16_rows_pow2() { return RM <= 1 ? 1 : RM <= 2 ?
 template <int RM, int NW> constexpr int d16_gpt() { return 16 / d16_rows_pow2<RM>() < 2 * NW ? 16 / d16_rows_pow2<RM>() : 2 * NW; }
 template <int RM, int NW> constexpr int d16_mpl() { return d16_gpt<RM, NW>() >= 4 ? 1 : 4 / d16_gpt<RM, NW>(); }
 
-// LDS of a block: x in pair order, 64 bytes of zeros, the wavefronts' partial rows.
+// LDS of a block: x in pair order, 64 bytes of zeros per wavefront, the wavefronts' partial rows.
 template <int RM, int NW, int RT>
 __host__ __device__ constexpr size_t d16_lds_bytes(int waves) {
-    return (size_t)RM * (waves * 128 * NW * 2 + 16) + 64 + (size_t)RT * waves * d16_mpl<RM, NW>() * 64 * 4;
+    return (size_t)RM * (waves * 128 * NW * 2 + 16) + 64 * waves + (size_t)RT * waves * d16_mpl<RM, NW>() * 64 * 4;
 }
 
 template <typename T, int RM, int NW, int RT, bool BATCHED>
@@ -724,8 +724,8 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     // Rows of x lie one 16-byte piece more than their length apart: the lanes of an operand read take the same piece
     // of up to eight rows, which then fall on different banks.
     const int kRowPieces = kPieces + 1;
-    uint4 *xs = reinterpret_cast<uint4 *>(lds);                                       // [RM][kRowPieces] + 4 pieces of zeros
-    float *partial = reinterpret_cast<float *>(lds + (size_t)RM * kRowPieces * 16 + 64);                                       // [RT][waves][kMpl][64]
+    uint4 *xs = reinterpret_cast<uint4 *>(lds);                                       // [RM][kRowPieces] + 4 pieces of zeros per wavefront
+    float *partial = reinterpret_cast<float *>(lds + (size_t)RM * kRowPieces * 16 + 64 * waves);                                       // [RT][waves][kMpl][64]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nl = lane & 15, kq = lane >> 4;
@@ -747,7 +747,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
 #pragma unroll
     for (int i = 0; i < RM; i++)
         xq[i] = m0 + i < M ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * tid) : make_uint4(0, 0, 0, 0);
-    if (tid < 4) xs[RM * kRowPieces + tid] = make_uint4(0, 0, 0, 0);
+    if (lane < 4) xs[RM * kRowPieces + 4 * wave + lane] = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < RM; i++) {
             const uint4 q = xq[i];
@@ -789,13 +789,17 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
         }
     }
 
-    __syncthreads();
+    // A thread stages piece tid of every row of x, which lies in the K slice of its own wavefront, and a wavefront
+    // reads no other slice (nor another's zeros): its LDS accesses execute in order, so no block barrier is needed.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
 
     // A operands: tile row nl = row nl / kGpt of x, group nl % kGpt of the phase: window (nl % kGpt) / 2 of the
     // phase, from the lanes of half nl % 2 only.
     const int ma = nl / kGpt, da = (nl % kGpt) >> 1, sa = nl & 1;
     const bool alive = (kq >> 1) == sa && ma < RM;
-    const int a_live = ma * kRowPieces + ((wave * kSlice) >> 3) + 4 * kq, a_zero = RM * kRowPieces;
+    const int a_live = ma * kRowPieces + ((wave * kSlice) >> 3) + 4 * kq, a_zero = RM * kRowPieces + 4 * wave;
     const int me = (4 * kq) / kGpt;  // the first row of x among this lane's accumulator elements
     // The sums X of the groups come from the matrix cores as well: the same x operands against a weight operand of
     // ones, once per wavefront, land in the accumulator layout of P.
