@@ -868,17 +868,20 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     }
 }
 
-// Whether the 16x16x32 decode kernel takes the product: two to eight rows of x, groups of 64, K a multiple of 512
+// Whether the 16x16x32 decode kernel takes the product: one to eight rows of x, groups of 64, K a multiple of 512
 // (a wavefront per 512 values) up to 7168, 16-byte aligned scale and bias rows.  Measured against the vector kernel
 // and the 32x32x16 kernels (us per launch at 2 / 4 / 8 rows, old -> new): W[8192,1024] 5.6 / 8.7 / 7.0 -> 3.7 / 3.9 /
 // 5.1; W[18944,3584] 11.8 / 18.4 / 30.1 -> 10.9 / 13.4 / 15.6; W[14336,4096] 9.8 / 14.2 / 17.3 -> 10.6 / 11.1 / 12.3;
 // W[13824,5120] 15.8 / 25.7 / 22.0 -> 13.3 / 15.8 / 19.1; W[28672,8192] 32.0 / 46.0 / 52.7 -> 34.9 / 42.0 / 55.7.
 // Two rows with K in (2048, 4096] stay on the vector kernel, whose single step of 4096 values is ahead there
-// (W[6144,3072]: 5.2 against 6.3 us); K = 8192 stays where it was.
+// (W[6144,3072]: 5.2 against 6.3 us); K = 8192 stays where it was.  One row: only where the vector kernel's steps of
+// 4096 values fit K badly (W[32768,2048] 11.8 -> 8.9, W[8192,1024] 4.4 -> 3.6, W[13824,5120] 11.5 -> 10.3; behind at
+// W[18944,3584] 8.9 -> 9.6, W[4096,4096] 4.1 -> 4.7, W[8192,7168] 8.5 -> 8.7).
 inline bool d16_takes(const ProductArgs &a) {
     if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64) return false;
     if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || a.k > 14 * kD16Slice) return false;
-    if (a.m < 2 || a.m > 8 || (a.m == 2 && a.k > 2048 && a.k <= 4096)) return false;
+    if (a.m < 1 || a.m > 8 || (a.m == 2 && a.k > 2048 && a.k <= 4096)) return false;
+    if (a.m == 1 && !(a.k <= 2048 || (a.k > 4096 && a.k <= 6144))) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases) % 16 == 0;
 }
 
@@ -901,6 +904,7 @@ int32_t run_d16_sized(const ProductArgs &a, hipStream_t s) {
 
 template <typename T>
 int32_t run_d16(const ProductArgs &a, hipStream_t s) {
+    if (a.m == 1) return run_d16_sized<T, 1, 4, 1>(a, s);
     if (a.m == 2) return run_d16_sized<T, 2, 4, 1>(a, s);
     // Two tiles of weight rows per block halve the staging of x; with fewer than 8192 weight rows the blocks of one
     // tile are needed to fill the chip.
