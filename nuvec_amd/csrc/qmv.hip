@@ -816,11 +816,9 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     for (int u = 0; u < kMpl; u++) part[u] = 0.0f;
 #pragma unroll
     for (int ph = 0; ph < kPhases; ph++) {
-        floatx4_t acc[2];
+        floatx4_t acc;
 #pragma unroll
-        for (int u = 0; u < 2; u++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[u][e] = 0.0f;
+        for (int e = 0; e < 4; e++) acc[e] = 0.0f;
 #pragma unroll
         for (int dd = 0; dd < kGpt / 2; dd++) {
             const int d = ph * (kGpt / 2) + dd;
@@ -836,7 +834,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
                 b.y = ((dw >> 4) & mask) | magic;
                 b.z = ((dw >> 8) & mask) | magic;
                 b.w = ((dw >> 12) & mask) | magic;
-                acc[j & 1] = Mfma16<T>::run(xa[j], b, acc[j & 1]);
+                acc = Mfma16<T>::run(xa[j], b, acc);
                 if (rt == 0) accx[ph] = Mfma16<T>::run(xa[j], b_ones, accx[ph]);
             }
         }
@@ -848,7 +846,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
             const uint32_t sw = sraw[rt][gi >> 1], bw = braw[rt][gi >> 1];
             const float sc = (gi & 1) ? Pair<T>::hi(sw) : Pair<T>::lo(sw), bi = (gi & 1) ? Pair<T>::hi(bw) : Pair<T>::lo(bw);
             const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
-            part[u] = __builtin_fmaf(sc, acc[0][j] + acc[1][j], __builtin_fmaf(bb, accx[ph][j], part[u]));
+            part[u] = __builtin_fmaf(sc, acc[j], __builtin_fmaf(bb, accx[ph][j], part[u]));
         }
     }
 #pragma unroll
