@@ -855,13 +855,15 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     __syncthreads();
     for (int out = tid; out < RT * RM * 16; out += (int)blockDim.x) {
         const int rt = out / (RM * 16), m = (out >> 4) % RM, n = out & 15;
+        // Row m of x is tile rows kGpt m .. kGpt m + kGpt - 1: element u of the lanes of kQ quarters from q0 on.
+        constexpr int kQ = kGpt >= 4 ? kGpt / 4 : 1;
+        const int q0 = (m * kGpt) >> 2, u = kGpt >= 4 ? 0 : ((m * kGpt) & 3) / kGpt;
+        const float *src = partial + (rt * waves * kMpl + u) * 64 + 16 * q0 + n;
         float v = 0.0f;
+#pragma unroll 4
         for (int wv = 0; wv < waves; wv++)
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-#pragma unroll
-                for (int u = 0; u < kMpl; u++)
-                    if ((4 * q) / kGpt + u == m) v += partial[((rt * waves + wv) * kMpl + u) * 64 + 16 * q + n];
+            for (int q = 0; q < kQ; q++) v += src[wv * kMpl * 64 + 16 * q];
         if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, v);
     }
 }
