@@ -869,18 +869,20 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
 }
 
 // Whether the 16x16x32 decode kernel takes the product: one to eight rows of x, groups of 64, K a multiple of 512
-// (a wavefront per 512 values) up to 7168, 16-byte aligned scale and bias rows.  Measured against the vector kernel
-// and the 32x32x16 kernels (us per launch at 2 / 4 / 8 rows, old -> new): W[8192,1024] 5.6 / 8.7 / 7.0 -> 3.7 / 3.9 /
-// 5.1; W[18944,3584] 11.8 / 18.4 / 30.1 -> 10.9 / 13.4 / 15.6; W[14336,4096] 9.8 / 14.2 / 17.3 -> 10.6 / 11.1 / 12.3;
-// W[13824,5120] 15.8 / 25.7 / 22.0 -> 13.3 / 15.8 / 19.1; W[28672,8192] 32.0 / 46.0 / 52.7 -> 34.9 / 42.0 / 55.7.
-// Two rows with K in (2048, 4096] stay on the vector kernel, whose single step of 4096 values is ahead there
-// (W[6144,3072]: 5.2 against 6.3 us); K = 8192 stays where it was.  One row: only where the vector kernel's steps of
-// 4096 values fit K badly (W[32768,2048] 11.8 -> 8.9, W[8192,1024] 4.4 -> 3.6, W[13824,5120] 11.5 -> 10.3; behind at
-// W[18944,3584] 8.9 -> 9.6, W[4096,4096] 4.1 -> 4.7, W[8192,7168] 8.5 -> 8.7).
+// (a wavefront per 512 values) up to 8192, 16-byte aligned scale and bias rows.  Measured against the vector kernel
+// and the 32x32x16 kernels (us per launch at 1 / 2 / 4 / 8 rows, old -> new):
+//   W[8192,1024]   4.2 /  5.6 /  8.6 /  7.0 ->  3.3 /  3.4 /  3.7 /  4.1     W[32768,2048] 11.8 / 15.8 / 16.2 / 21.9 ->  8.8 /  9.2 /  9.3 / 10.0
+//   W[6144,3072]   4.3 /  5.0 /  7.4 /  8.7 ->  5.1 /  5.5 /  5.6 /  6.5     W[18944,3584]  8.9 / 11.7 / 18.2 / 30.1 ->  9.2 / 10.0 / 11.5 / 12.7
+//   W[14336,4096]  7.9 /  9.7 / 12.8 / 17.3 ->  9.2 /  9.4 /  9.9 / 10.4     W[4096,4096]   3.9 /  4.2 /  7.2 /  9.9 ->  4.6 /  5.0 /  5.1 /  5.3
+//   W[13824,5120] 11.5 / 15.2 / 24.9 / 21.9 -> 10.3 / 11.7 / 11.8 / 14.0     W[8192,7168]   8.3 / 10.8 / 16.8 / 14.9 ->  8.6 /  9.0 /  9.4 / 10.1
+//   W[8192,8192]   8.6 / 11.1 / 13.5 / 16.5 -> 10.3 / 11.0 / 11.0 / 11.6     W[28672,8192] 23.9 / 32.4 / 45.5 / 52.0 -> 27.2 / 30.8 / 34.2 / 38.1
+// Three rows and more: always.  Two rows: not for 2048 < K <= 4096 with fewer than 8192 weight rows.  One row: only
+// where the vector kernel's steps of 4096 values fit K badly (K <= 2048, 4096 < K <= 6144).
 inline bool d16_takes(const ProductArgs &a) {
     if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64) return false;
-    if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || a.k > 14 * kD16Slice) return false;
-    if (a.m < 1 || a.m > 8 || (a.m == 2 && a.k > 2048 && a.k <= 4096)) return false;
+    if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || a.k > 16 * kD16Slice) return false;
+    if (a.m < 1 || a.m > 8) return false;
+    if (a.m == 2 && a.k > 2048 && a.k <= 4096 && a.n < 8192) return false;
     if (a.m == 1 && !(a.k <= 2048 || (a.k > 4096 && a.k <= 6144))) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases) % 16 == 0;
 }
