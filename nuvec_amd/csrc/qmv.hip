@@ -710,12 +710,14 @@ __host__ __device__ constexpr size_t d16_lds_bytes(int waves) {
     return (size_t)RM * (waves * 128 * NW * 2 + 16) + 64 * waves + (size_t)RT * waves * d16_mpl<RM, NW>() * 64 * 4;
 }
 
-template <typename T, int RM, int NW, int RT, bool BATCHED>
+template <typename T, int RM, int NW, int RT, bool BATCHED, bool CHUNKED>
 __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     constexpr int kSlice = 128 * NW, kSliceGroups = 2 * NW;
     static_assert(kSlice == kD16Slice, "the host sizes the block by the slice");
-    const int waves = __builtin_amdgcn_readfirstlane(blockDim.x >> 6);  // K / kSlice
-    const int K = waves * kSlice, kPieces = K >> 3, kGroups = K >> 6;
+    const int waves = __builtin_amdgcn_readfirstlane(blockDim.x >> 6);
+    // The block walks K in chunks of one slice per wavefront (a single chunk up to K = 8192).
+    const int K = (int)a.k, chunk_k = waves * kSlice, chunks = CHUNKED ? K / chunk_k : 1;  // one chunk: no loop is compiled
+    const int kPieces = chunk_k >> 3, kGroups = K >> 6;  // 16-byte pieces of x per row and chunk; groups per weight row
     constexpr int kGpt = d16_gpt<RM, NW>();          // groups per tile and row of x: 2, 4, 8 or 16
     constexpr int kPhases = kSliceGroups / kGpt;     // accumulators a slice goes through, one after the other
     constexpr int kMpl = d16_mpl<RM, NW>();          // rows of x per lane of the accumulator
@@ -742,12 +744,20 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
 
-    // x first: a row is one 16-byte piece per thread (K / 8 pieces, K / 8 threads).
+    if (lane < 4) xs[RM * kRowPieces + 4 * wave + lane] = make_uint4(0, 0, 0, 0);
+    const int me = (4 * kq) / kGpt;  // the first row of x among this lane's accumulator elements
+    float part[RT][kMpl];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int u = 0; u < kMpl; u++) part[rt][u] = 0.0f;
+#pragma unroll 1
+    for (int c = 0; c < chunks; c++) {
+    // x first: a row of the chunk is one 16-byte piece per thread.
     uint4 xq[RM];
 #pragma unroll
     for (int i = 0; i < RM; i++)
-        xq[i] = m0 + i < M ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * tid) : make_uint4(0, 0, 0, 0);
-    if (lane < 4) xs[RM * kRowPieces + 4 * wave + lane] = make_uint4(0, 0, 0, 0);
+        xq[i] = m0 + i < M ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + 8 * (c * kPieces + tid)) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < RM; i++) {
             const uint4 q = xq[i];
@@ -765,7 +775,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
         rows[rt] = n0 + 16 * rt + nl < N ? n0 + 16 * rt + nl : N - 1;  // tail rows are computed, not stored
-        const uint4 *wp = reinterpret_cast<const uint4 *>(w + (int64_t)rows[rt] * kwords) + ((wave * kSlice + 32 * kq) >> 5);
+        const uint4 *wp = reinterpret_cast<const uint4 *>(w + (int64_t)rows[rt] * kwords) + ((c * chunk_k + wave * kSlice + 32 * kq) >> 5);
 #pragma unroll
         for (int d = 0; d < NW; d++) wq[rt][d] = wp[4 * d];
     }
@@ -777,7 +787,8 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     uint32_t sraw[RT][kScaleWords], braw[RT][kScaleWords];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        const T *sp = scales + (int64_t)rows[rt] * kGroups + wave * kSliceGroups + gl0, *bp = biases + (int64_t)rows[rt] * kGroups + wave * kSliceGroups + gl0;
+        const int g0 = (c * chunk_k >> 6) + wave * kSliceGroups + gl0;
+        const T *sp = scales + (int64_t)rows[rt] * kGroups + g0, *bp = biases + (int64_t)rows[rt] * kGroups + g0;
         if constexpr (kScaleWords == 4) {
             const uint4 sv = *reinterpret_cast<const uint4 *>(sp), bv = *reinterpret_cast<const uint4 *>(bp);
             sraw[rt][0] = sv.x; sraw[rt][1] = sv.y; sraw[rt][2] = sv.z; sraw[rt][3] = sv.w;
@@ -800,7 +811,6 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     const int ma = nl / kGpt, da = (nl % kGpt) >> 1, sa = nl & 1;
     const bool alive = (kq >> 1) == sa && ma < RM;
     const int a_live = ma * kRowPieces + ((wave * kSlice) >> 3) + 4 * kq, a_zero = RM * kRowPieces + 4 * wave;
-    const int me = (4 * kq) / kGpt;  // the first row of x among this lane's accumulator elements
     // The sums X of the groups come from the matrix cores as well: the same x operands against a weight operand of
     // ones, once per wavefront, land in the accumulator layout of P.
     const uint4 b_ones = make_uint4(ones, ones, ones, ones);
@@ -811,9 +821,6 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
         for (int e = 0; e < 4; e++) accx[ph][e] = 0.0f;
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-    float part[kMpl];
-#pragma unroll
-    for (int u = 0; u < kMpl; u++) part[u] = 0.0f;
 #pragma unroll
     for (int ph = 0; ph < kPhases; ph++) {
         floatx4_t acc;
@@ -846,12 +853,16 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
             const uint32_t sw = sraw[rt][gi >> 1], bw = braw[rt][gi >> 1];
             const float sc = (gi & 1) ? Pair<T>::hi(sw) : Pair<T>::lo(sw), bi = (gi & 1) ? Pair<T>::hi(bw) : Pair<T>::lo(bw);
             const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
-            part[u] = __builtin_fmaf(sc, acc[j], __builtin_fmaf(bb, accx[ph][j], part[u]));
+            part[rt][u] = __builtin_fmaf(sc, acc[j], __builtin_fmaf(bb, accx[ph][j], part[rt][u]));
         }
     }
-#pragma unroll
-    for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[u] : 0.0f;
     }
+    asm volatile("" ::: "memory");  // the next chunk's x is written after this chunk's reads (same wavefront: in order)
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[rt][u] : 0.0f;
     __syncthreads();
     for (int out = tid; out < RT * RM * 16; out += (int)blockDim.x) {
         const int rt = out / (RM * 16), m = (out >> 4) % RM, n = out & 15;
@@ -868,6 +879,15 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     }
 }
 
+// Wavefronts of a block: one per 512 values of K up to 8192; beyond, the largest divisor of K / 512 up to 16 (the
+// block then walks K in chunks of that many slices).
+inline int d16_waves(int64_t k) {
+    const int slices = (int)(k / kD16Slice);
+    for (int wv = slices < 16 ? slices : 16; wv >= 1; wv--)
+        if (slices % wv == 0) return wv;
+    return 1;
+}
+
 // Whether the 16x16x32 decode kernel takes the product: one to eight rows of x, groups of 64, K a multiple of 512
 // (a wavefront per 512 values) up to 8192, 16-byte aligned scale and bias rows.  Measured against the vector kernel
 // and the 32x32x16 kernels (us per launch at 1 / 2 / 4 / 8 rows, old -> new):
@@ -880,8 +900,8 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
 // where the vector kernel's steps of 4096 values fit K badly (K <= 2048, 4096 < K <= 6144).
 inline bool d16_takes(const ProductArgs &a) {
     if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64) return false;
-    if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || a.k > 16 * kD16Slice) return false;
-    if (a.m < 1 || a.m > 8) return false;
+    if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || (a.k > 16 * kD16Slice && d16_waves(a.k) < 7)) return false;
+    if (a.m < 1 || a.m > 8 || (a.k > 16 * kD16Slice && a.m < 3)) return false;
     if (a.m == 2 && a.k > 2048 && a.k <= 4096 && a.n < 8192) return false;
     if (a.m == 1 && !(a.k <= 2048 || (a.k > 4096 && a.k <= 6144))) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases) % 16 == 0;
@@ -889,15 +909,22 @@ inline bool d16_takes(const ProductArgs &a) {
 
 template <typename T, int RM, int NW, int RT>
 int32_t run_d16_sized(const ProductArgs &a, hipStream_t s) {
-    const int waves = (int)(a.k / kD16Slice);
+    const int waves = d16_waves(a.k);
     const size_t lds_bytes = d16_lds_bytes<RM, NW, RT>(waves);
     dim3 grid((unsigned)((a.n + kD16Rows * RT - 1) / (kD16Rows * RT)), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
     const bool batched = !(a.batch == 1 && a.rhs == nullptr);
-    void (*kernel)(const ProductArgs) = batched ? qmv4_mm16_kernel<T, RM, NW, RT, true> : qmv4_mm16_kernel<T, RM, NW, RT, false>;
-    static bool configured[2] = {false, false};
-    if (lds_bytes > 64 * 1024 && !configured[batched]) {
+    const bool chunked = a.k > (int64_t)waves * kD16Slice;
+    void (*kernel)(const ProductArgs);
+    if constexpr (RM >= 4) {  // K beyond 8192 is taken from three rows on
+        kernel = chunked ? (batched ? qmv4_mm16_kernel<T, RM, NW, RT, true, true> : qmv4_mm16_kernel<T, RM, NW, RT, false, true>)
+                         : (batched ? qmv4_mm16_kernel<T, RM, NW, RT, true, false> : qmv4_mm16_kernel<T, RM, NW, RT, false, false>);
+    } else {
+        kernel = batched ? qmv4_mm16_kernel<T, RM, NW, RT, true, false> : qmv4_mm16_kernel<T, RM, NW, RT, false, false>;
+    }
+    static bool configured[2][2] = {{false, false}, {false, false}};
+    if (lds_bytes > 64 * 1024 && !configured[batched][chunked]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured[batched] = true;
+        configured[batched][chunked] = true;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmv4_mm16");

@@ -626,10 +626,10 @@ def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 @pytest.mark.parametrize("m,n,k", [(2, 100, 4096), (3, 33, 4096), (4, 64, 4096), (5, 47, 4096), (8, 130, 4096), (2, 40, 1024), (7, 33, 1536),
-                                   (4, 50, 8192), (8, 20, 8192), (6, 36, 3584), (1, 70, 1024), (1, 33, 2048), (1, 24, 5120)])
+                                   (4, 50, 8192), (8, 20, 8192), (6, 36, 3584), (1, 70, 1024), (1, 33, 2048), (1, 24, 5120), (4, 40, 14336), (8, 17, 12288), (3, 20, 28672)])
 def test_decode_rows_on_16x16x32(dtype, m, n, k):
     """One to eight rows of x at 4 bits, groups of 64, K a multiple of 512 up to 8192 (the 16x16x32 matrix-core decode
-    kernel, a wavefront per 512 values): every tile-row layout (rows of x times groups), the smallest and the largest
+    kernel, a wavefront per 512 values, chunks of K beyond 8192): every tile-row layout (rows of x times groups), the smallest and the largest
     block, N not a multiple of a block's weight rows, and a matrix per item."""
     group = 64
     rng = np.random.default_rng(5200 + 16 * m + n + k + dtype)
