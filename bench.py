@@ -33,8 +33,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_201_351   # read 32,367 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
-QMM_TRAFFIC_BYTES = 275_990_323  # read 212,175 KiB + written 57,346 KiB (profiles/qmm_kernel__prefill_c3_m2048.txt)
+QMV_TRAFFIC_BYTES = 33_213_687   # read 32,379 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
+QMM_TRAFFIC_BYTES = 275_968_746  # read 212,154 KiB + written 57,347 KiB (profiles/qmm_kernel__prefill_c3_m2048.txt)
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
