@@ -856,13 +856,19 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
             part[rt][u] = __builtin_fmaf(sc, acc[j], __builtin_fmaf(bb, accx[ph][j], part[rt][u]));
         }
     }
+    if constexpr (!CHUNKED) {  // a single chunk: the tile's partial rows leave the registers right away
+#pragma unroll
+        for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[rt][u] : 0.0f;
+    }
     }
     asm volatile("" ::: "memory");  // the next chunk's x is written after this chunk's reads (same wavefront: in order)
     }
+    if constexpr (CHUNKED) {
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++)
+        for (int rt = 0; rt < RT; rt++)
 #pragma unroll
-        for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[rt][u] : 0.0f;
+            for (int u = 0; u < kMpl; u++) partial[((rt * waves + wave) * kMpl + u) * 64 + lane] = me + u < RM ? part[rt][u] : 0.0f;
+    }
     __syncthreads();
     for (int out = tid; out < RT * RM * 16; out += (int)blockDim.x) {
         const int rt = out / (RM * 16), m = (out >> 4) % RM, n = out & 15;
