@@ -86,7 +86,7 @@ class GatherProduct:
     def __init__(self, lib, x, q, lhs, rhs, offsets, y, n, k, experts):
         from nuvec_amd import _lib
         pairs = rhs.numel()
-        self.d = _lib.GatherDescC(q.quant._c(), _lib.BF16, 1, 1, n, k, pairs, x.shape[0], experts)
+        self.d = _lib.GatherDescC(q.quant._c(), _lib.BF16, 1, 0, 0, 1, n, k, pairs, x.shape[0], experts)
         self.fn = lib.nvq_gather_qmm
         biases = q.biases.data_ptr() if q.biases is not None else None
         self.args = (C.byref(self.d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),

@@ -93,8 +93,13 @@ typedef struct nvq_qmm_desc {
     nvq_quant quant;
     int32_t dtype;     /* NVQ_F16 / NVQ_BF16 / NVQ_F32: x, y and (affine) scales, biases */
     int32_t transpose; /* 1: y = x . dequantize(w)^T  (MLX's default) */
-    int32_t row_exact; /* Primitive::QuantizedMatmul::row_exact (primitive.rs:491-493) */
-    int32_t rows;      /* Primitive::QuantizedMatmul::rows (primitive.rs:489-490) */
+    int32_t row_exact; /* Primitive::QuantizedMatmul::row_exact (primitive.rs:491-493; lib.rs:159-193): a product of up to
+                          8 rows per item gives each row the bits of its one-row product (itself computed with the flag
+                          set): it runs on the vector kernels, whose per-row arithmetic does not depend on the rows
+                          that share a pass, and an untransposed product splits K by the weight's shape alone
+                          (gpu.rs:6956-6981) */
+    int32_t rows;      /* Primitive::QuantizedMatmul::rows (primitive.rs:489-490): every row count takes the
+                          matrix-vector kernels, rows independent as above (qqmm's products) */
     int64_t m, n, k;
     int64_t item_rows; /* 0 = m */
     int32_t batch_ndim;
@@ -113,6 +118,10 @@ typedef struct nvq_gather_desc {
     nvq_quant quant;
     int32_t dtype;
     int32_t transpose;
+    int32_t row_exact; /* crate::row_exact() at the gather (gpu.rs:7325-7340): every pair on the vector kernels, so that a
+                          pair has the bits of its one-row product, sorted or not; the caller's grouped rule
+                          (nvq_gather_grouped) then asks for 65 rows before it passes `offsets` */
+    int32_t reserved;  /* 0 */
     int64_t m, n, k;
     int64_t pairs;
     int64_t x_batches;

@@ -54,9 +54,9 @@ class QmmDescC(C.Structure):
 
 
 class GatherDescC(C.Structure):
-    _fields_ = [("quant", QuantC), ("dtype", C.c_int32), ("transpose", C.c_int32), ("m", C.c_int64),
-                ("n", C.c_int64), ("k", C.c_int64), ("pairs", C.c_int64), ("x_batches", C.c_int64),
-                ("experts", C.c_int64)]
+    _fields_ = [("quant", QuantC), ("dtype", C.c_int32), ("transpose", C.c_int32), ("row_exact", C.c_int32),
+                ("reserved", C.c_int32), ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64), ("pairs", C.c_int64),
+                ("x_batches", C.c_int64), ("experts", C.c_int64)]
 
 
 # name -> (restype, argtypes): every symbol include/nuvec_hip.h declares.

@@ -18,10 +18,12 @@ namespace nvq {
 namespace {
 thread_local char g_error[512] = "";
 
+// Written under the mutex by nvq_init; `ready`, `device` and `units` are read without it on every call.
 struct DeviceRecord {
     std::mutex mutex;
-    bool ready = false;
-    int device = -1;
+    std::atomic<bool> ready{false};
+    std::atomic<int> device{-1};
+    std::atomic<int> units{0};
     hipDeviceProp_t prop;
 } g_device;
 
@@ -58,12 +60,22 @@ const char *mode_name(int32_t m) {
     }
 }
 
+// The bound device must also be the calling thread's current one: kernels launch on the current device, and the
+// caller's stream and buffers belong to the device it bound.
 int32_t require_device() {
-    if (!g_device.ready) return fail(NVQ_NO_DEVICE, "no device bound: call nvq_init first");
+    if (!g_device.ready.load(std::memory_order_acquire)) return fail(NVQ_NO_DEVICE, "no device bound: call nvq_init first");
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(NVQ_NO_DEVICE, "no current HIP device");
+    }
+    const int bound = g_device.device.load(std::memory_order_relaxed);
+    if (current != bound)
+        return fail(NVQ_INVALID_ARGUMENT, "the calling thread's current device is %d but the library is bound to device %d", current, bound);
     return NVQ_OK;
 }
 
-int32_t compute_units() { return g_device.ready ? g_device.prop.multiProcessorCount : 0; }
+int32_t compute_units() { return g_device.ready.load(std::memory_order_acquire) ? g_device.units.load(std::memory_order_relaxed) : 0; }
 
 // Quant::checked (quantized.rs:133-168), messages included.
 int32_t check_quant(const nvq_quant *q, const char *op) {
@@ -107,12 +119,20 @@ int32_t check_float(const char *op, int32_t dtype) {
     return NVQ_OK;
 }
 
-// The kernels use 16-byte vector accesses on every operand; allocations from hipMalloc (and
-// any sub-buffer at a multiple of 16 bytes) satisfy this.
-int32_t check_aligned(const char *op, const char *what, const void *p) {
-    if (p != nullptr && !aligned(p, 16))
-        return fail(NVQ_UNSUPPORTED, "%s: %s is not 16-byte aligned", op, what);
+// The kernels use 16-byte vector accesses on x, the packed weights, y and the workspace; allocations from
+// hipMalloc (and any sub-buffer at a multiple of 16 bytes) satisfy this.  Scales and biases are read at element
+// granularity (the kernels that fetch them in wider pieces start at the enclosing aligned piece), so they need
+// only the alignment of their element type.
+int32_t check_aligned(const char *op, const char *what, const void *p, size_t to = 16) {
+    if (p != nullptr && !aligned(p, to))
+        return fail(NVQ_UNSUPPORTED, "%s: %s is not %zu-byte aligned", op, what, to);
     return NVQ_OK;
+}
+
+int32_t check_groups_aligned(const char *op, const nvq_quant &q, int32_t dtype, const void *scales, const void *biases) {
+    const size_t to = q.mode == NVQ_AFFINE ? (size_t)dtype_size(dtype) : 1;
+    int32_t rc = check_aligned(op, "scales", scales, to);
+    return rc != NVQ_OK ? rc : check_aligned(op, "biases", biases, to);
 }
 
 #define NVQ_TRY(expr)                     \
@@ -156,6 +176,11 @@ static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
     a.m = d->m; a.n = d->n; a.k = d->k;
     a.batch = batch;
+    // Row-exact products of up to ROW_INDEPENDENT_ROWS = 8 rows per item, and products built with `rows` (every row
+    // count on the matrix-vector kernels), give each row the bits of its one-row product (lib.rs:159-193,
+    // gpu.rs:6956-6981, primitive.rs:489-493).
+    const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
+    a.row_exact = d->rows != 0 || (d->row_exact != 0 && item <= 8);
     a.batch_ndim = d->batch_ndim;
     for (int i = 0; i < d->batch_ndim; i++) {
         a.batch_shape[i] = d->batch_shape[i];
@@ -186,14 +211,16 @@ int32_t nvq_init(int32_t device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(NVQ_NO_DEVICE, "device %d is %s: this library holds gfx950 code only", device, prop.gcnArchName);
     g_device.prop = prop;
-    g_device.device = device;
-    g_device.ready = true;
+    g_device.device.store(device, std::memory_order_relaxed);
+    g_device.units.store(prop.multiProcessorCount, std::memory_order_relaxed);
+    g_device.ready.store(true, std::memory_order_release);
     return NVQ_OK;
 }
 
 int32_t nvq_get_device_info(nvq_device_info *info) {
     if (info == nullptr) return fail(NVQ_INVALID_ARGUMENT, "device_info: null output");
     NVQ_TRY(require_device());
+    std::lock_guard<std::mutex> lock(g_device.mutex);
     memset(info, 0, sizeof *info);
     info->device = g_device.device;
     info->compute_units = g_device.prop.multiProcessorCount;
@@ -238,6 +265,7 @@ static int32_t quantize_any(const nvq_quant *quant, int32_t dtype, const void *w
     NVQ_TRY(require_device());
     NVQ_TRY(check_aligned("quantize", "w", w));
     NVQ_TRY(check_aligned("quantize", "packed", packed));
+    NVQ_TRY(check_groups_aligned("quantize", *quant, dtype, scales, biases));
     const int64_t n = rows * cols;
     if (n >= (1LL << 32)) return fail(NVQ_INVALID_ARGUMENT, "quantize: %lld elements; an operand holds fewer than 2^32", (long long)n);
     if (quant->mode == NVQ_AFFINE)
@@ -295,6 +323,7 @@ static int32_t dequantize_any(const char *op, const nvq_quant *quant, int32_t dt
     NVQ_TRY(require_device());
     NVQ_TRY(check_aligned(op, "packed", packed));
     NVQ_TRY(check_aligned(op, "out", out));
+    NVQ_TRY(check_groups_aligned(op, *quant, dtype, scales, biases));
     const int64_t n = count * cols;
     if (n >= (1LL << 32) || table_rows * cols >= (1LL << 32))  // gpu.rs:1582-1590
         return fail(NVQ_INVALID_ARGUMENT, "%s: %lld elements; an operand holds fewer than 2^32", op, (long long)n);
@@ -335,9 +364,30 @@ static int32_t check_qmm(const nvq_qmm_desc *d, const char *op) {
     return NVQ_OK;
 }
 
+// The limits of the launch grids, the same ones the launch meets: batches and passes of rows travel in grid y and z
+// (at most 65535 each).  Every mode, width, element type and both orientations have a kernel: the matrix-core kernels
+// take affine and MXFP4 transposed, the general kernels the rest.
+static int32_t check_grid(const nvq_qmm_desc *d) {
+    int64_t batch = 1;
+    for (int i = 0; i < d->batch_ndim; i++) batch *= d->batch_shape[i];
+    if (batch == 0 || d->m == 0 || d->n == 0 || d->k == 0) return NVQ_OK;
+    if (batch > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld batches exceed the grid limit", (long long)batch);
+    const int64_t passes = (d->m + 3) / 4;  // the vector kernels take four rows of x per pass
+    if (!d->transpose) {
+        if (batch * (d->m == 1 ? 1 : passes) > 65535)
+            return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld row passes exceed the grid limit", (long long)(batch * passes));
+        return NVQ_OK;
+    }
+    const ProductArgs a = product_args(d, batch);
+    const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
+    if (!a.row_exact && item > 32 && qmm_supported(a)) return NVQ_OK;  // tiled: rows travel in grid x
+    if (passes > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld rows exceed the grid limit", (long long)d->m);
+    return NVQ_OK;
+}
+
 int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
     if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
-    return 1;  // every mode and both orientations: the matrix-core kernels take affine and MXFP4 transposed, the general kernels the rest
+    return check_grid(d) == NVQ_OK;
 }
 
 // Whether a transposed product goes to the tiled kernel: routed by one item's rows, as the reference does
@@ -355,7 +405,7 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
     const ProductArgs a = product_args(d, batch);
     // float32 partial sums of the splits of K: weights stored [K, N], or few tiles of a long K
     if (!d->transpose) return qvm_workspace_bytes(a);
-    return takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
+    return !a.row_exact && takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
 }
 
 static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
@@ -368,11 +418,12 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr)
         return fail(NVQ_INVALID_ARGUMENT, "quantized_matmul: null operand");
     NVQ_TRY(require_device());
-    if (!nvq_quantized_matmul_supported(d))
-        return fail(NVQ_UNSUPPORTED, "quantized_matmul: no gfx950 kernel for mode %s, transpose=%d", mode_name(d->quant.mode), d->transpose);
+    NVQ_TRY(check_grid(d));
     NVQ_TRY(check_aligned("quantized_matmul", "x", x));
     NVQ_TRY(check_aligned("quantized_matmul", "w", w));
     NVQ_TRY(check_aligned("quantized_matmul", "y", y));
+    NVQ_TRY(check_aligned("quantized_matmul", "workspace", workspace));
+    NVQ_TRY(check_groups_aligned("quantized_matmul", d->quant, d->dtype, scales, biases));
     if (d->k == 0) {  // an empty reduction is zero (crates/nuvec-cpu/src/matmul.rs:237-240)
         return launch_fill_zero(y, batch * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
     }
@@ -381,6 +432,7 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     a.global_scale = global_scale;
     if (global_scale != nullptr) return launch_qmv(a, (hipStream_t)stream);  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
+    if (a.row_exact) return launch_qmv(a, (hipStream_t)stream);  // the vector kernels: a row's bits do not depend on its neighbours
     if (takes_tiled(d, a)) return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
     // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the decode kernel (per-row work on the vector units, which is
     // cheaper than the matrix-core kernel's full dequantization up to there).  A single row of the other affine
@@ -424,6 +476,7 @@ size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *d) {
     a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
     a.m = d->m; a.n = d->n; a.k = d->k;
     a.batch = d->pairs;
+    a.row_exact = d->row_exact != 0;
     return qvm_workspace_bytes(a);
 }
 
@@ -513,6 +566,11 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(check_aligned("gather_qmm", "x", x));
     NVQ_TRY(check_aligned("gather_qmm", "w", w));
     NVQ_TRY(check_aligned("gather_qmm", "y", y));
+    NVQ_TRY(check_aligned("gather_qmm", "workspace", workspace));
+    NVQ_TRY(check_groups_aligned("gather_qmm", d->quant, d->dtype, scales, biases));
+    NVQ_TRY(check_aligned("gather_qmm", "lhs", lhs, 4));
+    NVQ_TRY(check_aligned("gather_qmm", "rhs", rhs, 4));
+    NVQ_TRY(check_aligned("gather_qmm", "offsets", offsets, 4));
     if (d->k == 0) {
         return launch_fill_zero(y, d->pairs * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
     }
@@ -525,13 +583,16 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.x_batches = d->x_batches; a.experts = d->experts;
     a.global_scale = global_scale;
     a.out_rows = out_rows;
+    a.row_exact = d->row_exact != 0;
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;
     if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     a.offsets = nullptr;
-    if (qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
+    // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
+    // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
+    if (!a.row_exact && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }
 

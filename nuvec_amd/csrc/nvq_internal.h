@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "nuvec_hip.h"
 
 namespace nvq {
@@ -82,6 +84,8 @@ struct ProductArgs {
     float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
     const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (general kernel only)
     const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
+    int32_t row_exact;              // every row takes the arithmetic of its one-row product: the vector kernels only, K split
+                                    // (weights stored [K, N]) by the weight's shape alone
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 // Whether the 16x16x32 matrix-core decode kernel takes the product (4-bit affine, groups of 64, K = 4096).

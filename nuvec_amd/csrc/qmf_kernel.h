@@ -456,7 +456,7 @@ inline int row_groups(const ProductArgs &a) {
 template <typename T, int BITS, bool FP4, int RG>
 int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS, RG>;
-    static bool configured = false;
+    static std::atomic<bool> configured = false;
     auto kernel = qmf_kernel<T, BITS, FP4, RG>;
     if (!configured) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));

@@ -296,7 +296,7 @@ inline size_t table_bytes(const ProductArgs &a) { return qmf::table_bytes(a, kRo
 template <typename T, int BITS, bool FP4>
 int32_t run(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS>;
-    static bool configured = false;
+    static std::atomic<bool> configured = false;
     auto kernel = qmg_kernel<T, BITS, FP4>;
     const size_t lds_bytes = G::kFixedLdsBytes + table_bytes(a);
     if (!configured) {

@@ -493,7 +493,7 @@ inline int k_splits(const ProductArgs &a, int cus, int *steps_per_split = nullpt
 template <typename T, int BITS, bool FP4, class TL>
 int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     using G = Geometry<BITS, TL>;
-    static bool configured[2] = {false, false};
+    static std::atomic<bool> configured[2] = {false, false};
     const bool batched = a.batch > 1;
     auto kernel = batched ? qmm_kernel<T, BITS, FP4, true, TL> : qmm_kernel<T, BITS, FP4, false, TL>;
     if (!configured[batched]) {

@@ -927,7 +927,7 @@ int32_t run_d16_sized(const ProductArgs &a, hipStream_t s) {
     } else {
         kernel = batched ? qmv4_mm16_kernel<T, RM, NW, RT, true, false> : qmv4_mm16_kernel<T, RM, NW, RT, false, false>;
     }
-    static bool configured[2][2] = {{false, false}, {false, false}};
+    static std::atomic<bool> configured[2][2] = {{false, false}, {false, false}};
     if (lds_bytes > 64 * 1024 && !configured[batched][chunked]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         configured[batched][chunked] = true;
@@ -962,7 +962,7 @@ int32_t run_mfma4(const ProductArgs &a, hipStream_t s) {
     const bool batched = !(a.batch == 1 && a.rhs == nullptr), g128 = a.group == 128;
     void (*kernel)(const ProductArgs) = g128 ? (batched ? qmv4_mfma_kernel<T, RM, true, true> : qmv4_mfma_kernel<T, RM, true, false>)
                                              : (batched ? qmv4_mfma_kernel<T, RM, false, true> : qmv4_mfma_kernel<T, RM, false, false>);
-    static bool configured[2][2] = {{false, false}, {false, false}};
+    static std::atomic<bool> configured[2][2] = {{false, false}, {false, false}};
     if (!configured[g128][batched]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         configured[g128][batched] = true;
@@ -1007,8 +1007,10 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
             // 10.4 us at one row).
-            if (d16_takes(a)) return run_d16<T>(a, s);  // 9.8 / 10.6 / 12.1 us at 2 / 4 / 8 rows of W[14336,4096] (vector and 32x32x16 kernels: 10.0 / 12.7 / 17.3)
-            if (a.m >= 4 && mfma_decode_takes<4>(a)) return run_mfma4<T, 4>(a, s);  // more rows: passes of four over grid.y
+            // Row-exact products stay on the vector kernel at every row count: a row's arithmetic there does not depend
+            // on the rows that share its pass.
+            if (!a.row_exact && d16_takes(a)) return run_d16<T>(a, s);  // 9.8 / 10.6 / 12.1 us at 2 / 4 / 8 rows of W[14336,4096] (vector and 32x32x16 kernels: 10.0 / 12.7 / 17.3)
+            if (!a.row_exact && a.m >= 4 && mfma_decode_takes<4>(a)) return run_mfma4<T, 4>(a, s);  // more rows: passes of four over grid.y
             if (a.m == 1) return run_lds4<T, 1, 1, 8>(a, s);
             if (a.m == 2) return run_lds4<T, 2, 1, 8>(a, s);
             if (a.m == 3) return run_lds4<T, 3, 1, 8>(a, s);
@@ -1031,7 +1033,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 
 }  // namespace
 
-bool qmv_d16_takes(const ProductArgs &a) { return d16_takes(a); }
+bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
 
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s) {
     if (a.batch > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld batches exceed the grid limit", (long long)a.batch);

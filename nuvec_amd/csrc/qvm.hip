@@ -230,7 +230,8 @@ int32_t run_qvm_typed(const ProductArgs &a, void *workspace, hipStream_t s) {
 // Splits of K: enough blocks for about four wavefronts per compute unit, at least 32 rows per split.
 int qvm_splits(const ProductArgs &a) {
     const int rm = a.m == 1 ? 1 : 4;
-    const int64_t base = ((a.n + 2047) / 2048) * a.batch * ((a.m + rm - 1) / rm);
+    // row-exact: the split is the one-row product's, whatever the rows and batches, so that every row keeps its bits
+    const int64_t base = ((a.n + 2047) / 2048) * (a.row_exact ? 1 : a.batch * ((a.m + rm - 1) / rm));
     const int64_t want = ((int64_t)compute_units() * 4 + base - 1) / base;
     const int64_t most = a.k / 32 > 1 ? a.k / 32 : 1;
     const int64_t splits = want < 1 ? 1 : (want > most ? most : want);

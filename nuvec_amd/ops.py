@@ -341,8 +341,11 @@ def _strides(t: torch.Tensor, nbatch: int):
     return [int(t.stride(i)) for i in range(nbatch)]
 
 
-def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, row_exact: bool = False) -> torch.Tensor:
-    """ops.rs:1031-1045, quantized.rs:446-537, primitive.rs:1279-1320."""
+def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, row_exact: bool = False, rows: bool = False,
+                     scratch: bool = True) -> torch.Tensor:
+    """ops.rs:1031-1045, quantized.rs:446-537, primitive.rs:1279-1320.  `row_exact` and `rows` are the primitive's
+    routing flags (primitive.rs:489-493; `with_row_exact`, lib.rs:159-193).  `scratch=False` hands the library no
+    workspace (a transposed product then runs without splitting K)."""
     op = "quantized_matmul"
     quant = q.quant
     group, bits = quant.checked(op)
@@ -383,7 +386,7 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     _init(x)
     out = torch.empty(x.shape[:-1] + (outer,), dtype=dtype, device=x.device)
     d = _lib.QmmDescC()
-    d.quant, d.dtype, d.transpose, d.row_exact, d.rows = quant._c(), _CODE[dtype], int(transpose), int(row_exact), 0
+    d.quant, d.dtype, d.transpose, d.row_exact, d.rows = quant._c(), _CODE[dtype], int(transpose), int(row_exact), int(rows)
     d.n, d.k = outer, inner
     if wn == 2:  # the reference's "flat" rule: every leading row of x is a row of one product
         d.m = 1
@@ -402,7 +405,7 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
             d.x_strides[i], d.w_strides[i], d.s_strides[i] = x.stride(i), w.stride(i), scales.stride(i)
     lib = _lib.load()
     need = lib.nvq_quantized_matmul_workspace_bytes(C.byref(d))
-    workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
+    workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need and scratch else None
     if g is not None:
         _lib.check(lib.nvq_quantized_matmul_scaled(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(g), _ptr(out),
                                                    _ptr(workspace), _stream()))
@@ -518,7 +521,7 @@ def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted
     if lhs.numel() != rhs.numel() or offsets.numel() != w.shape[0] or offsets.dtype != torch.int32:
         raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
     out = torch.empty((rhs.numel(), w.shape[-2]), dtype=dtype, device=x.device)
-    d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 1, w.shape[-2], columns, rhs.numel(), x.shape[0], w.shape[0])
+    d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 0, 0, 1, w.shape[-2], columns, rhs.numel(), x.shape[0], w.shape[0])
     scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
     if scatter is not None:
         _lib.check(_lib.load().nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(None),
@@ -575,6 +578,15 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
     except RuntimeError:
         raise InvalidArgument(f"{op}: index shapes {list(lhs.shape)} and {list(rhs.shape)} do not broadcast") from None
     lhs, rhs = lhs.contiguous(), rhs.contiguous()
+    gs = q.global_scale
+    if gs is not None:  # quantized.rs:620-636: one float32 value per expert
+        if quant.mode != QuantMode.NVFP4:
+            raise InvalidArgument(f"{op}: global scale is only supported for 'nvfp4' quantization mode")
+        if gs.dtype != torch.float32:
+            raise InvalidArgument(f"{op}: global scale must have dtype float32 but got {_name(gs.dtype)}")
+        if tuple(gs.shape) != tuple(w.shape[:-2]):
+            raise InvalidArgument(f"{op}: global scale must have one entry per expert with shape {list(w.shape[:-2])} but got {list(gs.shape)}")
+        gs = gs.to(x.device).contiguous()
     _init(x)
     m = x.shape[-2]
     x_batches = x.numel() // (m * inner) if m * inner else 0
@@ -586,22 +598,13 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
     if is_sorted and m == 1 and x.ndim == 3 and rhs.ndim == 1:  # quantized.rs:772-782
         offsets = sorted_offsets(rhs, experts)
     out = torch.empty(tuple(rhs.shape) + (m, outer), dtype=dtype, device=x.device)
-    d = _lib.GatherDescC(quant._c(), _CODE[dtype], int(options.transpose), m, outer, inner, rhs.numel(), x_batches, experts)
+    d = _lib.GatherDescC(quant._c(), _CODE[dtype], int(options.transpose), int(row_exact), 0, m, outer, inner, rhs.numel(), x_batches, experts)
     lib = _lib.load()
     need = lib.nvq_gather_qmm_workspace_bytes(C.byref(d))
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need else None
-    gs = q.global_scale
     scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
     if scatter is not None and lhs_indices is None and rhs_indices is None:
         raise InvalidArgument(f"{op}: output rows need indices")
-    if gs is not None:  # quantized.rs:620-636: one float32 value per expert
-        if quant.mode != QuantMode.NVFP4:
-            raise InvalidArgument(f"{op}: global scale is only supported for 'nvfp4' quantization mode")
-        if gs.dtype != torch.float32:
-            raise InvalidArgument(f"{op}: global scale must have dtype float32 but got {_name(gs.dtype)}")
-        if tuple(gs.shape) != tuple(w.shape[:-2]):
-            raise InvalidArgument(f"{op}: global scale must have one entry per expert with shape {list(w.shape[:-2])} but got {list(gs.shape)}")
-        gs = gs.to(x.device).contiguous()
     if scatter is not None:
         _lib.check(lib.nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs), _ptr(lhs),
                                               _ptr(rhs), _ptr(offsets), _ptr(scatter), _ptr(out), _ptr(workspace), _stream()))

@@ -116,8 +116,8 @@ def test_hip_conversion_matches_the_oracle(fmt, bits, group, inputs, outputs, dt
     x = ref.from_f32(rng.standard_normal((3, inputs), dtype=np.float32), dtype)
     y = to_host(nv.quantized_matmul(to_dev(x), q))
     want = ref.quantized_matmul(x, want_w, want_s, want_b, group=group, bits=bits, dtype=dtype)
-    bound = (1e-2 if dtype != ref.F32 else 1e-4) * np.max(np.abs(ref.to_f32(want, dtype)), axis=-1, keepdims=True)
-    assert np.all(np.abs(ref.to_f32(y, dtype) - ref.to_f32(want, dtype)) <= 1.5 * bound + 1e-6)
+    from tests.test_gpu_parity import assert_rows_close
+    assert_rows_close(y, want, dtype, f"converted {fmt} layer b{bits} g{group} {inputs}x{outputs}")
     with pytest.raises(nv.InvalidArgument, match="reorders the inputs"):
         bad = dict(tensors)
         bad["l.g_idx"] = torch.flip(tensors["l.g_idx"], dims=[0])

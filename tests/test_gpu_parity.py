@@ -7,20 +7,16 @@ of the formats' unit roundoffs (2.56 output ulps at the row maximum in both), 1.
 times two because the float16 dequantized weights are themselves rounded once here and twice on
 the CPU: 2.5e-3 * max|row|.
 
-How the half-precision bar is applied.  The kernels compute in the arithmetic of the reference's
-device kernels: weights dequantized with one rounding of fma(code, scale, bias) (or not rounded at
-all in the decode kernels).  The reference's CPU path rounds the dequantized weights twice in the
-element type, which changes every second bfloat16 weight by one unit in the last place.  Measured
-on the BASELINE shapes, that alone moves an output by a zero-mean error of about 0.2 x the bar
-(standard deviation), i.e. the exact products of the two weight sets already differ by 0.7-0.95 x
-the bar at the worst of 1e5 outputs, while the kernels sit within 0.4 x the bar of the exact
-product of their own weights.  So two checks are made:
-  * against the device-arithmetic oracle (`ref.quantized_matmul_device`): EVERY output within
-    half the bar;
-  * against the CPU oracle: at least 99.9 % of the outputs within the bar and none beyond 1.5 x
-    it (the tail of the weights' second rounding, not of the kernels).
-float32 has no such effect and every float32 output is held to its bar.
+How the half-precision bar is applied.  EVERY output of every product is held to the bar against the
+CPU oracle (`assert_rows_close`), and the worst ratio error / bar of each case is printed and appended to
+`gpurun_out/parity_ratios.txt` so that a run's record holds the margin.  The kernels compute in the
+arithmetic of the reference's device kernels (weights dequantized with one rounding of
+fma(code, scale, bias), or not rounded at all in the decode kernels) while the reference's CPU path rounds
+the dequantized weights twice in the element type; a second check (`assert_device_arithmetic`) holds every
+output to HALF the bar against an oracle in that device arithmetic.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -51,16 +47,37 @@ def _excess(got, want, dtype):
     return np.abs(g - w) / np.maximum(bound, 1e-30)
 
 
-def assert_rows_close(got, want, dtype, what):
-    """Against the CPU oracle (see the module docstring for the half-precision form of the bar)."""
+RATIOS = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out", "parity_ratios.txt")
+
+
+def record_ratio(what, worst, count):
+    """The worst error of a case as a fraction of its bar: printed (pytest -rA shows it) and kept on file."""
+    line = f"{what}: worst error {worst:.3f} x the bar over {count} outputs"
+    print(line, flush=True)
+    try:
+        os.makedirs(os.path.dirname(RATIOS), exist_ok=True)
+        with open(RATIOS, "a") as f:
+            f.write(line + "\n")
+    except OSError:
+        pass
+
+
+def assert_rows_close(got, want, dtype, what, exact_weights=False):
+    """Against the CPU oracle: every output within the bar of its row (1e-2 * max|row| for bfloat16).
+
+    The one exception, recorded with its ratio like every case: half-precision affine products whose rows hold fewer
+    than 512 outputs.  The bar scales with the largest of a row's outputs, about four standard deviations of an output
+    in a row of thousands (the BASELINE shapes) but only two in a row of 32; the difference between the device's single
+    rounding of a dequantized weight and the CPU's two has a standard deviation of 0.14 x the bar at the BASELINE shapes
+    and twice that in such short rows, so their worst output is allowed 1.5 x the bar.  `exact_weights` (block formats,
+    whose weights both sides hold exactly) takes the exception away."""
     ratio = _excess(got, want, dtype)
     worst = float(np.max(ratio)) if ratio.size else 0.0
-    if dtype == ref.F32:
-        assert worst <= 1.0, f"{what}: max error is {worst:.3f} x the bound"
-        return
+    record_ratio(what, worst, ratio.size)
     beyond = int(np.count_nonzero(ratio > 1.0))
-    assert worst <= 1.5 and beyond <= max(1, ratio.size // 1000), \
-        f"{what}: max error is {worst:.3f} x the bound, {beyond} of {ratio.size} outputs beyond it"
+    columns = np.asarray(want).shape[-1]
+    limit = 1.5 if dtype != ref.F32 and columns < 512 and not exact_weights else 1.0
+    assert worst <= limit, f"{what}: max error is {worst:.3f} x the bound, {beyond} of {ratio.size} outputs beyond it"
 
 
 def assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what):
@@ -178,6 +195,46 @@ def test_config4_odd_bit_widths(group, bits, m):
     assert_device_arithmetic(got, x, packed, scales, biases, group, bits, ref.BF16, f"config 4 b{bits} g{group} M={m}")
 
 
+@pytest.mark.parametrize("group,bits", [(64, 3), (32, 8)])
+def test_config4_odd_bit_widths_512_rows(group, bits):
+    """BASELINE config 4 at M = 512: the tiled kernel with K split over the grid and the partial sums added from the
+    caller's workspace, and the same product handed no workspace (K not split).  The whole product against the oracle."""
+    import ctypes as C
+
+    from nuvec_amd import _lib
+    rng = np.random.default_rng(20260104 + bits)
+    m, n, k = 512, 4096, 4096
+    w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, group, bits)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(group, bits))
+    assert np.array_equal(to_host(q.weight), packed)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=ref.BF16, threads=8)
+    d = _lib.QmmDescC()
+    d.quant, d.dtype, d.transpose = nv.Quant.affine(group, bits)._c(), _lib.BF16, 1
+    d.m, d.n, d.k, d.item_rows = m, n, k, m
+    need = _lib.load().nvq_quantized_matmul_workspace_bytes(C.byref(d))
+    assert need > 0, "this product is expected to split K through a workspace"
+    xd = to_dev(x)
+    split = to_host(nv.quantized_matmul(xd, q))
+    assert_rows_close(split, want, ref.BF16, f"config 4 b{bits} g{group} M=512, K split through the workspace")
+    some = np.sort(rng.choice(m, 48, replace=False))
+    assert_device_arithmetic(split[some], x[some], packed, scales, biases, group, bits, ref.BF16, f"config 4 b{bits} g{group} M=512")
+    unsplit = to_host(nv.quantized_matmul(xd, q, scratch=False))
+    assert_rows_close(unsplit, want, ref.BF16, f"config 4 b{bits} g{group} M=512, no workspace")
+
+
+def test_untransposed_product_needs_its_workspace():
+    """Weights stored [K, N] split K through the caller's workspace: handed none, the call is refused, not run."""
+    rng = np.random.default_rng(3)
+    k, n, m = 512, 256, 3
+    w, x = make_w(rng, k, n, ref.BF16), make_x(rng, m, k, ref.BF16)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(64, 4))
+    y = nv.quantized_matmul(to_dev(x), q, transpose=False)
+    assert y.shape == (m, n)
+    with pytest.raises((nv.InvalidArgument, nv.Unsupported)):
+        nv.quantized_matmul(to_dev(x), q, transpose=False, scratch=False)
+
+
 @pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
 @pytest.mark.parametrize("group,bits", [(64, 4), (32, 2), (128, 6), (64, 5), (128, 1), (32, 3), (64, 8)])
 def test_ragged_shapes_every_width(dtype, group, bits):
@@ -206,7 +263,7 @@ def test_mxfp4_quantize_and_products():
         x = make_x(rng, m, k, ref.BF16)
         want = ref.quantized_matmul(x, packed, scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16)
         got = to_host(nv.quantized_matmul(to_dev(x), q))
-        assert_rows_close(got, want, ref.BF16, f"mxfp4 M={m}")
+        assert_rows_close(got, want, ref.BF16, f"mxfp4 M={m}", exact_weights=True)
 
 
 def test_empty_and_degenerate_products():
@@ -237,7 +294,7 @@ def test_sorted_offsets_and_gather_pairs():
     want = ref.gather_qmm(x, packed, scales, None, np.arange(rows, dtype=np.uint32), rhs, mode=ref.MXFP4, group=32,
                           bits=4, dtype=ref.BF16)
     assert got.shape == (rows, 1, n)
-    assert_rows_close(got, want, ref.BF16, "sorted gather")
+    assert_rows_close(got, want, ref.BF16, "sorted gather", exact_weights=True)
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
@@ -289,8 +346,12 @@ def test_config3_prefill_bf16_4bit_g64():
     g32 = ref.to_f32(got, ref.BF16)
     row_max = np.max(np.abs(g32), axis=1)
     ratio = np.abs(g32[rows, cols].astype(np.float64) - want.astype(np.float64)) / (1e-2 * row_max[rows])
-    assert float(np.max(ratio)) <= 1.5 and np.count_nonzero(ratio > 1.0) <= 1, f"max sample error {float(np.max(ratio)):.3f} x the bound"
-    some = np.sort(rng.choice(m, 64, replace=False))  # whole rows against the device arithmetic
+    record_ratio("config 3, 6000 sampled outputs", float(np.max(ratio)), ratio.size)
+    assert float(np.max(ratio)) <= 1.0, f"max sample error {float(np.max(ratio)):.3f} x the bound"
+    some = np.sort(rng.choice(m, 256, replace=False))  # whole rows against the CPU oracle (3.7 million outputs) ...
+    want_rows = ref.quantized_matmul(x[some], packed, scales, biases, group=64, bits=4, dtype=ref.BF16, threads=16)
+    assert_rows_close(got[some], want_rows, ref.BF16, "config 3, 256 whole rows")
+    some = some[::4]  # ... and against the device arithmetic
     assert_device_arithmetic(got[some], x[some], packed, scales, biases, 64, 4, ref.BF16, "config 3, 64 whole rows")
     for i in (0, 777, m - 1):
         one = ref.to_f32(to_host(nv.quantized_matmul(xd[i:i + 1], q)), ref.BF16)[0]
@@ -322,9 +383,9 @@ def test_config5_moe_gather_mxfp4():
     assert got.shape == (1024, 1, n)
     want = ref.gather_qmm(x, packed, scales, None, np.arange(1024, dtype=np.uint32), rhs, mode=ref.MXFP4, group=32, bits=4,
                           dtype=ref.BF16, threads=8)
-    assert_rows_close(got, want, ref.BF16, "config 5 grouped")
+    assert_rows_close(got, want, ref.BF16, "config 5 grouped", exact_weights=True)
     unsorted = to_host(nv.gather_qmm(to_dev(x[:40]), q, None, rhs_dev[:40], nv.GatherQmm(sorted_indices=False)))
-    assert_rows_close(unsorted, want[:40], ref.BF16, "config 5 per pair")
+    assert_rows_close(unsorted, want[:40], ref.BF16, "config 5 per pair", exact_weights=True)
 
 
 def test_grouped_gather_edge_cases():
@@ -411,7 +472,7 @@ def test_tiled_mxfp4():
     q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.mxfp4()) if hasattr(nv.Quant, "mxfp4") else nv.quantize(to_dev(w), nv.QuantMode.MXFP4)
     want = ref.quantized_matmul(x, packed, scales, None, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16, threads=8)
     got = to_host(nv.quantized_matmul(to_dev(x), q))
-    assert_rows_close(got, want, ref.BF16, "tiled mxfp4")
+    assert_rows_close(got, want, ref.BF16, "tiled mxfp4", exact_weights=True)
 
 
 @pytest.mark.parametrize("mode,qmode", [(ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])

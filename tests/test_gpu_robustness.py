@@ -1,0 +1,180 @@
+"""Row independence, run-to-run determinism and re-entrancy of the HIP path, through the C ABI.
+
+Mirrors the reference's tests of the same contracts:
+  * `few_row_products_equal_one_row_products_bit_for_bit` (crates/nuvec-core/tests/quantized.rs:794-831) and
+    `sorted_few_row_gathers_keep_the_one_row_bits` (:1798-1900): under `row_exact` a product of up to eight rows gives
+    every row the bits of its one-row product, and a sorted gather the bits of the unsorted one;
+  * `kernels_are_deterministic` (crates/nuvec-core/tests/determinism.rs:47-88): every route, run again into reused
+    buffers, gives identical bits;
+  * many host threads evaluate at once (eval.rs:129-137): eight threads on their own streams get the serial results.
+"""
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+import nuvec_amd as nv
+from oracle import ref
+from tests.hip_backend import TORCH, to_dev, to_host
+from tests.test_gpu_parity import assert_rows_close, make_w, make_x
+
+pytestmark = pytest.mark.gpu
+
+
+def bits_of(t):
+    return to_host(t).view(np.uint8)
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16, ref.F32])
+@pytest.mark.parametrize("m,k,n,group,bits", [(6, 4096, 512, 64, 4), (5, 1024, 1000, 32, 4), (4, 2048, 256, 128, 4),
+                                              (8, 4096, 14336, 64, 4), (7, 1024, 130, 64, 3), (3, 512, 96, 32, 8),
+                                              (8, 768, 64, 64, 2), (2, 640, 72, 128, 6)])
+def test_row_exact_rows_equal_their_one_row_products(dtype, m, k, n, group, bits):
+    """tests/quantized.rs:794-831, widened to the other code widths: odd and even row counts, N off the block size."""
+    rng = np.random.default_rng(m * 1000 + bits)
+    w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(group, bits))
+    xd = to_dev(x)
+    both = bits_of(nv.quantized_matmul(xd, q, row_exact=True))
+    for r in range(m):
+        one = bits_of(nv.quantized_matmul(xd[r:r + 1], q, row_exact=True))
+        assert np.array_equal(one[0], both[r]), f"row {r} of {m} differs from its one-row product"
+    # the values are the product's
+    packed, scales, biases = to_host(q.weight), to_host(q.scales), to_host(q.biases)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype)
+    assert_rows_close(to_host(nv.quantized_matmul(xd, q, row_exact=True)), want, dtype, f"row-exact b{bits} g{group} M={m} K={k} N={n}")
+    # `rows` (every row count on the matrix-vector kernels) keeps rows independent at any count
+    many = np.concatenate([x, x[::-1], x, x[:1]])
+    wide = bits_of(nv.quantized_matmul(to_dev(many), q, rows=True))
+    assert np.array_equal(wide[:m], both) and np.array_equal(wide[-1], both[0])
+
+
+@pytest.mark.parametrize("mode", ["MXFP4", "MXFP8", "NVFP4"])
+def test_row_exact_block_formats_and_untransposed(mode):
+    rng = np.random.default_rng(5)
+    m, k, n = 7, 1024, 200
+    w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+    q = nv.quantize(to_dev(w), nv.QuantMode[mode])
+    xd = to_dev(x)
+    both = bits_of(nv.quantized_matmul(xd, q, row_exact=True))
+    for r in range(m):
+        assert np.array_equal(bits_of(nv.quantized_matmul(xd[r:r + 1], q, row_exact=True))[0], both[r]), f"{mode}: row {r}"
+    # weights stored [K, N]: K is split over the grid by the weight's shape alone
+    wt = make_w(rng, k, 256, ref.BF16)
+    qt = nv.quantize(to_dev(wt), nv.QuantMode[mode])
+    both = bits_of(nv.quantized_matmul(xd, qt, transpose=False, row_exact=True))
+    for r in range(m):
+        one = bits_of(nv.quantized_matmul(xd[r:r + 1], qt, transpose=False, row_exact=True))
+        assert np.array_equal(one[0], both[r]), f"{mode} untransposed: row {r}"
+
+
+@pytest.mark.parametrize("dtype", [ref.F16, ref.BF16])
+@pytest.mark.parametrize("bits", [2, 3, 4, 8])
+def test_sorted_few_row_gathers_keep_the_one_row_bits(dtype, bits):
+    """tests/quantized.rs:1798-1900: 2 to 8 tokens' top-8 of 16 experts, sorted by expert as a mixture-of-experts
+    layer sorts them, against the unsorted per-pair gather and against each token alone."""
+    rng = np.random.default_rng(0x1D5 + bits)
+    experts, n, k, top = 16, 256, 512, 8
+    w = ref.from_f32((rng.standard_normal((experts, n, k)) * 0.1).astype(np.float32), dtype)
+    q = nv.quantize(to_dev(w), nv.Quant.affine(64, bits))
+    for tokens in (2, 5, 8):
+        ids = np.stack([rng.permutation(experts)[:top] for _ in range(tokens)]).astype(np.int64)
+        x = to_dev(make_x(rng, tokens, k, dtype)).reshape(1, tokens, 1, 1, k)
+        idx = torch.from_numpy(ids).cuda().reshape(1, tokens, top)
+        unsorted = nv.gather_qmm(x, q, None, idx, nv.GatherQmm(), row_exact=True)
+        assert unsorted.shape == (1, tokens, top, 1, n)
+        flat = idx.reshape(-1)
+        order = torch.argsort(flat, stable=True)
+        token_of = torch.arange(tokens * top, device="cuda") // top
+        rows = x.reshape(-1, 1, k)[token_of[order]]
+        got = nv.gather_qmm(rows, q, None, flat[order], nv.GatherQmm(sorted_indices=True), row_exact=True)
+        restored = got[torch.argsort(order)].reshape(1, tokens, top, 1, n)
+        assert np.array_equal(bits_of(restored), bits_of(unsorted)), f"b{bits}, {tokens} tokens: the sorted gather differs"
+        for t in range(tokens):
+            one = nv.gather_qmm(x[:, t:t + 1], q, None, idx[:, t:t + 1], nv.GatherQmm(), row_exact=True)
+            assert np.array_equal(bits_of(one)[0, 0], bits_of(restored)[0, t]), f"b{bits}, token {t} of {tokens} alone differs"
+
+
+def determinism_cases():
+    """One product per route (determinism.rs:47-88 for this path): decode, few rows on both matrix-core kernels, tiled
+    with and without a split of K, weights stored [K, N], batched, the general kernel's modes, grouped and per-pair
+    gathers, quantize and dequantize."""
+    rng = np.random.default_rng(123)
+    w = make_w(rng, 4096, 4096, ref.BF16)
+    wd = to_dev(w)
+    q4 = nv.quantize(wd, nv.Quant.affine(64, 4))
+    cases = {}
+    for rows in (1, 2, 4, 8, 16, 40, 256, 512):
+        x = to_dev(make_x(rng, rows, 4096, ref.BF16))
+        cases[f"b4 M={rows}"] = lambda x=x: nv.quantized_matmul(x, q4)
+    x1, x512 = to_dev(make_x(rng, 1, 4096, ref.BF16)), to_dev(make_x(rng, 512, 4096, ref.BF16))
+    cases["b4 M=512 unsplit"] = lambda: nv.quantized_matmul(x512, q4, scratch=False)
+    cases["b4 untransposed"] = lambda: nv.quantized_matmul(x1, q4, transpose=False)
+    cases["b4 row-exact M=8"] = lambda: nv.quantized_matmul(x512[:8], q4, row_exact=True)
+    for group, bits in ((64, 3), (32, 8), (128, 2), (64, 6), (64, 5)):
+        q = nv.quantize(wd[:1024], nv.Quant.affine(group, bits))
+        for rows in (1, 16, 300):
+            cases[f"b{bits} M={rows}"] = lambda q=q, rows=rows: nv.quantized_matmul(x512[:rows], q)
+    xf = to_dev(make_x(rng, 3, 4096, ref.F32))
+    qf = nv.quantize(wd[:512].float(), nv.Quant.affine(64, 4))
+    cases["f32 M=3"] = lambda: nv.quantized_matmul(xf, qf)
+    experts = to_dev(make_w(rng, 16 * 512, 1024, ref.BF16)).reshape(16, 512, 1024)
+    ids = (torch.arange(512, device="cuda") * 16 // 512)
+    xe = to_dev(make_x(rng, 512, 1024, ref.BF16)).reshape(512, 1, 1024)
+    eq = nv.quantize(experts, nv.Quant.affine(64, 4))
+    cases["grouped gather b4"] = lambda: nv.gather_qmm(xe, eq, None, ids, nv.GatherQmm(sorted_indices=True))
+    cases["pair gather b4"] = lambda: nv.gather_qmm(xe[:24], eq, None, ids[:24].flip(0), nv.GatherQmm())
+    for mode in ("MXFP4", "MXFP8", "NVFP4"):
+        qm = nv.quantize(wd[:512], nv.QuantMode[mode])
+        cases[f"{mode} M=64"] = lambda qm=qm: nv.quantized_matmul(x512[:64], qm)
+        em = nv.quantize(experts, nv.QuantMode[mode])
+        if mode == "NVFP4":
+            em = nv.Quantized(em.weight, em.scales, None, em.quant, torch.full((16,), 0.5, device="cuda"))
+        cases[f"{mode} grouped gather"] = lambda em=em: nv.gather_qmm(xe, em, None, ids, nv.GatherQmm(sorted_indices=True))
+    cases["quantize b4"] = lambda: nv.quantize(wd, nv.Quant.affine(64, 4)).weight
+    cases["quantize mxfp4"] = lambda: nv.quantize(wd, nv.QuantMode.MXFP4).weight
+    cases["dequantize b4"] = lambda: nv.dequantize(q4)
+    return cases
+
+
+def test_kernels_are_deterministic_under_buffer_reuse():
+    """Every route three times; between the runs the outputs are dropped, so the allocator hands the same buffers out
+    again (and scratch memory holds the previous run's partial sums)."""
+    cases = determinism_cases()
+    first = {name: bits_of(run()).copy() for name, run in cases.items()}
+    torch.cuda.synchronize()
+    for again in range(2):
+        for name, run in cases.items():
+            assert np.array_equal(bits_of(run()), first[name]), f"{name}: run {again + 2} differs from the first"
+
+
+def test_eight_host_threads_on_their_own_streams():
+    """The library is re-entrant: eight threads call the C ABI at once, each on a stream of its own, and every one
+    gets the bits of the serial run."""
+    cases = determinism_cases()
+    names = list(cases)
+    serial = {name: bits_of(cases[name]()).copy() for name in names}
+    torch.cuda.synchronize()
+    failures, barrier = [], threading.Barrier(8)
+
+    def work(t):
+        try:
+            stream = torch.cuda.Stream()
+            barrier.wait()
+            with torch.cuda.stream(stream):
+                for rep in range(3):
+                    for name in names[t % 3::3] + names:  # threads walk the routes in different orders
+                        out = cases[name]()
+                        stream.synchronize()
+                        if not np.array_equal(bits_of(out), serial[name]):
+                            failures.append(f"thread {t}: {name} differs from the serial run")
+        except Exception as e:  # noqa: BLE001 - reported below
+            failures.append(f"thread {t}: {type(e).__name__}: {e}")
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(8)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not failures, failures[:5]
