@@ -10,7 +10,7 @@ stream through the C ABI and rotate through enough distinct weight copies that n
 its weights in the 256 MB last-level cache.  The prefill-shaped product (configs[2], M = 2048)
 is timed the same way and reported in the same line as `qmm`.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-qmm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-qmm] [--no-configs] [--no-peaks]
 
 Prints one JSON line.
 """
@@ -139,9 +139,10 @@ def time_launches(calls, steps, warmup, graph=True):
     return start.elapsed_time(stop) / (reps * n), reps * n
 
 
-def cpu_baseline(seconds_budget=20.0):
-    """The CPU restatement of nuvec's path (dequantize the whole matrix, then the fixed-order
-    few-row product) on this host's cores, on a bounded sample of the same workload."""
+def cpu_baseline(seconds_budget=24.0):
+    """The CPU restatement of nuvec's path (dequantize the whole matrix on one thread as the reference does, then the
+    product) on this host's cores, on a bounded sample of the same workload: the decode product of configs[1] on one
+    thread and on all cores, and rows of the prefill product of configs[2] (the path for more than 16 rows)."""
     import numpy as np
 
     from oracle import ref
@@ -149,19 +150,73 @@ def cpu_baseline(seconds_budget=20.0):
     w = ref.from_f32((rng.standard_normal((N, K)) * 0.02).astype(np.float32), ref.BF16)
     x = ref.from_f32(rng.standard_normal((1, K)).astype(np.float32), ref.BF16)
     packed, scales, biases = ref.affine_quantize(w, ref.BF16, GROUP, BITS)
-    threads = max(1, min(ref.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1)))
-    run = lambda: ref.quantized_matmul(x, packed, scales, biases, group=GROUP, bits=BITS, dtype=ref.BF16, threads=threads)
-    run()
-    done, t0 = 0, time.perf_counter()
-    while done < 3 or (time.perf_counter() - t0 < seconds_budget / 2 and done < 50):
+    cores = max(1, min(ref.max_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or os.cpu_count() or 1)))
+
+    def timed(run, budget, least=2, most=40):
         run()
-        done += 1
-    dt = (time.perf_counter() - t0) / done
-    return {"value": WEIGHT_BYTES / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "ms_per_step": dt * 1e3,
-            "sample": f"{done} products of the same workload (x bf16 [1,{K}], W [{N},{K}] affine 4-bit g64): whole-matrix "
-                      f"dequantize on one thread as the reference does, then the 8-lane fixed-order product over "
-                      f"64-column blocks on {threads} threads"}
+        done, t0 = 0, time.perf_counter()
+        while done < least or (time.perf_counter() - t0 < budget and done < most):
+            run()
+            done += 1
+        return (time.perf_counter() - t0) / done, done
+
+    legs = {}
+    for name, threads in (("single_thread", 1), ("all_cores", cores)):
+        dt, done = timed(lambda: ref.quantized_matmul(x, packed, scales, biases, group=GROUP, bits=BITS, dtype=ref.BF16, threads=threads),
+                         seconds_budget / 4)
+        legs[name] = {"value": WEIGHT_BYTES / dt / 1e9, "unit": "GB/s", "cores": threads, "ms_per_step": dt * 1e3, "products": done}
+    rows = 64  # of the 2048 of configs[2]: more than 16 rows, so the many-row product (float32 products summed in order)
+    xm = ref.from_f32(rng.standard_normal((rows, K)).astype(np.float32), ref.BF16)
+    dt, done = timed(lambda: ref.quantized_matmul(xm, packed, scales, biases, group=GROUP, bits=BITS, dtype=ref.BF16, threads=cores),
+                     seconds_budget / 4, least=1, most=10)
+    legs["prefill_all_cores"] = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "ms_per_step": dt * 1e3,
+                                 "products": done, "sample": f"{rows} of the 2048 rows of configs[2] per product (dequantize included)"}
+    return {"value": legs["all_cores"]["value"], "unit": "GB/s", "cores": cores, "kind": "port",
+            "ms_per_step": legs["all_cores"]["ms_per_step"],
+            "sample": f"{legs['all_cores']['products']} products of the same workload (x bf16 [1,{K}], W [{N},{K}] affine 4-bit g64): "
+                      f"whole-matrix dequantize on one thread as the reference does, then the 8-lane fixed-order product over "
+                      f"64-column blocks on {cores} threads; `single_thread` is the same on one thread, `prefill_all_cores` "
+                      f"{rows} rows of configs[2]",
+            **legs}
+
+
+def measured_peaks(lib, device, qs):
+    """What this box gives the simplest kernels, measured in this run with the same event timing: the ceilings the
+    roofline fractions can be read against besides the published peaks."""
+    import torch
+
+    from nuvec_amd import _lib
+    work = C.c_int64(0)
+    out = {}
+
+    def best_of(calls, steps):
+        return min(time_launches(calls, steps, len(calls), graph=False)[0] for _ in range(3))
+
+    # the decode kernel's grid reading the 29.4 MB of packed codes and nothing else, weights rotated like the headline
+    code_bytes = N * K * BITS // 8
+    reads = [(lambda stream, q=q: _lib.check(lib.nvq_calibrate(0, C.c_void_p(q.weight.data_ptr()), code_bytes, 0, None, C.byref(work), stream)))
+             for q in qs]
+    ms = best_of(reads, 2000)
+    out["read_codes_decode_grid"] = {"us_per_launch": ms * 1e3, "gbps": code_bytes / (ms * 1e-3) / 1e9, "bytes": code_bytes,
+                                     "note": "plain read of one product's packed codes (no scales, no arithmetic), rotating buffers"}
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    ms = best_of([lambda stream: _lib.check(lib.nvq_calibrate(0, C.c_void_p(big.data_ptr()), 1 << 30, 0, None, C.byref(work), stream))], 30)
+    out["stream_read_1gib"] = {"us_per_launch": ms * 1e3, "gbps": (1 << 30) / (ms * 1e-3) / 1e9}
+    del big
+    empty = torch.empty(16384, dtype=torch.uint8, device=device)
+    ms = best_of([lambda stream: _lib.check(lib.nvq_calibrate(0, C.c_void_p(empty.data_ptr()), 16384, 0, None, C.byref(work), stream))], 2000)
+    out["one_block_launch"] = {"us_per_launch": ms * 1e3, "note": "a launch of one block: the floor of any back-to-back kernel here"}
+    iters = 4096
+    ms = best_of([lambda stream: _lib.check(lib.nvq_calibrate(1, None, 0, iters, None, C.byref(work), stream))], 10)
+    out["mfma_only_loop"] = {"us_per_launch": ms * 1e3, "tflops": work.value / (ms * 1e-3) / 1e12,
+                             "note": "v_mfma_f32_32x32x16_bf16 on constant operands, two wavefronts per SIMD"}
+    a = torch.randn(2048, K, device=device).to(torch.bfloat16)
+    b = torch.randn(N, K, device=device).to(torch.bfloat16)
+    c = torch.empty(2048, N, dtype=torch.bfloat16, device=device)
+    ms = best_of([lambda stream: torch.matmul(a, b.t(), out=c)], 20)
+    out["vendor_dense_gemm"] = {"us_per_launch": ms * 1e3, "tflops": 2.0 * 2048 * N * K / (ms * 1e-3) / 1e12,
+                                "note": "torch.matmul bf16 [2048,4096] x [4096,14336] (hipBLASLt, nothing to dequantize): baseline only"}
+    return out
 
 
 def all_configs(lib, device, qs):
@@ -258,8 +313,9 @@ def main():
     ap.add_argument("--qmm-steps", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-qmm", action="store_true", help="skip the M=2048 leg")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time every configuration of the reference's benchmark list (C1..C5) and report them under \"configs\"")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip timing every configuration of the reference's benchmark list (C1..C5), reported under \"configs\"")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the calibration kernels reported under \"measured_peaks\"")
     ap.add_argument("--only", choices=["qmv", "qmm", "copy"], default=None,
                     help="profiling aid: run just the rotating decode leg, just the prefill leg, or a plain 1 GiB "
                          "device copy (the known-size kernel the HBM counters are scaled by)")
@@ -319,17 +375,22 @@ def main():
         xm = torch.randn(m, K, device=device).to(torch.bfloat16)
         ym = torch.empty(m, N, dtype=torch.bfloat16, device=device)
         qcalls = [Product(lib, m, xm, q, ym) for q in qs[:4]]
-        # best of three runs of `qmm_steps` launches: the first run of a process sits on the clock ramp
-        qms, qsteps = min(time_launches(qcalls, args.qmm_steps, 4, graph=False) for _ in range(3))
+        # four runs of `qmm_steps` launches; the first sits on the clock ramp and is dropped, the others are averaged
+        runs = [time_launches(qcalls, args.qmm_steps, 4, graph=False) for _ in range(4)][1:]
+        qms, qsteps = sum(r[0] for r in runs) / len(runs), sum(r[1] for r in runs)
+        best_ms = min(r[0] for r in runs)
         flop = 2.0 * m * N * K
         tflops = flop / (qms * 1e-3) / 1e12
         record["qmm"] = {"workload": "configs[2]: prefill QMM, affine 4-bit g64, x bf16 [2048,4096], W [14336,4096]",
                          "value": tflops, "unit": "TFLOP/s", "ms_per_step": qms, "steps": qsteps,
+                         "best_run": {"ms_per_step": best_ms, "tflops": flop / (best_ms * 1e-3) / 1e12},
                          "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                       "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": QMM_TRAFFIC_BYTES,
                                       "kernel": "qmm_kernel (256x256 tile)", "flop_per_launch": flop}}
 
-    if only is None and args.all_configs:
+    if only is None and not args.no_peaks:
+        record["measured_peaks"] = measured_peaks(lib, device, qs)
+    if only is None and not args.no_configs:
         record["configs"] = all_configs(lib, device, qs)
     if only is None and not args.no_cpu:
         record["cpu_baseline"] = cpu_baseline()

@@ -139,6 +139,18 @@ NVQ_API int32_t nvq_get_device_info(nvq_device_info *info);
 NVQ_API const char *nvq_last_error(void);
 NVQ_API const char *nvq_version(void);
 
+/* No counterpart in the reference: two calibration kernels for the measurement harness, so that a benchmark can state
+ * what this machine gives a kernel that does nothing but read memory or nothing but issue matrix instructions.
+ *   NVQ_CALIBRATE_READ: every byte of `buffer` (`bytes`, a multiple of 16384) is read once with non-temporal 16-byte
+ *     loads, 32 bytes per thread in blocks of 512 threads (bytes = N * K / 2 gives the decode kernel's grid);
+ *   NVQ_CALIBRATE_MFMA: two wavefronts per SIMD issue `iters` rounds of eight independent v_mfma_f32_32x32x16_bf16.
+ * `*work` (host, may be NULL) receives the bytes read or the floating-point operations of the launch; `sink` (device,
+ * may be NULL) exists so that the compiler keeps the work. */
+#define NVQ_CALIBRATE_READ 0
+#define NVQ_CALIBRATE_MFMA 1
+NVQ_API int32_t nvq_calibrate(int32_t kind, const void *buffer, int64_t bytes, int32_t iters, void *sink, int64_t *work,
+                      void *stream);
+
 /* ── validation mirrors (usable without a device) ────────────────────────────────── */
 
 /* Quant::checked (quantized.rs:133-168): NVQ_OK or NVQ_INVALID_ARGUMENT with the
@@ -194,6 +206,18 @@ NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
  * `workspace` may be NULL when nvq_quantized_matmul_workspace_bytes(desc) == 0 (and for transposed products). */
 NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
                              const void *biases, void *y, void *workspace, void *stream);
+
+/* No counterpart in the reference: nvq_quantized_matmul for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot bring the workspace.  Same operands,
+ * same routing and bit for bit the same results as nvq_quantized_matmul given the workspace its size query names; the
+ * partial sums of a split K go to a scratch array inside the library (NVQ_STATIC_SCRATCH_BYTES of device memory, held
+ * by every device the library is loaded on until the process ends).  A product whose partial sums need more is refused
+ * with NVQ_UNSUPPORTED.  The call allocates and frees nothing.  All calls on a device share the one array (nothing in
+ * it needs clearing: every partial sum a call reads it has written first), so calls that overlap in time on one device,
+ * from several streams or threads, race: serialise them, or use nvq_quantized_matmul with a workspace per stream. */
+#define NVQ_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+NVQ_API int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
+                                    const void *biases, void *y, void *stream);
 
 /* GpuEval::sorted_offsets (gpu.rs:6732-6756); kernels::sorted_offsets (kernels.rs:873-892):
  * per row of `indices` u32[rows, m], offsets[row, g] = first position whose value is >= g. */

@@ -15,6 +15,7 @@ OK, INVALID_ARGUMENT, UNSUPPORTED, OUT_OF_MEMORY, BACKEND, NO_DEVICE = range(6)
 U8, U32, I32, F16, BF16, F32 = 1, 3, 7, 9, 10, 11
 AFFINE, MXFP4, MXFP8, NVFP4 = 0, 1, 2, 3
 MAX_BATCH_DIMS = 6
+STATIC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 
 class InvalidArgument(ValueError):
@@ -65,6 +66,7 @@ SIGNATURES = {
     "nvq_get_device_info": (C.c_int32, [C.POINTER(DeviceInfoC)]),
     "nvq_last_error": (C.c_char_p, []),
     "nvq_version": (C.c_char_p, []),
+    "nvq_calibrate": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.POINTER(C.c_int64), C.c_void_p]),
     "nvq_quant_check": (C.c_int32, [C.POINTER(QuantC), C.c_char_p]),
     "nvq_gather_grouped": (C.c_int32, [C.c_int64, C.c_int64, C.c_int32]),
     "nvq_quantized_matmul_supported": (C.c_int32, [C.POINTER(QmmDescC)]),
@@ -77,6 +79,8 @@ SIGNATURES = {
     "nvq_quantized_matmul_workspace_bytes": (C.c_size_t, [C.POINTER(QmmDescC)]),
     "nvq_quantized_matmul": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nvq_quantized_matmul_static": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                C.c_void_p, C.c_void_p]),
     "nvq_sorted_offsets": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
     "nvq_quantize_scaled": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_dequantize_scaled": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),

@@ -15,8 +15,16 @@
 
 namespace nvq {
 
+// Scratch for nvq_quantized_matmul_static, the entry point for callers that cannot allocate: the float32 partial sums of
+// a product whose K is split over the grid.  Every device the library is loaded on holds its own copy of the array at its
+// own address; host code never passes the array's name to a kernel, only the address hipGetSymbolAddress reported
+// for the bound device (g_scratch).
+static __device__ __align__(256) unsigned char scratch[NVQ_STATIC_SCRATCH_BYTES];
+
 namespace {
 thread_local char g_error[512] = "";
+constexpr int kMaxDevices = 64;
+void *g_scratch[kMaxDevices] = {};  // device address of `scratch` per device, written under the device record's mutex
 
 // Written under the mutex by nvq_init; `ready`, `device` and `units` are read without it on every call.
 struct DeviceRecord {
@@ -210,6 +218,20 @@ int32_t nvq_init(int32_t device) {
     NVQ_HIP_TRY(hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(NVQ_NO_DEVICE, "device %d is %s: this library holds gfx950 code only", device, prop.gcnArchName);
+    if (device >= kMaxDevices) return fail(NVQ_NO_DEVICE, "device %d: at most %d devices", device, kMaxDevices);
+    if (g_scratch[device] == nullptr) {  // once per device, with that device current
+        int current = -1;
+        NVQ_HIP_TRY(hipGetDevice(&current));
+        if (current != device) NVQ_HIP_TRY(hipSetDevice(device));
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (current != device) (void)hipSetDevice(current);
+        if (e != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            return fail(NVQ_BACKEND, "hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
+        }
+        g_scratch[device] = ptr;
+    }
     g_device.prop = prop;
     g_device.device.store(device, std::memory_order_relaxed);
     g_device.units.store(prop.multiProcessorCount, std::memory_order_relaxed);
@@ -230,6 +252,11 @@ int32_t nvq_get_device_info(nvq_device_info *info) {
     snprintf(info->arch, sizeof info->arch, "%s", g_device.prop.gcnArchName);
     snprintf(info->name, sizeof info->name, "%s", g_device.prop.name);
     return NVQ_OK;
+}
+
+int32_t nvq_calibrate(int32_t kind, const void *buffer, int64_t bytes, int32_t iters, void *sink, int64_t *work, void *stream) {
+    NVQ_TRY(require_device());
+    return launch_calibrate(kind, buffer, bytes, iters, sink, work, (hipStream_t)stream);
 }
 
 int32_t nvq_quant_check(const nvq_quant *quant, const char *op) { return check_quant(quant, op ? op : "quant"); }
@@ -446,6 +473,21 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
 
 int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                              void *y, void *workspace, void *stream) {
+    return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream);
+}
+
+int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                                    void *y, void *stream) {
+    NVQ_TRY(check_qmm(d, "quantized_matmul"));
+    const size_t need = nvq_quantized_matmul_workspace_bytes(d);  // 0 without a device: the launch below says so
+    if (need > (size_t)NVQ_STATIC_SCRATCH_BYTES)
+        return fail(NVQ_UNSUPPORTED, "quantized_matmul: this product splits K through %zu bytes of partial sums; the static scratch holds %d",
+                    need, NVQ_STATIC_SCRATCH_BYTES);
+    void *workspace = nullptr;
+    if (need > 0) {
+        NVQ_TRY(require_device());
+        workspace = g_scratch[g_device.device.load(std::memory_order_relaxed)];
+    }
     return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream);
 }
 
