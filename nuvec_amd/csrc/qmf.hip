@@ -12,8 +12,10 @@ bool qmf_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.k < 64 || a.k % 64 != 0) return false;
     size_t lds = 0;
-    if (a.mode == NVQ_MXFP4) {
+    if (a.mode == NVQ_MXFP4 || (a.mode == NVQ_NVFP4 && a.global_scale == nullptr)) {
         lds = qmf::lds_needed<4>(a);
+    } else if (a.mode == NVQ_MXFP8) {
+        lds = qmf::lds_needed<8>(a);
     } else if (a.mode == NVQ_AFFINE) {
         switch (a.bits) {
         case 2: lds = qmf::lds_needed<2>(a); break;
@@ -36,6 +38,8 @@ bool qmf_supported(const ProductArgs &a) {
 
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s) {
     if (a.mode == NVQ_MXFP4) return launch_qmf_fp4(a, s);
+    if (a.mode == NVQ_MXFP8) return launch_qmf_fp8(a, s);
+    if (a.mode == NVQ_NVFP4) return launch_qmf_nvfp4(a, s);
     switch (a.bits) {
     case 2: return launch_qmf_b2(a, s);
     case 3: return launch_qmf_b3(a, s);

@@ -42,6 +42,11 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2v_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2v_t __attribute__((ext_vector_type(2)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
+// The FP4 template parameter of the kernels below names the code format: 0 affine integers with a scale and a bias per
+// group, 1 MXFP4 (E2M1 codes, an E8M0 scale per 32), 2 MXFP8 (E4M3 codes, an E8M0 scale per 32), 3 NVFP4 (E2M1 codes, an
+// E4M3 scale per 16; without a global scale).  Every weight of the block formats is exact in bfloat16 and float16 (at
+// most six significant bits times a power of two).
+constexpr int kAffine = 0, kMxfp4 = 1, kMxfp8 = 2, kNvfp4 = 3;
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
@@ -101,6 +106,10 @@ template <> struct Ops<bf16_t> {
     template <int B> __device__ static __forceinline__ uint32_t fp4_pair(uint32_t word, float scale) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, scale, B));
     }
+    // The two E4M3 codes of the low or high half of `word` times the power of two `scale`.
+    template <bool HIGH> __device__ static __forceinline__ uint32_t fp8_pair(uint32_t word, float scale) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(word, scale, HIGH));
+    }
 };
 template <> struct Ops<f16_t> {
     __device__ static __forceinline__ floatx16_t mfma(uint4 a, uint4 b, floatx16_t c) {
@@ -113,7 +122,18 @@ template <> struct Ops<f16_t> {
     template <int B> __device__ static __forceinline__ uint32_t fp4_pair(uint32_t word, float scale) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(word, scale, B));
     }
+    template <bool HIGH> __device__ static __forceinline__ uint32_t fp8_pair(uint32_t word, float scale) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, scale, HIGH));
+    }
 };
+
+// The two E2M1 codes of byte B of `word` times any `scale` (NVFP4: the scale is no power of two, so the scaled
+// conversion, which takes the scale's exponent only, does not apply): decoded to float, multiplied, packed.
+template <typename T, int B>
+__device__ __forceinline__ uint32_t fp4_pair_times(uint32_t word, float scale) {
+    const floatx2_t v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, B);
+    return Ops<T>::pack(v.x * scale, v.y * scale);
+}
 
 // Code J of a lane's 32 codes (BITS dwords, value i in bits i BITS .. of the stream) as a float.
 template <int BITS, int J>
@@ -130,10 +150,22 @@ __device__ __forceinline__ float code_to_float(const uint32_t (&dw)[BITS]) {
 }
 
 // Piece KK (eight codes, stream order) of a lane's 32 codes as one matrix operand.
-template <typename T, int BITS, bool FP4, int KK>
+template <typename T, int BITS, int FP4, int KK>
 __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float s, float b) {
     uint4 r;
-    if constexpr (FP4) {
+    if constexpr (FP4 == kMxfp8) {
+        const uint32_t w0 = dw[2 * KK], w1 = dw[2 * KK + 1];
+        r.x = Ops<T>::template fp8_pair<false>(w0, s);
+        r.y = Ops<T>::template fp8_pair<true>(w0, s);
+        r.z = Ops<T>::template fp8_pair<false>(w1, s);
+        r.w = Ops<T>::template fp8_pair<true>(w1, s);
+    } else if constexpr (FP4 == kNvfp4) {
+        const uint32_t word = dw[KK];
+        r.x = fp4_pair_times<T, 0>(word, s);
+        r.y = fp4_pair_times<T, 1>(word, s);
+        r.z = fp4_pair_times<T, 2>(word, s);
+        r.w = fp4_pair_times<T, 3>(word, s);
+    } else if constexpr (FP4) {
         const uint32_t word = dw[KK];
         r.x = Ops<T>::template fp4_pair<0>(word, s);
         r.y = Ops<T>::template fp4_pair<1>(word, s);
@@ -186,19 +218,19 @@ __device__ __forceinline__ void fill_table(unsigned char *table, const S *src, i
 }
 
 // blockIdx.z is a batch with one stride per operand, or a gathered pair; blockIdx.y a pass of 32 rows.
-template <typename T, int BITS, bool FP4, int RG>
+template <typename T, int BITS, int FP4, int RG>
 __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     using G = Geometry<BITS, RG>;
     constexpr int kRows = G::kRows, kDepth = G::kDepth, kLoads = G::kLoads;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     float *partial = reinterpret_cast<float *>(lds);  // [4][RG][values][64]
-    using S = std::conditional_t<FP4, uint8_t, T>;    // stored scale type
+    using S = std::conditional_t<FP4 != 0, uint8_t, T>;    // stored scale type
     unsigned char *table_s = lds + G::kFixedLdsBytes;  // scales [rows][groups, padded]; the biases follow
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = lane >> 5, l32 = lane & 31;
     const int K = (int)a.k, N = (int)a.n;
-    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int kgroups = K >> gshift;
     const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
     const int tstride = table_stride(kgroups, (int)sizeof(S));
@@ -273,17 +305,22 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         }
     static_assert(G::swizzle(32) == 0 && G::swizzle(33) == G::swizzle(1), "row groups share the swizzle of their rows");
 
-    auto load_scales = [&](int step, float (&scale)[RG], float (&bias)[RG]) {
+    // The scale (NVFP4: the two scales, one per 16 values) and bias of this lane's 32 values of a step.
+    auto load_scales = [&](int step, float (&scale)[RG][2], float (&bias)[RG]) {
         const int g = (step * 64 + 32 * h) >> gshift;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             const int at = (32 * rg + l32) * tstride + g * (int)sizeof(S);
             const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
-            if constexpr (FP4) {
-                scale[rg] = ftz(e8m0_to_f32(*sp));
+            if constexpr (FP4 == kNvfp4) {
+                scale[rg][0] = ftz(e4m3_to_f32(sp[0]));
+                scale[rg][1] = ftz(e4m3_to_f32(sp[1]));
+                bias[rg] = 0.0f;
+            } else if constexpr (FP4) {
+                scale[rg][0] = scale[rg][1] = ftz(e8m0_to_f32(*sp));
                 bias[rg] = 0.0f;
             } else {
-                scale[rg] = Elem<T>::load(sp, 0);
+                scale[rg][0] = scale[rg][1] = Elem<T>::load(sp, 0);
                 bias[rg] = Elem<T>::load(bp, 0);
             }
         }
@@ -366,7 +403,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     if (step + t < s_end) {
-                        float scale[RG], bias[RG];
+                        float scale[RG][2], bias[RG];
                         load_scales(step + t, scale, bias);
                         static_for<4>([&](auto kk_tag) {
                             constexpr int kk = decltype(kk_tag)::value;
@@ -377,7 +414,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
                             }
 #pragma unroll
                             for (int rg = 0; rg < RG; rg++)
-                                acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg], bias[rg]), acc[rg]);
+                                acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg][kk >> 1], bias[rg]), acc[rg]);
                         });
                     }
                 }
@@ -442,8 +479,8 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
 
 // Bytes of the LDS table of scales (and biases) for `rows` weight rows.
 inline size_t table_bytes(const ProductArgs &a, int rows) {
-    const bool fp4 = a.mode == NVQ_MXFP4;
-    const int64_t bytes = (int64_t)rows * table_stride((int)(a.k / (fp4 ? 32 : a.group)), fp4 ? 1 : 2) * (fp4 ? 1 : 2);
+    const bool block = a.mode != NVQ_AFFINE;  // one-byte scale codes, no biases
+    const int64_t bytes = (int64_t)rows * table_stride((int)(a.k / a.group), block ? 1 : 2) * (block ? 1 : 2);
     return (size_t)((bytes + 15) & ~(int64_t)15);
 }
 
@@ -453,7 +490,7 @@ inline int row_groups(const ProductArgs &a) {
     return blocks >= 192 ? 2 : 1;
 }
 
-template <typename T, int BITS, bool FP4, int RG>
+template <typename T, int BITS, int FP4, int RG>
 int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS, RG>;
     static std::atomic<bool> configured = false;
@@ -471,12 +508,12 @@ int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int BITS, bool FP4>
+template <typename T, int BITS, int FP4>
 int32_t run_width(const ProductArgs &a, hipStream_t s) {
     return row_groups(a) == 2 ? run_variant<T, BITS, FP4, 2>(a, s) : run_variant<T, BITS, FP4, 1>(a, s);
 }
 
-template <int BITS, bool FP4>
+template <int BITS, int FP4>
 int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
     return a.dtype == NVQ_BF16 ? run_width<bf16_t, BITS, FP4>(a, s) : run_width<f16_t, BITS, FP4>(a, s);
 }
@@ -490,6 +527,8 @@ inline size_t lds_needed(const ProductArgs &a) {
 }  // namespace qmf
 
 // One per code width, each in its own translation unit.
+int32_t launch_qmf_fp8(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_nvfp4(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b2(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b3(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b4(const ProductArgs &a, hipStream_t s);

@@ -45,20 +45,20 @@ struct Geometry {
     __host__ __device__ static constexpr int swizzle(int row) { return kPow2 ? (row / (BITS >= 16 ? 1 : 16 / BITS)) % BITS : 0; }
 };
 
-template <typename T, int BITS, bool FP4>
+template <typename T, int BITS, int FP4>
 // Three blocks per compute unit (three wavefronts per SIMD): the registers are capped for that, and the LDS of a
 // block (two x stages, the weight stages, the table) fits three times.
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) qmg_kernel(const ProductArgs a) {
     using G = Geometry<BITS>;
     constexpr int kDepth = G::kDepth, kLoads = G::kLoads;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    using S = std::conditional_t<FP4, uint8_t, T>;  // stored scale type
+    using S = std::conditional_t<FP4 != 0, uint8_t, T>;  // stored scale type
     unsigned char *table_s = lds + G::kFixedLdsBytes;  // scales [rows][groups, padded]; the biases follow
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = lane >> 5, l32 = lane & 31;
     const int K = (int)a.k, N = (int)a.n;
-    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int kgroups = K >> gshift;
     const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
     const int tstride = table_stride(kgroups, (int)sizeof(S));
@@ -113,15 +113,28 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
             wread[t][p] = l32 * G::kRowBytes + 16 * ((byte >> 4) ^ G::swizzle(l32)) + (byte & 15);
         }
 
-    auto load_scales = [&](int step, float &scale, float &bias) {
+    // The first windows of weights are requested before anything waits: they depend on nothing but the block's place.
+    u32x4_t ring[kDepth][kLoads];  // weight windows in flight
+    static_for<kDepth>([&](auto d_tag) {
+        constexpr int d = decltype(d_tag)::value;
+        load_window(d, ring[d]);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+
+    // The scale (NVFP4: the two scales, one per 16 values) and bias of this lane's 32 values of a step.
+    auto load_scales = [&](int step, float (&scale)[2], float &bias) {
         const int g = (step * 64 + 32 * h) >> gshift;
         const int at = (32 * wave + l32) * tstride + g * (int)sizeof(S);
         const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
-        if constexpr (FP4) {
-            scale = ftz(e8m0_to_f32(*sp));
+        if constexpr (FP4 == kNvfp4) {
+            scale[0] = ftz(e4m3_to_f32(sp[0]));
+            scale[1] = ftz(e4m3_to_f32(sp[1]));
+            bias = 0.0f;
+        } else if constexpr (FP4) {
+            scale[0] = scale[1] = ftz(e8m0_to_f32(*sp));
             bias = 0.0f;
         } else {
-            scale = Elem<T>::load(sp, 0);
+            scale[0] = scale[1] = Elem<T>::load(sp, 0);
             bias = Elem<T>::load(bp, 0);
         }
     };
@@ -185,13 +198,14 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
             for (int el = 0; el < 16; el++) acc[u][el] = 0.0f;
 
         u32x4_t xq[2][4];                   // x chunks of the next two windows
-        u32x4_t ring[kDepth][kLoads] = {};  // weight windows in flight
         load_x(0, xq[0]);
         load_x(1, xq[1]);
-        static_for<kDepth>([&](auto d_tag) {
-            constexpr int d = decltype(d_tag)::value;
-            load_window(d, ring[d]);
-        });
+        if (pass != row_begin) {  // (the first pass found its windows on the way already)
+            static_for<kDepth>([&](auto d_tag) {
+                constexpr int d = decltype(d_tag)::value;
+                load_window(d, ring[d]);
+            });
+        }
         store_x(0, xq[0]);
         load_x(2, xq[0]);
         __syncthreads();  // window 0 of x is in LDS (first pass: the table too)
@@ -239,11 +253,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
                         for (int kk = 0; kk < 4; kk++) xf[t][kk] = *reinterpret_cast<const uint4 *>(xs + xread[t][kk]);
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        float scale, bias;
+                        float scale[2], bias;
                         load_scales(2 * win + (t == 0 || second_step ? t : 0), scale, bias);
                         static_for<4>([&](auto kk_tag) {
                             constexpr int kk = decltype(kk_tag)::value;
-                            wb[t][kk] = expand_piece<T, BITS, FP4, kk>(codes[t], scale, bias);
+                            wb[t][kk] = expand_piece<T, BITS, FP4, kk>(codes[t], scale[kk >> 1], bias);
                         });
                     }
 #pragma unroll
@@ -293,7 +307,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
 // Bytes of the LDS table of scales (and biases) for the block's rows.
 inline size_t table_bytes(const ProductArgs &a) { return qmf::table_bytes(a, kRows); }
 
-template <typename T, int BITS, bool FP4>
+template <typename T, int BITS, int FP4>
 int32_t run(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS>;
     static std::atomic<bool> configured = false;
@@ -310,7 +324,7 @@ int32_t run(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <int BITS, bool FP4>
+template <int BITS, int FP4>
 int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
     return a.dtype == NVQ_BF16 ? run<bf16_t, BITS, FP4>(a, s) : run<f16_t, BITS, FP4>(a, s);
 }

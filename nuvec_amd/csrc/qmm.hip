@@ -10,8 +10,8 @@ bool qmm_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.mode == NVQ_AFFINE) {
         if (a.bits != 2 && a.bits != 3 && a.bits != 4 && a.bits != 6 && a.bits != 8) return false;
-    } else if (a.mode != NVQ_MXFP4) {
-        return false;
+    } else if (a.mode == NVQ_NVFP4 && a.global_scale != nullptr) {
+        return false;  // the scaled weights are not exact in the element type: the general kernel keeps them in float32
     }
     if (a.rhs != nullptr) return false;
     if (a.batch > 1 && a.batch_ndim != 1) return false;
@@ -33,6 +33,8 @@ size_t qmm_workspace_bytes(const ProductArgs &a) {
 
 int32_t launch_qmm(const ProductArgs &a, void *workspace, hipStream_t s) {
     if (a.mode == NVQ_MXFP4) return launch_qmm_fp4(a, workspace, s);
+    if (a.mode == NVQ_MXFP8) return launch_qmm_fp8(a, workspace, s);
+    if (a.mode == NVQ_NVFP4) return launch_qmm_nvfp4(a, workspace, s);
     switch (a.bits) {
     case 2: return launch_qmm_b2(a, workspace, s);
     case 3: return launch_qmm_b3(a, workspace, s);

@@ -125,9 +125,13 @@ __device__ __forceinline__ void pin() { __builtin_amdgcn_sched_barrier(0); }
 __device__ __forceinline__ void keep(const uint4 &v) { asm volatile("" : : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)); }
 
 // Dword D (two elements) of piece KK of a lane's 32 codes: expand_piece, one register at a time.
-template <typename T, int BITS, bool FP4, int KK, int D>
+template <typename T, int BITS, int FP4, int KK, int D>
 __device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], float s, float b) {
-    if constexpr (FP4) {
+    if constexpr (FP4 == kMxfp8) {
+        return Ops<T>::template fp8_pair<(D & 1) != 0>(dw[2 * KK + D / 2], s);
+    } else if constexpr (FP4 == kNvfp4) {
+        return fp4_pair_times<T, D>(dw[KK], s);
+    } else if constexpr (FP4) {
         return Ops<T>::template fp4_pair<D>(dw[KK], s);
     } else if constexpr (BITS == 4) {
         const uint32_t word = dw[KK];
@@ -139,14 +143,14 @@ __device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], flo
     }
 }
 
-template <typename T, int BITS, bool FP4, bool BATCHED, class TL>
+template <typename T, int BITS, int FP4, bool BATCHED, class TL>
 __global__ void __launch_bounds__(TL::kThreads) __attribute__((amdgpu_waves_per_eu(TL::kWavesPerSimd, TL::kWavesPerSimd)))
 qmm_kernel(const ProductArgs a) {
     using G = Geometry<BITS, TL>;
     constexpr int BM = TL::BM, BN = TL::BN, kThreads = TL::kThreads, kXBytes = TL::kXBytes, kSbBytes = TL::kSbBytes;
     constexpr int TI = TL::TI, TJ = TL::TJ;
     using P = Pieces<BITS>;
-    using S = std::conditional_t<FP4, uint8_t, T>;  // stored scale type
+    using S = std::conditional_t<FP4 != 0, uint8_t, T>;  // stored scale type
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
     // Scale and bias tables, two buffers of [scale | bias][group 0..3][row] dwords (the element in the low bits).
@@ -155,10 +159,12 @@ qmm_kernel(const ProductArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / TL::WN, wn = wave % TL::WN;  // wavefront grid WM x WN: 32 TI x 32 TJ each
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
-    const int gshift = FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int row_dwords = (K >> 5) * BITS, kgroups = K >> gshift;
-    // A table covers a period of 4 groups (2 of 128): two steps for groups of 32, else four.
-    const int pshift = gshift == 5 ? 1 : 2, psteps = 1 << pshift;
+    // A table covers a period of 4 groups (2 of 128; NVFP4, which has no biases: 8 of 16): two steps for groups of 16
+    // and 32, else four.
+    constexpr int kTableGroups = FP4 == kNvfp4 ? 8 : 4;
+    const int pshift = gshift <= 5 ? 1 : 2, psteps = 1 << pshift;
     const int gper = (psteps * BK) >> gshift;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     // A single product may split K over grid z (few tiles, long K): this block takes the steps
@@ -241,7 +247,7 @@ qmm_kernel(const ProductArgs a) {
     };
     // The table of period `period`: every wavefront brings kTableLoads times 64 consecutive rows of one group's
     // scales or biases (groups past the row's last one repeat it: they are never read).
-    constexpr int kKinds = FP4 ? 1 : 2, kTableLoads = kKinds * 4 * BN / kThreads;
+    constexpr int kKinds = FP4 ? 1 : 2, kTableLoads = kKinds * kTableGroups * BN / kThreads;
     const int trow = n0 + tid % BN < N ? tid % BN : N - 1 - n0;
     const uint32_t toff = (uint32_t)trow * (uint32_t)kgroups * (uint32_t)sizeof(S);
     const int g0 = (step0 * BK) >> gshift, groups_left = kgroups - g0;  // this block's first group
@@ -252,7 +258,7 @@ qmm_kernel(const ProductArgs a) {
 #pragma unroll
         for (int i = 0; i < kTableLoads; i++) {
             const int entry = i * kThreads + wave * 64;  // of this wavefront's first lane: [kind][group][row]
-            const int kind = entry / (4 * BN), g = (entry / BN) % 4;
+            const int kind = entry / (kTableGroups * BN), g = (entry / BN) % kTableGroups;
             const int gi = period * gper + g < groups_left ? period * gper + g : groups_left - 1;
             dma_element<sizeof(S)>((kind ? bbase : sbase) + gi * (int)sizeof(S), toff, tbase + entry * 4);
         }
@@ -267,8 +273,8 @@ qmm_kernel(const ProductArgs a) {
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     const int h = lane >> 5, l32 = lane & 31;
-    uint32_t raw[TJ][BITS], sraw[TJ], braw[TJ];  // codes and table entries as read: converted where first used
-    float sc[TJ], bi[TJ];
+    uint32_t raw[TJ][BITS], sraw[TJ], braw[TJ];  // codes and table entries as read: converted where first used (NVFP4: braw is the second scale)
+    float sc[TJ][2], bi[TJ];
     uint4 af[2][TI], bf[2][TJ];
     // The packed codes, scales and biases of this lane's TJ columns for `step` (its stage and table are visible).
     auto read_codes = [&](int step, int stage) {
@@ -290,14 +296,19 @@ qmm_kernel(const ProductArgs a) {
             }
             sraw[j] = sbt[col];
             if constexpr (!FP4) braw[j] = sbt[4 * BN + col];
+            if constexpr (FP4 == kNvfp4) braw[j] = sbt[BN + col];  // the lane's second group of 16
         }
     };
     auto convert_scales = [&](int j) {
-        if constexpr (FP4) {
-            sc[j] = ftz(e8m0_to_f32((uint8_t)sraw[j]));
+        if constexpr (FP4 == kNvfp4) {
+            sc[j][0] = ftz(e4m3_to_f32((uint8_t)sraw[j]));
+            sc[j][1] = ftz(e4m3_to_f32((uint8_t)braw[j]));
+            bi[j] = 0.0f;
+        } else if constexpr (FP4) {
+            sc[j][0] = sc[j][1] = ftz(e8m0_to_f32((uint8_t)sraw[j]));
             bi[j] = 0.0f;
         } else {
-            sc[j] = half_lo<T>(sraw[j]);
+            sc[j][0] = sc[j][1] = half_lo<T>(sraw[j]);
             bi[j] = half_lo<T>(braw[j]);
         }
     };
@@ -319,7 +330,7 @@ qmm_kernel(const ProductArgs a) {
         } else {
             constexpr int j = index / 4, d = index % 4;
             if constexpr (KK == 0 && d == 0) convert_scales(j);
-            const uint32_t v = expand_dword<T, BITS, FP4, KK, d>(raw[j], sc[j], bi[j]);
+            const uint32_t v = expand_dword<T, BITS, FP4, KK, d>(raw[j], sc[j][KK >> 1], bi[j]);
             if constexpr (d == 0) bf[KK & 1][j].x = v;
             else if constexpr (d == 1) bf[KK & 1][j].y = v;
             else if constexpr (d == 2) bf[KK & 1][j].z = v;
@@ -490,7 +501,7 @@ inline int k_splits(const ProductArgs &a, int cus, int *steps_per_split = nullpt
     return best;
 }
 
-template <typename T, int BITS, bool FP4, class TL>
+template <typename T, int BITS, int FP4, class TL>
 int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     using G = Geometry<BITS, TL>;
     static std::atomic<bool> configured[2] = {false, false};
@@ -516,13 +527,13 @@ int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int BITS, bool FP4>
+template <typename T, int BITS, int FP4>
 int32_t run(const ProductArgs &a, void *workspace, hipStream_t s) {
     return small_tile_is_faster(a, compute_units()) ? run_tile<T, BITS, FP4, SmallTile>(a, workspace, s)
                                                     : run_tile<T, BITS, FP4, BigTile>(a, workspace, s);
 }
 
-template <int BITS, bool FP4>
+template <int BITS, int FP4>
 int32_t run_dtype(const ProductArgs &a, void *workspace, hipStream_t s) {
     return a.dtype == NVQ_BF16 ? run<bf16_t, BITS, FP4>(a, workspace, s) : run<f16_t, BITS, FP4>(a, workspace, s);
 }
@@ -536,5 +547,7 @@ int32_t launch_qmm_b4(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b6(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b8(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_fp4(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_fp8(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_nvfp4(const ProductArgs &a, void *workspace, hipStream_t s);
 
 }  // namespace nvq

@@ -499,6 +499,48 @@ def test_mxfp8_nvfp4_quantize_and_products(mode, qmode, dtype):
         assert float(np.max(ratio)) <= 1.0, f"{qmode} M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
 
 
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_block_formats_on_the_matrix_cores(mode, qmode, dtype):
+    """MXFP4, MXFP8 and NVFP4 (no global scale) through the few-row, the tiled and the grouped matrix-core kernels: few rows,
+    passes of 32 rows, tiles off the 256 x 256 shape with K split and unsplit, a batch, sorted experts.  Their weights are
+    exact in the element type (a few significant bits times a scale of few bits), so the bar holds for every output."""
+    rng = np.random.default_rng(4100 + 10 * mode + dtype)
+    group, bits = ref.FP_PARAMS[mode]
+    for m, n, k in [(1, 200, 1152), (5, 77, 2880), (33, 130, 640), (100, 96, 1024), (300, 260, 1152), (520, 64, 4096)]:
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales = ref.fp_quantize(w, dtype, mode)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8)
+        for scratch in (True, False):
+            got = to_host(nv.quantized_matmul(to_dev(x), q, scratch=scratch))
+            assert_rows_close(got, want, dtype, f"{qmode} M={m} N={n} K={k} scratch={scratch}", exact_weights=True)
+    # a batch with one stride per operand
+    b, m, n, k = 3, 40, 96, 512
+    w, x = make_w(rng, b * n, k, dtype), make_x(rng, b * m, k, dtype)
+    packed, scales = ref.fp_quantize(w, dtype, mode)
+    q = nv.Quantized(to_dev(packed.reshape(b, n, -1)), to_dev(scales.reshape(b, n, -1)), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+    got = to_host(nv.quantized_matmul(to_dev(x.reshape(b, m, k)), q))
+    for i in range(b):
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n], None, mode=mode,
+                                    group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[i], want, dtype, f"{qmode} batch item {i}", exact_weights=True)
+    # experts: rows sorted by expert (the grouped kernel), an expert without rows, one with more than 64
+    experts, n, k = 5, 136, 768
+    w = make_w(rng, experts * n, k, dtype).reshape(experts, n, k)
+    packed, scales = ref.fp_quantize(w, dtype, mode)
+    rhs = np.sort(np.array([0] * 7 + [1] * 70 + [3] * 33 + [4] * 18, np.uint32))
+    x = make_x(rng, rhs.size, k, dtype).reshape(-1, 1, k)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+    got = to_host(nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs.astype(np.int64)).cuda(), nv.GatherQmm(sorted_indices=True)))
+    want = ref.gather_qmm(x, packed, scales, None, np.arange(rhs.size, dtype=np.uint32), rhs, mode=mode, group=group, bits=bits, dtype=dtype)
+    assert_rows_close(got, want, dtype, f"{qmode} grouped gather", exact_weights=True)
+    some = rng.permutation(rhs.size)[:20]
+    got = to_host(nv.gather_qmm(to_dev(x), q, torch.from_numpy(some.astype(np.int64)).cuda(),
+                                torch.from_numpy(rhs[some].astype(np.int64)).cuda(), nv.GatherQmm()))
+    assert_rows_close(got, want[some], dtype, f"{qmode} gather per pair", exact_weights=True)
+
+
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
 def test_nvfp4_global_scale(dtype):
     """NVFP4 with a global scale (MLX's `quantize(..., global_scale=)`): codes, scales and dequantized values bit for
