@@ -207,6 +207,14 @@ NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
 NVQ_API int32_t nvq_quantized_matmul(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
                              const void *biases, void *y, void *workspace, void *stream);
 
+/* QuantizedLinear::forward (crates/nuvec-nn/src/layers.rs:155-162): `x . dequantize(w)^T + bias` in one launch.  The
+ * reference records the product and a separate addition; here the product kernels' epilogues add `bias` (element type
+ * `desc->dtype`, one value per column of y, [n]) to the product already rounded to the element type and round again, so
+ * the result has the bits of the two operations.  `bias` NULL: nvq_quantized_matmul.  A bias of another element type is
+ * the caller's promotion (it then adds separately, as the reference does). */
+NVQ_API int32_t nvq_quantized_linear(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
+                             const void *biases, const void *bias, void *y, void *workspace, void *stream);
+
 /* No counterpart in the reference: nvq_quantized_matmul for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot bring the workspace.  Same operands,
  * same routing and bit for bit the same results as nvq_quantized_matmul given the workspace its size query names; the

@@ -79,6 +79,7 @@ SIGNATURES = {
     "nvq_quantized_matmul_workspace_bytes": (C.c_size_t, [C.POINTER(QmmDescC)]),
     "nvq_quantized_matmul": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                          C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nvq_quantized_linear": (C.c_int32, [C.POINTER(QmmDescC)] + [C.c_void_p] * 8),
     "nvq_quantized_matmul_static": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                                 C.c_void_p, C.c_void_p]),
     "nvq_sorted_offsets": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),

@@ -436,7 +436,7 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
 }
 
 static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
-                                    const float *global_scale, void *y, void *workspace, void *stream) {
+                                    const float *global_scale, void *y, void *workspace, void *stream, const void *row_bias = nullptr) {
     NVQ_TRY(check_qmm(d, "quantized_matmul"));
     NVQ_TRY(check_groups("quantized_matmul", d->quant.mode, biases));
     int64_t batch = 1;
@@ -457,6 +457,7 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     ProductArgs a = product_args(d, batch);
     a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
     a.global_scale = global_scale;
+    a.row_bias = row_bias;
     if (global_scale != nullptr) return launch_qmv(a, (hipStream_t)stream);  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
     if (a.row_exact) return launch_qmv(a, (hipStream_t)stream);  // the vector kernels: a row's bits do not depend on its neighbours
@@ -474,6 +475,15 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
 int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                              void *y, void *workspace, void *stream) {
     return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream);
+}
+
+int32_t nvq_quantized_linear(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                             const void *bias, void *y, void *workspace, void *stream) {
+    NVQ_TRY(check_qmm(d, "quantized_linear"));
+    if (bias != nullptr && d->k == 0)  // an empty reduction is zero: the fill kernel has no bias epilogue
+        return fail(NVQ_UNSUPPORTED, "quantized_linear: a bias over an empty reduction");
+    NVQ_TRY(check_aligned("quantized_linear", "bias", bias, (size_t)dtype_size(d->dtype)));
+    return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream, bias);
 }
 
 int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,

@@ -77,6 +77,14 @@ template <> struct Elem<f16_t> {
     __device__ static __forceinline__ float add(float a, float b) { return (float)((f16_t)a + (f16_t)b); }
 };
 
+// A product's value for column n with the layer's bias, as QuantizedLinear::forward computes it
+// (crates/nuvec-nn/src/layers.rs:155-162: the product, rounded to the element type, then a separate addition, rounded
+// again).  The result is exact in the element type, so storing it rounds nothing.
+template <typename T>
+__device__ __forceinline__ float add_row_bias(const void *row_bias, float v, int64_t n) {
+    return row_bias == nullptr ? v : Elem<T>::add(Elem<T>::mul(v, 1.0f), Elem<T>::load((const T *)row_bias, n));
+}
+
 // Rust's f32::min / f32::max as the reference's hosts evaluate them: the other operand
 // when one is NaN, and -0 ordered below +0.
 __device__ __forceinline__ float rs_min(float a, float b) {

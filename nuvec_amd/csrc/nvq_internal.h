@@ -84,6 +84,8 @@ struct ProductArgs {
     float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
     const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (general kernel only)
     const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
+    const void *row_bias;           // NULL, or one value of the element type per column of y, added to the rounded product
+                                    // (QuantizedLinear's bias)
     int32_t row_exact;              // every row takes the arithmetic of its one-row product: the vector kernels only, K split
                                     // (weights stored [K, N]) by the weight's shape alone
 };

@@ -464,7 +464,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
             const int l = idx & 63, v = (idx >> 6) % NV, rg = idx / (64 * NV);
             const float sum = ((slot_of(0, rg, v)[l] + slot_of(1, rg, v)[l]) + slot_of(2, rg, v)[l]) + slot_of(3, rg, v)[l];
             const int m = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), col = n0 + 32 * rg + (l & 31);
-            if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, sum);
+            if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, add_row_bias<T>(a.row_bias, sum, col));
         }
         __syncthreads();
     };

@@ -405,7 +405,8 @@ qmm_kernel(const ProductArgs a) {
                 const int row0 = m0 + wm * (32 * TI) + i * 32 + 4 * h;
 #pragma unroll
                 for (int e = 0; e < 16; e += 2) {
-                    const uint32_t pair = Ops<T>::pack(acc[i][j][e], acc[i][j][e + 1]);  // rounded to nearest even
+                    const uint32_t pair = Ops<T>::pack(add_row_bias<T>(a.row_bias, acc[i][j][e], col),
+                                                       add_row_bias<T>(a.row_bias, acc[i][j][e + 1], col));  // rounded to nearest even
                     const int r = i * 32 + 8 * (e >> 2) + (e & 3);
                     uint16_t *out = out0 + (int64_t)r * N + j * 32;
                     if (whole || (row0 + r - i * 32 < M && col < N)) out[0] = (uint16_t)pair;
@@ -437,7 +438,8 @@ qmm_kernel(const ProductArgs a) {
 
 // y = the splits' partial sums added in split order, rounded once.
 template <typename T>
-__global__ void __launch_bounds__(256) qmm_reduce_kernel(const float *__restrict__ partials, T *__restrict__ y, int splits, int64_t total) {
+__global__ void __launch_bounds__(256) qmm_reduce_kernel(const float *__restrict__ partials, T *__restrict__ y, int splits, int64_t total,
+                                                         const void *row_bias, int64_t n) {
     const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (idx >= total) return;
     if (idx + 4 <= total) {
@@ -446,12 +448,14 @@ __global__ void __launch_bounds__(256) qmm_reduce_kernel(const float *__restrict
             const float4 v = *reinterpret_cast<const float4 *>(partials + s * total + idx);
             sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
         }
-        Elem<T>::store(y, idx, sum.x), Elem<T>::store(y, idx + 1, sum.y), Elem<T>::store(y, idx + 2, sum.z), Elem<T>::store(y, idx + 3, sum.w);
+        const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) Elem<T>::store(y, idx + j, add_row_bias<T>(row_bias, v[j], (idx + j) % n));
     } else {
         for (int64_t i = idx; i < total; i++) {
             float sum = 0.0f;
             for (int s = 0; s < splits; s++) sum += partials[s * total + i];
-            Elem<T>::store(y, i, sum);
+            Elem<T>::store(y, i, add_row_bias<T>(row_bias, sum, i % n));
         }
     }
 }
@@ -521,7 +525,7 @@ int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     NVQ_LAUNCH_CHECK("qmm");
     if (splits > 1) {
         const int64_t total = a.m * a.n;
-        hipLaunchKernelGGL((qmm_reduce_kernel<T>), dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s, a.partials, (T *)a.y, splits, total);
+        hipLaunchKernelGGL((qmm_reduce_kernel<T>), dim3((unsigned)((total / 4 + 256) / 256)), dim3(256), 0, s, a.partials, (T *)a.y, splits, total, a.row_bias, a.n);
         NVQ_LAUNCH_CHECK("qmm_reduce");
     }
     return NVQ_OK;

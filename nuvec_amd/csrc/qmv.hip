@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 #pragma unroll
     for (int i = 0; i < RM; i++) {
         const float v = wave_sum_lane63(acc[i]);
-        if (lane == 63 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, v);
+        if (lane == 63 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, add_row_bias<T>(a.row_bias, v, n));
     }
 }
 
@@ -441,7 +441,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
 #pragma unroll
         for (int i = 0; i < RM; i++) {
             const float v = wave_sum_lane63(acc[r][i]);
-            if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, v);
+            if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, add_row_bias<T>(a.row_bias, v, n0 + r));
         }
 }
 
@@ -664,7 +664,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
         float v = 0.0f;
 #pragma unroll
         for (int wv = 0; wv < kMmWaves; wv++) v += partial[(wv * RM + i) * kMmRows + col];
-        if (m0 + i < M && n0 + col < N) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + col, v);
+        if (m0 + i < M && n0 + col < N) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + col, add_row_bias<T>(a.row_bias, v, n0 + col));
     }
 }
 
@@ -881,7 +881,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
         for (int wv = 0; wv < waves; wv++)
 #pragma unroll
             for (int q = 0; q < kQ; q++) v += src[wv * kMpl * 64 + 16 * q];
-        if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, v);
+        if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, add_row_bias<T>(a.row_bias, v, n0 + 16 * rt + n));
     }
 }
 

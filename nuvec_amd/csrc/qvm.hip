@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
             T *out = (T *)a.y + (o.y * M + m0 + i) * N + n0;
 #pragma unroll
             for (int j = 0; j < 32; j++)
-                if (j < 16 || whole) Elem<T>::store(out, j, acc[i][j] + accb[i]);
+                if (j < 16 || whole) Elem<T>::store(out, j, add_row_bias<T>(a.row_bias, acc[i][j] + accb[i], n0 + j));
         } else {
             float *out = partial + (((int64_t)bz * splits + blockIdx.y) * M + m0 + i) * N + n0;
 #pragma unroll
@@ -174,13 +174,14 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
 
 // y[b, m, n] = the splits' partial sums added in split order, rounded once.
 template <typename T>
-__global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T *y, int splits, int64_t per_batch, int64_t total) {
+__global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T *y, int splits, int64_t per_batch, int64_t total,
+                                                         const void *row_bias, int64_t n) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int64_t b = idx / per_batch, rest = idx - b * per_batch;
     float sum = 0.0f;
     for (int s = 0; s < splits; s++) sum += partial[(b * splits + s) * per_batch + rest];
-    Elem<T>::store(y, idx, sum);
+    Elem<T>::store(y, idx, add_row_bias<T>(row_bias, sum, idx % n));
 }
 
 template <typename T, int BITS, int MODE>
@@ -199,7 +200,7 @@ int32_t run_qvm(const ProductArgs &a, void *workspace, hipStream_t s) {
     if (splits > 1) {
         const int64_t per_batch = a.m * a.n, total = a.batch * per_batch;
         hipLaunchKernelGGL((qvm_reduce_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const float *)workspace,
-                           (T *)a.y, splits, per_batch, total);
+                           (T *)a.y, splits, per_batch, total, a.row_bias, a.n);
         NVQ_LAUNCH_CHECK("qvm_reduce");
     }
     return NVQ_OK;

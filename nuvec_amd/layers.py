@@ -41,9 +41,17 @@ class QuantizedLinear:
         return ops.dequantize(self.quantized(), dtype)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """layers.rs:155-162: the product, then the bias added as a separate rounded addition."""
-        y = ops.quantized_matmul(x, self.quantized(), transpose=True)
-        return y if self.bias is None else y + self.bias
+        """layers.rs:155-162: the product, then the bias added as a separate rounded addition: here in the product
+        kernels' epilogues (same two roundings, one launch) when the bias has the product's dtype and the mode no global
+        scale; otherwise the addition stays separate, as in the reference, and promotes."""
+        q = self.quantized()
+        if self.bias is None:
+            return ops.quantized_matmul(x, q, transpose=True)
+        affine = self.quant.mode == QuantMode.AFFINE
+        dtype = torch.promote_types(torch.promote_types(x.dtype, self.scales.dtype), self.biases.dtype) if affine else x.dtype
+        if self.bias.dtype == dtype and self.bias.ndim == 1 and x.shape[-1] > 0 and getattr(q, "global_scale", None) is None:
+            return ops.quantized_matmul(x, q, transpose=True, bias=self.bias)
+        return ops.quantized_matmul(x, q, transpose=True) + self.bias
 
     __call__ = forward
 

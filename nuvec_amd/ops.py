@@ -342,10 +342,11 @@ def _strides(t: torch.Tensor, nbatch: int):
 
 
 def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, row_exact: bool = False, rows: bool = False,
-                     scratch: bool = True) -> torch.Tensor:
+                     scratch: bool = True, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """ops.rs:1031-1045, quantized.rs:446-537, primitive.rs:1279-1320.  `row_exact` and `rows` are the primitive's
     routing flags (primitive.rs:489-493; `with_row_exact`, lib.rs:159-193).  `scratch=False` hands the library no
-    workspace (a transposed product then runs without splitting K)."""
+    workspace (a transposed product then runs without splitting K).  `bias` ([N], the product's dtype) is added in the
+    kernels' epilogues as `QuantizedLinear::forward` adds it (layers.rs:155-162)."""
     op = "quantized_matmul"
     quant = q.quant
     group, bits = quant.checked(op)
@@ -406,7 +407,13 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     lib = _lib.load()
     need = lib.nvq_quantized_matmul_workspace_bytes(C.byref(d))
     workspace = torch.empty(need, dtype=torch.uint8, device=x.device) if need and scratch else None
-    if g is not None:
+    if bias is not None:
+        if g is not None or bias.dtype != dtype or bias.ndim != 1 or bias.shape[0] != outer:
+            raise InvalidArgument(f"{op}: the fused bias must be [{outer}] of {_name(dtype)} and the mode without a global scale")
+        bias = bias.contiguous()
+        _lib.check(lib.nvq_quantized_linear(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(bias), _ptr(out),
+                                            _ptr(workspace), _stream()))
+    elif g is not None:
         _lib.check(lib.nvq_quantized_matmul_scaled(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(g), _ptr(out),
                                                    _ptr(workspace), _stream()))
     else:

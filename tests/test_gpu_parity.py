@@ -701,6 +701,36 @@ def test_layers_mirror_the_reference_callers():
     assert_rows_close(tied, want, ref.BF16, "tied embedding")
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16, ref.F32])
+def test_linear_bias_in_the_product_epilogues(dtype):
+    """nvq_quantized_linear on every product route (decode kernels, both matrix-core few-row kernels, the tiled kernel with
+    and without a split of K, the general kernel's widths and block formats, weights stored [K, N]): bit for bit the
+    product this library returns followed by the separate rounded addition of the reference (layers.rs:155-162)."""
+    rng = np.random.default_rng(5200 + dtype)
+    cases = [(nv.Quant.affine(64, 4), 4096, 1024, (1, 2, 3, 4, 8, 16, 40, 300)), (nv.Quant.affine(64, 4), 4096, 4096, (512,)),
+             (nv.Quant.affine(64, 3), 1024, 200, (1, 5, 33, 260)), (nv.Quant.affine(32, 8), 512, 96, (1, 7, 200)),
+             (nv.Quant.affine(128, 5), 1024, 77, (1, 9)), (nv.Quant.new(nv.QuantMode.MXFP4), 2880, 360, (1, 6, 70, 300)),
+             (nv.Quant.new(nv.QuantMode.MXFP8), 1024, 130, (1, 12)), (nv.Quant.new(nv.QuantMode.NVFP4), 1024, 130, (1, 12, 300))]
+    for quant, k, n, ms in cases:
+        q = nv.quantize(to_dev(make_w(rng, n, k, dtype)), quant)
+        bias = to_dev(make_x(rng, 1, n, dtype).reshape(n))
+        for m in ms:
+            x = to_dev(make_x(rng, m, k, dtype))
+            plain = nv.quantized_matmul(x, q)
+            fused = nv.quantized_matmul(x, q, bias=bias)
+            assert np.array_equal(to_host(fused).view(np.uint8), to_host(plain + bias).view(np.uint8)), f"{quant} M={m} N={n} K={k}"
+    # weights stored [K, N]
+    k, n = 512, 256
+    q = nv.quantize(to_dev(make_w(rng, k, n, dtype)), nv.Quant.affine(64, 4))
+    bias = to_dev(make_x(rng, 1, n, dtype).reshape(n))
+    for m in (1, 6):
+        x = to_dev(make_x(rng, m, k, dtype))
+        fused = nv.quantized_matmul(x, q, transpose=False, bias=bias)
+        assert np.array_equal(to_host(fused).view(np.uint8), to_host(nv.quantized_matmul(x, q, transpose=False) + bias).view(np.uint8))
+    with pytest.raises(nv.InvalidArgument):
+        nv.quantized_matmul(x, q, transpose=False, bias=bias[:-1])
+
+
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 @pytest.mark.parametrize("group,k,n", [(64, 2048, 100), (128, 4096, 96), (64, 6144, 33), (128, 10240, 64)])
 def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
