@@ -128,6 +128,20 @@ typedef struct nvq_gather_desc {
     int64_t experts;
 } nvq_gather_desc;
 
+/* FastOp::QuantizedAttention (crates/nuvec-core/src/fast.rs:694-718; fit rule fast/imp.rs:3944-3992): one query row per
+ * head over an affine-quantized key / value cache.
+ *   q dtype [batch, query_heads, 1, head_dim];  k_w, v_w u32 [batch, key_heads, positions, head_dim*bits/32];
+ *   k_s, k_b, v_s, v_b dtype [batch, key_heads, positions, head_dim/group_size];  sinks dtype [query_heads] or NULL;
+ *   out dtype [batch, query_heads, 1, head_dim], all contiguous. */
+typedef struct nvq_attention_desc {
+    int32_t dtype;      /* NVQ_F16 / NVQ_BF16 / NVQ_F32: q, scales, biases, sinks, out */
+    int32_t bits;       /* 4 or 8 (3 bits: NVQ_UNSUPPORTED, the caller's composition) */
+    int32_t group_size; /* 32, 64 or 128, dividing head_dim */
+    int32_t head_dim;   /* 64 or 128 */
+    int64_t batch, query_heads, key_heads, positions;
+    float scale;
+} nvq_attention_desc;
+
 /* ── runtime ─────────────────────────────────────────────────────────────────────── */
 
 /* Binds the library to HIP device `device` (idempotent; the process-wide device record,
@@ -226,6 +240,15 @@ NVQ_API int32_t nvq_quantized_linear(const nvq_qmm_desc *desc, const void *x, co
 #define NVQ_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
 NVQ_API int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *desc, const void *x, const void *w, const void *scales,
                                     const void *biases, void *y, void *stream);
+
+/* GpuEval::quantized_attention (gpu.rs:4969-5040): softmax(scale * q . K^T [, sinks]) . V in one kernel, the codes
+ * dequantized in registers (never rounded), float32 products and sums; within the float bound of the dequantized
+ * attention, as the reference's kernel.  What the fit rule excludes (several query rows, a mask, other head sizes,
+ * 3 bits, query heads that are not 1, 2, 4 or 8 per key head) answers NVQ_UNSUPPORTED: the caller then records the
+ * composition of two quantized products and a softmax, as the reference does (fast/imp.rs:3996-4035). */
+NVQ_API int32_t nvq_quantized_attention(const nvq_attention_desc *desc, const void *q, const void *k_w, const void *k_s,
+                                const void *k_b, const void *v_w, const void *v_s, const void *v_b, const void *sinks,
+                                void *out, void *stream);
 
 /* GpuEval::sorted_offsets (gpu.rs:6732-6756); kernels::sorted_offsets (kernels.rs:873-892):
  * per row of `indices` u32[rows, m], offsets[row, g] = first position whose value is >= g. */

@@ -54,6 +54,12 @@ class QmmDescC(C.Structure):
                 ("x_strides", _DIMS), ("w_strides", _DIMS), ("s_strides", _DIMS)]
 
 
+class AttentionDescC(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("bits", C.c_int32), ("group_size", C.c_int32), ("head_dim", C.c_int32),
+                ("batch", C.c_int64), ("query_heads", C.c_int64), ("key_heads", C.c_int64), ("positions", C.c_int64),
+                ("scale", C.c_float)]
+
+
 class GatherDescC(C.Structure):
     _fields_ = [("quant", QuantC), ("dtype", C.c_int32), ("transpose", C.c_int32), ("row_exact", C.c_int32),
                 ("reserved", C.c_int32), ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64), ("pairs", C.c_int64),
@@ -82,6 +88,7 @@ SIGNATURES = {
     "nvq_quantized_linear": (C.c_int32, [C.POINTER(QmmDescC)] + [C.c_void_p] * 8),
     "nvq_quantized_matmul_static": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                                 C.c_void_p, C.c_void_p]),
+    "nvq_quantized_attention": (C.c_int32, [C.POINTER(AttentionDescC)] + [C.c_void_p] * 10),
     "nvq_sorted_offsets": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),
     "nvq_quantize_scaled": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_dequantize_scaled": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),

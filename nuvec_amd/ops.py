@@ -422,6 +422,46 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     return out.squeeze(-2) if vector else out
 
 
+def quantized_attention_fits(q: torch.Tensor, k: Quantized, v: Quantized, sinks: Optional[torch.Tensor] = None) -> bool:
+    """fast/imp.rs:3944-3992: whether the fused kernel takes these operands (else the composition)."""
+    if q.ndim != 4 or k.weight.ndim != 4 or v.weight.ndim != 4 or k.quant != v.quant or k.quant.mode != QuantMode.AFFINE:
+        return False
+    b, hq, l, d = q.shape
+    group, bits = k.quant.group_size, k.quant.bits
+    if q.dtype not in _FLOATS or l != 1 or d not in (64, 128) or bits not in (4, 8) or group not in (32, 64, 128) or d % group:
+        return False
+    hkv, n = k.weight.shape[1], k.weight.shape[2]
+    for t in (k, v):
+        if t.biases is None or t.weight.dtype != torch.uint32 or tuple(t.weight.shape) != (b, hkv, n, d * bits // 32):
+            return False
+        if tuple(t.scales.shape) != (b, hkv, n, d // group) or t.biases.shape != t.scales.shape:
+            return False
+        if t.scales.dtype != q.dtype or t.biases.dtype != q.dtype:
+            return False
+    if hkv == 0 or n < 1 or hq % hkv or hq // hkv not in (1, 2, 4, 8):
+        return False
+    return sinks is None or (sinks.ndim == 1 and sinks.numel() == hq and sinks.dtype == q.dtype)
+
+
+def quantized_attention(q: torch.Tensor, k: Quantized, v: Quantized, scale: float,
+                        sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fast.rs:694-718 where the kernel fits (`quantized_attention_fits`): one query row per head over the quantized
+    cache in one launch."""
+    if not quantized_attention_fits(q, k, v, sinks):
+        raise Unsupported("quantized_attention: the operands do not fit the kernel")
+    _init(q)
+    b, hq, _, d = q.shape
+    q = q.contiguous()
+    kw, ks, kb = _u32(k.weight).contiguous(), k.scales.contiguous(), k.biases.contiguous()
+    vw, vs, vb = _u32(v.weight).contiguous(), v.scales.contiguous(), v.biases.contiguous()
+    sinks = None if sinks is None else sinks.contiguous()
+    out = torch.empty_like(q)
+    desc = _lib.AttentionDescC(_CODE[q.dtype], k.quant.bits, k.quant.group_size, d, b, hq, kw.shape[1], kw.shape[2], float(scale))
+    _lib.check(_lib.load().nvq_quantized_attention(C.byref(desc), _ptr(q), _ptr(kw), _ptr(ks), _ptr(kb), _ptr(vw), _ptr(vs), _ptr(vb),
+                                                   _ptr(sinks), _ptr(out), _stream()))
+    return out
+
+
 def sorted_offsets(rhs: torch.Tensor, groups: int) -> torch.Tensor:
     """kernels.rs:873-892: per row of the last axis, where each group's indices start."""
     _init(rhs)

@@ -1031,7 +1031,7 @@ def test_quantized_attention_composition(dtype, group, bits, d):
     oracle's dequantized cache in float64 (the bound the reference states for it: that of the dequantized attention)."""
     from nuvec_amd.layers import quantized_attention
     rng = np.random.default_rng(8100 + bits + dtype)
-    b, hkv, rep, s = 2, 2, 4, 192
+    b, hkv, rep, s = 2, 2, 4, 203  # positions that fill no tile of keys
     hq = hkv * rep
     kd, vd = make_x(rng, b * hkv * s, d, dtype).reshape(b, hkv, s, d), make_x(rng, b * hkv * s, d, dtype).reshape(b, hkv, s, d)
     kq, vq = ref.affine_quantize(kd, dtype, group, bits), ref.affine_quantize(vd, dtype, group, bits)
@@ -1046,6 +1046,9 @@ def test_quantized_attention_composition(dtype, group, bits, d):
     qf = ref.to_f32(q, dtype).astype(np.float64).reshape(b, hkv, rep, d)
     logits = scale * np.einsum("bhrd,bhsd->bhrs", qf, kf)
     tol = {ref.BF16: 2e-2, ref.F32: 2e-5}[dtype]
+    from nuvec_amd import ops as nv_ops
+    fits = nv_ops.quantized_attention_fits(to_dev(q), K, V)
+    assert fits == (bits in (4, 8) and d in (64, 128))  # the fused kernel's rule (fast/imp.rs:3944-3992) less its 3 bits
     for use_sinks in (False, True):
         full = logits
         if use_sinks:
@@ -1053,9 +1056,10 @@ def test_quantized_attention_composition(dtype, group, bits, d):
         p = np.exp(full - full.max(-1, keepdims=True))
         p = (p / p.sum(-1, keepdims=True))[..., :s]
         want = np.einsum("bhrs,bhsd->bhrd", p, vf).reshape(b, hq, 1, d)
-        got = quantized_attention(to_dev(q), K, V, scale, to_dev(sinks) if use_sinks else None)
-        assert tuple(got.shape) == (b, hq, 1, d)
-        err = np.abs(ref.to_f32(to_host(got), dtype).astype(np.float64) - want).max()
-        assert err <= tol * max(1.0, np.abs(want).max()), f"sinks={use_sinks}: {err}"
+        for fused in (True, False):  # the kernel where it fits, and the composition
+            got = quantized_attention(to_dev(q), K, V, scale, to_dev(sinks) if use_sinks else None, fused=fused)
+            assert tuple(got.shape) == (b, hq, 1, d)
+            err = np.abs(ref.to_f32(to_host(got), dtype).astype(np.float64) - want).max()
+            assert err <= tol * max(1.0, np.abs(want).max()), f"sinks={use_sinks} fused={fused}: {err}"
     with pytest.raises(nv.InvalidArgument):
         quantized_attention(to_dev(q), K, nv.Quantized(V.weight, V.scales, V.biases, nv.Quant.affine(group, 2 if bits != 2 else 4)), scale)

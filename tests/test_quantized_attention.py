@@ -60,7 +60,10 @@ def test_quantized_attention_matches_the_recorded_outputs(recorded, dt, bits, l)
     g = lambda k: recorded[f"{dt}_b{bits}_l{l}_{k}"].cuda()
     quant = nv.Quant.affine(GROUP, bits)
     k, v = nv.Quantized(g("k0"), g("k1"), g("k2"), quant), nv.Quantized(g("v0"), g("v1"), g("v2"), quant)
-    got = quantized_attention(g("q"), k, v, SCALE, causal=l > 1)
     want = recorded[f"{dt}_b{bits}_l{l}_out"]
-    assert got.shape == want.shape and got.dtype == want.dtype
-    assert (got.cpu().float() - want.float()).abs().max().item() < TOL[dt]
+    for fused in (True, False):  # one query row: the fused kernel and the composition; several: the composition twice
+        got = quantized_attention(g("q"), k, v, SCALE, causal=l > 1, fused=fused)
+        assert got.shape == want.shape and got.dtype == want.dtype
+        assert (got.cpu().float() - want.float()).abs().max().item() < TOL[dt]
+    from nuvec_amd import ops
+    assert ops.quantized_attention_fits(g("q"), k, v) == (l == 1)
