@@ -245,10 +245,14 @@ NVQ_API int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *desc, const void
  * dequantized in registers (never rounded), float32 products and sums; within the float bound of the dequantized
  * attention, as the reference's kernel.  What the fit rule excludes (several query rows, a mask, other head sizes,
  * 3 bits, query heads that are not 1, 2, 4 or 8 per key head) answers NVQ_UNSUPPORTED: the caller then records the
- * composition of two quantized products and a softmax, as the reference does (fast/imp.rs:3996-4035). */
+ * composition of two quantized products and a softmax, as the reference does (fast/imp.rs:3996-4035).
+ * With the workspace the size query names (float32 states of the splits: maximum, denominator and weighted sum per
+ * split and head) the positions are split over the grid and a second kernel merges the splits; with NULL one block
+ * walks all positions of a head. */
+NVQ_API size_t nvq_quantized_attention_workspace_bytes(const nvq_attention_desc *desc);
 NVQ_API int32_t nvq_quantized_attention(const nvq_attention_desc *desc, const void *q, const void *k_w, const void *k_s,
                                 const void *k_b, const void *v_w, const void *v_s, const void *v_b, const void *sinks,
-                                void *out, void *stream);
+                                void *out, void *workspace, void *stream);
 
 /* GpuEval::sorted_offsets (gpu.rs:6732-6756); kernels::sorted_offsets (kernels.rs:873-892):
  * per row of `indices` u32[rows, m], offsets[row, g] = first position whose value is >= g. */

@@ -512,8 +512,8 @@ int32_t nvq_quantized_matmul_scaled(const nvq_qmm_desc *d, const void *x, const 
     return quantized_matmul_any(d, x, w, scales, nullptr, global_scale, y, workspace, stream);
 }
 
-int32_t nvq_quantized_attention(const nvq_attention_desc *d, const void *q, const void *k_w, const void *k_s, const void *k_b,
-                                const void *v_w, const void *v_s, const void *v_b, const void *sinks, void *out, void *stream) {
+// The argument checks and the fit rule of the fused attention kernel (fast/imp.rs:3944-3992, 4037-4075).
+static int32_t check_attention(const nvq_attention_desc *d) {
     const char *op = "quantized_attention";
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null descriptor", op);
     NVQ_TRY(check_float(op, d->dtype));
@@ -521,21 +521,34 @@ int32_t nvq_quantized_attention(const nvq_attention_desc *d, const void *q, cons
     NVQ_TRY(check_quant(&quant, op));
     if (d->batch < 0 || d->query_heads < 0 || d->key_heads < 0 || d->positions < 0 || d->head_dim < 0)
         return fail(NVQ_INVALID_ARGUMENT, "%s: negative size", op);
-    if (d->key_heads == 0 || d->query_heads % d->key_heads != 0)  // fast/imp.rs:4060-4070
+    if (d->key_heads == 0 || d->query_heads % d->key_heads != 0)
         return fail(NVQ_INVALID_ARGUMENT, "%s: %lld query heads over %lld key heads", op, (long long)d->query_heads, (long long)d->key_heads);
-    // the kernel's fit rule (fast/imp.rs:3944-3992); beyond it the caller composes
     const int64_t rep = d->query_heads / d->key_heads;
     if ((d->head_dim != 64 && d->head_dim != 128) || (d->bits != 4 && d->bits != 8) || d->head_dim % d->group_size != 0 ||
         !(rep == 1 || rep == 2 || rep == 4 || rep == 8) || d->positions < 1 || d->batch > 65535 ||
         d->batch * d->key_heads * d->positions * d->head_dim >= (1LL << 31))
         return fail(NVQ_UNSUPPORTED, "%s: the kernel takes head sizes 64 and 128, 4 or 8 bits, 1, 2, 4 or 8 query heads per key head", op);
+    return NVQ_OK;
+}
+
+size_t nvq_quantized_attention_workspace_bytes(const nvq_attention_desc *d) {
+    if (check_attention(d) != NVQ_OK || require_device() != NVQ_OK) return 0;
+    return attention_workspace_bytes(*d);
+}
+
+int32_t nvq_quantized_attention(const nvq_attention_desc *d, const void *q, const void *k_w, const void *k_s, const void *k_b,
+                                const void *v_w, const void *v_s, const void *v_b, const void *sinks, void *out, void *workspace,
+                                void *stream) {
+    const char *op = "quantized_attention";
+    NVQ_TRY(check_attention(d));
     if (d->batch == 0 || d->query_heads == 0) return NVQ_OK;
     if (q == nullptr || k_w == nullptr || k_s == nullptr || k_b == nullptr || v_w == nullptr || v_s == nullptr || v_b == nullptr || out == nullptr)
         return fail(NVQ_INVALID_ARGUMENT, "%s: null operand", op);
     NVQ_TRY(require_device());
     NVQ_TRY(check_aligned(op, "keys", k_w));
     NVQ_TRY(check_aligned(op, "values", v_w));
-    return launch_quantized_attention(*d, q, k_w, k_s, k_b, v_w, v_s, v_b, sinks, out, (hipStream_t)stream);
+    NVQ_TRY(check_aligned(op, "workspace", workspace));
+    return launch_quantized_attention(*d, q, k_w, k_s, k_b, v_w, v_s, v_b, sinks, out, workspace, (hipStream_t)stream);
 }
 
 int32_t nvq_sorted_offsets(const uint32_t *indices, int64_t rows, int64_t m, int32_t groups, int32_t *offsets, void *stream) {

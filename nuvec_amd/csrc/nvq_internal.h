@@ -102,7 +102,9 @@ bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);
 int32_t launch_fill_zero(void *p, int64_t bytes, hipStream_t s);
 int32_t launch_quantized_attention(const nvq_attention_desc &d, const void *q, const void *kw, const void *ks, const void *kb,
-                                   const void *vw, const void *vs, const void *vb, const void *sinks, void *out, hipStream_t s);
+                                   const void *vw, const void *vs, const void *vb, const void *sinks, void *out, void *workspace,
+                                   hipStream_t s);
+size_t attention_workspace_bytes(const nvq_attention_desc &d);  // float32 states of the splits of the positions, or 0
 int32_t launch_calibrate(int32_t kind, const void *buffer, int64_t bytes, int32_t iters, void *sink, int64_t *work, hipStream_t s);
 // Products with the weights stored [K, N] (transpose = false); K is split over the grid through a float32 workspace.
 int qvm_splits(const ProductArgs &a);

@@ -444,7 +444,7 @@ def quantized_attention_fits(q: torch.Tensor, k: Quantized, v: Quantized, sinks:
 
 
 def quantized_attention(q: torch.Tensor, k: Quantized, v: Quantized, scale: float,
-                        sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        sinks: Optional[torch.Tensor] = None, scratch: bool = True) -> torch.Tensor:
     """fast.rs:694-718 where the kernel fits (`quantized_attention_fits`): one query row per head over the quantized
     cache in one launch."""
     if not quantized_attention_fits(q, k, v, sinks):
@@ -457,8 +457,11 @@ def quantized_attention(q: torch.Tensor, k: Quantized, v: Quantized, scale: floa
     sinks = None if sinks is None else sinks.contiguous()
     out = torch.empty_like(q)
     desc = _lib.AttentionDescC(_CODE[q.dtype], k.quant.bits, k.quant.group_size, d, b, hq, kw.shape[1], kw.shape[2], float(scale))
-    _lib.check(_lib.load().nvq_quantized_attention(C.byref(desc), _ptr(q), _ptr(kw), _ptr(ks), _ptr(kb), _ptr(vw), _ptr(vs), _ptr(vb),
-                                                   _ptr(sinks), _ptr(out), _stream()))
+    lib = _lib.load()
+    need = lib.nvq_quantized_attention_workspace_bytes(C.byref(desc)) if scratch else 0
+    workspace = torch.empty(need, dtype=torch.uint8, device=q.device) if need else None
+    _lib.check(lib.nvq_quantized_attention(C.byref(desc), _ptr(q), _ptr(kw), _ptr(ks), _ptr(kb), _ptr(vw), _ptr(vs), _ptr(vb),
+                                           _ptr(sinks), _ptr(out), _ptr(workspace), _stream()))
     return out
 
 

@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 import torch
 
+import nuvec_amd as nv
 from nuvec_amd import checkpoint as ck
 from oracle import ref
 
@@ -67,3 +68,34 @@ def test_quantized_attention_matches_the_recorded_outputs(recorded, dt, bits, l)
         assert (got.cpu().float() - want.float()).abs().max().item() < TOL[dt]
     from nuvec_amd import ops
     assert ops.quantized_attention_fits(g("q"), k, v) == (l == 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch,hq,hkv,s,d,bits,group,with_sinks", [
+    (1, 32, 8, 8192, 128, 4, 64, False), (2, 8, 8, 1000, 64, 8, 32, True), (1, 4, 1, 777, 128, 8, 128, True),
+    (3, 16, 2, 2049, 64, 4, 64, False), (1, 2, 2, 513, 128, 4, 32, True)])
+def test_positions_split_over_the_grid(batch, hq, hkv, s, d, bits, group, with_sinks):
+    """Long caches: the positions split over the grid and merged (with the workspace) against one block per head
+    (without) and against float32 attention over the dequantized cache; lengths off the tile size, grouped heads,
+    sinks.  Bound: 2e-3 of the largest output, far under the bfloat16 step of the recorded cases' tolerance."""
+    from nuvec_amd import ops
+    torch.manual_seed(s)
+    kd, vd = torch.randn(batch, hkv, s, d, device="cuda"), torch.randn(batch, hkv, s, d, device="cuda")
+    quant = nv.Quant.affine(group, bits)
+    k, v = nv.quantize(kd, quant), nv.quantize(vd, quant)
+    q = torch.randn(batch, hq, 1, d, device="cuda")
+    sinks = torch.randn(hq, device="cuda") if with_sinks else None
+    scale = d ** -0.5
+    assert ops.quantized_attention_fits(q, k, v)
+    split = ops.quantized_attention(q, k, v, scale, sinks)
+    whole = ops.quantized_attention(q, k, v, scale, sinks, scratch=False)
+    kf = nv.dequantize(k).repeat_interleave(hq // hkv, dim=1)
+    vf = nv.dequantize(v).repeat_interleave(hq // hkv, dim=1)
+    scores = scale * q @ kf.transpose(-1, -2)
+    if with_sinks:
+        scores = torch.cat([scores, sinks.view(1, hq, 1, 1).expand(batch, hq, 1, 1)], dim=-1)
+    p = torch.softmax(scores, dim=-1)[..., :s]
+    want = p @ vf
+    bound = 2e-3 * want.abs().max().item()
+    assert (split - want).abs().max().item() <= bound, "split"
+    assert (whole - want).abs().max().item() <= bound, "one block per head"
