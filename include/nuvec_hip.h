@@ -213,6 +213,12 @@ NVQ_API int32_t nvq_dequantize_rows(const nvq_quant *quant, int32_t dtype, const
  * split over the grid (float32 partial sums): transpose = 0, and transpose = 1 products of many rows with few
  * output tiles and a long K (the counterpart of the reference's qmm_t_splitk, gpu.rs:7507-7590).  A transposed
  * product given no workspace runs unsplit. */
+/* The kernel a product of this descriptor runs on with operands aligned as hipMalloc aligns them ("qmm_kernel",
+ * "qmf_kernel", "qmd_kernel", "qmv4_lds_kernel", ...), from the same routing code as the launch; NULL with
+ * nvq_last_error for a descriptor the launch would refuse.  The reference names its kernels by route as well
+ * (gpu.rs:7022, "nuvec_affine_qmv_mma_..."; its tests check the names, crates/nuvec-core/tests/quantized.rs:843-861).
+ * Needs nvq_init. */
+NVQ_API const char *nvq_quantized_matmul_route(const nvq_qmm_desc *desc);
 NVQ_API size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *desc);
 
 /* GpuEval::quantized_matmul / fp_quantized_matmul (gpu.rs:6934-7168, 6336-6577); values of

@@ -88,6 +88,7 @@ SIGNATURES = {
     "nvq_quantized_linear": (C.c_int32, [C.POINTER(QmmDescC)] + [C.c_void_p] * 8),
     "nvq_quantized_matmul_static": (C.c_int32, [C.POINTER(QmmDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                                 C.c_void_p, C.c_void_p]),
+    "nvq_quantized_matmul_route": (C.c_char_p, [C.POINTER(QmmDescC)]),
     "nvq_quantized_attention_workspace_bytes": (C.c_size_t, [C.POINTER(AttentionDescC)]),
     "nvq_quantized_attention": (C.c_int32, [C.POINTER(AttentionDescC)] + [C.c_void_p] * 11),
     "nvq_sorted_offsets": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]),

@@ -178,6 +178,29 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
     return nvq::qmm_estimate_us(a) < few_us;
 }
 
+// Whether the 16x16x32 kernel with directly loaded weight operands takes a few-row product, from its measured times
+// against the kernels it replaces (bf16, us per launch, new / old):
+//   3 bits g64   W[4096,4096]  2 rows 6.0 / 10.5, 16 rows 6.9 / 11.5;  W[14336,4096] 16 rows 11.9 / 19.9;  W[151936,1024] 4 rows 22.6 / 72.8
+//   8 bits g32   W[4096,4096] 16 rows 11.1 / 12.9;  W[4096,14336] 8 rows 23.6 / 28.1;  W[151936,1024] 8 rows 47.8 / 74.5
+//   4 bits g64   W[14336,4096] 12 rows 12.8 / 17.5;  W[32768,2048] 16 rows 13.3 / 26.0  (up to 8 rows the 4-bit decode kernels are ahead: 13.1 / 11.1)
+//   4 bits g128  W[14336,4096]  4 rows 10.4 / 13.5, 8 rows 10.8 / 16.4;  W[151936,1024] 1 row 19.9 / 50.1
+// One row stays on the vector kernels except for very tall matrices; 17 to 32 rows (two passes) where K fits one chunk
+// and the matrix is small enough that the second pass reads it from the caches.
+static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
+    if (!nvq::qmd_supported(a)) return false;
+    const int64_t rows = a.n * a.batch;
+    if (a.m > 16) return a.m <= 32 && a.k <= 4096 && rows * a.k * a.bits <= (int64_t)32 * 8 * 1024 * 1024 && !(a.group == 32 && rows > 4096);
+    switch (a.bits) {
+    case 2: return true;
+    case 3: return a.group == 128 || a.m >= 2 || rows >= 16384;
+    case 8: return a.m >= 2 || rows >= (a.group == 128 ? 32768 : 65536);
+    default:  // 4 bits: beside the 4-bit decode kernels
+        if (a.group == 64) return a.m > 8 || (a.m > 4 && !nvq::qmv_d16_takes(a));
+        if (a.group == 128) return a.m >= 3 || rows >= 32768;
+        return a.m >= 5 || (rows >= 32768 && a.m >= 2) || rows >= 65536;
+    }
+}
+
 // The kernels' view of a product descriptor.
 static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     nvq::ProductArgs a{};
@@ -435,6 +458,25 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
     return !a.row_exact && takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
 }
 
+// The kernel family of a product (the counterpart of the routing in GpuEval::quantized_matmul, gpu.rs:6934-7168).
+enum class Route { kUntransposed, kVector, kTiled, kFewRowsDirect, kFewRows };
+
+static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
+    if (a.global_scale != nullptr) return Route::kVector;  // NVFP4, transposed, one matrix: the general kernel
+    if (!d->transpose) return Route::kUntransposed;        // weights stored [K, N]
+    if (a.row_exact) return Route::kVector;                // the vector kernels: a row's bits do not depend on its neighbours
+    if (takes_tiled(d, a)) return Route::kTiled;
+    if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;
+    // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the
+    // decode kernels (per-row work on the vector units, which is cheaper than the matrix-core kernel's full
+    // dequantization up to there).  A single row of the other affine widths from 3 bits: the general vector kernel
+    // (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against 11.7 us with 8 bits in groups of 32).  Other
+    // few-row products share one weight decode on the matrix cores where those kernels take them.
+    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || qmv_d16_takes(a) : a.bits >= 3 && a.m == 1);
+    if (!decode && qmf_supported(a)) return Route::kFewRows;
+    return Route::kVector;
+}
+
 static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                                     const float *global_scale, void *y, void *workspace, void *stream, const void *row_bias = nullptr) {
     NVQ_TRY(check_qmm(d, "quantized_matmul"));
@@ -458,18 +500,29 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
     a.global_scale = global_scale;
     a.row_bias = row_bias;
-    if (global_scale != nullptr) return launch_qmv(a, (hipStream_t)stream);  // NVFP4, transposed, one matrix: the general kernel
-    if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]
-    if (a.row_exact) return launch_qmv(a, (hipStream_t)stream);  // the vector kernels: a row's bits do not depend on its neighbours
-    if (takes_tiled(d, a)) return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
-    // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the decode kernel (per-row work on the vector units, which is
-    // cheaper than the matrix-core kernel's full dequantization up to there).  A single row of the other affine
-    // widths from 3 bits: the general vector kernel (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against
-    // 11.7 us with 8 bits in groups of 32; from two rows on the matrix-core kernel is ahead).  Other few-row
-    // products share one weight decode on the matrix cores where that kernel takes them.
-    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || qmv_d16_takes(a) : a.bits >= 3 && a.m == 1);
-    if (!decode && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
-    return launch_qmv(a, (hipStream_t)stream);
+    switch (pick_route(d, a)) {
+    case Route::kUntransposed: return launch_qvm(a, workspace, (hipStream_t)stream);
+    case Route::kTiled: return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
+    case Route::kFewRowsDirect: return launch_qmd(a, (hipStream_t)stream);
+    case Route::kFewRows: return launch_qmf(a, (hipStream_t)stream);
+    default: return launch_qmv(a, (hipStream_t)stream);
+    }
+}
+
+const char *nvq_quantized_matmul_route(const nvq_qmm_desc *d) {
+    if (check_qmm(d, "quantized_matmul") != NVQ_OK || check_grid(d) != NVQ_OK || require_device() != NVQ_OK) return nullptr;
+    int64_t batch = 1;
+    for (int i = 0; i < d->batch_ndim; i++) batch *= d->batch_shape[i];
+    ProductArgs a = product_args(d, batch);
+    a.x = a.w = a.scales = a.biases = reinterpret_cast<const void *>(uintptr_t{256});  // operands aligned as hipMalloc aligns them
+    a.y = reinterpret_cast<void *>(uintptr_t{256});
+    switch (pick_route(d, a)) {
+    case Route::kUntransposed: return "qvm_kernel";
+    case Route::kTiled: return "qmm_kernel";
+    case Route::kFewRowsDirect: return "qmd_kernel";
+    case Route::kFewRows: return "qmf_kernel";
+    default: return qmv_kernel_name(a);
+    }
 }
 
 int32_t nvq_quantized_matmul(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
@@ -683,6 +736,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.offsets = nullptr;
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
     // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
+    if (!a.row_exact && global_scale == nullptr && takes_few_rows_direct(a)) return launch_qmd(a, (hipStream_t)stream);
     if (!a.row_exact && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }

@@ -90,8 +90,12 @@ struct ProductArgs {
                                     // (weights stored [K, N]) by the weight's shape alone
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
+const char *qmv_kernel_name(const ProductArgs &a);  // which of the vector / decode kernels launch_qmv runs for `a`
 // Whether the 16x16x32 matrix-core decode kernel takes the product (4-bit affine, groups of 64, K = 4096).
 bool qmv_d16_takes(const ProductArgs &a);
+// The 16x16x32 matrix-core kernel for passes of up to 16 rows of x (affine 2, 3, 4 and 8 bits, every group size).
+bool qmd_supported(const ProductArgs &a);
+int32_t launch_qmd(const ProductArgs &a, hipStream_t s);
 // The tiled matrix-core kernel (many rows of x); `qmm_supported` says whether it takes `a`.
 bool qmm_supported(const ProductArgs &a);
 size_t qmm_workspace_bytes(const ProductArgs &a);  // float32 partial sums when K is split over the grid, else 0

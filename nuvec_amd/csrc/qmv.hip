@@ -15,45 +15,12 @@
 #include "nvq_device.h"
 #include "nvq_internal.h"
 #include "qmf_kernel.h"  // matrix-instruction wrappers
+#include "qmv_common.h"
 
 namespace nvq {
 namespace {
 
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
-typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
-
 constexpr int kStep = 64 * 32;        // values of K per wavefront step
-
-// Element offsets of batch `z` for x, w (in packed dwords), scales/biases and y.
-struct BatchOffsets { int64_t x, w, s, y; };
-
-__device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int64_t z, int64_t kwords, int64_t kgroups) {
-    BatchOffsets o{0, 0, 0, z * a.m * a.n};
-    if (a.rhs != nullptr) {  // gathered pairs
-        // An index outside its operand is the caller's error; it is clamped so that it cannot
-        // fault the device.
-        const int64_t l = min((int64_t)a.lhs[z], a.x_batches - 1), r = min((int64_t)a.rhs[z], a.experts - 1);
-        o.x = l * a.m * a.k;
-        o.w = r * a.n * kwords;
-        o.s = r * a.n * kgroups;
-        if (a.out_rows != nullptr) o.y = min((int64_t)a.out_rows[z], a.batch - 1) * a.m * a.n;
-        return o;
-    }
-    if (a.batch_ndim == 0) return o;
-    int64_t rest = z;
-#pragma unroll
-    for (int d = NVQ_MAX_BATCH_DIMS - 1; d >= 0; d--) {  // constant indices: the arrays stay in kernel arguments
-        if (d < a.batch_ndim) {
-            const int64_t i = rest % a.batch_shape[d];
-            rest /= a.batch_shape[d];
-            o.x += i * a.x_strides[d];
-            o.w += i * a.w_strides[d];
-            o.s += i * a.s_strides[d];
-        }
-    }
-    return o;
-}
-
 
 // v + (v moved across lanes by a DPP control); lanes the control does not feed add 0.
 template <int CTRL, int ROW_MASK>
@@ -283,30 +250,6 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 }
 
 // ── 4-bit affine, bf16 / f16: packed-pair dot products ────────────────────────────────────
-// Two codes become two element-type values in one instruction: code c in the low mantissa
-// bits of the constant 128 (bf16, 0x4300) or 1024 (f16, 0x6400) is exactly 128 + c or 1024 + c.
-// `v_dot2_f32_{bf16,f16}` then accumulates x0*(B + c0) + x1*(B + c1) in float32, and the
-// offset is removed with the group's sum of x:  sum x*c = dot - B * sum x.
-template <typename T> struct Pair;
-template <> struct Pair<bf16_t> {
-    static constexpr uint32_t magic = 0x43004300u;
-    static constexpr float base = 128.0f;
-    __device__ static __forceinline__ float dot2(uint32_t x, uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, w), acc, false);
-    }
-    __device__ static __forceinline__ float lo(uint32_t p) { return u2f(p << 16); }
-    __device__ static __forceinline__ float hi(uint32_t p) { return u2f(p & 0xFFFF0000u); }
-};
-template <> struct Pair<f16_t> {
-    static constexpr uint32_t magic = 0x64006400u;
-    static constexpr float base = 1024.0f;
-    __device__ static __forceinline__ float dot2(uint32_t x, uint32_t w, float acc) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, x), __builtin_bit_cast(f16x2_t, w), acc, false);
-    }
-    __device__ static __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[0]; }
-    __device__ static __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2_t, p)[1]; }
-};
-
 // ── 4-bit affine, bf16 / f16, one or two rows of x: the decode kernel ─────────────────────
 // A block of WAVES wavefronts shares the x slice of one K step (4096 values) through LDS, stored
 // once in the pair order the nibbles need together with the sums of its 32-value slices, so the
@@ -683,20 +626,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
 // X comes from the same operands of x against a weight operand of ones, once per wavefront.
 // x is staged once per block in LDS in the pair order of the nibbles; dead tile rows read a zero piece (one
 // address: a broadcast).  The wavefronts' partial rows are added in a fixed order.
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 constexpr int kD16Rows = 16, kD16Slice = 512;  // weight rows of a tile; values of K per wavefront (a block has K / 512 wavefronts)
-
-template <typename T> struct Mfma16;
-template <> struct Mfma16<bf16_t> {
-    __device__ static __forceinline__ floatx4_t run(uint4 a, uint4 b, floatx4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(qmf::bf16x8_t, a), __builtin_bit_cast(qmf::bf16x8_t, b), c, 0, 0, 0);
-    }
-};
-template <> struct Mfma16<f16_t> {
-    __device__ static __forceinline__ floatx4_t run(uint4 a, uint4 b, floatx4_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(qmf::f16x8_t, a), __builtin_bit_cast(qmf::f16x8_t, b), c, 0, 0, 0);
-    }
-};
 
 // Rows of x a tile carries (RM rounded up to a power of two), the groups of the slice it carries for each
 // (kGpt), and the rows of x one lane's four accumulator elements belong to.
@@ -1034,6 +964,16 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 }  // namespace
 
 bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
+
+// Mirrors run_typed.
+const char *qmv_kernel_name(const ProductArgs &a) {
+    if (a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32) {
+        if (!a.row_exact && d16_takes(a)) return "qmv4_mm16_kernel";
+        if (!a.row_exact && a.m >= 4 && mfma_decode_takes<4>(a)) return "qmv4_mfma_kernel";
+        return "qmv4_lds_kernel";
+    }
+    return "qmv_lds_kernel";
+}
 
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s) {
     if (a.batch > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld batches exceed the grid limit", (long long)a.batch);

@@ -367,8 +367,8 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     if vector:
         x = x.unsqueeze(0)
     columns = _quantized_columns(op, w, scales, biases, quant)
-    rows = w.shape[-2]
-    inner, outer = (columns, rows) if transpose else (rows, columns)
+    w_rows = w.shape[-2]
+    inner, outer = (columns, w_rows) if transpose else (w_rows, columns)
     # Dense last two dimensions for every operand; batch dimensions broadcast by stride 0.
     x, w, scales = x.contiguous(), w.contiguous(), scales.contiguous()
     biases = biases.contiguous() if affine else None
@@ -420,6 +420,26 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
         _lib.check(lib.nvq_quantized_matmul(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(out),
                                             _ptr(workspace), _stream()))
     return out.squeeze(-2) if vector else out
+
+
+def quantized_matmul_route(m: int, n: int, k: int, quant: Quant, dtype: torch.dtype, *, batch: int = 1, transpose: bool = True,
+                           row_exact: bool = False, rows: bool = False, device: int = 0) -> str:
+    """The kernel a product of `m` rows of x per item ([.., m, k] times `batch` weight matrices [n, k], or one matrix
+    when `batch` is 1) runs on, from the library's own routing code: what the reference's tests read from the kernel
+    names (tests/quantized.rs:843-861)."""
+    _lib.check(_lib.load().nvq_init(device))
+    d = _lib.QmmDescC()
+    d.quant, d.dtype, d.transpose, d.row_exact, d.rows = quant._c(), _CODE[dtype], int(transpose), int(row_exact), int(rows)
+    d.m = d.item_rows = m
+    d.n, d.k = n, k
+    d.batch_ndim = 0 if batch == 1 else 1
+    if batch != 1:
+        d.batch_shape[0] = batch
+        d.x_strides[0], d.w_strides[0], d.s_strides[0] = m * k, n * k * quant.bits // 32, n * k // quant.group_size
+    name = _lib.load().nvq_quantized_matmul_route(C.byref(d))
+    if name is None:
+        raise Unsupported(_lib.last_error())
+    return name.decode()
 
 
 def quantized_attention_fits(q: torch.Tensor, k: Quantized, v: Quantized, sinks: Optional[torch.Tensor] = None) -> bool:

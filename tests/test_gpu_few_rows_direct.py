@@ -1,0 +1,111 @@
+"""The few-row kernel on the 16x16x32 matrix instruction with directly loaded weight operands (`qmd_kernel`: the
+counterpart of the reference's `affine_qmv_mma`, crates/nuvec-kernels/src/metal/quantized.h:1722-1905, routed at
+crates/nuvec-core/src/gpu.rs:6978-7024), and the routing of the BASELINE configurations.
+
+Like the reference's `few_row_mma_products_match_the_dequantized_product` (crates/nuvec-core/tests/quantized.rs:881-935)
+the tests name the kernel a product must run on and hold its values to the CPU's product: every output within the
+bar of its row against the CPU oracle, and within half of it against the device arithmetic."""
+import numpy as np
+import pytest
+import torch
+
+import nuvec_amd as nv
+from nuvec_amd import ops
+from oracle import ref
+from tests.hip_backend import TORCH, to_dev, to_host
+from tests.test_gpu_parity import assert_device_arithmetic, assert_rows_close, make_w, make_x
+
+pytestmark = pytest.mark.gpu
+
+WIDTHS = [(2, 64), (2, 128), (3, 64), (3, 128), (4, 32), (4, 64), (4, 128), (8, 32), (8, 64), (8, 128)]
+
+
+def test_routes_of_the_baseline_configurations():
+    """Which kernel each BASELINE configuration runs on (the routing code answers, not a table of the test)."""
+    bf16 = torch.bfloat16
+    c2 = lambda m, **kw: ops.quantized_matmul_route(m, 14336, 4096, nv.Quant.affine(64, 4), bf16, **kw)
+    assert ops.quantized_matmul_route(1, 4096, 4096, nv.Quant.affine(64, 4), torch.float32) == "qmv_lds_kernel"
+    assert c2(1) == "qmv4_lds_kernel"
+    assert c2(4) == "qmv4_mm16_kernel" and c2(8) == "qmv4_mm16_kernel"
+    assert c2(12) == "qmd_kernel" and c2(16) == "qmd_kernel"
+    assert c2(2048) == "qmm_kernel"
+    assert c2(8, row_exact=True) == "qmv4_lds_kernel" and c2(300, rows=True) == "qmv4_lds_kernel"
+    for group, bits in ((64, 3), (32, 8)):
+        c4 = lambda m, **kw: ops.quantized_matmul_route(m, 4096, 4096, nv.Quant.affine(group, bits), bf16, **kw)
+        assert c4(1) == "qmv_lds_kernel"
+        assert c4(16) == "qmd_kernel" and c4(2) == "qmd_kernel"
+        assert c4(512) == "qmm_kernel"
+        assert c4(16, transpose=False) == "qvm_kernel"
+        assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
+    assert ops.quantized_matmul_route(24, 1000, 4096, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
+    assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
+    assert ops.quantized_matmul_route(64, 2880, 2880, nv.Quant.new(nv.QuantMode.MXFP4), bf16) in ("qmf_kernel", "qmm_kernel")
+
+
+SHAPES = [(2, 200, 512), (9, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (11, 48, 14336), (23, 64, 1536), (16, 5000, 512),
+          (12, 40, 7168)]
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("bits,group", WIDTHS)
+def test_direct_few_row_kernel_every_width(dtype, bits, group):
+    """One and two passes of rows, K of one chunk, of several (8192: 2 chunks of 8 slices; 14336: 4 of 7; 7168: 2 of 7),
+    N off the tile and with several tiles per block, tails of rows."""
+    rng = np.random.default_rng(4000 + 10 * bits + group)
+    quant = nv.Quant.affine(group, bits)
+    for m, n, k in SHAPES:
+        route = ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
+        if bits == 4 and m <= 8:
+            continue  # the 4-bit decode kernels' rows
+        assert route == "qmd_kernel", f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, threads=8)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        what = f"direct few rows b{bits} g{group} M={m} N={n} K={k}"
+        assert_rows_close(got, want, dtype, what)
+        assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what)
+
+
+@pytest.mark.parametrize("bits,group", [(3, 64), (8, 32), (4, 128)])
+def test_direct_few_row_kernel_batched_with_bias(bits, group):
+    """A batch of weight matrices (one stride per operand) and the layer's bias in the epilogue."""
+    rng = np.random.default_rng(4100 + bits)
+    b, m, n, k = 3, 10, 96, 1024
+    quant = nv.Quant.affine(group, bits)
+    assert ops.quantized_matmul_route(m, n, k, quant, torch.bfloat16, batch=b) == "qmd_kernel"
+    w, x = make_w(rng, b * n, k, ref.BF16), make_x(rng, b * m, k, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, group, bits)
+    q = nv.Quantized(to_dev(packed.reshape(b, n, -1)), to_dev(scales.reshape(b, n, -1)), to_dev(biases.reshape(b, n, -1)), quant)
+    got = to_host(nv.quantized_matmul(to_dev(x.reshape(b, m, k)), q))
+    for i in range(b):
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n],
+                                    biases[i * n:(i + 1) * n], group=group, bits=bits, dtype=ref.BF16)
+        assert_rows_close(got[i], want, ref.BF16, f"direct few rows batched b{bits} item {i}")
+    # bias: the rounded product plus the bias, rounded (layers.rs:155-162), bit for bit the separate addition
+    q0 = nv.Quantized(q.weight[0].contiguous(), q.scales[0].contiguous(), q.biases[0].contiguous(), quant)
+    bias = to_dev(make_x(rng, 1, n, ref.BF16)[0])
+    xd = to_dev(x[:m])
+    fused = nv.quantized_matmul(xd, q0, bias=bias)
+    assert np.array_equal(to_host(fused).view(np.uint8), to_host(nv.quantized_matmul(xd, q0) + bias).view(np.uint8))
+
+
+def test_direct_few_row_kernel_per_pair_gather():
+    """gather_qmm without offsets: one product per pair on the same kernel (pairs over grid z)."""
+    rng = np.random.default_rng(4200)
+    experts, n, k, m, pairs = 5, 80, 1024, 6, 7
+    w = make_w(rng, experts * n, k, ref.BF16)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 3)
+    q = nv.Quantized(to_dev(packed.reshape(experts, n, -1)), to_dev(scales.reshape(experts, n, -1)),
+                     to_dev(biases.reshape(experts, n, -1)), nv.Quant.affine(64, 3))
+    x = make_x(rng, 4 * m, k, ref.BF16)
+    lhs = rng.integers(0, 4, pairs).astype(np.uint32)
+    rhs = rng.integers(0, experts, pairs).astype(np.uint32)
+    got = to_host(nv.gather_qmm(to_dev(x.reshape(4, m, k)), q, torch.from_numpy(lhs.astype(np.int64)).cuda(),
+                                torch.from_numpy(rhs.astype(np.int64)).cuda(), nv.GatherQmm()))
+    for z in range(pairs):
+        e = int(rhs[z])
+        want = ref.quantized_matmul(x[lhs[z] * m:(lhs[z] + 1) * m], packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n],
+                                    biases[e * n:(e + 1) * n], group=64, bits=3, dtype=ref.BF16)
+        assert_rows_close(got[z], want, ref.BF16, f"direct few rows, pair {z}")
