@@ -33,8 +33,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_213_687   # read 32,379 KiB + written 56 KiB (profiles/qmv4_lds_kernel__decode_c2_m1.txt)
-QMM_TRAFFIC_BYTES = 275_968_746  # read 212,154 KiB + written 57,347 KiB (profiles/qmm_kernel__prefill_c3_m2048.txt)
+QMV_TRAFFIC_BYTES = 33_216_732   # rocprofv3 FETCH_SIZE + WRITE_SIZE per launch, scaled by a plain 1 GiB copy (profiles/)
+QMM_TRAFFIC_BYTES = 297_183_146  # the same for the tiled kernel at configs[2]
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -244,8 +244,9 @@ def all_configs(lib, device, qs):
             ys = [torch.empty(m, n, dtype=tdtype, device=device) for _ in weights]
             calls = [Product(lib, m, x, q, y, n, k, code) for q, y in zip(weights, ys)]
             ms = best_of(calls, 600 if m <= 64 else 48)
-            out.append({"config": label, "m": m, "us_per_launch": ms * 1e3, "weight_gbps": wbytes / (ms * 1e-3) / 1e9,
-                        "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12})
+            kernel = lib.nvq_quantized_matmul_route(C.byref(calls[0].d))  # from the library's routing code
+            out.append({"config": label, "m": m, "kernel": kernel.decode() if kernel else None, "us_per_launch": ms * 1e3,
+                        "weight_gbps": wbytes / (ms * 1e-3) / 1e9, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12})
 
     products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1], 48, 10_485_760)
     products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 2048], 0, WEIGHT_BYTES,
@@ -267,7 +268,7 @@ def all_configs(lib, device, qs):
     offsets = nv.sorted_offsets(rhs, experts)
     calls = [GatherProduct(lib, x, q, lhs, rhs, offsets, y, n, k, experts) for q in weights]
     ms = best_of(calls, 200)
-    out.append({"config": "C5 MXFP4 gather_qmm 32 experts W[2880,2880], 1024 sorted rows", "m": tokens * top,
+    out.append({"config": "C5 MXFP4 gather_qmm 32 experts W[2880,2880], 1024 sorted rows", "m": tokens * top, "kernel": "qmg_kernel",
                 "us_per_launch": ms * 1e3, "weight_gbps": 141_004_800 / (ms * 1e-3) / 1e9,
                 "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12})
     del weights, calls
@@ -316,9 +317,9 @@ def main():
     ap.add_argument("--no-configs", action="store_true",
                     help="skip timing every configuration of the reference's benchmark list (C1..C5), reported under \"configs\"")
     ap.add_argument("--no-peaks", action="store_true", help="skip the calibration kernels reported under \"measured_peaks\"")
-    ap.add_argument("--only", choices=["qmv", "qmm", "copy"], default=None,
-                    help="profiling aid: run just the rotating decode leg, just the prefill leg, or a plain 1 GiB "
-                         "device copy (the known-size kernel the HBM counters are scaled by)")
+    ap.add_argument("--only", choices=["qmv", "qmm", "copy", "configs"], default=None,
+                    help="profiling aid: run just the rotating decode leg, just the prefill leg, just the table of every "
+                         "configuration, or a plain 1 GiB device copy (the known-size kernel the HBM counters are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (the path shards along N without exchange: "
@@ -344,6 +345,9 @@ def main():
 
     only = args.only
     qs = make_weights(args.copies if only != "qmm" else 4, device)
+    if only == "configs":
+        print(json.dumps({"configs": all_configs(lib, device, qs)}))
+        return
     record = {"metric": METRIC, "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "scaling": "weak",
               "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
 
