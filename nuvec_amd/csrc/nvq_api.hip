@@ -184,12 +184,21 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 //   8 bits g32   W[4096,4096] 16 rows 11.1 / 12.9;  W[4096,14336] 8 rows 23.6 / 28.1;  W[151936,1024] 8 rows 47.8 / 74.5
 //   4 bits g64   W[14336,4096] 12 rows 12.8 / 17.5;  W[32768,2048] 16 rows 13.3 / 26.0  (up to 8 rows the 4-bit decode kernels are ahead: 13.1 / 11.1)
 //   4 bits g128  W[14336,4096]  4 rows 10.4 / 13.5, 8 rows 10.8 / 16.4;  W[151936,1024] 1 row 19.9 / 50.1
-// One row stays on the vector kernels except for very tall matrices; 17 to 32 rows (two passes) where K fits one chunk
-// and the matrix is small enough that the second pass reads it from the caches.
+// One row stays on the vector kernels except for very tall matrices.  More than 16 rows are passes of 16 that read
+// the weights again (from the caches, if the matrix is small enough): measured up to 192 rows at five shapes, e.g.
+// 4 bits g64 W[4096,4096] 64 rows 11.8 / 14.6, 96 rows 18.2 / 18.6; W[14336,4096] 64 rows 33.7 / 35.3, 96 rows 49.3 / 33.9;
+// W[1024,4096] 128 rows 8.2 / 15.5; 8 bits g32 W[4096,4096] 32 rows 13.0 / 16.9, 48 rows 19.5 / 17.1.  The rule below is
+// passes x megabytes of weights, fitted to those tables.
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     if (!nvq::qmd_supported(a)) return false;
     const int64_t rows = a.n * a.batch;
-    if (a.m > 16) return a.m <= 32 && a.k <= 4096 && rows * a.k * a.bits <= (int64_t)32 * 8 * 1024 * 1024 && !(a.group == 32 && rows > 4096);
+    if (a.m > 16) {
+        if (a.k > 4096 || a.m > 192) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
+        const double passes = (double)((a.m + 15) / 16), mb = (double)rows * (double)a.k * a.bits / 8.0 / 1048576.0;
+        if (a.bits == 8) return passes * mb <= (a.group == 32 ? 34.0 : 40.0);
+        if (a.group == 32) return passes * mb <= 30.0;
+        return passes * mb <= 50.0 || (passes <= 4.0 && mb <= 32.0);
+    }
     switch (a.bits) {
     case 2: return true;
     case 3: return a.group == 128 || a.m >= 2 || rows >= 16384;
@@ -465,8 +474,8 @@ static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     if (a.global_scale != nullptr) return Route::kVector;  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return Route::kUntransposed;        // weights stored [K, N]
     if (a.row_exact) return Route::kVector;                // the vector kernels: a row's bits do not depend on its neighbours
+    if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;  // (also passes of 16 rows of small matrices, ahead of the tiles)
     if (takes_tiled(d, a)) return Route::kTiled;
-    if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;
     // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the
     // decode kernels (per-row work on the vector units, which is cheaper than the matrix-core kernel's full
     // dequantization up to there).  A single row of the other affine widths from 3 bits: the general vector kernel

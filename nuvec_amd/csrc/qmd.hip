@@ -355,15 +355,20 @@ int32_t run_qmd_sized(const ProductArgs &a, hipStream_t s) {
     const int slices = qmd_slices(a.k);
     const bool chunked = a.k > (int64_t)slices * kQmdSlice;
     const size_t lds_bytes = qmd_lds_bytes<RM, RT, GROUP>(slices, chunked);
-    // Groups of RT tiles of 16 weight rows; a block that stages x once walks several where there are more groups than
-    // compute units, so that x is staged less often.  Measured at W[14336,4096], 3 bits, 16 rows of x: 21.8 / 14.3 /
-    // 11.8 / 18.3 us with 1 / 2 / 4 / 8 groups a block.
+    // Groups of RT tiles of 16 weight rows; a block that stages x once walks several where there are more blocks than
+    // compute units, so that x is staged less often and the blocks are one round on the chip.  Measured at
+    // W[14336,4096], 3 bits, 16 rows of x: 21.8 / 14.3 / 11.8 / 18.3 us with 1 / 2 / 4 / 8 groups a block.
     const int64_t groups = (a.n + 16 * RT - 1) / (16 * RT), passes = (a.m + RM - 1) / RM;
     int tiles = 1;
     if (!chunked) {
+        // rounds of blocks on the chip x (staging of x: about 2.5 us, plus 1.5 us a group walked)
         const int64_t slots = compute_units();
-        tiles = (int)((groups * passes * a.batch + slots - 1) / slots);
-        tiles = tiles < 1 ? 1 : tiles > 8 ? 8 : tiles;
+        double best = 0.0;
+        for (int t = 1; t <= 8; t++) {
+            const int64_t blocks = (groups + t - 1) / t * passes * a.batch;
+            const double cost = (double)((blocks + slots - 1) / slots) * (2.5 + 1.5 * t);
+            if (t == 1 || cost < best) best = cost, tiles = t;
+        }
 #ifdef QMD_LAB
         if (const char *e = getenv("NVQ_LAB_TILES")) tiles = atoi(e);
 #endif

@@ -40,16 +40,23 @@ def test_routes_of_the_baseline_configurations():
     assert ops.quantized_matmul_route(24, 1000, 4096, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
     assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
     assert ops.quantized_matmul_route(64, 2880, 2880, nv.Quant.new(nv.QuantMode.MXFP4), bf16) in ("qmf_kernel", "qmm_kernel")
+    # passes of 16 rows where the matrix is small enough to be read again from the caches; the tiles beyond
+    small = lambda m: ops.quantized_matmul_route(m, 1024, 4096, nv.Quant.affine(64, 4), bf16)
+    assert small(64) == "qmd_kernel" and small(192) == "qmd_kernel" and small(512) in ("qmf_kernel", "qmm_kernel")
+    assert c2(64) == "qmd_kernel" and c2(96) == "qmm_kernel"
+    # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
+    for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (30, 64, 128, 64, 4), (20, 1000, 4096, 64, 6)):
+        assert ops.quantized_matmul_route(m, n, k, nv.Quant.affine(group, bits), bf16) == "qmf_kernel", (m, n, k, group, bits)
 
 
 SHAPES = [(2, 200, 512), (9, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (11, 48, 14336), (23, 64, 1536), (16, 5000, 512),
-          (12, 40, 7168)]
+          (12, 40, 7168), (77, 300, 2048), (130, 48, 512)]
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 @pytest.mark.parametrize("bits,group", WIDTHS)
 def test_direct_few_row_kernel_every_width(dtype, bits, group):
-    """One and two passes of rows, K of one chunk, of several (8192: 2 chunks of 8 slices; 14336: 4 of 7; 7168: 2 of 7),
+    """One to nine passes of rows, K of one chunk, of several (8192: 2 chunks of 8 slices; 14336: 4 of 7; 7168: 2 of 7),
     N off the tile and with several tiles per block, tails of rows."""
     rng = np.random.default_rng(4000 + 10 * bits + group)
     quant = nv.Quant.affine(group, bits)
@@ -65,7 +72,8 @@ def test_direct_few_row_kernel_every_width(dtype, bits, group):
         got = to_host(nv.quantized_matmul(to_dev(x), q))
         what = f"direct few rows b{bits} g{group} M={m} N={n} K={k}"
         assert_rows_close(got, want, dtype, what)
-        assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what)
+        if m <= 32:  # (half the bar leaves no room for one rounding step of the largest outputs: not over thousands of short rows)
+            assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what)
 
 
 @pytest.mark.parametrize("bits,group", [(3, 64), (8, 32), (4, 128)])
