@@ -192,6 +192,10 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     if (!nvq::qmd_supported(a)) return false;
     const int64_t rows = a.n * a.batch;
+    // The block formats (bf16, new / the few-row kernel of the 32x32x16 instruction): MXFP4 W[14336,4096] 1 row 11.1 / 13.4,
+    // 16 rows 11.3 / 14.6; W[4096,4096] 1 row 5.4 / 6.9, 32 rows 7.0 / 14.2; NVFP4 W[14336,4096] 1 row 13.2 / 17.7;
+    // MXFP8 W[4096,14336] 16 rows 18.8 / 29.4: every row count up to 16, 32 where K or the matrix is short.
+    if (a.mode != NVQ_AFFINE && a.m <= 32) return a.m <= 16 || a.k <= 4096 || rows <= 4096;
     if (a.m > 16) {
         if (a.k > 4096 || a.m > 192) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
         const double passes = (double)((a.m + 15) / 16), mb = (double)rows * (double)a.k * a.bits / 8.0 / 1048576.0;

@@ -31,7 +31,8 @@ constexpr int kQmdSlices = 8;                  // slices of a block: what the LD
 // Codes per lane and span: 32 (a span of 128 values: a lane's load is 4 BITS bytes, a wavefront's 64 BITS / 8 bytes of
 // each of 16 rows) for groups of 64 and 128, 16 for groups of 32 (where that is whole dwords).  Measured at
 // W[14336,4096], 4 bits, groups of 64: 13.6 us with 16 codes (loads of 8 bytes a lane), 11.2 us with 32.
-template <int BITS, int GROUP> constexpr int qmd_chunk() {
+template <int MODE, int BITS, int GROUP> constexpr int qmd_chunk() {
+    if (MODE != NVQ_AFFINE) return BITS == 8 ? 16 : 32;  // the block formats: 16 bytes of codes a lane (one or two groups)
     constexpr int want = GROUP == 32 ? 16 : 32;
     return (want * BITS) % 32 == 0 ? want : 32;
 }
@@ -132,20 +133,26 @@ __device__ __forceinline__ void qmd_load(const uint32_t *p, uint32_t (&out)[DW])
 // slice ([group][quarter] x 4 rows, float32); its partial rows — twice where the block walks several tiles (one barrier
 // each: a tile's sums are read while the next tile's are written).
 template <int RM, int RT, int GROUP>
-__host__ __device__ constexpr size_t qmd_lds_bytes(int slices, bool chunked) {
-    return (size_t)slices * ((RM * kQmdRowPieces + 1) * 16 + (kQmdSlice / GROUP) * 64 + (chunked ? 1 : 2) * (size_t)RT * RM * 16 * 4);
+__host__ __device__ constexpr size_t qmd_lds_bytes(int slices, bool chunked, bool sums) {
+    return (size_t)slices * ((RM * kQmdRowPieces + 1) * 16 + (sums ? (kQmdSlice / GROUP) * 64 : 0) + (chunked ? 1 : 2) * (size_t)RT * RM * 16 * 4);
 }
 
 // CHUNKED: K is longer than the block's wavefronts cover at once; the block owns one group of RT tiles of weight rows
 // and walks K in chunks, staging x anew for each.  Otherwise x is staged once and the block walks `tiles` groups of
 // tiles, the weights of a group requested one step ahead.
-template <typename T, int BITS, int GROUP, int RM, int RT, bool CHUNKED>
+//
+// The block formats (MXFP4, MXFP8, NVFP4 without a global scale) take the same walk with less arithmetic: the scaled
+// conversion instructions give the dequantized elements themselves (exact: a code times a power of two; NVFP4's E4M3
+// scale by one multiplication in float32), so the accumulators run over all of K and there are no sums of x.
+template <typename T, int MODE, int BITS, int GROUP, int RM, int RT, bool CHUNKED>
 __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs a, const int tiles) {
-    constexpr int C = qmd_chunk<BITS, GROUP>(), kSpan = 4 * C, kSpans = kQmdSlice / kSpan, J = C / 8;
-    constexpr int NG = kSpan / GROUP;            // groups (accumulators) per span: 1, 2 or 4
+    constexpr bool kBlock = MODE != NVQ_AFFINE;
+    constexpr int C = qmd_chunk<MODE, BITS, GROUP>(), kSpan = 4 * C, kSpans = kQmdSlice / kSpan, J = C / 8;
+    constexpr int NG = kBlock ? 1 : kSpan / GROUP;  // groups (accumulators) per span: 1, 2 or 4
     constexpr int DW = C * BITS / 32;            // dwords of codes per lane and span
-    constexpr int SG = kQmdSlice / GROUP;        // groups per slice: a lane holds their scales and biases
-    static_assert(NG >= 1 && NG <= 4 && NG * GROUP == kSpan && J >= 1, "a span is one, two or four whole groups");
+    constexpr int SG = kQmdSlice / GROUP;        // groups per slice: a lane holds their scales (and biases)
+    constexpr int SW = kBlock ? SG / 4 : SG / 2; // dwords of scales of a slice (one byte a group in the block formats)
+    static_assert(kBlock || (NG >= 1 && NG <= 4 && NG * GROUP == kSpan && J >= 1), "a span is one, two or four whole groups");
     const int slices = __builtin_amdgcn_readfirstlane(blockDim.x >> 6);  // one wavefront per slice
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int chunk_k = slices * kQmdSlice;
@@ -157,14 +164,15 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     const int slice = wave;
     const int nl = lane & 15, kq = lane >> 4;
     uint4 *xs = reinterpret_cast<uint4 *>(lds) + slice * (RM * kQmdRowPieces + 1);  // this slice's rows of x, then a piece of zeros
-    floatx4_t *xsum = reinterpret_cast<floatx4_t *>(lds + (size_t)slices * (RM * kQmdRowPieces + 1) * 16) + wave * SG * 4;  // [SG][4 quarters]
-    float *partial = reinterpret_cast<float *>(lds + (size_t)slices * ((RM * kQmdRowPieces + 1) * 16 + SG * 64));  // [2][RT][slices][RM][16] (chunked: one)
+    floatx4_t *xsum = reinterpret_cast<floatx4_t *>(lds + (size_t)slices * (RM * kQmdRowPieces + 1) * 16) + wave * SG * 4;  // [SG][4 quarters] (affine)
+    float *partial = reinterpret_cast<float *>(lds + (size_t)slices * ((RM * kQmdRowPieces + 1) * 16 + (kBlock ? 0 : SG * 64)));  // [2][RT][slices][RM][16] (chunked: one)
     const int m0 = blockIdx.y * RM;
     const bool batched = !(a.batch == 1 && a.rhs == nullptr);
     const BatchOffsets o = batched ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
-    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
+    using S = std::conditional_t<kBlock, uint8_t, T>;  // a scale: the element type, or one byte (E8M0; NVFP4: E4M3)
+    const S *scales = (const S *)a.scales + o.s, *biases = kBlock ? nullptr : (const S *)a.biases + o.s;
     T *y = (T *)a.y + o.y;
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     constexpr float base = qmd_magic<T, BITS>() ? Pair<T>::base : 0.0f;
@@ -182,7 +190,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     // What a step reads from memory: the codes, scales and biases of RT tiles of weight rows for this wavefront's slice.
     struct Tile {
         uint32_t w[RT][kSpans][DW];
-        uint32_t s[RT][SG / 2], b[RT][SG / 2];
+        uint32_t s[RT][SW], b[RT][kBlock ? 1 : SW];
     };
     // The group of RT tiles this wavefront takes in a step.
     auto group_of = [&](int step) { return CHUNKED ? (int)blockIdx.x : (int)blockIdx.x * tiles + step; };
@@ -200,8 +208,8 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
 #pragma unroll
             for (int sp = 0; sp < kSpans; sp++) qmd_load<DW>(wp + sp * stride, t.w[rt][sp]);
             const int64_t g0 = real ? (int64_t)row * kgroups + k0 / GROUP : 0;
-            qmd_load<SG / 2>(reinterpret_cast<const uint32_t *>(scales + g0), t.s[rt]);
-            qmd_load<SG / 2>(reinterpret_cast<const uint32_t *>(biases + g0), t.b[rt]);
+            qmd_load<SW>(reinterpret_cast<const uint32_t *>(scales + g0), t.s[rt]);
+            if constexpr (!kBlock) qmd_load<SW>(reinterpret_cast<const uint32_t *>(biases + g0), t.b[rt]);
         }
     };
     // x of a step: a row of the slice is one 16-byte piece per lane.  A wavefront reads only what it staged itself, and
@@ -214,7 +222,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
             xq[i] = m0 + i < M ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + k0 + 8 * lane) : make_uint4(0, 0, 0, 0);
         asm volatile("" ::: "memory");
 #pragma unroll
-        for (int i = 0; i < RM; i++) xs[i * kQmdRowPieces + lane] = qmd_pair_order<BITS>(xq[i]);
+        for (int i = 0; i < RM; i++) xs[i * kQmdRowPieces + lane] = kBlock ? xq[i] : qmd_pair_order<BITS>(xq[i]);  // (the conversions give the elements in order)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_wave_barrier();
         asm volatile("" ::: "memory");
@@ -222,6 +230,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     // The sums X of the slice's groups: the x operands against a weight operand of ones give them in the accumulator
     // layout of P (the same values in the 16 lanes of a quarter); they wait in the LDS for the tiles.
     auto sums = [&]() {
+        if constexpr (kBlock) return;
 #pragma unroll
         for (int sp = 0; sp < kSpans; sp++)
 #pragma unroll
@@ -248,6 +257,59 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
             for (int e = 0; e < 4; e++) part[rt][e] = 0.0f;
     };
     auto compute = [&](const Tile &t) {
+        if constexpr (kBlock) {
+            // Byte g of the slice's scales is group g; the lane's chunk of span sp lies in group (sp kSpan + C q) / GROUP
+            // (NVFP4: and in the next one).
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                floatx4_t even = part[rt], odd;
+#pragma unroll
+                for (int e = 0; e < 4; e++) odd[e] = 0.0f;
+#pragma unroll
+                for (int sp = 0; sp < kSpans; sp++) {
+                    const int g = (sp * kSpan) / GROUP + (C * kq) / GROUP;  // (sp kSpan / GROUP is a compile-time constant)
+                    const uint32_t word = MODE == NVQ_NVFP4 ? (kq < 2 ? t.s[rt][2 * sp] : t.s[rt][2 * sp + 1])
+                                          : MODE == NVQ_MXFP8 ? t.s[rt][sp / 2] : t.s[rt][sp];
+                    float sc0, sc1;
+                    if constexpr (MODE == NVQ_NVFP4) {
+                        const uint32_t two = word >> (16 * (kq & 1));
+                        sc0 = ftz(e4m3_to_f32(two & 255u)), sc1 = ftz(e4m3_to_f32((two >> 8) & 255u));
+                    } else {
+                        sc0 = sc1 = ftz(e8m0_to_f32((word >> (8 * (g & 3))) & 255u));
+                    }
+                    const uint4 *xa = xs + a_live + (sp * 4 * J) * a_step;
+#pragma unroll
+                    for (int j = 0; j < J; j++) {
+                        uint4 b;
+                        if constexpr (MODE == NVQ_MXFP8) {
+                            const uint32_t w0 = t.w[rt][sp][2 * j], w1 = t.w[rt][sp][2 * j + 1];
+                            b.x = qmf::Ops<T>::template fp8_pair<false>(w0, sc0);
+                            b.y = qmf::Ops<T>::template fp8_pair<true>(w0, sc0);
+                            b.z = qmf::Ops<T>::template fp8_pair<false>(w1, sc0);
+                            b.w = qmf::Ops<T>::template fp8_pair<true>(w1, sc0);
+                        } else if constexpr (MODE == NVQ_MXFP4) {
+                            const uint32_t w0 = t.w[rt][sp][j];
+                            b.x = qmf::Ops<T>::template fp4_pair<0>(w0, sc0);
+                            b.y = qmf::Ops<T>::template fp4_pair<1>(w0, sc0);
+                            b.z = qmf::Ops<T>::template fp4_pair<2>(w0, sc0);
+                            b.w = qmf::Ops<T>::template fp4_pair<3>(w0, sc0);
+                        } else {
+                            const uint32_t w0 = t.w[rt][sp][j];
+                            const float sc = j < 2 ? sc0 : sc1;  // codes 0..15 of the chunk, 16..31
+                            b.x = qmf::fp4_pair_times<T, 0>(w0, sc);
+                            b.y = qmf::fp4_pair_times<T, 1>(w0, sc);
+                            b.z = qmf::fp4_pair_times<T, 2>(w0, sc);
+                            b.w = qmf::fp4_pair_times<T, 3>(w0, sc);
+                        }
+                        if (j & 1) odd = Mfma16<T>::run(xa[j * a_step], b, odd);
+                        else even = Mfma16<T>::run(xa[j * a_step], b, even);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) part[rt][e] = even[e] + odd[e];
+            }
+            return;
+        }
 #pragma unroll
         for (int sp = 0; sp < kSpans; sp++) {
 #pragma unroll
@@ -350,11 +412,11 @@ inline int qmd_slices(int64_t k) {
     return 1;
 }
 
-template <typename T, int BITS, int GROUP, int RM, int RT>
+template <typename T, int MODE, int BITS, int GROUP, int RM, int RT>
 int32_t run_qmd_sized(const ProductArgs &a, hipStream_t s) {
     const int slices = qmd_slices(a.k);
     const bool chunked = a.k > (int64_t)slices * kQmdSlice;
-    const size_t lds_bytes = qmd_lds_bytes<RM, RT, GROUP>(slices, chunked);
+    const size_t lds_bytes = qmd_lds_bytes<RM, RT, GROUP>(slices, chunked, MODE == NVQ_AFFINE);
     // Groups of RT tiles of 16 weight rows; a block that stages x once walks several where there are more blocks than
     // compute units, so that x is staged less often and the blocks are one round on the chip.  Measured at
     // W[14336,4096], 3 bits, 16 rows of x: 21.8 / 14.3 / 11.8 / 18.3 us with 1 / 2 / 4 / 8 groups a block.
@@ -375,8 +437,8 @@ int32_t run_qmd_sized(const ProductArgs &a, hipStream_t s) {
     }
     const dim3 grid((unsigned)((groups + tiles - 1) / tiles), (unsigned)passes, (unsigned)a.batch);
     void (*kernel)(const ProductArgs, int);
-    if constexpr (RT == 1) kernel = chunked ? qmd_kernel<T, BITS, GROUP, RM, RT, true> : qmd_kernel<T, BITS, GROUP, RM, RT, false>;
-    else kernel = qmd_kernel<T, BITS, GROUP, RM, RT, true>;  // (two tiles a wavefront: only where K is walked in chunks)
+    if constexpr (RT == 1) kernel = chunked ? qmd_kernel<T, MODE, BITS, GROUP, RM, RT, true> : qmd_kernel<T, MODE, BITS, GROUP, RM, RT, false>;
+    else kernel = qmd_kernel<T, MODE, BITS, GROUP, RM, RT, true>;  // (two tiles a wavefront: only where K is walked in chunks)
     static std::atomic<bool> configured[2] = {false, false};
     if (lds_bytes > 64 * 1024 && !configured[chunked]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
@@ -387,29 +449,32 @@ int32_t run_qmd_sized(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int BITS, int GROUP>
+template <typename T, int MODE, int BITS, int GROUP>
 int32_t run_qmd_rows(const ProductArgs &a, hipStream_t s) {
     const bool chunked = a.k > (int64_t)qmd_slices(a.k) * kQmdSlice;
     if (chunked) {
         // A long K (walked in chunks, x staged per chunk): two tiles of weight rows per wavefront halve the staging
         // where there are weight rows enough to fill the chip with such blocks.
         const bool two = a.n * a.batch >= 8192;
-        if (a.m <= 8) return two ? run_qmd_sized<T, BITS, GROUP, 8, 2>(a, s) : run_qmd_sized<T, BITS, GROUP, 8, 1>(a, s);
-        return two ? run_qmd_sized<T, BITS, GROUP, 16, 2>(a, s) : run_qmd_sized<T, BITS, GROUP, 16, 1>(a, s);
+        if (a.m <= 8) return two ? run_qmd_sized<T, MODE, BITS, GROUP, 8, 2>(a, s) : run_qmd_sized<T, MODE, BITS, GROUP, 8, 1>(a, s);
+        return two ? run_qmd_sized<T, MODE, BITS, GROUP, 16, 2>(a, s) : run_qmd_sized<T, MODE, BITS, GROUP, 16, 1>(a, s);
     }
-    return a.m <= 8 ? run_qmd_sized<T, BITS, GROUP, 8, 1>(a, s) : run_qmd_sized<T, BITS, GROUP, 16, 1>(a, s);
+    return a.m <= 8 ? run_qmd_sized<T, MODE, BITS, GROUP, 8, 1>(a, s) : run_qmd_sized<T, MODE, BITS, GROUP, 16, 1>(a, s);
 }
 
 template <typename T, int BITS>
 int32_t run_qmd_group(const ProductArgs &a, hipStream_t s) {
     if constexpr (BITS == 4 || BITS == 8) {
-        if (a.group == 32) return run_qmd_rows<T, BITS, 32>(a, s);
+        if (a.group == 32) return run_qmd_rows<T, NVQ_AFFINE, BITS, 32>(a, s);
     }
-    return a.group == 64 ? run_qmd_rows<T, BITS, 64>(a, s) : run_qmd_rows<T, BITS, 128>(a, s);
+    return a.group == 64 ? run_qmd_rows<T, NVQ_AFFINE, BITS, 64>(a, s) : run_qmd_rows<T, NVQ_AFFINE, BITS, 128>(a, s);
 }
 
 template <typename T>
 int32_t run_qmd(const ProductArgs &a, hipStream_t s) {
+    if (a.mode == NVQ_MXFP4) return run_qmd_rows<T, NVQ_MXFP4, 4, 32>(a, s);
+    if (a.mode == NVQ_MXFP8) return run_qmd_rows<T, NVQ_MXFP8, 8, 32>(a, s);
+    if (a.mode == NVQ_NVFP4) return run_qmd_rows<T, NVQ_NVFP4, 4, 16>(a, s);
     switch (a.bits) {
     case 2: return run_qmd_group<T, 2>(a, s);
     case 3: return run_qmd_group<T, 3>(a, s);
@@ -423,12 +488,14 @@ int32_t run_qmd(const ProductArgs &a, hipStream_t s) {
 // Whether the kernel takes the product: bf16 / f16, affine 2, 3, 4 or 8 bits, K in slices of 512, 16-byte aligned
 // scale and bias rows (a lane reads the scales of its slice with vector loads).
 bool qmd_supported(const ProductArgs &a) {
-    if (a.mode != NVQ_AFFINE || a.dtype == NVQ_F32 || a.row_exact) return false;
-    if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 8)) return false;
-    if (!(a.group == 64 || a.group == 128 || (a.group == 32 && a.bits >= 4))) return false;  // 2 and 3 bits in groups of 32: four groups per span
+    if (a.dtype == NVQ_F32 || a.row_exact || a.global_scale != nullptr) return false;
+    if (a.mode == NVQ_AFFINE) {
+        if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 8)) return false;
+        if (!(a.group == 64 || a.group == 128 || (a.group == 32 && a.bits >= 4))) return false;  // 2 and 3 bits in groups of 32: four groups per span
+    }
     if (a.k < kQmdSlice || a.k % kQmdSlice != 0 || a.m < 1) return false;
     if ((a.m + 15) / 16 > 65535 || a.batch > 65535) return false;
-    return ((uintptr_t)a.scales | (uintptr_t)a.biases | (uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
+    return ((uintptr_t)a.scales | (uintptr_t)(a.mode == NVQ_AFFINE ? a.biases : nullptr) | (uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
 }
 
 int32_t launch_qmd(const ProductArgs &a, hipStream_t s) {

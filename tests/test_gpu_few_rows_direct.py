@@ -117,3 +117,40 @@ def test_direct_few_row_kernel_per_pair_gather():
         want = ref.quantized_matmul(x[lhs[z] * m:(lhs[z] + 1) * m], packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n],
                                     biases[e * n:(e + 1) * n], group=64, bits=3, dtype=ref.BF16)
         assert_rows_close(got[z], want, ref.BF16, f"direct few rows, pair {z}")
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_direct_few_row_kernel_block_formats(mode, qmode, dtype):
+    """MXFP4, MXFP8 and NVFP4 (no global scale) on the same kernel: the scaled conversions give the dequantized elements
+    themselves, exact in the element type, so the bar holds for every output; a batch; pairs of a gather."""
+    rng = np.random.default_rng(4300 + 10 * mode + dtype)
+    group, bits = ref.FP_PARAMS[mode]
+    quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
+    for m, n, k in [(1, 200, 512), (3, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (11, 48, 14336), (23, 64, 1536), (8, 5000, 512),
+                    (50, 300, 2048)]:
+        assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmd_kernel", (qmode, m, n, k)
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales = ref.fp_quantize(w, dtype, mode)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, dtype, f"direct few rows {qmode} M={m} N={n} K={k}", exact_weights=True)
+    b, m, n, k = 3, 6, 96, 512
+    assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype], batch=b) == "qmd_kernel"
+    w, x = make_w(rng, b * n, k, dtype), make_x(rng, b * m, k, dtype)
+    packed, scales = ref.fp_quantize(w, dtype, mode)
+    q = nv.Quantized(to_dev(packed.reshape(b, n, -1)), to_dev(scales.reshape(b, n, -1)), None, quant)
+    got = to_host(nv.quantized_matmul(to_dev(x.reshape(b, m, k)), q))
+    for i in range(b):
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n], None, mode=mode,
+                                    group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[i], want, dtype, f"direct few rows {qmode} batch item {i}", exact_weights=True)
+    pairs = rng.integers(0, b, 5)
+    got = to_host(nv.gather_qmm(to_dev(x.reshape(b, m, k)), q, torch.from_numpy(pairs.astype(np.int64)).cuda(),
+                                torch.from_numpy(pairs[::-1].copy().astype(np.int64)).cuda(), nv.GatherQmm()))
+    for z in range(5):
+        i, e = int(pairs[z]), int(pairs[::-1][z])
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n], None, mode=mode,
+                                    group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[z], want, dtype, f"direct few rows {qmode} pair {z}", exact_weights=True)
