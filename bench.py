@@ -245,8 +245,12 @@ def all_configs(lib, device, qs):
             calls = [Product(lib, m, x, q, y, n, k, code) for q, y in zip(weights, ys)]
             ms = best_of(calls, 600 if m <= 64 else 48)
             kernel = lib.nvq_quantized_matmul_route(C.byref(calls[0].d))  # from the library's routing code
+            gbps, tflops = wbytes / (ms * 1e-3) / 1e9, 2.0 * m * n * k / (ms * 1e-3) / 1e12
             out.append({"config": label, "m": m, "kernel": kernel.decode() if kernel else None, "us_per_launch": ms * 1e3,
-                        "weight_gbps": wbytes / (ms * 1e-3) / 1e9, "tflops": 2.0 * m * n * k / (ms * 1e-3) / 1e12})
+                        "weight_gbps": gbps, "tflops": tflops,
+                        # the roof that bounds the row: weight bytes over HBM for few rows, the bf16 matrix peak for many
+                        "frac_of_peak": gbps / HBM_PEAK_GBPS if m <= 64 else tflops / MFMA_BF16_PEAK_TFLOPS,
+                        "bound": "hbm" if m <= 64 else "mfma"})
 
     products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1], 48, 10_485_760)
     products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 2048], 0, WEIGHT_BYTES,
@@ -270,7 +274,8 @@ def all_configs(lib, device, qs):
     ms = best_of(calls, 200)
     out.append({"config": "C5 MXFP4 gather_qmm 32 experts W[2880,2880], 1024 sorted rows", "m": tokens * top, "kernel": "qmg_kernel",
                 "us_per_launch": ms * 1e3, "weight_gbps": 141_004_800 / (ms * 1e-3) / 1e9,
-                "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12})
+                "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12, "frac_of_peak": 141_004_800 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                "bound": "hbm"})
     del weights, calls
 
     # The weights' own kernels at the same shapes: quantize (dense in, packed out) and dequantize (packed in, dense out),
@@ -289,7 +294,8 @@ def all_configs(lib, device, qs):
                                                               ptr(q.biases), stream))
         ms = best_of([quantize_call(w) for w in dense], 60)
         out.append({"config": f"quantize {label}", "m": 0, "us_per_launch": ms * 1e3,
-                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0})
+                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0,
+                    "frac_of_peak": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "bound": "hbm"})
         qs_ = [nv.quantize(w, quant) for w in dense]
 
         def dequantize_call(qq, o):
@@ -297,7 +303,8 @@ def all_configs(lib, device, qs):
                                                                 cols, ptr(o), stream))
         ms = best_of([dequantize_call(qq, w) for qq, w in zip(qs_, dense)], 60)
         out.append({"config": f"dequantize {label}", "m": 0, "us_per_launch": ms * 1e3,
-                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0})
+                    "weight_gbps": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9, "tflops": 0.0,
+                    "frac_of_peak": (dense_bytes + packed_bytes) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "bound": "hbm"})
 
     quantizers("C2 W[14336,4096] bf16 <-> 4-bit g64", (N, K), torch.bfloat16, _lib.BF16, nv.Quant.affine(GROUP, BITS), 4)
     quantizers("C1 W[4096,4096] f32 <-> 4-bit g64", (4096, 4096), torch.float32, _lib.F32, nv.Quant.affine(64, 4), 8)

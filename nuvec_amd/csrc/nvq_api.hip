@@ -225,13 +225,22 @@ static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     // gpu.rs:6956-6981, primitive.rs:489-493).
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
     a.row_exact = d->rows != 0 || (d->row_exact != 0 && item <= 8);
-    a.batch_ndim = d->batch_ndim;
+    // Batch dimensions that one stride per operand describes together are merged (dimension i with i + 1 where every
+    // operand's stride of i is its stride of i + 1 times the extent of i + 1; extents of 1 vanish): a [B, H] batch of
+    // dense operands is one dimension, which the matrix-core kernels take.
+    int nd = 0;
     for (int i = 0; i < d->batch_ndim; i++) {
-        a.batch_shape[i] = d->batch_shape[i];
-        a.x_strides[i] = d->x_strides[i];
-        a.w_strides[i] = d->w_strides[i];
-        a.s_strides[i] = d->s_strides[i];
+        if (d->batch_shape[i] == 1) continue;
+        const int64_t e = d->batch_shape[i], xs = d->x_strides[i], ws = d->w_strides[i], ss = d->s_strides[i];
+        if (nd > 0 && a.x_strides[nd - 1] == xs * e && a.w_strides[nd - 1] == ws * e && a.s_strides[nd - 1] == ss * e) {
+            a.batch_shape[nd - 1] *= e;
+            a.x_strides[nd - 1] = xs, a.w_strides[nd - 1] = ws, a.s_strides[nd - 1] = ss;
+        } else {
+            a.batch_shape[nd] = e, a.x_strides[nd] = xs, a.w_strides[nd] = ws, a.s_strides[nd] = ss;
+            nd++;
+        }
     }
+    a.batch_ndim = nd;
     return a;
 }
 

@@ -422,20 +422,23 @@ def quantized_matmul(x: torch.Tensor, q: Quantized, transpose: bool = True, *, r
     return out.squeeze(-2) if vector else out
 
 
-def quantized_matmul_route(m: int, n: int, k: int, quant: Quant, dtype: torch.dtype, *, batch: int = 1, transpose: bool = True,
+def quantized_matmul_route(m: int, n: int, k: int, quant: Quant, dtype: torch.dtype, *, batch=1, transpose: bool = True,
                            row_exact: bool = False, rows: bool = False, device: int = 0) -> str:
-    """The kernel a product of `m` rows of x per item ([.., m, k] times `batch` weight matrices [n, k], or one matrix
-    when `batch` is 1) runs on, from the library's own routing code: what the reference's tests read from the kernel
+    """The kernel a product of `m` rows of x per item ([.., m, k] times `batch` weight matrices [n, k] — a count or a
+    tuple of batch dimensions —, or one matrix when `batch` is 1) runs on, from the library's own routing code: what the reference's tests read from the kernel
     names (tests/quantized.rs:843-861)."""
     _lib.check(_lib.load().nvq_init(device))
     d = _lib.QmmDescC()
     d.quant, d.dtype, d.transpose, d.row_exact, d.rows = quant._c(), _CODE[dtype], int(transpose), int(row_exact), int(rows)
     d.m = d.item_rows = m
     d.n, d.k = n, k
-    d.batch_ndim = 0 if batch == 1 else 1
-    if batch != 1:
-        d.batch_shape[0] = batch
-        d.x_strides[0], d.w_strides[0], d.s_strides[0] = m * k, n * k * quant.bits // 32, n * k // quant.group_size
+    dims = () if batch == 1 else tuple(batch) if isinstance(batch, (tuple, list)) else (batch,)
+    d.batch_ndim = len(dims)
+    items = 1
+    for i in reversed(range(len(dims))):  # dense operands
+        d.batch_shape[i] = dims[i]
+        d.x_strides[i], d.w_strides[i], d.s_strides[i] = items * m * k, items * n * k * quant.bits // 32, items * n * k // quant.group_size
+        items *= dims[i]
     name = _lib.load().nvq_quantized_matmul_route(C.byref(d))
     if name is None:
         raise Unsupported(_lib.last_error())

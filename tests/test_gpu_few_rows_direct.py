@@ -91,6 +91,17 @@ def test_direct_few_row_kernel_batched_with_bias(bits, group):
         want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n],
                                     biases[i * n:(i + 1) * n], group=group, bits=bits, dtype=ref.BF16)
         assert_rows_close(got[i], want, ref.BF16, f"direct few rows batched b{bits} item {i}")
+    # two batch dimensions of dense operands are one to the kernels (not the vector kernels' business)
+    assert ops.quantized_matmul_route(m, n, k, quant, torch.bfloat16, batch=(3, 1)) == "qmd_kernel"
+    assert ops.quantized_matmul_route(40, n, k, nv.Quant.affine(64, 6), torch.bfloat16, batch=(2, 3)) == "qmf_kernel"
+    w2, x2 = make_w(rng, 6 * n, k, ref.BF16), make_x(rng, 6 * m, k, ref.BF16)
+    p2, s2, b2 = ref.affine_quantize(w2, ref.BF16, group, bits)
+    q2 = nv.Quantized(to_dev(p2.reshape(2, 3, n, -1)), to_dev(s2.reshape(2, 3, n, -1)), to_dev(b2.reshape(2, 3, n, -1)), quant)
+    got2 = to_host(nv.quantized_matmul(to_dev(x2.reshape(2, 3, m, k)), q2)).reshape(6, m, n)
+    for i in range(6):
+        want = ref.quantized_matmul(x2[i * m:(i + 1) * m], p2[i * n:(i + 1) * n], s2[i * n:(i + 1) * n], b2[i * n:(i + 1) * n],
+                                    group=group, bits=bits, dtype=ref.BF16)
+        assert_rows_close(got2[i], want, ref.BF16, f"direct few rows, batch [2,3] b{bits} item {i}")
     # bias: the rounded product plus the bias, rounded (layers.rs:155-162), bit for bit the separate addition
     q0 = nv.Quantized(q.weight[0].contiguous(), q.scales[0].contiguous(), q.biases[0].contiguous(), quant)
     bias = to_dev(make_x(rng, 1, n, ref.BF16)[0])
