@@ -539,7 +539,7 @@ const char *nvq_quantized_matmul_route(const nvq_qmm_desc *d) {
     a.x = a.w = a.scales = a.biases = reinterpret_cast<const void *>(uintptr_t{256});  // operands aligned as hipMalloc aligns them
     a.y = reinterpret_cast<void *>(uintptr_t{256});
     switch (pick_route(d, a)) {
-    case Route::kUntransposed: return "qvm_kernel";
+    case Route::kUntransposed: return qvm_kernel_name(a);
     case Route::kTiled: return "qmm_kernel";
     case Route::kFewRowsDirect: return "qmd_kernel";
     case Route::kFewRows: return "qmf_kernel";

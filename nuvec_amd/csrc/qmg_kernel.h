@@ -63,8 +63,14 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
     const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
     const int tstride = table_stride(kgroups, (int)sizeof(S));
     unsigned char *table_b = table_s + kRows * tstride;
-    const int n0 = blockIdx.x * kRows;
-    const int e = blockIdx.z;
+    // Blocks are handed to the 8 XCDs in turn, each with an L2 of its own: block p takes work item
+    // (p % 8) * ceil(items / 8) + p / 8 of the expert-major list, so that the blocks of an expert — which all read
+    // the expert's rows of x — sit on one XCD.
+    const int tiles = (N + kRows - 1) / kRows, items = tiles * (int)a.experts, per = (items + 7) >> 3;
+    const int item = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+    if (item >= items) return;  // the whole block: no barrier has been reached
+    const int n0 = (item % tiles) * kRows;
+    const int e = item / tiles;
     const int row_begin = a.offsets[e];
     const int row_end = e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch;
     if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
@@ -318,7 +324,8 @@ int32_t run(const ProductArgs &a, hipStream_t s) {
                                         G::kFixedLdsBytes + kTableMaxBytes));
         configured = true;
     }
-    const dim3 grid((unsigned)((a.n + kRows - 1) / kRows), 1, (unsigned)a.experts);
+    const int64_t items = (a.n + kRows - 1) / kRows * a.experts;
+    const dim3 grid((unsigned)((items + 7) / 8 * 8));
     hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmg");
     return NVQ_OK;

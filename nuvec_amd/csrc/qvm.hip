@@ -11,8 +11,12 @@
 // in split order (deterministic), rounding once.
 #include "nvq_device.h"
 #include "nvq_internal.h"
+#include "qmf_kernel.h"
 
 namespace nvq {
+
+bool qvm_takes_tiled(const ProductArgs &a);
+
 namespace {
 
 template <int BITS>
@@ -184,6 +188,277 @@ __global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T
     Elem<T>::store(y, idx, add_row_bias<T>(row_bias, sum, idx % n));
 }
 
+
+// ---- Many rows of x: the same product on the matrix cores ---------------------------------------------------------
+// A block of four wavefronts (2 x 2, each 64 x 64 of y as 2 x 2 tiles of the 32x32x16 instruction) owns 128 x 128 of
+// y and walks K in steps of 64 rows of w through two LDS stages, one barrier per step, two blocks per compute unit.
+// The matrix instruction wants eight consecutive k per lane and column, the storage gives eight consecutive columns
+// per row and word, so the weights are turned on the way into LDS: thread (q = t / 16, c = t % 16) loads the codes of
+// columns 8 c .. 8 c + 7 of rows 4 q .. 4 q + 3 of the step (one word per row at 4 bits: sixteen lanes cover the
+// row's 64 bytes) two steps ahead, expands each row with its scale and bias to the element type (one rounding of
+// fma(code, scale, bias), as the tiled kernel of the transposed storage) between the matrix instructions of the
+// running step, swaps the 4 x 8 block in registers (one byte permute per output word) and writes, per column, its
+// four k as one 8-byte piece.  x travels through registers into the other half of the stage.
+// LDS layouts, both in 16-byte slots of eight k: x row r, slot ch at r * 8 + (ch ^ (r >> 1) % 8); w column n, slot ch
+// at (n / 16 * 8 + ch) * 16 + (n + n / 16 + 8 (ch / 4)) % 16.  Sixteen lanes reading one slot index of consecutive
+// rows (columns) touch sixteen different bank groups in either layout, and so do the writes of sixteen lanes whose
+// columns are eight apart (the rotation by n / 16).  A substep of the matrix instructions takes slot ks for the
+// lanes' lower half and slot 4 + ks for the upper one, which the layouts keep in different banks.
+// Products of few tiles split K over the grid (float32 partial sums in the caller's workspace, added in split order
+// by the reduction kernel above); without a workspace K is not split.
+namespace qmn {
+
+using namespace qmf;
+
+constexpr int BM = 128, BN = 128, BK = 64, kThreads = 256;
+constexpr int kXBytes = BM * BK * 2, kWBytes = BN * BK * 2, kStageBytes = kXBytes + kWBytes;
+
+__device__ __forceinline__ int x_slot(int row, int ch) { return (row * 8 + (ch ^ ((row >> 1) & 7))) * 16; }
+__device__ __forceinline__ int w_slot(int n, int ch) { return (((n >> 4) * 8 + ch) * 16 + ((n + (n >> 4) + 2 * (ch & 4)) & 15)) * 16; }
+
+// The codes of eight columns of one row: BITS bytes.
+template <int BITS>
+__device__ __forceinline__ void load_run(const unsigned char *p, uint32_t (&d)[BITS]) {
+#pragma unroll
+    for (int i = 0; i < BITS; i++) d[i] = 0;
+    if constexpr (BITS == 8) {
+        const uint2 v = *reinterpret_cast<const uint2 *>(p);
+        d[0] = v.x, d[1] = v.y;
+    } else if constexpr (BITS == 4) {
+        d[0] = *reinterpret_cast<const uint32_t *>(p);
+    } else {
+        static_assert(BITS == 2, "runs of eight codes of 2, 4 or 8 bits");
+        d[0] = *reinterpret_cast<const uint16_t *>(p);
+    }
+}
+
+template <typename T, int BITS, int FP4>
+__global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, int splits, float *partial) {
+    using S = std::conditional_t<FP4 != 0, uint8_t, T>;  // stored scale type
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kStageBytes];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1, h = lane >> 5, l32 = lane & 31;
+    const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
+    const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
+    const int ngroups = N >> gshift;
+    const int64_t row_bytes = ((int64_t)N * BITS) >> 3;
+    // Blocks are handed to the 8 XCDs (an L2 each) in turn: block p takes item (p % 8) * ceil(items / 8) + p / 8 of the
+    // tile list, whose order walks bands of 8 tiles of rows column tile by column tile, so that an XCD's 64 resident
+    // blocks are 8 x 8 tiles that share 8 tiles of x and 8 of w.
+    const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN, items = mtiles * ntiles, per = (items + 7) >> 3;
+    const int item = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+    if (item >= items) return;  // the whole block, before any barrier
+    const int band = item / (8 * ntiles), in_band = item - band * 8 * ntiles;
+    const int band_rows = mtiles - 8 * band < 8 ? mtiles - 8 * band : 8;
+    const int m0 = (8 * band + in_band % band_rows) * BM, n0 = (in_band / band_rows) * BN;
+    const Offsets o = batch_offsets(a, blockIdx.y);
+    const T *x = (const T *)a.x + o.x;
+
+    // Addresses are a base that is the same for the whole block (scalar registers, advanced per step by scalar
+    // arithmetic) plus a 32-bit offset per lane that never changes.
+    // This thread's part of a step of w: columns n0 + 8 c .. + 7 (a run past N reads the block's first run; its
+    // columns are not stored), rows 4 q .. 4 q + 3.
+    const int c = tid & 15, q = tid >> 4;
+    const int run = n0 + 8 * c < N ? 8 * c : 0;  // within the tile
+    const unsigned char *wbase = (const unsigned char *)a.w + o.w * 4 + (((int64_t)n0 * BITS) >> 3);
+    const S *sbase = (const S *)a.scales + o.s + (n0 >> gshift);
+    const S *bbase = (const S *)a.biases + o.s + (n0 >> gshift);
+    const uint32_t woff = (uint32_t)(4 * q) * (uint32_t)row_bytes + (uint32_t)((run * BITS) >> 3);
+    const uint32_t soff = ((uint32_t)(4 * q * ngroups) + (uint32_t)(((n0 + run) >> gshift) - (n0 >> gshift))) * (uint32_t)sizeof(S);
+    int wdst[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) wdst[j] = kXBytes + w_slot(8 * c + j, q >> 1) + 8 * (q & 1);
+    // This thread's part of a step of x: 16-byte pieces t + 256 i (piece p: row p / 8, slot p % 8).
+    const unsigned char *xbase = (const unsigned char *)(x + (int64_t)m0 * K);
+    uint32_t xoff[4];
+    int xdst[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int p = tid + 256 * i, r = p >> 3, ch = p & 7;
+        const int row = m0 + r < M ? r : M - 1 - m0;  // rows past M are computed, not stored
+        xoff[i] = ((uint32_t)row * (uint32_t)K + 8u * ch) * 2u;
+        xdst[i] = x_slot(r, ch);
+    }
+
+    struct Regs {
+        u32x4_t x[4];
+        uint32_t w[4][BITS];
+        S s[4], b[4];
+    };
+    auto load = [&](int step, Regs &r) {
+        const int64_t k0 = (int64_t)step * BK;
+        const unsigned char *xs = xbase + k0 * 2;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.x[i] = *reinterpret_cast<const u32x4_t *>(xs + xoff[i]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            load_run<BITS>(wbase + (k0 + i) * row_bytes + woff, r.w[i]);
+            const int64_t srow = (k0 + i) * ngroups * (int64_t)sizeof(S);
+            r.s[i] = *reinterpret_cast<const S *>((const unsigned char *)sbase + srow + soff);
+            if constexpr (!FP4) r.b[i] = *reinterpret_cast<const S *>((const unsigned char *)bbase + srow + soff);
+        }
+    };
+    // Row I of the thread's block of a step: eight columns, two per word, in the element type.
+    auto row = [&](const Regs &r, auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        const S sv = r.s[i], bv = r.b[i];
+        float scale, bias = 0.0f;
+        if constexpr (FP4 == kNvfp4) scale = ftz(e4m3_to_f32(sv));
+        else if constexpr (FP4) scale = ftz(e8m0_to_f32(sv));
+        else scale = Elem<T>::load(&sv, 0), bias = Elem<T>::load(&bv, 0);
+        return expand_piece<T, BITS, FP4, 0>(r.w[i], scale, bias);
+    };
+    // The four expanded rows turned (columns 2 d: the words' low halves, 2 d + 1: the high halves; rows (0, 1) and (2, 3)
+    // as two words each) and written to a stage together with the thread's pieces of x.
+    auto store = [&](int stage_at, const Regs &r, const uint4 &v0, const uint4 &v1, const uint4 &v2, const uint4 &v3) {
+        unsigned char *stage = lds + stage_at * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4_t *>(stage + xdst[i]) = r.x[i];
+        auto turn = [&](uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, int even_at, int odd_at) {
+            const uint2 even = {__builtin_amdgcn_perm(a1, a0, 0x05040100u), __builtin_amdgcn_perm(a3, a2, 0x05040100u)};
+            const uint2 odd = {__builtin_amdgcn_perm(a1, a0, 0x07060302u), __builtin_amdgcn_perm(a3, a2, 0x07060302u)};
+            *reinterpret_cast<uint2 *>(stage + even_at) = even;
+            *reinterpret_cast<uint2 *>(stage + odd_at) = odd;
+        };
+        turn(v0.x, v1.x, v2.x, v3.x, wdst[0], wdst[1]);
+        turn(v0.y, v1.y, v2.y, v3.y, wdst[2], wdst[3]);
+        turn(v0.z, v1.z, v2.z, v3.z, wdst[4], wdst[5]);
+        turn(v0.w, v1.w, v2.w, v3.w, wdst[6], wdst[7]);
+    };
+
+    int xread[2], wread[2];  // of the first slot of the lane's half; the others are an XOR (x) or a constant (w) away
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        xread[t] = (64 * wm + 32 * t + l32) * 128;
+        wread[t] = kXBytes + w_slot(64 * wn + 32 * t + l32, 4 * h);
+    }
+    const int xswz = ((l32 >> 1) & 7) ^ (4 * h);  // (the tile bases are multiples of 16 rows) slot s of the lane's half: s ^ xswz
+
+    floatx16_t acc[2][2];
+#pragma unroll
+    for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+        for (int tj = 0; tj < 2; tj++)
+#pragma unroll
+            for (int el = 0; el < 16; el++) acc[ti][tj][el] = 0.0f;
+
+    // This block's steps of K (all of them without a split), loaded two steps ahead into two sets of registers.
+    const int all_steps = K / BK, per_split = (all_steps + splits - 1) / splits;
+    const int first = (int)blockIdx.z * per_split, steps = all_steps - first < per_split ? all_steps - first : per_split;
+    const int last = first + steps - 1;
+    auto at = [&](int step) { return step < last ? step : last; };  // a step past the end loads the last one again
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    Regs ra, rb;
+    load(first, ra);
+    load(at(first + 1), rb);
+    store(0, ra, row(ra, I0{}), row(ra, I1{}), row(ra, I2{}), row(ra, I3{}));
+    load(at(first + 2), ra);
+    __syncthreads();
+    // One step.  Its four substeps of 16 k each read their operands from the stage a substep ahead and run four
+    // matrix instructions, between which one row of the next step's registers is expanded (register work only: the
+    // order of LDS reads and writes stays the written one, reads first).  Then the expanded block is turned and
+    // written to the other stage (last read a step ago, before the barrier) and the registers take the step after
+    // the next but one.  Nothing branches (a step past the end is stored and never read).
+    auto step = [&](int stage_at, Regs &next, int refill) {
+        const unsigned char *stage = lds + stage_at * kStageBytes;
+        uint4 v[4];
+        static_for<4>([&](auto ks_tag) {
+            constexpr int ks = decltype(ks_tag)::value;
+            // substep ks takes the eight k of slot ks for the lanes' lower half and of slot 4 + ks for the upper one (any
+            // order of k serves as long as x and w agree): the two halves then never meet in a bank
+            uint4 xa[2], wb[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                xa[t] = *reinterpret_cast<const uint4 *>(stage + xread[t] + ((ks ^ xswz) << 4));
+                wb[t] = *reinterpret_cast<const uint4 *>(stage + wread[t] + ks * 256);
+            }
+#pragma unroll
+            for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+                for (int tj = 0; tj < 2; tj++) acc[ti][tj] = Ops<T>::mfma(xa[ti], wb[tj], acc[ti][tj]);
+            v[ks] = row(next, ks_tag);
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        store(stage_at ^ 1, next, v[0], v[1], v[2], v[3]);
+        load(at(refill), next);
+        __syncthreads();
+    };
+    for (int s = 0; s < steps; s += 2) {
+        step(0, rb, first + s + 3);
+        if (s + 1 >= steps) break;
+        step(1, ra, first + s + 4);
+    }
+
+    // Accumulator element el of lane l is tile row 8 (el / 4) + 4 (l / 32) + el % 4 (a row of x), column l % 32.
+    T *y = (T *)a.y + o.y * M * N;
+    float *part = partial + ((int64_t)blockIdx.y * splits + blockIdx.z) * M * N;  // (used with a split only)
+    const bool biased = a.row_bias != nullptr;
+#pragma unroll
+    for (int tj = 0; tj < 2; tj++) {
+        const int col = n0 + 64 * wn + 32 * tj + l32;
+        if (col >= N) continue;
+        const float bias = biased && splits == 1 ? Elem<T>::load((const T *)a.row_bias, col) : 0.0f;
+#pragma unroll
+        for (int ti = 0; ti < 2; ti++)
+#pragma unroll
+            for (int el = 0; el < 16; el++) {
+                const int m = m0 + 64 * wm + 32 * ti + 8 * (el >> 2) + 4 * h + (el & 3);
+                if (m >= M) continue;
+                const float v = acc[ti][tj][el];
+                if (splits > 1) part[(int64_t)m * N + col] = v;
+                else Elem<T>::store(y, (int64_t)m * N + col, biased ? Elem<T>::add(Elem<T>::mul(v, 1.0f), bias) : v);  // as add_row_bias
+            }
+    }
+}
+
+// Splits of K for a product of few tiles: about two blocks per compute unit, eight steps or more per split.
+inline int splits_of(const ProductArgs &a) {
+    const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
+    const int64_t want = (2 * (int64_t)compute_units() + tiles - 1) / tiles, most = steps / 8;
+    const int64_t splits = want < most ? want : most;
+    if (splits <= 1) return 1;
+    const int64_t per_split = (steps + splits - 1) / splits;
+    return (int)((steps + per_split - 1) / per_split);  // every split holds a step
+}
+
+template <typename T, int BITS, int FP4>
+int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
+    const int splits = workspace != nullptr ? splits_of(a) : 1;  // without a workspace K is not split
+    const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN);
+    const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)a.batch, (unsigned)splits);
+    hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4>), grid, dim3(kThreads), 0, s, a, splits, workspace);
+    NVQ_LAUNCH_CHECK("qmn");
+    if (splits > 1) {
+        const int64_t per_batch = a.m * a.n, total = a.batch * per_batch;
+        hipLaunchKernelGGL((qvm_reduce_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, (const float *)workspace,
+                           (T *)a.y, splits, per_batch, total, a.row_bias, a.n);
+        NVQ_LAUNCH_CHECK("qvm_reduce");
+    }
+    return NVQ_OK;
+}
+
+template <typename T>
+int32_t run_typed(const ProductArgs &a, float *ws, hipStream_t s) {
+    switch (a.mode) {
+    case NVQ_MXFP4: return run<T, 4, kMxfp4>(a, ws, s);
+    case NVQ_MXFP8: return run<T, 8, kMxfp8>(a, ws, s);
+    case NVQ_NVFP4: return run<T, 4, kNvfp4>(a, ws, s);
+    default: break;
+    }
+    return a.bits == 2 ? run<T, 2, kAffine>(a, ws, s) : a.bits == 4 ? run<T, 4, kAffine>(a, ws, s) : run<T, 8, kAffine>(a, ws, s);
+}
+
+}  // namespace qmn
+
 template <typename T, int BITS, int MODE>
 int32_t run_qvm(const ProductArgs &a, void *workspace, hipStream_t s) {
     const int splits = qvm_splits(a);
@@ -240,11 +515,33 @@ int qvm_splits(const ProductArgs &a) {
 }
 
 size_t qvm_workspace_bytes(const ProductArgs &a) {
+    if (qvm_takes_tiled(a)) {
+        const int splits = qmn::splits_of(a);
+        return splits > 1 ? (size_t)splits * (size_t)a.batch * (size_t)a.m * (size_t)a.n * sizeof(float) : 0;
+    }
     const int splits = qvm_splits(a);
     return splits > 1 ? (size_t)splits * (size_t)a.batch * (size_t)a.m * (size_t)a.n * sizeof(float) : 0;
 }
 
+// The matrix-core kernel takes the 16-bit products whose codes come in whole runs of eight columns (2, 4 and 8 bits,
+// the block formats without a global scale) and whose K is whole steps of 64, whatever the rows of x: measured
+// against the vector kernel above (bf16, 4-bit g64, both with their split of K and its reduction, us per call of the
+// Python wrapper) w[4096,14336] 1 row 42 / 55, 8 rows 42 / 91, 32 rows 45 / 246, 512 rows 128 / 1890; w[14336,4096]
+// 1 row 35 / 131; w[1024,1024] 1 row 24 / 24, 32 rows 24 / 37; MXFP4 w[4096,4096] 1 row 22 / 94, 128 rows 26 / 588.
+bool qvm_takes_tiled(const ProductArgs &a) {
+    if (a.dtype == NVQ_F32 || a.row_exact || a.global_scale != nullptr || a.m < 1) return false;
+    if (a.mode == NVQ_AFFINE && !(a.bits == 2 || a.bits == 4 || a.bits == 8)) return false;
+    if (a.k < qmn::BK || a.k % qmn::BK != 0 || a.batch > 65535) return false;
+    for (int d = 0; d < a.batch_ndim; d++)
+        if (a.x_strides[d] % 8 != 0 || a.w_strides[d] % 4 != 0) return false;  // 16-byte pieces of x, 8-byte runs of codes
+    return ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
+}
+
+const char *qvm_kernel_name(const ProductArgs &a) { return qvm_takes_tiled(a) ? "qmn_kernel" : "qvm_kernel"; }
+
 int32_t launch_qvm(const ProductArgs &a, void *workspace, hipStream_t s) {
+    if (qvm_takes_tiled(a))
+        return a.dtype == NVQ_BF16 ? qmn::run_typed<bf16_t>(a, (float *)workspace, s) : qmn::run_typed<f16_t>(a, (float *)workspace, s);
     switch (a.dtype) {
     case NVQ_F32: return run_qvm_typed<float>(a, workspace, s);
     case NVQ_BF16: return run_qvm_typed<bf16_t>(a, workspace, s);

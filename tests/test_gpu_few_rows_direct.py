@@ -35,7 +35,7 @@ def test_routes_of_the_baseline_configurations():
         assert c4(1) == "qmv_lds_kernel"
         assert c4(16) == "qmd_kernel" and c4(2) == "qmd_kernel"
         assert c4(512) == "qmm_kernel"
-        assert c4(16, transpose=False) == "qvm_kernel"
+        assert c4(16, transpose=False) == ("qmn_kernel" if bits == 8 else "qvm_kernel")  # runs of eight codes: 2, 4, 8 bits
         assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
     assert ops.quantized_matmul_route(24, 1000, 4096, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
     assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices

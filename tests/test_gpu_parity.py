@@ -226,9 +226,10 @@ def test_config4_odd_bit_widths_512_rows(group, bits):
 def test_untransposed_product_needs_its_workspace():
     """Weights stored [K, N] split K through the caller's workspace: handed none, the call is refused, not run."""
     rng = np.random.default_rng(3)
-    k, n, m = 512, 256, 3
+    k, n, m = 480, 256, 3  # (K is no multiple of 64: the vector kernel, which cannot run unsplit)
     w, x = make_w(rng, k, n, ref.BF16), make_x(rng, m, k, ref.BF16)
     q = nv.quantize(to_dev(w), nv.Quant.affine(64, 4))
+    assert nv.quantized_matmul_route(m, n, k, q.quant, torch.bfloat16, transpose=False) == "qvm_kernel"
     y = nv.quantized_matmul(to_dev(x), q, transpose=False)
     assert y.shape == (m, n)
     with pytest.raises((nv.InvalidArgument, nv.Unsupported)):
@@ -633,6 +634,68 @@ def test_untransposed_products_batched():
     got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
     assert got.shape == (b, m, n)
     assert_rows_close(got, want, ref.F32, "batched x.w")
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("group,bits", [(64, 4), (32, 4), (128, 8), (32, 8), (64, 2), (128, 2)])
+def test_untransposed_products_on_the_matrix_cores(dtype, group, bits):
+    """Weights stored [K, N] with K in whole steps of 64 and codes in runs of eight columns: the tiled matrix-core
+    kernel, for one row of x and for several tiles of rows, ragged M and N, K split over the grid (through the
+    workspace) and not (without one)."""
+    rng = np.random.default_rng(2100 + 10 * bits + group + dtype)
+    tdtype = torch.bfloat16 if dtype == ref.BF16 else torch.float16
+    for m, k, n in [(1, 64, 128), (5, 128, 2048 + 3 * 128), (130, 192, 384), (300, 2048, 640), (33, 4096, 128)]:
+        w = make_w(rng, k, n, dtype)  # quantized along N
+        x = make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+        assert nv.quantized_matmul_route(m, n, k, q.quant, tdtype, transpose=False) == "qmn_kernel"
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, transpose=False)
+        got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
+        assert got.shape == (m, n)
+        assert_rows_close(got, want, dtype, f"x.w tiled b{bits} g{group} M={m} K={k} N={n}")
+        unsplit = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False, scratch=False))
+        assert_rows_close(unsplit, want, dtype, f"x.w tiled b{bits} g{group} M={m} K={k} N={n}, no workspace")
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+def test_untransposed_block_formats_on_the_matrix_cores(mode, qmode):
+    """The block formats of the same kernel (NVFP4: also a last group of 16 columns); their weights are exact in the
+    element type, so the bar has no exception for short rows."""
+    rng = np.random.default_rng(2200 + mode)
+    group, bits = ref.FP_PARAMS[mode]
+    for dtype, tdtype in ((ref.BF16, torch.bfloat16), (ref.F16, torch.float16)):
+        for m, k, n in [(1, 128, 256), (70, 320, 2048 + 64), (260, 1024, 96 + (16 if mode == ref.NVFP4 else 0))]:
+            w, x = make_w(rng, k, n, dtype), make_x(rng, m, k, dtype)
+            packed, scales = ref.fp_quantize(w, dtype, mode)
+            q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+            assert nv.quantized_matmul_route(m, n, k, q.quant, tdtype, transpose=False) == "qmn_kernel"
+            want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, transpose=False)
+            got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=False))
+            assert_rows_close(got, want, dtype, f"x.w tiled {qmode} M={m} K={k} N={n}", exact_weights=True)
+
+
+def test_untransposed_products_on_the_matrix_cores_batched_with_bias():
+    """x [B, M, K] against w [B, K, N / 8] on the tiled kernel, with and without the layer's bias (the separate rounded
+    addition, bit for bit) and with one weight for every batch item."""
+    rng = np.random.default_rng(2300)
+    b, m, k, n = 3, 40, 256, 384
+    w = make_w(rng, b * k, n, ref.BF16).reshape(b, k, n)
+    x = make_x(rng, b * m, k, ref.BF16).reshape(b, m, k)
+    packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+    assert nv.quantized_matmul_route(m, n, k, q.quant, torch.bfloat16, batch=b, transpose=False) == "qmn_kernel"
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16, transpose=False)
+    plain = nv.quantized_matmul(to_dev(x), q, transpose=False)
+    assert plain.shape == (b, m, n)
+    assert_rows_close(to_host(plain), want, ref.BF16, "batched x.w tiled")
+    bias = to_dev(make_x(rng, 1, n, ref.BF16).reshape(n))
+    fused = nv.quantized_matmul(to_dev(x), q, transpose=False, bias=bias)
+    assert np.array_equal(to_host(fused).view(np.uint8), to_host(plain + bias).view(np.uint8))
+    shared = nv.Quantized(q.weight[1], q.scales[1], q.biases[1], q.quant)  # broadcast over the batch
+    got = to_host(nv.quantized_matmul(to_dev(x), shared, transpose=False))
+    want1 = ref.quantized_matmul(x, packed[1], scales[1], biases[1], group=64, bits=4, dtype=ref.BF16, transpose=False)
+    assert_rows_close(got, want1, ref.BF16, "batched x against one w, tiled")
 
 
 @pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
