@@ -341,6 +341,27 @@ NVQ_API int32_t nvq_moe_route(int32_t dtype, const void *probs, int64_t rows, in
 NVQ_API int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out,
                          void *stream);
 
+/* The experts' gated activation between their gate / up products and their down product (`SwitchGlu::through`,
+ * crates/nuvec-lm/src/model.rs:2157-2170), with each row's expert's bias added to either product first
+ * (`SwitchProjection::forward`, model.rs:2139-2143): out[r, c] = act(gate[r, c] + gate_bias[ids[r], c],
+ * up[r, c] + up_bias[ids[r], c]), every operation rounded to `dtype` in the reference's order.
+ *   NVQ_GLU_SWIGLU      gate * sigmoid(gate) * up                     (crates/nuvec-nn/src/lib.rs:343-345, 513-519)
+ *   NVQ_GLU_SWIGLU_OAI  (clip(up, -limit, limit) + 1) * g * sigmoid(alpha * g), g = min(gate, limit)   (lib.rs:564-570)
+ *   gate, up dtype[rows, hidden] with `gate_stride` / `up_stride` elements between rows (so the two halves of one
+ *   product [rows, 2 * hidden] of fused gate / up weights serve);  out dtype[rows, hidden];  gate_bias, up_bias
+ *   dtype[experts, hidden], both or neither, with ids i32[rows] (an id outside is clamped). */
+enum { NVQ_GLU_SWIGLU = 0, NVQ_GLU_SWIGLU_OAI = 1 };
+typedef struct nvq_glu_desc {
+    int32_t dtype;       /* NVQ_F32, NVQ_F16 or NVQ_BF16 */
+    int32_t activation;  /* NVQ_GLU_* */
+    float alpha, limit;  /* NVQ_GLU_SWIGLU_OAI (gpt-oss: 1.702 and 7) */
+    int64_t rows, hidden;
+    int64_t gate_stride, up_stride;
+    int64_t experts;     /* rows of the biases; 0 without */
+} nvq_glu_desc;
+NVQ_API int32_t nvq_glu(const nvq_glu_desc *desc, const void *gate, const void *up, const void *gate_bias, const void *up_bias,
+                const int32_t *ids, void *out, void *stream);
+
 /* Bytes of float32 partial sums nvq_gather_qmm wants in `workspace`: with the weights stored [K, N] (transpose = 0) K is
  * split over the grid (the reference's split-K scratch, gpu.rs:7562); 0 for transposed weights. */
 NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);

@@ -60,6 +60,12 @@ class AttentionDescC(C.Structure):
                 ("scale", C.c_float)]
 
 
+class GluDescC(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("activation", C.c_int32), ("alpha", C.c_float), ("limit", C.c_float),
+                ("rows", C.c_int64), ("hidden", C.c_int64), ("gate_stride", C.c_int64), ("up_stride", C.c_int64),
+                ("experts", C.c_int64)]
+
+
 class GatherDescC(C.Structure):
     _fields_ = [("quant", QuantC), ("dtype", C.c_int32), ("transpose", C.c_int32), ("row_exact", C.c_int32),
                 ("reserved", C.c_int32), ("m", C.c_int64), ("n", C.c_int64), ("k", C.c_int64), ("pairs", C.c_int64),
@@ -100,6 +106,7 @@ SIGNATURES = {
     "nvq_gather_qmm_scatter": (C.c_int32, [C.c_void_p] * 13),
     "nvq_quantize_dequantize": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_moe_route": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nvq_glu": (C.c_int32, [C.POINTER(GluDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_weighted_sum": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
     "nvq_moe_order": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                   C.c_void_p, C.c_void_p]),

@@ -712,6 +712,26 @@ int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t ro
     return launch_weighted_sum(dtype, x, w, rows, k, d, out, (hipStream_t)stream);
 }
 
+int32_t nvq_glu(const nvq_glu_desc *d, const void *gate, const void *up, const void *gate_bias, const void *up_bias, const int32_t *ids,
+                void *out, void *stream) {
+    // model.rs:2139-2143, 2157-2170
+    if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "glu: null descriptor");
+    if (!float_dtype(d->dtype)) return fail(NVQ_INVALID_ARGUMENT, "glu: unsupported dtype %s", dtype_name(d->dtype));
+    if (d->activation != NVQ_GLU_SWIGLU && d->activation != NVQ_GLU_SWIGLU_OAI)
+        return fail(NVQ_INVALID_ARGUMENT, "glu: unknown activation %d", d->activation);
+    if (d->rows < 0 || d->hidden < 0 || d->experts < 0) return fail(NVQ_INVALID_ARGUMENT, "glu: negative size");
+    if (d->gate_stride < d->hidden || d->up_stride < d->hidden)
+        return fail(NVQ_INVALID_ARGUMENT, "glu: a row stride (%lld, %lld) below the %lld columns", (long long)d->gate_stride,
+                    (long long)d->up_stride, (long long)d->hidden);
+    if ((gate_bias == nullptr) != (up_bias == nullptr)) return fail(NVQ_INVALID_ARGUMENT, "glu: one bias without the other");
+    if (gate_bias != nullptr && (ids == nullptr || d->experts < 1)) return fail(NVQ_INVALID_ARGUMENT, "glu: biases need the rows' expert ids");
+    if (d->rows == 0 || d->hidden == 0) return NVQ_OK;
+    if (d->rows * d->hidden >= (1LL << 40)) return fail(NVQ_INVALID_ARGUMENT, "glu: more than 2^40 outputs");
+    if (gate == nullptr || up == nullptr || out == nullptr) return fail(NVQ_INVALID_ARGUMENT, "glu: null operand");
+    NVQ_TRY(require_device());
+    return launch_glu(*d, gate, up, gate_bias, up_bias, ids, out, (hipStream_t)stream);
+}
+
 static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                               const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
                               const uint32_t *out_rows, void *y, void *workspace, void *stream) {

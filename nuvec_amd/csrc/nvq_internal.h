@@ -62,6 +62,8 @@ int32_t launch_convert_packed(int32_t format, int32_t bits, int32_t dtype, const
 size_t moe_order_lds_bytes(int32_t experts);
 int32_t launch_moe_route(int32_t dtype, const void *probs, int64_t rows, int32_t experts, int32_t k, int32_t normalize,
                          uint32_t *indices, void *scores, hipStream_t s);
+int32_t launch_glu(const nvq_glu_desc &d, const void *gate, const void *up, const void *gate_bias, const void *up_bias,
+                   const int32_t *ids, void *out, hipStream_t s);
 int32_t launch_weighted_sum(int32_t dtype, const void *x, const void *w, int64_t rows, int32_t k, int64_t d, void *out, hipStream_t s);
 size_t moe_order_workspace_bytes(int64_t pairs, int32_t experts);
 int32_t launch_moe_order(const uint32_t *ids, int64_t pairs, int32_t experts, uint32_t *order, uint32_t *restore,

@@ -99,30 +99,26 @@ class SwitchProjection:
     def quantized(self) -> Quantized:
         return Quantized(self.weight, self.scales, self.biases, self.quant)
 
-    def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False, add_bias: bool = True) -> torch.Tensor:
         """model.rs:2113-2146: `x` (`[..., 1, input_dims]` batches) through the experts `indices`."""
         y = ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices))
-        return y if self.bias is None else y + self.bias[indices.long()].unsqueeze(-2)
+        return y if self.bias is None or not add_bias else y + self.bias[indices.long()].unsqueeze(-2)
 
     def forward_sorted_rows(self, x: torch.Tensor, rows, sorted_ids: torch.Tensor, offsets: torch.Tensor,
-                            out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out_rows: Optional[torch.Tensor] = None, add_bias: bool = True) -> torch.Tensor:
         """Rows `rows` of `x` (`[T, input_dims]`; None: its rows in order) through experts sorted by id.  With
-        `out_rows` (a permutation) result row i is written at row `out_rows[i]`."""
+        `out_rows` (a permutation) result row i is written at row `out_rows[i]`.  `add_bias` False leaves the experts'
+        bias to the caller (the gated activation adds it in its own pass)."""
         if rows is None:
             rows = torch.arange(x.shape[0], dtype=torch.int32, device=x.device)
         y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows)
-        if self.bias is None:
+        if self.bias is None or not add_bias:
             return y
         if out_rows is None:
             return y + self.bias[sorted_ids.long()]
         ids = torch.empty_like(sorted_ids)
         ids[out_rows.long()] = sorted_ids  # the expert of each output row
         return y + self.bias[ids.long()]
-
-
-def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """silu(gate) * up in the activations' type (elementwise; not part of the quantized path)."""
-    return torch.nn.functional.silu(gate) * up
 
 
 @dataclass
@@ -132,6 +128,22 @@ class SwitchGlu:
     up_proj: SwitchProjection
     down_proj: SwitchProjection
     gate_up_proj: Optional[SwitchProjection] = None  # `fuse_gate_up`: both projections' rows, gate first
+    activation: str = "swiglu"  # or "swiglu_oai" with `alpha` and `limit` (model.rs:2161-2166; gpt-oss: 1.702 and 7)
+    alpha: float = 1.702
+    limit: float = 7.0
+
+    def gated(self, gate: torch.Tensor, up: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        """model.rs:2157-2169 between the products: the experts' biases (model.rs:2139-2143) and the activation in one
+        pass over the two products, which arrive without their biases."""
+        gb, ub = self.gate_proj.bias, self.up_proj.bias
+        if (gb is None) != (ub is None):  # one projection with a bias: added on its own, as SwitchProjection does
+            rows = ids.reshape(-1).long()
+            if gb is not None:
+                gate = (gate.reshape(rows.numel(), -1) + gb[rows]).reshape(gate.shape)
+            else:
+                up = (up.reshape(rows.numel(), -1) + ub[rows]).reshape(up.shape)
+            gb = ub = None
+        return ops.glu(gate, up, self.activation, alpha=self.alpha, limit=self.limit, gate_bias=gb, up_bias=ub, ids=ids)
 
     def fuse_gate_up(self) -> "SwitchGlu":
         """Stores the gate and up projections as one weight `[experts, 2 * hidden, ...]` (rows of the gate, then rows of
@@ -154,20 +166,20 @@ class SwitchGlu:
         k = indices.shape[2]
         if indices.numel() < 64:  # model.rs:2189-2192
             xe = x.reshape(b, l, 1, 1, d)
-            up, gate = self.up_proj.forward(xe, indices), self.gate_proj.forward(xe, indices)
-            return self.down_proj.forward(swiglu(gate, up), indices).squeeze(-2)
+            up, gate = self.up_proj.forward(xe, indices, add_bias=False), self.gate_proj.forward(xe, indices, add_bias=False)
+            return self.down_proj.forward(self.gated(gate, up, indices), indices).squeeze(-2)
         experts = self.up_proj.weight.shape[0]
         order, restore, sorted_ids, offsets = ops.moe_order(indices, experts)
         tokens = torch.div(order, k, rounding_mode="floor").to(torch.int32)  # pair t*k + j belongs to token t
         xt = x.reshape(b * l, d)
         if self.gate_up_proj is not None:
-            both = self.gate_up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
+            both = self.gate_up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
             hidden = both.shape[-1] // 2
-            gate, up = both[:, :hidden], both[:, hidden:]
+            gate, up = both[:, :hidden], both[:, hidden:]  # (read in place: the activation takes a row stride)
         else:
-            up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
-            gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets)
-        out = self.down_proj.forward_sorted_rows(swiglu(gate, up), None, sorted_ids, offsets, out_rows=order)
+            up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
+            gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
+        out = self.down_proj.forward_sorted_rows(self.gated(gate, up, sorted_ids), None, sorted_ids, offsets, out_rows=order)
         return out.reshape(b, l, k, -1)
 
     __call__ = forward

@@ -554,6 +554,53 @@ def weighted_sum(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+GLU_ACTIVATIONS = {"swiglu": 0, "swiglu_oai": 1}
+
+
+def glu(gate: torch.Tensor, up: torch.Tensor, activation: str = "swiglu", *, alpha: float = 1.702, limit: float = 7.0,
+        gate_bias: Optional[torch.Tensor] = None, up_bias: Optional[torch.Tensor] = None,
+        ids: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The experts' gated activation (`SwitchGlu::through`, model.rs:2157-2170): `swiglu` is nuvec-nn's
+    `silu(gate) * up` (lib.rs:513-519), `swiglu_oai` gpt-oss's clamped form (lib.rs:564-570), every operation rounded
+    to the activations' type in the reference's order.  `gate` and `up` are `[..., hidden]` with unit stride along
+    the last axis and one stride between rows (views of the two halves of one fused product serve); with `gate_bias`
+    and `up_bias` (`[experts, hidden]`) and `ids` (one expert per row) each row's expert's biases are added first
+    (model.rs:2139-2143)."""
+    if activation not in GLU_ACTIVATIONS:
+        raise InvalidArgument(f"glu: unknown activation {activation!r}")
+    if gate.dtype not in _CODE or up.dtype != gate.dtype or gate.shape != up.shape or gate.ndim < 1:
+        raise InvalidArgument(f"glu: gate and up must share a floating-point type and a shape, got {gate.dtype} {list(gate.shape)} "
+                              f"and {up.dtype} {list(up.shape)}")
+    _init(gate)
+    hidden = gate.shape[-1]
+    rows = gate.numel() // hidden if hidden else 0
+
+    def as_rows(t):  # [rows, hidden] with unit stride along the columns and one stride between the rows; a copy only if needed
+        t2 = t.reshape(rows, hidden)
+        ok = hidden <= 1 or t2.stride(1) == 1
+        if rows > 1 and hidden > 0:
+            ok = ok and t2.stride(0) >= hidden
+        return t2 if ok else t2.contiguous()
+    g2, u2 = as_rows(gate), as_rows(up)
+    d = _lib.GluDescC(_CODE[gate.dtype], GLU_ACTIVATIONS[activation], float(alpha), float(limit), rows, hidden,
+                      g2.stride(0) if rows > 1 else hidden, u2.stride(0) if rows > 1 else hidden, 0)
+    gb = ub = idp = None
+    if (gate_bias is None) != (up_bias is None):
+        raise InvalidArgument("glu: one bias without the other")
+    if gate_bias is not None:
+        if ids is None or ids.numel() != rows or ids.dtype.is_floating_point:
+            raise InvalidArgument("glu: biases need one integer expert id per row")
+        if gate_bias.dtype != gate.dtype or up_bias.dtype != gate.dtype or gate_bias.ndim != 2 or gate_bias.shape != up_bias.shape \
+                or gate_bias.shape[1] != hidden:
+            raise InvalidArgument(f"glu: biases must be [experts, {hidden}] of {gate.dtype}")
+        gb, ub = gate_bias.contiguous(), up_bias.contiguous()
+        idp = ids.reshape(-1).to(torch.int32).contiguous()
+        d.experts = gb.shape[0]
+    out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    _lib.check(_lib.load().nvq_glu(C.byref(d), _ptr(g2), _ptr(u2), _ptr(gb), _ptr(ub), _ptr(idp), _ptr(out), _stream()))
+    return out
+
+
 def _out_rows(op: str, given: Optional[torch.Tensor], pairs: int, device) -> Optional[torch.Tensor]:
     """Where each pair's result goes (`nvq_gather_qmm_scatter`): one integer per pair, a permutation of the pairs."""
     if given is None:

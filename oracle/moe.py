@@ -5,7 +5,12 @@ reference defines both by that kernel's arithmetic, in the element type, in that
 source: the indices are the last k of a stable ascending sort with NaN last (numpy's stable argsort, a library routine,
 in tests/test_oracle_math.py), the documented example of crates/nuvec-core/src/fast.rs:733-737 and the NaN case of
 crates/nuvec-core/tests/fast.rs:900-911; the scores and sums are checked against float64 within the rounding of the
-element type.  Nothing here is imported by the product.
+element type.  `glu` restates the gated activations of crates/nuvec-nn/src/lib.rs (343-345, 513-519, 564-570) one
+operation at a time, each result rounded to the element type as the reference's element-wise graphs evaluate
+(crates/nuvec-core/src/fused.rs:190-215), with the experts' biases of crates/nuvec-lm/src/model.rs:2139-2143 added
+first; pinned by the documented example of lib.rs:555-560 and by the closed forms in float64 within the rounding of
+the element type.  Its last bit is PARITY UNPINNED: it depends on the host's `exp` (numpy's here, Rust's libm there).
+Nothing here is imported by the product.
 """
 from __future__ import annotations
 
@@ -71,3 +76,40 @@ def weighted_sum(x: np.ndarray, w: np.ndarray, dtype: int) -> np.ndarray:
             t = _round(product + t, dtype)
         total = t if y == 0 else _round(t + total, dtype)
     return ref.from_f32(total, dtype)
+
+
+SWIGLU, SWIGLU_OAI = 0, 1
+
+
+def _sigmoid(x: np.ndarray) -> np.ndarray:
+    """kernels.rs:1539-1543, in float32."""
+    x = np.asarray(x, np.float32)
+    with np.errstate(over="ignore"):
+        y = (np.float32(1.0) / (np.float32(1.0) + np.exp(np.abs(x), dtype=np.float32))).astype(np.float32)
+    return np.where(x < 0, y, np.float32(1.0) - y).astype(np.float32)
+
+
+def _nan_min(a, b):
+    """kernels.rs:1367-1368: NaN if either operand is NaN (numpy's minimum does the same)."""
+    return np.minimum(a, b).astype(np.float32)
+
+
+def glu(gate: np.ndarray, up: np.ndarray, dtype: int, activation: int = SWIGLU, alpha: float = 1.702, limit: float = 7.0,
+        gate_bias=None, up_bias=None, ids=None) -> np.ndarray:
+    """gate, up [rows, hidden] as stored (and biases [experts, hidden] with ids [rows]); returns [rows, hidden] as stored."""
+    with np.errstate(invalid="ignore", over="ignore"):  # inf * 0 and inf - inf are NaN, as in the reference
+        g, x = ref.to_f32(gate, dtype), ref.to_f32(up, dtype)
+        if gate_bias is not None:  # model.rs:2139-2143
+            ids = np.asarray(ids).astype(np.int64)
+            g = _round(g + ref.to_f32(gate_bias, dtype)[ids], dtype)
+            x = _round(x + ref.to_f32(up_bias, dtype)[ids], dtype)
+        if activation == SWIGLU:
+            s = _round(_sigmoid(g), dtype)              # lib.rs:344
+            y = _round(_round(g * s, dtype) * x, dtype)  # lib.rs:344, 517
+        else:
+            a, l = _round(np.float32(alpha), dtype), _round(np.float32(limit), dtype)  # lib.rs:505-507
+            g = _nan_min(g, l)                           # lib.rs:566
+            x = _nan_min(np.maximum(x, -l), l)           # lib.rs:567
+            s = _round(_sigmoid(_round(a * g, dtype)), dtype)
+            y = _round(_round(x + np.float32(1.0), dtype) * _round(g * s, dtype), dtype)  # lib.rs:568-569
+    return ref.from_f32(y, dtype)

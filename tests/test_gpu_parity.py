@@ -976,6 +976,67 @@ def test_moe_block_routes_multiplies_and_sums():
     assert torch.equal(glu(x, top).view(torch.int16), outputs.view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai"])
+def test_gated_activation_against_the_oracle(dtype, activation):
+    """`nvq_glu` (SwitchGlu::through between the products, model.rs:2157-2170; the experts' biases of model.rs:2139-2143)
+    against the oracle's operation-by-operation restatement.  The two differ only through `exp` (the device's and
+    numpy's, either within an ulp of float32), which the rounding of the sigmoid to a half type hides except at a tie:
+    there all but a few outputs in ten thousand agree bit for bit and none is off by more than one step of the type;
+    float32 outputs agree within four steps."""
+    from oracle import moe
+    rng = np.random.default_rng(7600 + dtype + len(activation))
+    tdtype = {ref.F32: torch.float32, ref.F16: torch.float16, ref.BF16: torch.bfloat16}[dtype]
+    act = moe.SWIGLU if activation == "swiglu" else moe.SWIGLU_OAI
+    rows, hidden, experts = 300, 360, 6
+    specials = np.array([0.0, -0.0, 7.0, -7.0, 7.5, -9.0, 60.0, -60.0, 100.0, -100.0, np.inf, -np.inf, np.nan, 1e-30, -1e-30], np.float32)
+    g = (rng.standard_normal((rows, 2 * hidden)) * 3).astype(np.float32)
+    g[0, :specials.size], g[0, hidden:hidden + specials.size] = specials, specials[::-1]
+    g[1, :specials.size], g[1, hidden:hidden + specials.size] = specials, 1.0
+    both = ref.from_f32(g, dtype)  # one product of fused gate / up weights: the gate's columns, then the up's
+    gate, up = both[:, :hidden], both[:, hidden:]
+    gb = ref.from_f32(rng.standard_normal((experts, hidden)).astype(np.float32), dtype)
+    ub = ref.from_f32(rng.standard_normal((experts, hidden)).astype(np.float32), dtype)
+    ids = np.sort(rng.integers(0, experts, rows)).astype(np.int32)
+
+    def check(got, want, what):
+        got, want = np.asarray(got), np.asarray(want)
+        gf, wf = ref.to_f32(got, dtype), ref.to_f32(want, dtype)
+        same = (got.view(np.uint8).reshape(got.shape + (-1,)) == want.view(np.uint8).reshape(want.shape + (-1,))).all(-1) | (np.isnan(gf) & np.isnan(wf))
+        if dtype != ref.F32:  # (float32 shows the last bits of exp itself: within four steps below)
+            assert np.count_nonzero(~same) <= max(1, same.size // 2000), f"{what}: {np.count_nonzero(~same)} of {same.size} outputs differ"
+        step = {ref.F32: 4 * 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+        off = np.abs(gf[~same].astype(np.float64) - wf[~same].astype(np.float64))
+        assert np.all(off <= step * np.abs(wf[~same]) + 2.0 ** -24), f"{what}: an output off by more than a step"
+
+    dboth = to_dev(both)
+    dgate, dup = dboth[:, :hidden], dboth[:, hidden:]  # strided views: read in place
+    check(to_host(nv.glu(dgate, dup, activation)), moe.glu(gate, up, dtype, act), f"{activation} {dtype}")
+    check(to_host(nv.glu(dgate.contiguous(), dup.contiguous(), activation, alpha=1.5, limit=5.0)),
+          moe.glu(gate, up, dtype, act, 1.5, 5.0), f"{activation} {dtype} alpha 1.5 limit 5")
+    got = nv.glu(dgate, dup, activation, gate_bias=to_dev(gb), up_bias=to_dev(ub), ids=torch.from_numpy(ids).cuda())
+    check(to_host(got), moe.glu(gate, up, dtype, act, gate_bias=gb, up_bias=ub, ids=ids), f"{activation} {dtype} with biases")
+    # batched shapes and the composition this library's SwitchGlu replaces: bias added by a separate rounded addition
+    lead = nv.glu(dgate.reshape(3, 100, hidden), dup.reshape(3, 100, hidden), activation)
+    assert tuple(lead.shape) == (3, 100, hidden) and lead.dtype == tdtype
+    assert torch.equal(lead.reshape(rows, hidden).view(torch.uint8), nv.glu(dgate, dup, activation).view(torch.uint8))
+    idl = torch.from_numpy(ids).cuda().long()
+    separate = nv.glu(dgate + to_dev(gb)[idl], dup + to_dev(ub)[idl], activation)
+    assert torch.equal(got.view(torch.uint8), separate.view(torch.uint8))
+    # empty, and what the op refuses
+    assert tuple(nv.glu(dgate[:0], dup[:0], activation).shape) == (0, hidden)
+    with pytest.raises(nv.InvalidArgument):
+        nv.glu(dgate, dup[:, :-1], activation)
+    with pytest.raises(nv.InvalidArgument):
+        nv.glu(dgate, dup, "geglu")
+    with pytest.raises(nv.InvalidArgument):
+        nv.glu(dgate, dup, activation, gate_bias=to_dev(gb))
+    with pytest.raises(nv.InvalidArgument):
+        nv.glu(dgate, dup, activation, gate_bias=to_dev(gb), up_bias=to_dev(ub))
+    with pytest.raises(nv.InvalidArgument):
+        nv.glu(dgate, dup.to(torch.float64), activation)
+
+
 @pytest.mark.parametrize("mode,qmode", [(ref.AFFINE, None), (ref.MXFP4, "MXFP4"), (ref.NVFP4, "NVFP4")])
 def test_untransposed_gathers(mode, qmode):
     """gather_qmm with the weights stored [K, N] (transpose=False): one product per pair, K split over the grid or not,

@@ -231,3 +231,54 @@ def test_weighted_sum_equals_multiply_and_sum(dtype):
     w = ref.from_f32(rng.standard_normal((2, 1)).astype(np.float32), dtype)
     want = ref.from_f32((ref.to_f32(x, dtype)[:, 0] * ref.to_f32(w, dtype)).astype(np.float32), dtype)
     assert np.array_equal(moe.weighted_sum(x, w, dtype).view(np.uint8), want.view(np.uint8))
+
+
+def test_glu_documented_example_and_clamps():
+    """crates/nuvec-nn/src/lib.rs:555-560: swiglu_oai([10, -1], [9, 0.5], 1.702, 7)[0] = 8 * 7 / (1 + exp(-1.702 * 7));
+    the gate is clamped from above only, the other operand on both sides; NaN stays NaN."""
+    from oracle import moe
+    y = moe.glu(np.array([[10.0, -1.0]], np.float32), np.array([[9.0, 0.5]], np.float32), ref.F32, moe.SWIGLU_OAI, 1.702, 7.0)
+    assert abs(float(y[0, 0]) - 8.0 * 7.0 / (1.0 + np.exp(-1.702 * 7.0))) < 1e-4
+    assert abs(float(y[0, 1]) - 1.5 * -1.0 / (1.0 + np.exp(1.702))) < 1e-6
+    low = moe.glu(np.array([[-20.0, 3.0]], np.float32), np.array([[-50.0, 50.0]], np.float32), ref.F32, moe.SWIGLU_OAI, 1.702, 7.0)
+    assert abs(float(low[0, 0]) - (-7.0 + 1.0) * -20.0 / (1.0 + np.exp(1.702 * 20.0))) < 1e-6  # gate below -limit is kept
+    assert abs(float(low[0, 1]) - 8.0 * 3.0 / (1.0 + np.exp(-1.702 * 3.0))) < 1e-5
+    nan = moe.glu(np.array([[np.nan, 1.0]], np.float32), np.array([[1.0, np.nan]], np.float32), ref.F32, moe.SWIGLU_OAI)
+    assert np.isnan(nan).all()
+    assert np.isnan(moe.glu(np.array([[np.nan]], np.float32), np.array([[1.0]], np.float32), ref.F32, moe.SWIGLU)).all()
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+def test_glu_equals_the_closed_forms(dtype):
+    """silu(g) * x and the clamped form in float64, within the roundings of the element type (three and five
+    operations); each row's expert's bias is added to both operands first."""
+    from oracle import moe
+    rng = np.random.default_rng(40 + dtype)
+    eps = {ref.F32: 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+    rows, hidden, experts = 37, 50, 5
+    g = ref.from_f32((rng.standard_normal((rows, hidden)) * 4).astype(np.float32), dtype)
+    x = ref.from_f32((rng.standard_normal((rows, hidden)) * 4).astype(np.float32), dtype)
+    gb = ref.from_f32(rng.standard_normal((experts, hidden)).astype(np.float32), dtype)
+    xb = ref.from_f32(rng.standard_normal((experts, hidden)).astype(np.float32), dtype)
+    ids = rng.integers(0, experts, rows)
+    for biased in (False, True):
+        g64, x64 = ref.to_f32(g, dtype).astype(np.float64), ref.to_f32(x, dtype).astype(np.float64)
+        if biased:  # the sums as the element type rounds them
+            g64 = ref.to_f32(ref.from_f32((g64 + ref.to_f32(gb, dtype)[ids]).astype(np.float32), dtype), dtype).astype(np.float64)
+            x64 = ref.to_f32(ref.from_f32((x64 + ref.to_f32(xb, dtype)[ids]).astype(np.float32), dtype), dtype).astype(np.float64)
+        kw = dict(gate_bias=gb, up_bias=xb, ids=ids) if biased else {}
+        got = ref.to_f32(moe.glu(g, x, dtype, moe.SWIGLU, **kw), dtype).astype(np.float64)
+        want = g64 / (1.0 + np.exp(-g64)) * x64
+        # (float16 rounds a sigmoid or a product below 2^-14 to a multiple of 2^-24)
+        tiny = 2.0 ** -24 if dtype == ref.F16 else 0.0
+        assert np.all(np.abs(got - want) <= 4 * eps * np.abs(want) + tiny * (np.abs(g64 * x64) + np.abs(x64) + 1.0) + 1e-30)
+        alpha = float(ref.to_f32(ref.from_f32(np.array([1.702], np.float32), dtype), dtype)[0])
+        got = ref.to_f32(moe.glu(g, x, dtype, moe.SWIGLU_OAI, 1.702, 7.0, **kw), dtype).astype(np.float64)
+        gc, xc = np.minimum(g64, 7.0), np.clip(x64, -7.0, 7.0)
+        want = (xc + 1.0) * gc / (1.0 + np.exp(-alpha * gc))
+        # (x + 1 may cancel: its rounding error is relative to |x| + 1, not to the sum)
+        slack = 6 * eps * np.abs(want) + 2 * eps * np.abs(gc / (1.0 + np.exp(-alpha * gc))) * (np.abs(xc) + 1.0)
+        # the rounded product alpha * g moves the sigmoid by up to |alpha g| eps / 4 (its slope is at most 1 / 4)
+        slack += np.abs(xc + 1.0) * np.abs(gc) * np.abs(alpha * gc) * eps / 4
+        slack += tiny * (np.abs((xc + 1.0) * gc) + np.abs(xc + 1.0) + 1.0)
+        assert np.all(np.abs(got - want) <= slack + 1e-30)
