@@ -362,6 +362,19 @@ typedef struct nvq_glu_desc {
 NVQ_API int32_t nvq_glu(const nvq_glu_desc *desc, const void *gate, const void *up, const void *gate_bias, const void *up_bias,
                 const int32_t *ids, void *out, void *stream);
 
+/* The grouped gathered product of the experts' gate and up projections with the gated activation as its epilogue:
+ * `SwitchGlu::through` up to its down projection (crates/nuvec-lm/src/model.rs:2157-2169) in one kernel.  w, scales,
+ * biases and expert_bias hold both projections in alternating runs of 64 rows (rows 128 b .. 128 b + 63: rows
+ * 64 b .. of the gate projection, rows 128 b + 64 .. 128 b + 127: the same rows of the up projection), desc->n is
+ * their total (a multiple of 128), desc->m is 1, rows sorted by expert with `offsets` as for nvq_gather_qmm.
+ *   y dtype[pairs, n / 2] = act(x[lhs] . gate^T + bias_gate[rhs], x[lhs] . up^T + bias_up[rhs]), the products rounded
+ *   to `dtype` as nvq_gather_qmm returns them, then nvq_glu's arithmetic: bit for bit that composition.
+ *   expert_bias dtype[experts, n] or NULL.  NVQ_UNSUPPORTED where the grouped matrix-core kernel does not take the
+ *   product (the caller then composes nvq_gather_qmm and nvq_glu). */
+NVQ_API int32_t nvq_gather_qmm_glu(const nvq_gather_desc *desc, int32_t activation, float alpha, float limit, const void *x,
+                           const void *w, const void *scales, const void *biases, const uint32_t *lhs, const uint32_t *rhs,
+                           const int32_t *offsets, const void *expert_bias, void *y, void *stream);
+
 /* Bytes of float32 partial sums nvq_gather_qmm wants in `workspace`: with the weights stored [K, N] (transpose = 0) K is
  * split over the grid (the reference's split-K scratch, gpu.rs:7562); 0 for transposed weights. */
 NVQ_API size_t nvq_gather_qmm_workspace_bytes(const nvq_gather_desc *desc);

@@ -7,5 +7,5 @@ nuvec-lm's mixture-of-experts blocks around the gathered products; `formats` and
 into `Quantized` operands in device memory.
 """
 from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, embedding,  # noqa: F401
-                  gather_qmm, gather_qmm_grouped, gather_qqmm, glu, moe_order, moe_route, qqmm, quantize, quantize_dequantize,
+                  gather_qmm, gather_qmm_glu, gather_qmm_grouped, gather_qqmm, glu, moe_order, pair_rows, moe_route, qqmm, quantize, quantize_dequantize,
                   quantized_matmul, quantized_matmul_route, sorted_offsets, weighted_sum)

@@ -106,6 +106,7 @@ SIGNATURES = {
     "nvq_gather_qmm_scatter": (C.c_int32, [C.c_void_p] * 13),
     "nvq_quantize_dequantize": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_moe_route": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nvq_gather_qmm_glu": (C.c_int32, [C.POINTER(GatherDescC), C.c_int32, C.c_float, C.c_float] + [C.c_void_p] * 10),
     "nvq_glu": (C.c_int32, [C.POINTER(GluDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_weighted_sum": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),
     "nvq_moe_order": (C.c_int32, [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,

@@ -732,9 +732,15 @@ int32_t nvq_glu(const nvq_glu_desc *d, const void *gate, const void *up, const v
     return launch_glu(*d, gate, up, gate_bias, up_bias, ids, out, (hipStream_t)stream);
 }
 
+struct GluEpilogue {
+    int32_t activation;
+    float alpha, limit;
+    const void *expert_bias;
+};
+
 static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                               const float *global_scale, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
-                              const uint32_t *out_rows, void *y, void *workspace, void *stream) {
+                              const uint32_t *out_rows, void *y, void *workspace, void *stream, const GluEpilogue *glu = nullptr) {
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null descriptor");
     NVQ_TRY(check_quant(&d->quant, "gather_qmm"));
     NVQ_TRY(check_groups("gather_qmm", d->quant.mode, biases));
@@ -757,6 +763,13 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(check_aligned("gather_qmm", "lhs", lhs, 4));
     NVQ_TRY(check_aligned("gather_qmm", "rhs", rhs, 4));
     NVQ_TRY(check_aligned("gather_qmm", "offsets", offsets, 4));
+    if (glu != nullptr) {
+        if (glu->activation != NVQ_GLU_SWIGLU && glu->activation != NVQ_GLU_SWIGLU_OAI)
+            return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: unknown activation %d", glu->activation);
+        if (!d->transpose || offsets == nullptr || d->m != 1 || d->k == 0 || d->n % 128 != 0)
+            return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue belongs to the grouped product of transposed weights whose "
+                                         "gate and up rows alternate in runs of 64");
+    }
     if (d->k == 0) {
         return launch_fill_zero(y, d->pairs * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
     }
@@ -774,6 +787,11 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;
+    if (glu != nullptr) {
+        a.glu = 1 + glu->activation; a.glu_alpha = glu->alpha; a.glu_limit = glu->limit; a.expert_bias = glu->expert_bias;
+        if (!qmf_supported(a)) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
+        return launch_qmf(a, (hipStream_t)stream);
+    }
     if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     a.offsets = nullptr;
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
@@ -806,6 +824,13 @@ int32_t nvq_gather_qmm_scatter(const nvq_gather_desc *d, const void *x, const vo
     if (global_scales != nullptr && d != nullptr && d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
     return gather_qmm_any(d, x, w, scales, biases, global_scales, lhs, rhs, offsets, out_rows, y, workspace, stream);
+}
+
+int32_t nvq_gather_qmm_glu(const nvq_gather_desc *d, int32_t activation, float alpha, float limit, const void *x, const void *w,
+                           const void *scales, const void *biases, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                           const void *expert_bias, void *y, void *stream) {
+    const GluEpilogue glu{activation, alpha, limit, expert_bias};
+    return gather_qmm_any(d, x, w, scales, biases, nullptr, lhs, rhs, offsets, nullptr, y, nullptr, stream, &glu);
 }
 
 }  // extern "C"

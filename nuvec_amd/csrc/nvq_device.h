@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "nuvec_hip.h"
+
 namespace nvq {
 
 struct bf16_t { uint16_t bits; };   // bfloat16 storage
@@ -162,5 +164,38 @@ __device__ __forceinline__ uint32_t e8m0_round_up_code(float x) {
     uint32_t c = (u >> 23) + ((u & 0x7FFFFFu) != 0u);
     return c > 254u ? 254u : c;
 }
+
+// ---- The gated activations of the experts' MLPs (crates/nuvec-nn/src/lib.rs:343-345, 513-519, 564-570), every
+// operation rounded to the element type as the reference's element-wise graphs evaluate them.
+// kernels.rs:1539-1543
+__device__ __forceinline__ float sigmoid_f32(float x) {
+    const float a = fabsf(x);
+    const float y = 1.0f / (1.0f + expf(a));
+    return x < 0.0f ? y : 1.0f - y;
+}
+
+// kernels.rs:1367-1368: a NaN operand gives NaN
+__device__ __forceinline__ float nan_min(float a, float b) { return (a != a || b != b) ? u2f(0x7FC00000u) : fminf(a, b); }
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a || b != b) ? u2f(0x7FC00000u) : fmaxf(a, b); }
+
+template <typename T>
+__device__ __forceinline__ float rounded(float v) { return Elem<T>::mul(v, 1.0f); }
+
+// `alpha` and `limit` are values of the activations' type (lib.rs:505-507: weak scalars): rounded first.
+template <typename T, int ACT>
+__device__ __forceinline__ float glu(float gate, float up, float alpha, float limit) {
+    alpha = rounded<T>(alpha), limit = rounded<T>(limit);
+    if constexpr (ACT == NVQ_GLU_SWIGLU) {
+        const float s = rounded<T>(sigmoid_f32(gate));
+        return Elem<T>::mul(Elem<T>::mul(gate, s), up);  // lib.rs:343-345, 516-517
+    } else {
+        // lib.rs:565-570
+        const float g = nan_min(gate, limit);
+        const float x = nan_min(nan_max(up, -limit), limit);
+        const float s = rounded<T>(sigmoid_f32(Elem<T>::mul(alpha, g)));
+        return Elem<T>::mul(Elem<T>::add(x, 1.0f), Elem<T>::mul(g, s));
+    }
+}
+
 
 }  // namespace nvq

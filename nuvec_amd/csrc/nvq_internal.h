@@ -90,6 +90,12 @@ struct ProductArgs {
                                     // (QuantizedLinear's bias)
     int32_t row_exact;              // every row takes the arithmetic of its one-row product: the vector kernels only, K split
                                     // (weights stored [K, N]) by the weight's shape alone
+    // Grouped gather with the gated activation as its epilogue (0: none, else 1 + NVQ_GLU_*): w holds the gate and up
+    // projections in alternating runs of 64 rows, y is [batch, n / 2]; expert_bias (NULL or [experts, n], rows as w) is
+    // added to the rounded products first.
+    int32_t glu;
+    float glu_alpha, glu_limit;
+    const void *expert_bias;
 };
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 const char *qmv_kernel_name(const ProductArgs &a);  // which of the vector / decode kernels launch_qmv runs for `a`

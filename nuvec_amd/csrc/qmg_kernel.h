@@ -45,7 +45,12 @@ struct Geometry {
     __host__ __device__ static constexpr int swizzle(int row) { return kPow2 ? (row / (BITS >= 16 ? 1 : 16 / BITS)) % BITS : 0; }
 };
 
-template <typename T, int BITS, int FP4>
+// GLU: the gated activation of the experts' MLPs as the epilogue (a.glu).  The weights then hold the gate and the up
+// projection in alternating runs of 64 rows, so that a block's wavefronts 0 and 1 own 64 columns of the gate product
+// and wavefronts 2 and 3 the same 64 columns of the up product, lane for lane: after a pass the latter leave their
+// values (rounded as the product's output, the expert's bias added) in LDS, the former combine them with their own
+// and write y [rows, N / 2].
+template <typename T, int BITS, int FP4, bool GLU = false>
 // Three blocks per compute unit (three wavefronts per SIMD): the registers are capped for that, and the LDS of a
 // block (two x stages, the weight stages, the table) fits three times.
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) qmg_kernel(const ProductArgs a) {
@@ -299,6 +304,41 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
         // place of the pass's row l (one load per wavefront) and the stores read it across lanes.
         uint32_t place = pass + lane;
         if (a.out_rows != nullptr) place = (uint32_t)min((int64_t)a.out_rows[pass + (lane < rows ? lane : 0)], a.batch - 1);
+        if constexpr (GLU) {
+            // (N is whole blocks here: checked on the host.)  The x stages are free: the loop ended with a barrier.
+            float *exchange = reinterpret_cast<float *>(lds) + ((wave & 1) * 32) * 64 + lane;  // [wavefront pair][value][lane]
+            const float bias = a.expert_bias != nullptr ? Elem<T>::load((const T *)a.expert_bias, (int64_t)e * N + col) : 0.0f;
+            auto value = [&](int u, int el) {  // the product as its output holds it, then the separate rounded addition
+                const float v = rounded<T>(acc[u][el]);
+                return a.expert_bias != nullptr ? Elem<T>::add(v, bias) : v;
+            };
+            if (wave >= 2) {
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int el = 0; el < 16; el++)
+                        if (u == 0 || two) exchange[(16 * u + el) * 64] = value(u, el);
+            }
+            __syncthreads();
+            if (wave < 2) {
+                const int H = N >> 1, hcol = (n0 >> 1) + 32 * wave + l32;
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int el = 0; el < 16; el++) {
+                        const int m0 = 32 * u + 8 * (el >> 2) + (el & 3), m = m0 + 4 * h;
+                        const uint32_t lo = __builtin_amdgcn_readlane(place, m0), hi = __builtin_amdgcn_readlane(place, m0 + 4);
+                        if (m < rows) {
+                            const float g = value(u, el), up = exchange[(16 * u + el) * 64];
+                            const float out = a.glu == 1 + NVQ_GLU_SWIGLU ? glu<T, NVQ_GLU_SWIGLU>(g, up, a.glu_alpha, a.glu_limit)
+                                                                          : glu<T, NVQ_GLU_SWIGLU_OAI>(g, up, a.glu_alpha, a.glu_limit);
+                            Elem<T>::store(y, (int64_t)(h ? hi : lo) * H + hcol, out);
+                        }
+                    }
+            }
+            __syncthreads();  // the next pass stores x where the values were exchanged
+            continue;
+        }
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
@@ -313,11 +353,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
 // Bytes of the LDS table of scales (and biases) for the block's rows.
 inline size_t table_bytes(const ProductArgs &a) { return qmf::table_bytes(a, kRows); }
 
-template <typename T, int BITS, int FP4>
-int32_t run(const ProductArgs &a, hipStream_t s) {
+template <typename T, int BITS, int FP4, bool GLU>
+int32_t run_kernel(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS>;
     static std::atomic<bool> configured = false;
-    auto kernel = qmg_kernel<T, BITS, FP4>;
+    auto kernel = qmg_kernel<T, BITS, FP4, GLU>;
     const size_t lds_bytes = G::kFixedLdsBytes + table_bytes(a);
     if (!configured) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -329,6 +369,13 @@ int32_t run(const ProductArgs &a, hipStream_t s) {
     hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmg");
     return NVQ_OK;
+}
+
+template <typename T, int BITS, int FP4>
+int32_t run(const ProductArgs &a, hipStream_t s) {
+    if (a.glu == 0) return run_kernel<T, BITS, FP4, false>(a, s);
+    if (a.n % kRows != 0) return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue takes gate and up rows in whole runs of 64");
+    return run_kernel<T, BITS, FP4, true>(a, s);
 }
 
 template <int BITS, int FP4>

@@ -128,6 +128,7 @@ class SwitchGlu:
     up_proj: SwitchProjection
     down_proj: SwitchProjection
     gate_up_proj: Optional[SwitchProjection] = None  # `fuse_gate_up`: both projections' rows, gate first
+    gate_up_paired: bool = False  # `gate_up_proj` alternates the two projections' rows in runs of 64
     activation: str = "swiglu"  # or "swiglu_oai" with `alpha` and `limit` (model.rs:2161-2166; gpt-oss: 1.702 and 7)
     alpha: float = 1.702
     limit: float = 7.0
@@ -146,13 +147,19 @@ class SwitchGlu:
         return ops.glu(gate, up, self.activation, alpha=self.alpha, limit=self.limit, gate_bias=gb, up_bias=ub, ids=ids)
 
     def fuse_gate_up(self) -> "SwitchGlu":
-        """Stores the gate and up projections as one weight `[experts, 2 * hidden, ...]` (rows of the gate, then rows of
-        the up projection; a copy made once, at load time), so that the ordered pairs take one product that reads x and
-        walks the experts once instead of two.  Every output column is computed as before: the results are bit-identical."""
+        """Stores the gate and up projections as one weight `[experts, 2 * hidden, ...]` (a copy made once, at load
+        time), so that the ordered pairs take one product that reads x and walks the experts once instead of two.  Where
+        `hidden` is a multiple of 64 the rows alternate in runs of 64 (`ops.pair_rows`) and the product applies the
+        activation itself (`ops.gather_qmm_glu`); otherwise the gate's rows come first, then the up projection's, and
+        the activation is a pass of its own.  Every output is computed as before: the results are bit-identical."""
         g, u = self.gate_proj, self.up_proj
         if g.quant != u.quant or g.weight.shape != u.weight.shape or (g.bias is None) != (u.bias is None):
             raise ops.InvalidArgument("fuse_gate_up: the gate and up projections differ in shape or quantization")
-        cat = lambda a, b: None if a is None else torch.cat([a, b], dim=1).contiguous()
+        self.gate_up_paired = g.weight.shape[1] % 64 == 0
+        if self.gate_up_paired:
+            cat = lambda a, b: None if a is None else ops.pair_rows(a, b, 1)
+        else:
+            cat = lambda a, b: None if a is None else torch.cat([a, b], dim=1).contiguous()
         self.gate_up_proj = SwitchProjection(cat(g.weight, u.weight), cat(g.scales, u.scales), cat(g.biases, u.biases),
                                              cat(g.bias, u.bias), g.quant)
         return self
@@ -172,14 +179,24 @@ class SwitchGlu:
         order, restore, sorted_ids, offsets = ops.moe_order(indices, experts)
         tokens = torch.div(order, k, rounding_mode="floor").to(torch.int32)  # pair t*k + j belongs to token t
         xt = x.reshape(b * l, d)
-        if self.gate_up_proj is not None:
+        hidden = None
+        if self.gate_up_proj is not None and self.gate_up_paired:
+            try:  # one kernel: both products and the activation
+                hidden = ops.gather_qmm_glu(xt, self.gate_up_proj.quantized(), tokens, sorted_ids, offsets, self.activation,
+                                            alpha=self.alpha, limit=self.limit, expert_bias=self.gate_up_proj.bias)
+            except ops.Unsupported:  # (a product the grouped matrix-core kernel does not take)
+                both = self.gate_up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
+                runs = both.reshape(both.shape[0], -1, 2, 64)
+                hidden = self.gated(runs[:, :, 0].reshape(both.shape[0], -1), runs[:, :, 1].reshape(both.shape[0], -1), sorted_ids)
+        elif self.gate_up_proj is not None:
             both = self.gate_up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
-            hidden = both.shape[-1] // 2
-            gate, up = both[:, :hidden], both[:, hidden:]  # (read in place: the activation takes a row stride)
+            half = both.shape[-1] // 2
+            hidden = self.gated(both[:, :half], both[:, half:], sorted_ids)  # (read in place: the activation takes a row stride)
         else:
             up = self.up_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
             gate = self.gate_proj.forward_sorted_rows(xt, tokens, sorted_ids, offsets, add_bias=False)
-        out = self.down_proj.forward_sorted_rows(self.gated(gate, up, sorted_ids), None, sorted_ids, offsets, out_rows=order)
+            hidden = self.gated(gate, up, sorted_ids)
+        out = self.down_proj.forward_sorted_rows(hidden, None, sorted_ids, offsets, out_rows=order)
         return out.reshape(b, l, k, -1)
 
     __call__ = forward

@@ -653,6 +653,58 @@ def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted
     return out
 
 
+def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor, offsets: torch.Tensor,
+                   activation: str = "swiglu", *, alpha: float = 1.702, limit: float = 7.0,
+                   expert_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`gather_qmm_grouped` of the experts' gate and up projections with `glu` as the kernel's epilogue
+    (`SwitchGlu::through` up to the down projection, model.rs:2157-2169): `q` (and `expert_bias` `[E, N]`) hold both
+    projections in alternating runs of 64 rows (`pair_rows`), the result is `[len(rows), N / 2]`, bit for bit
+    `glu(gate, up, ...)` of the two products.  Raises `Unsupported` where the grouped kernel does not take the product."""
+    op = "gather_qmm"
+    if activation not in GLU_ACTIVATIONS:
+        raise InvalidArgument(f"{op}: unknown activation {activation!r}")
+    quant = q.quant
+    quant.checked(op)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    affine = quant.mode == QuantMode.AFFINE
+    dtype = _promoted(op, x, q.scales, q.biases)
+    w = _u32(q.weight).contiguous()
+    if x.ndim != 2 or w.ndim != 3:
+        raise InvalidArgument(f"{op}: x must be [T, K] and w [E, N, K'], got {list(x.shape)} and {list(w.shape)}")
+    x = x.to(dtype).contiguous()
+    scales = (q.scales.to(dtype) if affine else q.scales).contiguous()
+    biases = q.biases.to(dtype).contiguous() if affine else None
+    columns = _quantized_columns(op, w, scales, biases, quant)
+    if x.shape[-1] != columns:
+        raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not match")
+    n = w.shape[-2]
+    if expert_bias is not None and (tuple(expert_bias.shape) != (w.shape[0], n) or expert_bias.dtype != dtype):
+        raise InvalidArgument(f"{op}: the experts' bias must be [{w.shape[0]}, {n}] of {dtype}")
+    _init(x)
+    lhs, rhs = _indices(op, x, rows.reshape(-1)).contiguous(), _indices(op, w, sorted_ids.reshape(-1)).contiguous()
+    if lhs.numel() != rhs.numel() or offsets.numel() != w.shape[0] or offsets.dtype != torch.int32:
+        raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
+    out = torch.empty((rhs.numel(), n // 2), dtype=dtype, device=x.device)
+    d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 0, 0, 1, n, columns, rhs.numel(), x.shape[0], w.shape[0])
+    eb = None if expert_bias is None else expert_bias.contiguous()
+    _lib.check(_lib.load().nvq_gather_qmm_glu(C.byref(d), GLU_ACTIVATIONS[activation], float(alpha), float(limit), _ptr(x), _ptr(w),
+                                              _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs), _ptr(offsets.contiguous()), _ptr(eb),
+                                              _ptr(out), _stream()))
+    return out
+
+
+def pair_rows(gate: torch.Tensor, up: torch.Tensor, dim: int) -> torch.Tensor:
+    """The gate and up projections' rows (along `dim`, a multiple of 64 long) in alternating runs of 64: the layout
+    `gather_qmm_glu` reads.  A copy, made once at load time."""
+    n = gate.shape[dim]
+    if up.shape != gate.shape or n % 64 != 0:
+        raise InvalidArgument(f"pair_rows: two tensors of one shape with a multiple of 64 rows, got {list(gate.shape)} and {list(up.shape)}")
+    dim = dim % gate.ndim
+    shape = gate.shape[:dim] + (n // 64, 64) + gate.shape[dim + 1:]
+    both = torch.stack([gate.reshape(shape), up.reshape(shape)], dim=dim + 1)  # [.., n / 64, 2, 64, ..]
+    return both.reshape(gate.shape[:dim] + (2 * n,) + gate.shape[dim + 1:]).contiguous()
+
+
 def _indices(op: str, a: torch.Tensor, given: Optional[torch.Tensor]) -> torch.Tensor:
     """quantized.rs:739-767: integer indices as uint32 (carried as int32 bit patterns)."""
     batch = a.shape[:-2]

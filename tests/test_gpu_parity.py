@@ -1037,6 +1037,46 @@ def test_gated_activation_against_the_oracle(dtype, activation):
         nv.glu(dgate, dup.to(torch.float64), activation)
 
 
+@pytest.mark.parametrize("quant", ["MXFP4", "affine4", "affine8", "NVFP4"])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai"])
+def test_grouped_gather_with_the_gated_epilogue(quant, activation):
+    """`nvq_gather_qmm_glu`: the gate and up products of the ordered pairs and the activation in one kernel, bit for bit
+    the two grouped products (`nvq_gather_qmm`) followed by `nvq_glu`; experts without rows, with one pass of one tile
+    (up to 32 rows), of two tiles (up to 64) and with several passes; with and without the experts' biases."""
+    rng = np.random.default_rng(7700 + len(quant) + len(activation))
+    experts, k, hidden = 7, 320, 192
+    q_of = {"MXFP4": nv.Quant.new(nv.QuantMode.MXFP4), "NVFP4": nv.Quant.new(nv.QuantMode.NVFP4), "affine4": nv.Quant.affine(64, 4),
+            "affine8": nv.Quant.affine(32, 8)}[quant]
+    for dtype in (ref.BF16, ref.F16):
+        gate = nv.quantize(to_dev(make_w(rng, experts * hidden, k, dtype).reshape(experts, hidden, k)), q_of)
+        up = nv.quantize(to_dev(make_w(rng, experts * hidden, k, dtype).reshape(experts, hidden, k)), q_of)
+        pair = lambda a, b: None if a is None else nv.pair_rows(a, b, 1)
+        both = nv.Quantized(pair(gate.weight, up.weight), pair(gate.scales, up.scales), pair(gate.biases, up.biases), q_of)
+        counts = [0, 5, 32, 33, 64, 150, 0]  # rows per expert
+        ids = np.repeat(np.arange(experts), counts).astype(np.int32)
+        pairs = ids.size
+        tokens = 40
+        x = to_dev(make_x(rng, tokens, k, dtype))
+        rows = torch.from_numpy(rng.integers(0, tokens, pairs).astype(np.int32)).cuda()
+        sorted_ids = torch.from_numpy(ids).cuda()
+        offsets = nv.sorted_offsets(sorted_ids, experts)
+        gb, ub = to_dev(make_x(rng, experts, hidden, dtype)), to_dev(make_x(rng, experts, hidden, dtype))
+        g = nv.gather_qmm_grouped(x, gate, rows, sorted_ids, offsets)
+        u = nv.gather_qmm_grouped(x, up, rows, sorted_ids, offsets)
+        for biased in (False, True):
+            kw = dict(gate_bias=gb, up_bias=ub, ids=sorted_ids) if biased else {}
+            want = nv.glu(g, u, activation, alpha=1.702, limit=7.0, **kw)
+            got = nv.gather_qmm_glu(x, both, rows, sorted_ids, offsets, activation, alpha=1.702, limit=7.0,
+                                    expert_bias=nv.pair_rows(gb, ub, 1) if biased else None)
+            assert tuple(got.shape) == (pairs, hidden)
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"{quant} {activation} dtype {dtype} biased {biased}"
+    with pytest.raises(nv.Unsupported):  # rows not in whole runs of 64
+        nv.gather_qmm_glu(x, nv.Quantized(both.weight[:, :320], both.scales[:, :320], None if both.biases is None else both.biases[:, :320], q_of),
+                          rows, sorted_ids, offsets, activation)
+    with pytest.raises(nv.InvalidArgument):
+        nv.gather_qmm_glu(x, both, rows, sorted_ids, offsets, "geglu")
+
+
 @pytest.mark.parametrize("mode,qmode", [(ref.AFFINE, None), (ref.MXFP4, "MXFP4"), (ref.NVFP4, "NVFP4")])
 def test_untransposed_gathers(mode, qmode):
     """gather_qmm with the weights stored [K, N] (transpose=False): one product per pair, K split over the grid or not,
