@@ -57,12 +57,12 @@ class Product:
     """One prepared nvq_quantized_matmul call: descriptor and pointers built once, so the timed
     loop is a bare C-ABI call per launch."""
 
-    def __init__(self, lib, m, x, q, y, n=N, k=K, dtype=None):
+    def __init__(self, lib, m, x, q, y, n=N, k=K, dtype=None, transpose=True):
         from nuvec_amd import _lib
         d = _lib.QmmDescC()
         d.quant = q.quant._c()
         d.dtype = _lib.BF16 if dtype is None else dtype
-        d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = 1, m, n, k, m, 0
+        d.transpose, d.m, d.n, d.k, d.item_rows, d.batch_ndim = int(transpose), m, n, k, m, 0
         self.d, self.fn = d, lib.nvq_quantized_matmul
         biases = q.biases.data_ptr() if q.biases is not None else None
         import torch
@@ -232,17 +232,18 @@ def all_configs(lib, device, qs):
     def best_of(calls, steps):
         return min(time_launches(calls, steps, len(calls), graph=False)[0] for _ in range(3))
 
-    def products(label, n, k, quant, tdtype, code, ms_list, copies, wbytes, weights=None):
+    def products(label, n, k, quant, tdtype, code, ms_list, copies, wbytes, weights=None, transpose=True):
         if weights is None:
             gen = torch.Generator(device=device)
             weights = []
             for i in range(copies):
                 gen.manual_seed(4321 + i)
-                weights.append(nv.quantize((torch.randn(n, k, device=device, generator=gen) * 0.02).to(tdtype), quant))
+                shape = (n, k) if transpose else (k, n)  # (stored [K, N]: quantized along N)
+                weights.append(nv.quantize((torch.randn(shape, device=device, generator=gen) * 0.02).to(tdtype), quant))
         for m in ms_list:
             x = torch.randn(m, k, device=device).to(tdtype)
             ys = [torch.empty(m, n, dtype=tdtype, device=device) for _ in weights]
-            calls = [Product(lib, m, x, q, y, n, k, code) for q, y in zip(weights, ys)]
+            calls = [Product(lib, m, x, q, y, n, k, code, transpose) for q, y in zip(weights, ys)]
             ms = best_of(calls, 600 if m <= 64 else 48)
             kernel = lib.nvq_quantized_matmul_route(C.byref(calls[0].d))  # from the library's routing code
             gbps, tflops = wbytes / (ms * 1e-3) / 1e9, 2.0 * m * n * k / (ms * 1e-3) / 1e12
@@ -259,6 +260,9 @@ def all_configs(lib, device, qs):
              7_340_032)
     products("C4 bf16 8-bit g32 W[4096,4096]", 4096, 4096, nv.Quant.affine(32, 8), torch.bfloat16, _lib.BF16, [1, 16, 512], 32,
              18_874_368)
+    # Beside the BASELINE configurations: C2's product with the weights stored [K, N] (transpose = false)
+    products("bf16 4-bit g64 w[4096,14336] stored [K, N]", N, K, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1, 16, 2048], 24,
+             WEIGHT_BYTES, transpose=False)
     # C5: 32 MXFP4 experts [2880,2880], 256 tokens x 4 distinct experts, pairs sorted by expert
     experts, n, k, tokens, top = 32, 2880, 2880, 256, 4
     weights = [nv.quantize((torch.randn(experts, n, k, device=device) * 0.02).to(torch.bfloat16), nv.QuantMode.MXFP4)

@@ -32,8 +32,9 @@ def test_static_scratch_matches_the_workspace_entry_point():
     rng = np.random.default_rng(77)
     quant = nv.Quant.affine(64, 4)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    # (rows, weight rows, K, transposed): tiled products that split K, then a smaller one, then weights stored [K, N]
-    for m, n, k, transpose in [(512, 4096, 4096, 1), (1024, 1024, 4096, 1), (3, 256, 512, 0)]:
+    # (rows, weight rows, K, transposed): tiled products that split K, then a smaller one, then weights stored [K, N] on
+    # the matrix-core kernel (K split) and on the vector kernel (K no multiple of 64)
+    for m, n, k, transpose in [(512, 4096, 4096, 1), (1024, 1024, 4096, 1), (40, 256, 2048, 0), (3, 256, 480, 0)]:
         w = make_w(rng, n, k, ref.BF16) if transpose else make_w(rng, k, n, ref.BF16)
         x = make_x(rng, m, k, ref.BF16)
         q = nv.quantize(to_dev(w), quant)
