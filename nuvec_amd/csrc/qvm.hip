@@ -420,14 +420,24 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     }
 }
 
-// Splits of K for a product of few tiles: about two blocks per compute unit, eight steps or more per split.
+// Splits of K for a product whose tiles do not fill the chip: the split with the least estimated time, counted as
+// rounds of resident blocks (two per compute unit) x (3 us to start + 1.2 us per step of the longest split) plus,
+// with a split, the reduction's launch and its float32 traffic at 4 TB/s.
 inline int splits_of(const ProductArgs &a) {
     const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
-    const int64_t want = (2 * (int64_t)compute_units() + tiles - 1) / tiles, most = steps / 8;
-    const int64_t splits = want < most ? want : most;
-    if (splits <= 1) return 1;
-    const int64_t per_split = (steps + splits - 1) / splits;
-    return (int)((steps + per_split - 1) / per_split);  // every split holds a step
+    const int64_t resident = 2 * (int64_t)compute_units();
+    if (tiles >= resident || steps < 4) return 1;
+    double best = 0.0;
+    int64_t pick = 1;
+    for (int64_t splits = 1; splits <= steps / 2 && splits <= 64; splits++) {
+        const int64_t per_split = (steps + splits - 1) / splits;
+        if ((steps + per_split - 1) / per_split != splits) continue;  // (another count gives the same longest split)
+        const int64_t rounds = (tiles * splits + resident - 1) / resident;
+        double us = (double)rounds * (3.0 + 1.2 * (double)per_split);
+        if (splits > 1) us += 2.0 + (double)splits * (double)(a.batch * a.m * a.n) * 4.0 / 4.0e6;
+        if (splits == 1 || us < best) best = us, pick = splits;
+    }
+    return (int)pick;
 }
 
 template <typename T, int BITS, int FP4>
