@@ -484,7 +484,6 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
 enum class Route { kUntransposed, kVector, kTiled, kFewRowsDirect, kFewRows };
 
 static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
-    if (a.global_scale != nullptr) return Route::kVector;  // NVFP4, transposed, one matrix: the general kernel
     if (!d->transpose) return Route::kUntransposed;        // weights stored [K, N]
     if (a.row_exact) return Route::kVector;                // the vector kernels: a row's bits do not depend on its neighbours
     if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;  // (also passes of 16 rows of small matrices, ahead of the tiles)
@@ -796,7 +795,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.offsets = nullptr;
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
     // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
-    if (!a.row_exact && global_scale == nullptr && takes_few_rows_direct(a)) return launch_qmd(a, (hipStream_t)stream);
+    if (!a.row_exact && takes_few_rows_direct(a)) return launch_qmd(a, (hipStream_t)stream);
     if (!a.row_exact && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }

@@ -84,7 +84,7 @@ struct ProductArgs {
     const int32_t *offsets;         // grouped gather: rows of expert e are [offsets[e], offsets[e+1]) of `batch` rows
     int32_t k_splits, k_split_steps;  // tiled kernel: K split over grid z (0 or 1: no split), steps of 64 values per split
     float *partials;                // tiled kernel with a split: float32 [k_splits][m][n], summed by a second kernel
-    const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (general kernel only)
+    const float *global_scale;      // NVFP4: NULL, one float32 value, or one per expert of a gather (weights stored [N, K] only)
     const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
     const void *row_bias;           // NULL, or one value of the element type per column of y, added to the rounded product
                                     // (QuantizedLinear's bias)

@@ -141,7 +141,7 @@ __host__ __device__ constexpr size_t qmd_lds_bytes(int slices, bool chunked, boo
 // and walks K in chunks, staging x anew for each.  Otherwise x is staged once and the block walks `tiles` groups of
 // tiles, the weights of a group requested one step ahead.
 //
-// The block formats (MXFP4, MXFP8, NVFP4 without a global scale) take the same walk with less arithmetic: the scaled
+// The block formats (MXFP4, MXFP8, NVFP4 with or without a global scale) take the same walk with less arithmetic: the scaled
 // conversion instructions give the dequantized elements themselves (exact: a code times a power of two; NVFP4's E4M3
 // scale by one multiplication in float32), so the accumulators run over all of K and there are no sums of x.
 template <typename T, int MODE, int BITS, int GROUP, int RM, int RT, bool CHUNKED>
@@ -169,6 +169,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     const int m0 = blockIdx.y * RM;
     const bool batched = !(a.batch == 1 && a.rhs == nullptr);
     const BatchOffsets o = batched ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
+    const float factor = MODE == NVQ_NVFP4 ? qmf::nvfp4_factor(a, a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0) : 1.0f;
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
     using S = std::conditional_t<kBlock, uint8_t, T>;  // a scale: the element type, or one byte (E8M0; NVFP4: E4M3)
@@ -273,7 +274,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
                     float sc0, sc1;
                     if constexpr (MODE == NVQ_NVFP4) {
                         const uint32_t two = word >> (16 * (kq & 1));
-                        sc0 = ftz(e4m3_to_f32(two & 255u)), sc1 = ftz(e4m3_to_f32((two >> 8) & 255u));
+                        sc0 = qmf::nvfp4_scale(two & 255u, factor), sc1 = qmf::nvfp4_scale((two >> 8) & 255u, factor);
                     } else {
                         sc0 = sc1 = ftz(e8m0_to_f32((word >> (8 * (g & 3))) & 255u));
                     }
@@ -488,7 +489,7 @@ int32_t run_qmd(const ProductArgs &a, hipStream_t s) {
 // Whether the kernel takes the product: bf16 / f16, affine 2, 3, 4 or 8 bits, K in slices of 512, 16-byte aligned
 // scale and bias rows (a lane reads the scales of its slice with vector loads).
 bool qmd_supported(const ProductArgs &a) {
-    if (a.dtype == NVQ_F32 || a.row_exact || a.global_scale != nullptr) return false;
+    if (a.dtype == NVQ_F32 || a.row_exact) return false;
     if (a.mode == NVQ_AFFINE) {
         if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 8)) return false;
         if (!(a.group == 64 || a.group == 128 || (a.group == 32 && a.bits >= 4))) return false;  // 2 and 3 bits in groups of 32: four groups per span

@@ -12,7 +12,7 @@ bool qmf_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.k < 64 || a.k % 64 != 0) return false;
     size_t lds = 0;
-    if (a.mode == NVQ_MXFP4 || (a.mode == NVQ_NVFP4 && a.global_scale == nullptr)) {
+    if (a.mode == NVQ_MXFP4 || a.mode == NVQ_NVFP4) {
         lds = qmf::lds_needed<4>(a);
     } else if (a.mode == NVQ_MXFP8) {
         lds = qmf::lds_needed<8>(a);

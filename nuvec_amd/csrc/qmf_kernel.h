@@ -44,8 +44,9 @@ typedef _Float16 f16x2v_t __attribute__((ext_vector_type(2)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 // The FP4 template parameter of the kernels below names the code format: 0 affine integers with a scale and a bias per
 // group, 1 MXFP4 (E2M1 codes, an E8M0 scale per 32), 2 MXFP8 (E4M3 codes, an E8M0 scale per 32), 3 NVFP4 (E2M1 codes, an
-// E4M3 scale per 16; without a global scale).  Every weight of the block formats is exact in bfloat16 and float16 (at
-// most six significant bits times a power of two).
+// E4M3 scale per 16, times the factor of a global scale where the product has one).  Every weight of the block formats
+// is exact in bfloat16 and float16 (at most six significant bits times a power of two) but for NVFP4 with a global
+// scale, whose weights are rounded once to the element type like the affine ones.
 constexpr int kAffine = 0, kMxfp4 = 1, kMxfp8 = 2, kNvfp4 = 3;
 typedef float floatx16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -134,6 +135,16 @@ __device__ __forceinline__ uint32_t fp4_pair_times(uint32_t word, float scale) {
     const floatx2_t v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, B);
     return Ops<T>::pack(v.x * scale, v.y * scale);
 }
+
+// NVFP4 with a global scale g (reference: crates/nuvec-core/src/kernels.rs:992-998): every group scale becomes
+// ftz(scale * ftz(g / (448 * 6))); a gather has one g per expert (quantized.rs:620-636).  Without one the factor is 1,
+// which changes no bit of a scale.
+__device__ __forceinline__ float nvfp4_factor(const ProductArgs &a, int64_t expert) {
+    if (a.global_scale == nullptr) return 1.0f;
+    const int64_t e = a.rhs != nullptr ? (expert < a.experts ? expert : a.experts - 1) : 0;
+    return ftz(a.global_scale[e] / (448.0f * 6.0f));
+}
+__device__ __forceinline__ float nvfp4_scale(uint32_t code, float factor) { return ftz(ftz(e4m3_to_f32(code)) * factor); }
 
 // Code J of a lane's 32 codes (BITS dwords, value i in bits i BITS .. of the stream) as a float.
 template <int BITS, int J>
@@ -305,6 +316,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         }
     static_assert(G::swizzle(32) == 0 && G::swizzle(33) == G::swizzle(1), "row groups share the swizzle of their rows");
 
+    const float factor = FP4 == kNvfp4 ? nvfp4_factor(a, a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0) : 1.0f;
     // The scale (NVFP4: the two scales, one per 16 values) and bias of this lane's 32 values of a step.
     auto load_scales = [&](int step, float (&scale)[RG][2], float (&bias)[RG]) {
         const int g = (step * 64 + 32 * h) >> gshift;
@@ -313,8 +325,8 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
             const int at = (32 * rg + l32) * tstride + g * (int)sizeof(S);
             const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
             if constexpr (FP4 == kNvfp4) {
-                scale[rg][0] = ftz(e4m3_to_f32(sp[0]));
-                scale[rg][1] = ftz(e4m3_to_f32(sp[1]));
+                scale[rg][0] = nvfp4_scale(sp[0], factor);
+                scale[rg][1] = nvfp4_scale(sp[1], factor);
                 bias[rg] = 0.0f;
             } else if constexpr (FP4) {
                 scale[rg][0] = scale[rg][1] = ftz(e8m0_to_f32(*sp));

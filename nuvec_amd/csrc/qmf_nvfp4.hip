@@ -1,4 +1,4 @@
-// The few-row, grouped and tiled matrix-core kernels for NVFP4 codes without a global scale (qmf_kernel.h, qmg_kernel.h,
+// The few-row, grouped and tiled matrix-core kernels for NVFP4 codes (a global scale folded into the group scales) (qmf_kernel.h, qmg_kernel.h,
 // qmm_kernel.h).
 #include "qmg_kernel.h"
 #include "qmm_kernel.h"

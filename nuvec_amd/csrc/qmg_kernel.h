@@ -132,14 +132,15 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
     });
     __builtin_amdgcn_sched_barrier(0);
 
+    const float factor = FP4 == kNvfp4 && a.global_scale != nullptr ? ftz(a.global_scale[e] / (448.0f * 6.0f)) : 1.0f;  // (one per expert)
     // The scale (NVFP4: the two scales, one per 16 values) and bias of this lane's 32 values of a step.
     auto load_scales = [&](int step, float (&scale)[2], float &bias) {
         const int g = (step * 64 + 32 * h) >> gshift;
         const int at = (32 * wave + l32) * tstride + g * (int)sizeof(S);
         const S *sp = reinterpret_cast<const S *>(table_s + at), *bp = reinterpret_cast<const S *>(table_b + at);
         if constexpr (FP4 == kNvfp4) {
-            scale[0] = ftz(e4m3_to_f32(sp[0]));
-            scale[1] = ftz(e4m3_to_f32(sp[1]));
+            scale[0] = nvfp4_scale(sp[0], factor);
+            scale[1] = nvfp4_scale(sp[1], factor);
             bias = 0.0f;
         } else if constexpr (FP4) {
             scale[0] = scale[1] = ftz(e8m0_to_f32(*sp));

@@ -10,9 +10,7 @@ bool qmm_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.mode == NVQ_AFFINE) {
         if (a.bits != 2 && a.bits != 3 && a.bits != 4 && a.bits != 6 && a.bits != 8) return false;
-    } else if (a.mode == NVQ_NVFP4 && a.global_scale != nullptr) {
-        return false;  // the scaled weights are not exact in the element type: the general kernel keeps them in float32
-    }
+    }  // (NVFP4 with a global scale: the scaled weights are rounded to the element type like the affine ones)
     if (a.rhs != nullptr) return false;
     if (a.batch > 1 && a.batch_ndim != 1) return false;
     return a.batch <= 65535 && a.k >= qmm::BK && a.k % qmm::BK == 0;

@@ -299,10 +299,11 @@ qmm_kernel(const ProductArgs a) {
             if constexpr (FP4 == kNvfp4) braw[j] = sbt[BN + col];  // the lane's second group of 16
         }
     };
+    const float factor = FP4 == kNvfp4 ? nvfp4_factor(a, 0) : 1.0f;  // (one matrix, or a batch that shares the scale)
     auto convert_scales = [&](int j) {
         if constexpr (FP4 == kNvfp4) {
-            sc[j][0] = ftz(e4m3_to_f32((uint8_t)sraw[j]));
-            sc[j][1] = ftz(e4m3_to_f32((uint8_t)braw[j]));
+            sc[j][0] = nvfp4_scale((uint8_t)sraw[j], factor);
+            sc[j][1] = nvfp4_scale((uint8_t)braw[j], factor);
             bi[j] = 0.0f;
         } else if constexpr (FP4) {
             sc[j][0] = sc[j][1] = ftz(e8m0_to_f32((uint8_t)sraw[j]));

@@ -559,12 +559,22 @@ def test_nvfp4_global_scale(dtype):
     for out in (ref.BF16, ref.F32, ref.F16):
         want = ref.fp_dequantize(packed, scales, ref.NVFP4, out, g)
         assert np.array_equal(to_host(nv.dequantize(q, TORCH[out])).view(np.uint8), want.view(np.uint8))
-    for m in (1, 5, 40):
+    for m in (1, 5, 40, 300):
         x = make_x(rng, m, k, dtype)
         want = ref.fp_quantized_matmul_scaled(x, packed, scales, ref.NVFP4, dtype, g)
         got = to_host(nv.quantized_matmul(to_dev(x), q))
-        ratio = _excess(got, want, dtype)
-        assert float(np.max(ratio)) <= 1.0, f"M={m}: max error is {float(np.max(ratio)):.3f} x the bound"
+        assert_rows_close(got, want, dtype, f"NVFP4 with a global scale M={m} K={k} N={n}")
+    if dtype != ref.F32:  # the matrix-core kernels fold the global scale into the group scales (kernels.rs:992-998)
+        n2, k2 = 640, 1024
+        w2 = make_w(rng, n2, k2, dtype)
+        p2, s2 = ref.fp_quantize(w2, dtype, ref.NVFP4, g)
+        q2 = nv.quantize(to_dev(w2), nv.QuantMode.NVFP4, gs)
+        for m, kernels in ((1, ("qmd_kernel",)), (16, ("qmd_kernel",)), (40, ("qmf_kernel", "qmd_kernel")), (600, ("qmm_kernel", "qmf_kernel"))):
+            x = make_x(rng, m, k2, dtype)
+            want = ref.fp_quantized_matmul_scaled(x, p2, s2, ref.NVFP4, dtype, g)
+            got = to_host(nv.quantized_matmul(to_dev(x), q2))
+            assert_rows_close(got, want, dtype, f"NVFP4 with a global scale on the matrix cores M={m} K={k2} N={n2}")
+            assert nv.quantized_matmul_route(m, n2, k2, q2.quant, TORCH[dtype]) in kernels  # (the scale does not change the route)
     # a batch of x: the reference dequantizes in x's type and multiplies densely (quantized.rs:481-491); so does the mirror
     xb = make_x(rng, 6, k, dtype).reshape(2, 3, k)
     got = to_host(nv.quantized_matmul(to_dev(xb), q)).reshape(6, n)
@@ -582,6 +592,13 @@ def test_nvfp4_global_scale(dtype):
     for i in range(pairs):
         want = ref.fp_quantized_matmul_scaled(xe[i], pe[rhs[i]], se[rhs[i]], ref.NVFP4, dtype, float(ge[rhs[i]]))
         assert float(np.max(_excess(got[i], want, dtype))) <= 1.0, f"pair {i}"
+    # many pairs sorted by expert: the grouped route, one scale per expert there too
+    many = 90
+    xm = make_x(rng, many, 256, dtype).reshape(many, 1, 256)
+    ids = np.sort(rng.integers(0, experts, many))
+    got = to_host(nv.gather_qmm(to_dev(xm), qe, None, torch.from_numpy(ids).cuda(), nv.GatherQmm(sorted_indices=True)))
+    want = np.stack([ref.fp_quantized_matmul_scaled(xm[i], pe[ids[i]], se[ids[i]], ref.NVFP4, dtype, float(ge[ids[i]])) for i in range(many)])
+    assert_rows_close(got.reshape(many, 64), want.reshape(many, 64), dtype, "NVFP4 experts with a global scale each, sorted pairs")
     with pytest.raises(nv.Unsupported):  # untransposed weights with a global scale: no kernel, and nothing else answers
         nv.gather_qmm(to_dev(xe[:, :, :64]), qe, None, torch.from_numpy(rhs).cuda(), nv.GatherQmm(transpose=False))
     with pytest.raises(nv.InvalidArgument):
