@@ -4,8 +4,8 @@
 
 namespace nvq {
 
-// Whether the few-row matrix-core kernel takes this product: MXFP4 or affine 2, 3, 4, 6 or 8 bits, bf16 or
-// f16, whole steps of 64 values (whole windows of 128 for 3 bits, whose 16-byte chunks straddle steps),
+// Whether the few-row matrix-core kernel takes this product: a block format or affine 1 to 6 or 8 bits, bf16 or
+// f16, whole steps of 64 values (whole windows of 128 for 1, 3 and 5 bits, whose 16-byte chunks straddle steps),
 // a scale table that fits in LDS, and either no batch, a batch with one stride per operand, gathered pairs,
 // or the grouped gather.
 bool qmf_supported(const ProductArgs &a) {
@@ -18,9 +18,11 @@ bool qmf_supported(const ProductArgs &a) {
         lds = qmf::lds_needed<8>(a);
     } else if (a.mode == NVQ_AFFINE) {
         switch (a.bits) {
+        case 1: lds = qmf::lds_needed<1>(a); break;
         case 2: lds = qmf::lds_needed<2>(a); break;
         case 3: lds = qmf::lds_needed<3>(a); break;
         case 4: lds = qmf::lds_needed<4>(a); break;
+        case 5: lds = qmf::lds_needed<5>(a); break;
         case 6: lds = qmf::lds_needed<6>(a); break;
         case 8: lds = qmf::lds_needed<8>(a); break;
         default: return false;
@@ -41,9 +43,11 @@ int32_t launch_qmf(const ProductArgs &a, hipStream_t s) {
     if (a.mode == NVQ_MXFP8) return launch_qmf_fp8(a, s);
     if (a.mode == NVQ_NVFP4) return launch_qmf_nvfp4(a, s);
     switch (a.bits) {
+    case 1: return launch_qmf_b1(a, s);
     case 2: return launch_qmf_b2(a, s);
     case 3: return launch_qmf_b3(a, s);
     case 4: return launch_qmf_b4(a, s);
+    case 5: return launch_qmf_b5(a, s);
     case 6: return launch_qmf_b6(a, s);
     default: return launch_qmf_b8(a, s);
     }

@@ -542,7 +542,9 @@ inline size_t lds_needed(const ProductArgs &a) {
 int32_t launch_qmf_fp8(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_nvfp4(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b2(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b1(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b3(const ProductArgs &a, hipStream_t s);
+int32_t launch_qmf_b5(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b4(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b6(const ProductArgs &a, hipStream_t s);
 int32_t launch_qmf_b8(const ProductArgs &a, hipStream_t s);

@@ -4,12 +4,12 @@
 
 namespace nvq {
 
-// Whether the tiled kernel takes this product: MXFP4 or affine 2, 3, 4, 6 or 8 bits, bf16 or f16, whole
+// Whether the tiled kernel takes this product: a block format or affine 1 to 6 or 8 bits, bf16 or f16, whole
 // steps of 64 values, and a batch that is a single stride per operand (or no batch).
 bool qmm_supported(const ProductArgs &a) {
     if (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16) return false;
     if (a.mode == NVQ_AFFINE) {
-        if (a.bits != 2 && a.bits != 3 && a.bits != 4 && a.bits != 6 && a.bits != 8) return false;
+        if (a.bits < 1 || a.bits > 8 || a.bits == 7) return false;
     }  // (NVFP4 with a global scale: the scaled weights are rounded to the element type like the affine ones)
     if (a.rhs != nullptr) return false;
     if (a.batch > 1 && a.batch_ndim != 1) return false;
@@ -34,9 +34,11 @@ int32_t launch_qmm(const ProductArgs &a, void *workspace, hipStream_t s) {
     if (a.mode == NVQ_MXFP8) return launch_qmm_fp8(a, workspace, s);
     if (a.mode == NVQ_NVFP4) return launch_qmm_nvfp4(a, workspace, s);
     switch (a.bits) {
+    case 1: return launch_qmm_b1(a, workspace, s);
     case 2: return launch_qmm_b2(a, workspace, s);
     case 3: return launch_qmm_b3(a, workspace, s);
     case 4: return launch_qmm_b4(a, workspace, s);
+    case 5: return launch_qmm_b5(a, workspace, s);
     case 6: return launch_qmm_b6(a, workspace, s);
     default: return launch_qmm_b8(a, workspace, s);
     }

@@ -1,5 +1,5 @@
 // Tiled quantized products y[M,N] = x[M,K] . dequantize(w[N,K])^T on the gfx950 matrix cores: the
-// prefill-shaped path, for affine 2, 3, 4, 6 and 8-bit codes and MXFP4 (this header holds the kernel template;
+// prefill-shaped path, for affine 1- to 6- and 8-bit codes and the block formats (this header holds the kernel template;
 // the per-width translation units instantiate it).  Values follow nuvec's CPU product (reference:
 // crates/nuvec-core/src/kernels.rs:1091-1142) within the stated tolerance; as in the reference's
 // device kernels the weights are dequantized on chip in the element type (one rounding of
@@ -61,9 +61,11 @@ using SmallTile = Tile<2, 2, 2, 2>;  // 128 x 128, 256 threads, two blocks per c
 
 // How a lane's BITS dwords travel into LDS: one or two pieces of 4, 3 or 1 dwords.
 template <int BITS> struct Pieces;
+template <> struct Pieces<1> { static constexpr int count = 1, dwords = 1; };
 template <> struct Pieces<2> { static constexpr int count = 2, dwords = 1; };
 template <> struct Pieces<3> { static constexpr int count = 1, dwords = 3; };
 template <> struct Pieces<4> { static constexpr int count = 1, dwords = 4; };
+template <> struct Pieces<5> { static constexpr int count = 5, dwords = 1; };
 template <> struct Pieces<6> { static constexpr int count = 2, dwords = 3; };
 template <> struct Pieces<8> { static constexpr int count = 2, dwords = 4; };
 
@@ -547,7 +549,9 @@ int32_t run_dtype(const ProductArgs &a, void *workspace, hipStream_t s) {
 
 // One per code width, each in its own translation unit.
 int32_t launch_qmm_b2(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b1(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b3(const ProductArgs &a, void *workspace, hipStream_t s);
+int32_t launch_qmm_b5(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b4(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b6(const ProductArgs &a, void *workspace, hipStream_t s);
 int32_t launch_qmm_b8(const ProductArgs &a, void *workspace, hipStream_t s);

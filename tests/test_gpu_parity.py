@@ -418,7 +418,7 @@ def test_few_rows_on_matrix_cores(m):
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("group,bits", [(32, 2), (64, 3), (128, 3), (64, 6), (32, 8), (128, 8), (32, 4)])
+@pytest.mark.parametrize("group,bits", [(32, 2), (64, 3), (128, 3), (64, 6), (32, 8), (128, 8), (32, 4), (64, 5), (32, 5), (128, 1), (32, 1)])
 def test_few_rows_every_width(dtype, group, bits):
     """The few-row matrix-core kernel at every code width it takes: K of whole and of half windows
     (128 and 64 values), N off the rows per block, passes of 8, 16 and 32 rows of x."""
@@ -431,6 +431,8 @@ def test_few_rows_every_width(dtype, group, bits):
         got = to_host(nv.quantized_matmul(to_dev(x), q))
         assert_rows_close(got, want, dtype, f"few rows b{bits} g{group} M={m} N={n} K={k}")
         assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, f"few rows b{bits} g{group} M={m} N={n} K={k}")
+        if m >= 5 and k % 128 == 0:  # (a single row of some widths stays on the vector kernels; odd widths need whole windows)
+            assert nv.quantized_matmul_route(m, n, k, q.quant, TORCH[dtype]) in ("qmf_kernel", "qmd_kernel", "qmm_kernel")
 
 
 @pytest.mark.parametrize("bits,group", [(3, 64), (8, 32)])
@@ -450,7 +452,7 @@ def test_few_rows_batched_widths(bits, group):
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("group,bits", [(32, 2), (64, 3), (128, 6), (32, 8), (64, 8)])
+@pytest.mark.parametrize("group,bits", [(32, 2), (64, 3), (128, 6), (32, 8), (64, 8), (64, 5), (128, 5), (64, 1), (32, 1)])
 def test_tiled_every_width(dtype, group, bits):
     """The tiled matrix-core kernel (M >= 193) at the other code widths, on shapes off its 256 x 256 x 64 tile."""
     rng = np.random.default_rng(1200 + 10 * bits + group)
@@ -462,6 +464,7 @@ def test_tiled_every_width(dtype, group, bits):
         got = to_host(nv.quantized_matmul(to_dev(x), q))
         assert_rows_close(got, want, dtype, f"tiled b{bits} g{group} {m}x{n}x{k}")
         assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, f"tiled b{bits} g{group} {m}x{n}x{k}")
+        assert nv.quantized_matmul_route(m, n, k, q.quant, TORCH[dtype]) in ("qmm_kernel", "qmf_kernel", "qmd_kernel")
 
 
 def test_tiled_mxfp4():
