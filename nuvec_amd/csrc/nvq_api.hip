@@ -215,6 +215,13 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 }
 
 // The kernels' view of a product descriptor.
+// Rows of few outputs: the bar of a product (a fraction of the row's largest output) is then so tight that the one
+// rounding the device kernels give a dequantized affine weight, against the CPU's two (kernels.rs:835-859), shows in
+// the worst output; such products materialise the CPU's weights instead, bit for bit.
+static bool wants_exact_weights(int32_t mode, int32_t dtype, int64_t n) {
+    return mode == NVQ_AFFINE && dtype != NVQ_F32 && n < 1024;
+}
+
 static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     nvq::ProductArgs a{};
     a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
@@ -225,6 +232,7 @@ static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     // gpu.rs:6956-6981, primitive.rs:489-493).
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
     a.row_exact = d->rows != 0 || (d->row_exact != 0 && item <= 8);
+    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
     // Batch dimensions that one stride per operand describes together are merged (dimension i with i + 1 where every
     // operand's stride of i is its stride of i + 1 times the extent of i + 1; extents of 1 vanish): a [B, H] batch of
     // dense operands is one dimension, which the matrix-core kernels take.
@@ -782,11 +790,16 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.global_scale = global_scale;
     a.out_rows = out_rows;
     a.row_exact = d->row_exact != 0;
+    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
     a.offsets = offsets;
     if (glu != nullptr) {
+        // (projections of fewer rows take the exact-weights kernels as separate products: the epilogue form would differ)
+        if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2))
+            return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue takes affine projections of 1024 rows or more each");
+        a.exact_weights = 0;
         a.glu = 1 + glu->activation; a.glu_alpha = glu->alpha; a.glu_limit = glu->limit; a.expert_bias = glu->expert_bias;
         if (!qmf_supported(a)) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
         return launch_qmf(a, (hipStream_t)stream);

@@ -90,6 +90,10 @@ struct ProductArgs {
                                     // (QuantizedLinear's bias)
     int32_t row_exact;              // every row takes the arithmetic of its one-row product: the vector kernels only, K split
                                     // (weights stored [K, N]) by the weight's shape alone
+    // Affine codes, 16-bit elements, rows of few outputs: the kernels materialise the weights with the CPU's two roundings
+    // (round(round(code * scale) + bias), kernels.rs:835-859) instead of one; the routes keep such products off the
+    // kernels that never materialise a weight.
+    int32_t exact_weights;
     // Grouped gather with the gated activation as its epilogue (0: none, else 1 + NVQ_GLU_*): w holds the gate and up
     // projections in alternating runs of 64 rows, y is [batch, n / 2]; expert_bias (NULL or [experts, n], rows as w) is
     // added to the rounded products first.

@@ -489,7 +489,7 @@ int32_t run_qmd(const ProductArgs &a, hipStream_t s) {
 // Whether the kernel takes the product: bf16 / f16, affine 2, 3, 4 or 8 bits, K in slices of 512, 16-byte aligned
 // scale and bias rows (a lane reads the scales of its slice with vector loads).
 bool qmd_supported(const ProductArgs &a) {
-    if (a.dtype == NVQ_F32 || a.row_exact) return false;
+    if (a.dtype == NVQ_F32 || a.row_exact || a.exact_weights) return false;  // (the factored form never materialises a weight)
     if (a.mode == NVQ_AFFINE) {
         if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 8)) return false;
         if (!(a.group == 64 || a.group == 128 || (a.group == 32 && a.bits >= 4))) return false;  // 2 and 3 bits in groups of 32: four groups per span

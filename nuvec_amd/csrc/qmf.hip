@@ -32,7 +32,7 @@ bool qmf_supported(const ProductArgs &a) {
         return false;
     }
     if (a.offsets != nullptr)  // the grouped kernel: one row of x per pair, its scale table within its LDS budget
-        return a.m == 1 && a.experts <= 65535 && qmg::table_bytes(a) <= (size_t)qmg::kTableMaxBytes;
+        return a.m == 1 && a.experts <= 65535 && !a.exact_weights && qmg::table_bytes(a) <= (size_t)qmg::kTableMaxBytes;
     if (lds > (size_t)qmf::kLdsLimit) return false;
     if (a.rhs != nullptr) return a.batch <= 65535 && (a.m + 31) / 32 <= 65535;  // gathered pairs, one per grid z
     return (a.batch == 1 || a.batch_ndim == 1) && a.batch <= 65535 && (a.m + 31) / 32 <= 65535;

@@ -128,6 +128,28 @@ template <> struct Ops<f16_t> {
     }
 };
 
+// Low / high 16 bits of a word as element-type values.
+template <typename T> __device__ __forceinline__ float half_lo(uint32_t p);
+template <typename T> __device__ __forceinline__ float half_hi(uint32_t p);
+template <> __device__ __forceinline__ float half_lo<bf16_t>(uint32_t p) { return u2f(p << 16); }
+template <> __device__ __forceinline__ float half_hi<bf16_t>(uint32_t p) { return u2f(p & 0xFFFF0000u); }
+template <> __device__ __forceinline__ float half_lo<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[0]; }
+template <> __device__ __forceinline__ float half_hi<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[1]; }
+
+// Two dequantized affine weights as the element type holds them.  As the reference's device kernels: one rounding of
+// fma(code, scale, bias).  EXACT: the CPU's two roundings, round(round(code * scale) + bias)
+// (crates/nuvec-core/src/kernels.rs:835-859; code * scale is exact in float32 and the sum of two elements rounds to
+// the element type as from the exact sum), so that the weights are bit for bit those nuvec's CPU product multiplies.
+template <typename T, bool EXACT>
+__device__ __forceinline__ uint32_t affine_pair(float c0, float c1, float s, float b) {
+    if constexpr (!EXACT) {
+        return Ops<T>::pack(__builtin_fmaf(c0, s, b), __builtin_fmaf(c1, s, b));
+    } else {
+        const uint32_t p = Ops<T>::pack(c0 * s, c1 * s);
+        return Ops<T>::pack(half_lo<T>(p) + b, half_hi<T>(p) + b);
+    }
+}
+
 // The two E2M1 codes of byte B of `word` times any `scale` (NVFP4: the scale is no power of two, so the scaled
 // conversion, which takes the scale's exponent only, does not apply): decoded to float, multiplied, packed.
 template <typename T, int B>
@@ -161,7 +183,7 @@ __device__ __forceinline__ float code_to_float(const uint32_t (&dw)[BITS]) {
 }
 
 // Piece KK (eight codes, stream order) of a lane's 32 codes as one matrix operand.
-template <typename T, int BITS, int FP4, int KK>
+template <typename T, int BITS, int FP4, int KK, bool EXACT = false>
 __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float s, float b) {
     uint4 r;
     if constexpr (FP4 == kMxfp8) {
@@ -185,16 +207,16 @@ __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float 
     } else if constexpr (BITS == 4) {
         const uint32_t word = dw[KK];
         const uint32_t even = opaque(word & 0x0F0F0F0Fu), odd = opaque((word >> 4) & 0x0F0F0F0Fu);
-        r.x = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<0>(even), s, b), __builtin_fmaf(ubyte_to_float<0>(odd), s, b));
-        r.y = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<1>(even), s, b), __builtin_fmaf(ubyte_to_float<1>(odd), s, b));
-        r.z = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<2>(even), s, b), __builtin_fmaf(ubyte_to_float<2>(odd), s, b));
-        r.w = Ops<T>::pack(__builtin_fmaf(ubyte_to_float<3>(even), s, b), __builtin_fmaf(ubyte_to_float<3>(odd), s, b));
+        r.x = affine_pair<T, EXACT>(ubyte_to_float<0>(even), ubyte_to_float<0>(odd), s, b);
+        r.y = affine_pair<T, EXACT>(ubyte_to_float<1>(even), ubyte_to_float<1>(odd), s, b);
+        r.z = affine_pair<T, EXACT>(ubyte_to_float<2>(even), ubyte_to_float<2>(odd), s, b);
+        r.w = affine_pair<T, EXACT>(ubyte_to_float<3>(even), ubyte_to_float<3>(odd), s, b);
     } else {
         constexpr int J = 8 * KK;
-        r.x = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 0>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 1>(dw), s, b));
-        r.y = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 2>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 3>(dw), s, b));
-        r.z = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 4>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 5>(dw), s, b));
-        r.w = Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J + 6>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 7>(dw), s, b));
+        r.x = affine_pair<T, EXACT>(code_to_float<BITS, J + 0>(dw), code_to_float<BITS, J + 1>(dw), s, b);
+        r.y = affine_pair<T, EXACT>(code_to_float<BITS, J + 2>(dw), code_to_float<BITS, J + 3>(dw), s, b);
+        r.z = affine_pair<T, EXACT>(code_to_float<BITS, J + 4>(dw), code_to_float<BITS, J + 5>(dw), s, b);
+        r.w = affine_pair<T, EXACT>(code_to_float<BITS, J + 6>(dw), code_to_float<BITS, J + 7>(dw), s, b);
     }
     return r;
 }
@@ -229,7 +251,8 @@ __device__ __forceinline__ void fill_table(unsigned char *table, const S *src, i
 }
 
 // blockIdx.z is a batch with one stride per operand, or a gathered pair; blockIdx.y a pass of 32 rows.
-template <typename T, int BITS, int FP4, int RG>
+// EXACT (affine codes): the weights as nuvec's CPU product holds them (affine_pair).
+template <typename T, int BITS, int FP4, int RG, bool EXACT = false>
 __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     using G = Geometry<BITS, RG>;
     constexpr int kRows = G::kRows, kDepth = G::kDepth, kLoads = G::kLoads;
@@ -426,7 +449,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
                             }
 #pragma unroll
                             for (int rg = 0; rg < RG; rg++)
-                                acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk>(codes[t][rg], scale[rg][kk >> 1], bias[rg]), acc[rg]);
+                                acc[rg] = Ops<T>::mfma(xa, expand_piece<T, BITS, FP4, kk, EXACT>(codes[t][rg], scale[rg][kk >> 1], bias[rg]), acc[rg]);
                         });
                     }
                 }
@@ -502,11 +525,11 @@ inline int row_groups(const ProductArgs &a) {
     return blocks >= 192 ? 2 : 1;
 }
 
-template <typename T, int BITS, int FP4, int RG>
+template <typename T, int BITS, int FP4, int RG, bool EXACT = false>
 int32_t run_variant(const ProductArgs &a, hipStream_t s) {
     using G = Geometry<BITS, RG>;
     static std::atomic<bool> configured = false;
-    auto kernel = qmf_kernel<T, BITS, FP4, RG>;
+    auto kernel = qmf_kernel<T, BITS, FP4, RG, EXACT>;
     if (!configured) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
         configured = true;
@@ -522,6 +545,8 @@ int32_t run_variant(const ProductArgs &a, hipStream_t s) {
 
 template <typename T, int BITS, int FP4>
 int32_t run_width(const ProductArgs &a, hipStream_t s) {
+    if constexpr (FP4 == kAffine)
+        if (a.exact_weights) return run_variant<T, BITS, FP4, 1, true>(a, s);  // (rows of few outputs: 32 weight rows per block)
     return row_groups(a) == 2 ? run_variant<T, BITS, FP4, 2>(a, s) : run_variant<T, BITS, FP4, 1>(a, s);
 }
 
@@ -533,7 +558,7 @@ int32_t run_dtype(const ProductArgs &a, hipStream_t s) {
 // LDS bytes of the variant `launch_qmf` would pick (for `qmf_supported`).
 template <int BITS>
 inline size_t lds_needed(const ProductArgs &a) {
-    return row_groups(a) == 2 ? Geometry<BITS, 2>::kFixedLdsBytes + table_bytes(a, 64) : Geometry<BITS, 1>::kFixedLdsBytes + table_bytes(a, 32);
+    return row_groups(a) == 2 && !a.exact_weights ? Geometry<BITS, 2>::kFixedLdsBytes + table_bytes(a, 64) : Geometry<BITS, 1>::kFixedLdsBytes + table_bytes(a, 32);
 }
 
 }  // namespace qmf

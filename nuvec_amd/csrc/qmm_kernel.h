@@ -86,14 +86,6 @@ struct Geometry {
 __device__ __forceinline__ int swizzle(int row) { return (row >> 1) & 7; }
 __device__ __forceinline__ int lds_offset(int row, int chunk) { return row * kRowBytes + ((chunk ^ swizzle(row)) << 4); }
 
-// Low / high 16 bits of a table entry as element-type values.
-template <typename T> __device__ __forceinline__ float half_lo(uint32_t p);
-template <typename T> __device__ __forceinline__ float half_hi(uint32_t p);
-template <> __device__ __forceinline__ float half_lo<bf16_t>(uint32_t p) { return u2f(p << 16); }
-template <> __device__ __forceinline__ float half_hi<bf16_t>(uint32_t p) { return u2f(p & 0xFFFF0000u); }
-template <> __device__ __forceinline__ float half_lo<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[0]; }
-template <> __device__ __forceinline__ float half_hi<f16_t>(uint32_t p) { return (float)__builtin_bit_cast(f16x2v_t, p)[1]; }
-
 // DWORDS x 4 bytes per lane from global memory straight into LDS: lane l of the wavefront reads base + offset
 // (a wavefront-uniform base, so the per-step address arithmetic is scalar) and writes lds_base + 16 l (4 l for
 // a single dword).  Issued as assembly so that the compiler keeps no account of it: the waits are placed by hand
@@ -127,7 +119,7 @@ __device__ __forceinline__ void pin() { __builtin_amdgcn_sched_barrier(0); }
 __device__ __forceinline__ void keep(const uint4 &v) { asm volatile("" : : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w)); }
 
 // Dword D (two elements) of piece KK of a lane's 32 codes: expand_piece, one register at a time.
-template <typename T, int BITS, int FP4, int KK, int D>
+template <typename T, int BITS, int FP4, int KK, int D, bool EXACT = false>
 __device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], float s, float b) {
     if constexpr (FP4 == kMxfp8) {
         return Ops<T>::template fp8_pair<(D & 1) != 0>(dw[2 * KK + D / 2], s);
@@ -138,14 +130,15 @@ __device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], flo
     } else if constexpr (BITS == 4) {
         const uint32_t word = dw[KK];
         const uint32_t even = opaque(word & 0x0F0F0F0Fu), odd = opaque((word >> 4) & 0x0F0F0F0Fu);
-        return Ops<T>::pack(__builtin_fmaf(ubyte_to_float<D>(even), s, b), __builtin_fmaf(ubyte_to_float<D>(odd), s, b));
+        return affine_pair<T, EXACT>(ubyte_to_float<D>(even), ubyte_to_float<D>(odd), s, b);
     } else {
         constexpr int J = 8 * KK + 2 * D;
-        return Ops<T>::pack(__builtin_fmaf(code_to_float<BITS, J>(dw), s, b), __builtin_fmaf(code_to_float<BITS, J + 1>(dw), s, b));
+        return affine_pair<T, EXACT>(code_to_float<BITS, J>(dw), code_to_float<BITS, J + 1>(dw), s, b);
     }
 }
 
-template <typename T, int BITS, int FP4, bool BATCHED, class TL>
+// EXACT (affine codes): the weights as nuvec's CPU product holds them (affine_pair).
+template <typename T, int BITS, int FP4, bool BATCHED, class TL, bool EXACT = false>
 __global__ void __launch_bounds__(TL::kThreads) __attribute__((amdgpu_waves_per_eu(TL::kWavesPerSimd, TL::kWavesPerSimd)))
 qmm_kernel(const ProductArgs a) {
     using G = Geometry<BITS, TL>;
@@ -333,7 +326,7 @@ qmm_kernel(const ProductArgs a) {
         } else {
             constexpr int j = index / 4, d = index % 4;
             if constexpr (KK == 0 && d == 0) convert_scales(j);
-            const uint32_t v = expand_dword<T, BITS, FP4, KK, d>(raw[j], sc[j][KK >> 1], bi[j]);
+            const uint32_t v = expand_dword<T, BITS, FP4, KK, d, EXACT>(raw[j], sc[j][KK >> 1], bi[j]);
             if constexpr (d == 0) bf[KK & 1][j].x = v;
             else if constexpr (d == 1) bf[KK & 1][j].y = v;
             else if constexpr (d == 2) bf[KK & 1][j].z = v;
@@ -477,7 +470,9 @@ inline double estimate_us(const ProductArgs &a, int cus) {
     const double tiles = (double)((a.m + TL::BM - 1) / TL::BM) * (double)((a.n + TL::BN - 1) / TL::BN) * (double)a.batch;
     return tiles_us<TL>(tiles, (double)(a.k / BK), cus);
 }
-inline bool small_tile_is_faster(const ProductArgs &a, int cus) { return estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus); }
+inline bool small_tile_is_faster(const ProductArgs &a, int cus) {
+    return a.exact_weights || estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus);
+}
 
 // How many ways a single product splits K over the grid, by estimate: the splits fill the chip's block slots
 // with its (few) tiles, and cost a second kernel that reads their float32 partial sums (about 3 us to launch and
@@ -508,12 +503,12 @@ inline int k_splits(const ProductArgs &a, int cus, int *steps_per_split = nullpt
     return best;
 }
 
-template <typename T, int BITS, int FP4, class TL>
+template <typename T, int BITS, int FP4, class TL, bool EXACT = false>
 int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     using G = Geometry<BITS, TL>;
     static std::atomic<bool> configured[2] = {false, false};
     const bool batched = a.batch > 1;
-    auto kernel = batched ? qmm_kernel<T, BITS, FP4, true, TL> : qmm_kernel<T, BITS, FP4, false, TL>;
+    auto kernel = batched ? qmm_kernel<T, BITS, FP4, true, TL, EXACT> : qmm_kernel<T, BITS, FP4, false, TL, EXACT>;
     if (!configured[batched]) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes));
         configured[batched] = true;
@@ -536,6 +531,8 @@ int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
 
 template <typename T, int BITS, int FP4>
 int32_t run(const ProductArgs &a, void *workspace, hipStream_t s) {
+    if constexpr (FP4 == kAffine)
+        if (a.exact_weights) return run_tile<T, BITS, FP4, SmallTile, true>(a, workspace, s);  // (rows of few outputs: the small tile)
     return small_tile_is_faster(a, compute_units()) ? run_tile<T, BITS, FP4, SmallTile>(a, workspace, s)
                                                     : run_tile<T, BITS, FP4, BigTile>(a, workspace, s);
 }

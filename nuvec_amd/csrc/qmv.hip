@@ -90,7 +90,9 @@ __device__ __forceinline__ uint32_t code_at(const uint32_t (&d)[BITS], int i) {
 // float32.  Every load of a step is issued before the first use.  MODE: NVQ_AFFINE, or NVQ_MXFP4 /
 // NVQ_MXFP8 / NVQ_NVFP4 (E2M1 or E4M3 values; E8M0 scales per 32 or E4M3 scales per 16 values, a lane's
 // slice then spanning two groups).
-template <typename T, int BITS, int MODE, int RM>
+// EXACT (affine codes, 16-bit elements): every weight is materialised as nuvec's CPU product holds it, round(round(code *
+// scale) + bias) in the element type (kernels.rs:835-859), instead of the factored float32 form.
+template <typename T, int BITS, int MODE, int RM, bool EXACT = false>
 __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
     constexpr int kBlockWaves = 8;
     constexpr int kPer = 4;  // values of one x row per thread and step: 2048 / 512
@@ -166,6 +168,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
         }
         return st;
     };
+    constexpr bool exact = EXACT;
     float inv_enc = 1.0f;
     bool scaled = false;
     if constexpr (MODE == NVQ_NVFP4) {
@@ -219,6 +222,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
             for (int j = 0; j < 4; j++) {
                 const uint32_t c = code_at<BITS>(d, 4 * p + j);
                 v[j] = kAffine ? (float)c : (MODE == NVQ_MXFP8 ? e4m3_to_f32(c) : e2m1_to_f32(c));
+                if constexpr (exact) v[j] = Elem<T>::add(Elem<T>::mul(v[j], sc[0]), bi);  // the weight as the CPU holds it
             }
 #pragma unroll
             for (int i = 0; i < RM; i++) {
@@ -234,7 +238,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 #pragma unroll
         for (int i = 0; i < RM; i++) {
             if constexpr (kAffine) {
-                acc[i] = __builtin_fmaf(sc[0], dot[i][0], __builtin_fmaf(bi, x_sums[i][lane], acc[i]));
+                acc[i] = exact ? acc[i] + dot[i][0] : __builtin_fmaf(sc[0], dot[i][0], __builtin_fmaf(bi, x_sums[i][lane], acc[i]));
             } else {
 #pragma unroll
                 for (int hf = 0; hf < kHalves; hf++) acc[i] = __builtin_fmaf(sc[hf], dot[i][hf], acc[i]);
@@ -835,7 +839,7 @@ inline int d16_waves(int64_t k) {
 // Three rows and more: always.  Two rows: not for 2048 < K <= 4096 with fewer than 8192 weight rows.  One row: only
 // where the vector kernel's steps of 4096 values fit K badly (K <= 2048, 4096 < K <= 6144).
 inline bool d16_takes(const ProductArgs &a) {
-    if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64) return false;
+    if (a.mode != NVQ_AFFINE || a.bits != 4 || a.dtype == NVQ_F32 || a.group != 64 || a.exact_weights) return false;
     if (a.k % kD16Slice != 0 || a.k < 2 * kD16Slice || (a.k > 16 * kD16Slice && d16_waves(a.k) < 7)) return false;
     if (a.m < 1 || a.m > 8 || (a.k > 16 * kD16Slice && a.m < 3)) return false;
     if (a.m == 2 && a.k > 2048 && a.k <= 4096 && a.n < 8192) return false;
@@ -917,11 +921,16 @@ int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
 template <typename T, int BITS, int MODE>
 int32_t run_general(const ProductArgs &a, hipStream_t s) {
     const unsigned gx = (unsigned)((a.n + 7) / 8);
-    if (a.m == 1) {
-        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 1>), dim3(gx, 1, (unsigned)a.batch), dim3(512), 0, s, a);
-    } else {  // passes of four rows over grid.y
-        if ((a.m + 3) / 4 > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld rows exceed the grid limit", (long long)a.m);
-        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 4>), dim3(gx, (unsigned)((a.m + 3) / 4), (unsigned)a.batch), dim3(512), 0, s, a);
+    constexpr bool kCanBeExact = MODE == NVQ_AFFINE && !std::is_same<T, float>::value;
+    if ((a.m + 3) / 4 > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld rows exceed the grid limit", (long long)a.m);
+    const dim3 grid(gx, a.m == 1 ? 1u : (unsigned)((a.m + 3) / 4), (unsigned)a.batch);  // one row, or passes of four rows over grid.y
+    if (kCanBeExact && a.exact_weights) {
+        if (a.m == 1) hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 1, kCanBeExact>), grid, dim3(512), 0, s, a);
+        else hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 4, kCanBeExact>), grid, dim3(512), 0, s, a);
+    } else if (a.m == 1) {
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 1>), grid, dim3(512), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((qmv_lds_kernel<T, BITS, MODE, 4>), grid, dim3(512), 0, s, a);
     }
     NVQ_LAUNCH_CHECK("qmv");
     return NVQ_OK;
@@ -933,7 +942,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
     if (a.mode == NVQ_MXFP8) return run_general<T, 8, NVQ_MXFP8>(a, s);
     if (a.mode == NVQ_NVFP4) return run_general<T, 4, NVQ_NVFP4>(a, s);
     if constexpr (!std::is_same<T, float>::value) {
-        if (a.bits == 4) {
+        if (a.bits == 4 && !a.exact_weights) {  // (the decode kernels never materialise a weight)
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
             // 10.4 us at one row).
@@ -967,7 +976,7 @@ bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); 
 
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
-    if (a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32) {
+    if (a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32 && !a.exact_weights) {
         if (!a.row_exact && d16_takes(a)) return "qmv4_mm16_kernel";
         if (!a.row_exact && a.m >= 4 && mfma_decode_takes<4>(a)) return "qmv4_mfma_kernel";
         return "qmv4_lds_kernel";

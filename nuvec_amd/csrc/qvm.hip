@@ -95,6 +95,7 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
     const int64_t s_at = o.s + (nc >> gshift);
     const int per = (K + splits - 1) / splits;
     const int k_begin = blockIdx.y * per, k_end = k_begin + per < K ? k_begin + per : K;
+    const bool exact = kAffine && a.exact_weights != 0;  // (the same for the whole launch)
 
     float acc[RM][32], accb[RM];
 #pragma unroll
@@ -144,13 +145,15 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
 #pragma unroll
                     for (int i = 0; i < RM; i++) {
 #pragma unroll
-                        for (int hf = 0; hf < kHalves; hf++) xs[i][hf] = r.x[i] * r.s[hf];
-                        accb[i] = __builtin_fmaf(r.x[i], r.b, accb[i]);
+                        for (int hf = 0; hf < kHalves; hf++) xs[i][hf] = exact ? r.x[i] : r.x[i] * r.s[hf];
+                        if (!exact) accb[i] = __builtin_fmaf(r.x[i], r.b, accb[i]);
                     }
 #pragma unroll
                     for (int j = 0; j < 32; j++) {
                         const uint32_t c = code_at<BITS>(r.d, j);
-                        const float v = kAffine ? (float)c : (MODE == NVQ_MXFP8 ? e4m3_to_f32(c) : e2m1_to_f32(c));
+                        float v = kAffine ? (float)c : (MODE == NVQ_MXFP8 ? e4m3_to_f32(c) : e2m1_to_f32(c));
+                        if constexpr (kAffine)
+                            if (exact) v = Elem<T>::add(Elem<T>::mul(v, r.s[0]), r.b);  // the weight as the CPU holds it (kernels.rs:835-859)
 #pragma unroll
                         for (int i = 0; i < RM; i++) acc[i][j] = __builtin_fmaf(xs[i][j * kHalves / 32], v, acc[i][j]);
                     }
@@ -232,7 +235,8 @@ __device__ __forceinline__ void load_run(const unsigned char *p, uint32_t (&d)[B
     }
 }
 
-template <typename T, int BITS, int FP4>
+// EXACT (affine codes): the weights as nuvec's CPU product holds them (qmf::affine_pair).
+template <typename T, int BITS, int FP4, bool EXACT>
 __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, int splits, float *partial) {
     using S = std::conditional_t<FP4 != 0, uint8_t, T>;  // stored scale type
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kStageBytes];
@@ -306,7 +310,7 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
         if constexpr (FP4 == kNvfp4) scale = ftz(e4m3_to_f32(sv));
         else if constexpr (FP4) scale = ftz(e8m0_to_f32(sv));
         else scale = Elem<T>::load(&sv, 0), bias = Elem<T>::load(&bv, 0);
-        return expand_piece<T, BITS, FP4, 0>(r.w[i], scale, bias);
+        return expand_piece<T, BITS, FP4, 0, EXACT>(r.w[i], scale, bias);
     };
     // The four expanded rows turned (columns 2 d: the words' low halves, 2 d + 1: the high halves; rows (0, 1) and (2, 3)
     // as two words each) and written to a stage together with the thread's pieces of x.
@@ -445,7 +449,8 @@ int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
     const int splits = workspace != nullptr ? splits_of(a) : 1;  // without a workspace K is not split
     const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN);
     const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)a.batch, (unsigned)splits);
-    hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4>), grid, dim3(kThreads), 0, s, a, splits, workspace);
+    if (FP4 == kAffine && a.exact_weights) hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, FP4 == kAffine>), grid, dim3(kThreads), 0, s, a, splits, workspace);
+    else hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, false>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     NVQ_LAUNCH_CHECK("qmn");
     if (splits > 1) {
         const int64_t per_batch = a.m * a.n, total = a.batch * per_batch;

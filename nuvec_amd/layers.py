@@ -155,7 +155,12 @@ class SwitchGlu:
         g, u = self.gate_proj, self.up_proj
         if g.quant != u.quant or g.weight.shape != u.weight.shape or (g.bias is None) != (u.bias is None):
             raise ops.InvalidArgument("fuse_gate_up: the gate and up projections differ in shape or quantization")
-        self.gate_up_paired = g.weight.shape[1] % 64 == 0
+        hidden = g.weight.shape[1]
+        if g.quant.mode == ops.QuantMode.AFFINE and 512 <= hidden < 1024:
+            # Affine products of fewer than 1024 outputs per row materialise the CPU's doubly rounded weights: one product
+            # of 2 * hidden rows would not, the two of `hidden` rows do.  Such projections stay apart.
+            return self
+        self.gate_up_paired = hidden % 64 == 0
         if self.gate_up_paired:
             cat = lambda a, b: None if a is None else ops.pair_rows(a, b, 1)
         else:

@@ -49,8 +49,9 @@ def test_routes_of_the_baseline_configurations():
         assert ops.quantized_matmul_route(m, n, k, nv.Quant.affine(group, bits), bf16) == "qmf_kernel", (m, n, k, group, bits)
 
 
-SHAPES = [(2, 200, 512), (9, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (11, 48, 14336), (23, 64, 1536), (16, 5000, 512),
-          (12, 40, 7168), (77, 300, 2048), (130, 48, 512)]
+# (rows of 1024 outputs or more: affine products of shorter rows take the kernels that materialise the CPU's weights)
+SHAPES = [(2, 1224, 512), (9, 2024, 1024), (16, 1154, 4096), (13, 1120, 8192), (11, 1072, 14336), (23, 1088, 1536), (16, 5000, 512),
+          (12, 1064, 7168), (77, 1324, 2048), (130, 1072, 512)]
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
@@ -72,15 +73,15 @@ def test_direct_few_row_kernel_every_width(dtype, bits, group):
         got = to_host(nv.quantized_matmul(to_dev(x), q))
         what = f"direct few rows b{bits} g{group} M={m} N={n} K={k}"
         assert_rows_close(got, want, dtype, what)
-        if m <= 32:  # (half the bar leaves no room for one rounding step of the largest outputs: not over thousands of short rows)
-            assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what)
+        if m <= 32:  # (one rounding step of a row's largest output is up to 0.78 x the bar: the float32 sums differ in order)
+            assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what, limit=0.8)
 
 
 @pytest.mark.parametrize("bits,group", [(3, 64), (8, 32), (4, 128)])
 def test_direct_few_row_kernel_batched_with_bias(bits, group):
     """A batch of weight matrices (one stride per operand) and the layer's bias in the epilogue."""
     rng = np.random.default_rng(4100 + bits)
-    b, m, n, k = 3, 10, 96, 1024
+    b, m, n, k = 3, 10, 1120, 1024
     quant = nv.Quant.affine(group, bits)
     assert ops.quantized_matmul_route(m, n, k, quant, torch.bfloat16, batch=b) == "qmd_kernel"
     w, x = make_w(rng, b * n, k, ref.BF16), make_x(rng, b * m, k, ref.BF16)
@@ -113,7 +114,7 @@ def test_direct_few_row_kernel_batched_with_bias(bits, group):
 def test_direct_few_row_kernel_per_pair_gather():
     """gather_qmm without offsets: one product per pair on the same kernel (pairs over grid z)."""
     rng = np.random.default_rng(4200)
-    experts, n, k, m, pairs = 5, 80, 1024, 6, 7
+    experts, n, k, m, pairs = 5, 1104, 1024, 6, 7
     w = make_w(rng, experts * n, k, ref.BF16)
     packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 3)
     q = nv.Quantized(to_dev(packed.reshape(experts, n, -1)), to_dev(scales.reshape(experts, n, -1)),

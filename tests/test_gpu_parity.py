@@ -63,30 +63,27 @@ def record_ratio(what, worst, count):
 
 
 def assert_rows_close(got, want, dtype, what, exact_weights=False):
-    """Against the CPU oracle: every output within the bar of its row (1e-2 * max|row| for bfloat16).
-
-    The one exception, recorded with its ratio like every case: half-precision affine products whose rows hold fewer
-    than 512 outputs.  The bar scales with the largest of a row's outputs, about four standard deviations of an output
-    in a row of thousands (the BASELINE shapes) but only two in a row of 32; the difference between the device's single
-    rounding of a dequantized weight and the CPU's two has a standard deviation of 0.14 x the bar at the BASELINE shapes
-    and twice that in such short rows, so their worst output is allowed 1.5 x the bar.  `exact_weights` (block formats,
-    whose weights both sides hold exactly) takes the exception away."""
+    """Against the CPU oracle: every output within the bar of its row (1e-2 * max|row| for bfloat16), whatever the
+    length of the row.  (Half-precision affine products of fewer than 1024 outputs per row, whose bar is tightest, run
+    on kernels that materialise the CPU's doubly rounded weights; `exact_weights` marks the block formats, whose weights
+    both sides hold exactly.)"""
     ratio = _excess(got, want, dtype)
     worst = float(np.max(ratio)) if ratio.size else 0.0
     record_ratio(what, worst, ratio.size)
     beyond = int(np.count_nonzero(ratio > 1.0))
-    columns = np.asarray(want).shape[-1]
-    limit = 1.5 if dtype != ref.F32 and columns < 512 and not exact_weights else 1.0
-    assert worst <= limit, f"{what}: max error is {worst:.3f} x the bound, {beyond} of {ratio.size} outputs beyond it"
+    assert worst <= 1.0, f"{what}: max error is {worst:.3f} x the bound, {beyond} of {ratio.size} outputs beyond it"
 
 
-def assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what):
-    """Against the device-arithmetic oracle: every output within half the bar.  The reference's device
-    kernels come in two forms (weights rounded once in the tiled kernels, never in the vector kernels); which
-    one a product takes here is a routing matter, so either is accepted."""
-    worst = min(float(np.max(_excess(got, ref.quantized_matmul_device(x, packed, scales, biases, group=group, bits=bits, dtype=dtype,
-                                                                       rounded_weights=r), dtype))) for r in (True, False))
-    assert worst <= 0.5, f"{what}: max error against the device arithmetic is {worst:.3f} x the bound"
+def assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, what, limit=0.5):
+    """Against the arithmetic of the kernel that ran: every output within half the bar.  The reference's device
+    kernels come in two forms (weights rounded once in the tiled kernels, never in the vector kernels); which one a
+    product takes here is a routing matter, so either is accepted, and rows of fewer than 1024 outputs take the
+    CPU's own weights (two roundings), i.e. the CPU oracle itself."""
+    forms = [ref.quantized_matmul_device(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, rounded_weights=r) for r in (True, False)]
+    if np.asarray(got).shape[-1] < 1024:
+        forms = [ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, threads=8)]
+    worst = min(float(np.max(_excess(got, form, dtype))) for form in forms)
+    assert worst <= limit, f"{what}: max error against the device arithmetic is {worst:.3f} x the bound"
 
 
 @pytest.mark.parametrize("dtype", [ref.F32, ref.BF16, ref.F16])
@@ -296,6 +293,46 @@ def test_sorted_offsets_and_gather_pairs():
                           bits=4, dtype=ref.BF16)
     assert got.shape == (rows, 1, n)
     assert_rows_close(got, want, ref.BF16, "sorted gather", exact_weights=True)
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_rows_of_few_outputs_take_the_cpu_weights(dtype):
+    """Half-precision affine products of fewer than 1024 outputs per row, on every kernel that serves them (few rows and
+    tiles on the matrix cores, the general vector kernel, both kernels of the [K, N] storage, gathered pairs): the
+    weights are the CPU's doubly rounded ones (kernels.rs:835-859), so the outputs differ from the CPU product only by
+    the order of the float32 sums: nearly all agree bit for bit, none is off by more than one rounding step (which is up to
+    0.78 x the bar for a row's largest output)."""
+    rng = np.random.default_rng(8800 + dtype)
+    tdtype = TORCH[dtype]
+    cases = [(5, 200, 1024, 4, 64, True, "qmf_kernel"), (1, 100, 4096, 4, 64, True, "qmv_lds_kernel"), (3, 64, 480, 8, 32, True, "qmv_lds_kernel"),
+             (2048, 768, 512, 4, 64, True, "qmm_kernel"), (300, 640, 1024, 4, 64, True, None), (260, 257, 192, 3, 64, True, None), (16, 48, 1536, 8, 128, True, "qmf_kernel"),
+             (40, 384, 256, 4, 64, False, "qmn_kernel"), (130, 992, 192, 8, 32, False, "qmn_kernel"), (7, 256, 200, 4, 64, False, "qvm_kernel"),
+             (9, 128, 320, 6, 64, False, "qvm_kernel")]
+    for m, n, k, bits, group, transpose, kernel in cases:
+        w = make_w(rng, n, k, dtype) if transpose else make_w(rng, k, n, dtype)
+        x = make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
+        if kernel is not None:
+            assert nv.quantized_matmul_route(m, n, k, q.quant, tdtype, transpose=transpose) == kernel
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, transpose=transpose, threads=8)
+        for rows_flag in (False, True):
+            got = to_host(nv.quantized_matmul(to_dev(x), q, transpose=transpose, rows=rows_flag))
+            what = f"CPU weights b{bits} g{group} M={m} N={n} K={k} transpose={transpose} rows={rows_flag}"
+            worst = float(np.max(_excess(got, want, dtype)))
+            record_ratio(what, worst, got.size)
+            differ = np.count_nonzero(got.view(np.uint16) != want.view(np.uint16))
+            assert worst <= 0.8 and differ <= max(2, got.size // 50), f"{what}: {worst:.3f} x the bar, {differ} of {got.size} outputs differ"
+    # gathered pairs: one product per pair
+    experts, n, k, m, pairs = 4, 96, 512, 3, 6
+    w = make_w(rng, experts * n, k, dtype).reshape(experts, n, k)
+    packed, scales, biases = ref.affine_quantize(w, dtype, 64, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+    x = make_x(rng, pairs * m, k, dtype).reshape(pairs, m, k)
+    rhs = rng.integers(0, experts, pairs)
+    got = to_host(nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs).cuda()))
+    want = ref.gather_qmm(x, packed, scales, biases, np.arange(pairs, dtype=np.uint32), rhs.astype(np.uint32), group=64, bits=4, dtype=dtype)
+    assert float(np.max(_excess(got.reshape(pairs * m, n), want.reshape(pairs * m, n), dtype))) <= 0.8
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
@@ -815,7 +852,7 @@ def test_linear_bias_in_the_product_epilogues(dtype):
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("group,k,n", [(64, 2048, 100), (128, 4096, 96), (64, 6144, 33), (128, 10240, 64)])
+@pytest.mark.parametrize("group,k,n", [(64, 2048, 1124), (128, 4096, 1120), (64, 6144, 1057), (128, 10240, 1088)])
 def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
     """Four rows of x at 4 bits, K a multiple of 2048 (the matrix-core decode kernel): N not a multiple of its 32
     weight rows, K beyond one staging round, both group sizes it takes, and a batch of products."""
@@ -841,8 +878,8 @@ def test_four_row_decode_on_matrix_cores(dtype, group, k, n):
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("m,n,k", [(2, 100, 4096), (3, 33, 4096), (4, 64, 4096), (5, 47, 4096), (8, 130, 4096), (2, 40, 1024), (7, 33, 1536),
-                                   (4, 50, 8192), (8, 20, 8192), (6, 36, 3584), (1, 70, 1024), (1, 33, 2048), (1, 24, 5120), (4, 40, 14336), (8, 17, 12288), (3, 20, 28672)])
+@pytest.mark.parametrize("m,n,k", [(2, 1124, 4096), (3, 1057, 4096), (4, 1088, 4096), (5, 1071, 4096), (8, 1154, 4096), (2, 1064, 1024), (7, 1057, 1536),
+                                   (4, 1074, 8192), (8, 1044, 8192), (6, 1060, 3584), (1, 1094, 1024), (1, 1057, 2048), (1, 1048, 5120), (4, 1064, 14336), (8, 1041, 12288), (3, 1044, 28672)])
 def test_decode_rows_on_16x16x32(dtype, m, n, k):
     """One to eight rows of x at 4 bits, groups of 64, K a multiple of 512 up to 8192 (the 16x16x32 matrix-core decode
     kernel, a wavefront per 512 values, chunks of K beyond 8192): every tile-row layout (rows of x times groups), the smallest and the largest
@@ -1064,7 +1101,7 @@ def test_grouped_gather_with_the_gated_epilogue(quant, activation):
     the two grouped products (`nvq_gather_qmm`) followed by `nvq_glu`; experts without rows, with one pass of one tile
     (up to 32 rows), of two tiles (up to 64) and with several passes; with and without the experts' biases."""
     rng = np.random.default_rng(7700 + len(quant) + len(activation))
-    experts, k, hidden = 7, 320, 192
+    experts, k, hidden = 7, 320, (1024 if quant.startswith("affine") else 192)  # (affine projections below 1024 rows stay apart)
     q_of = {"MXFP4": nv.Quant.new(nv.QuantMode.MXFP4), "NVFP4": nv.Quant.new(nv.QuantMode.NVFP4), "affine4": nv.Quant.affine(64, 4),
             "affine8": nv.Quant.affine(32, 8)}[quant]
     for dtype in (ref.BF16, ref.F16):
@@ -1090,7 +1127,7 @@ def test_grouped_gather_with_the_gated_epilogue(quant, activation):
                                     expert_bias=nv.pair_rows(gb, ub, 1) if biased else None)
             assert tuple(got.shape) == (pairs, hidden)
             assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"{quant} {activation} dtype {dtype} biased {biased}"
-    with pytest.raises(nv.Unsupported):  # rows not in whole runs of 64
+    with pytest.raises(nv.Unsupported):  # rows not in whole runs of 64 (affine: also fewer than 1024 rows each)
         nv.gather_qmm_glu(x, nv.Quantized(both.weight[:, :320], both.scales[:, :320], None if both.biases is None else both.biases[:, :320], q_of),
                           rows, sorted_ids, offsets, activation)
     with pytest.raises(nv.InvalidArgument):
