@@ -98,8 +98,8 @@ def test_sorted_few_row_gathers_keep_the_one_row_bits(dtype, bits):
 
 def determinism_cases():
     """One product per route (determinism.rs:47-88 for this path): decode, few rows on both matrix-core kernels, tiled
-    with and without a split of K, weights stored [K, N], batched, the general kernel's modes, grouped and per-pair
-    gathers, quantize and dequantize."""
+    with and without a split of K, weights stored [K, N] (both kernels), rows of few outputs, the general kernel's
+    modes, grouped and per-pair gathers, the gated activation, quantize and dequantize."""
     rng = np.random.default_rng(123)
     w = make_w(rng, 4096, 4096, ref.BF16)
     wd = to_dev(w)
@@ -132,6 +132,19 @@ def determinism_cases():
         if mode == "NVFP4":
             em = nv.Quantized(em.weight, em.scales, None, em.quant, torch.full((16,), 0.5, device="cuda"))
         cases[f"{mode} grouped gather"] = lambda em=em: nv.gather_qmm(xe, em, None, ids, nv.GatherQmm(sorted_indices=True))
+    # weights stored [K, N] on the matrix cores (K split through the workspace, and not), rows of few outputs on the
+    # exact-weights kernels, the gated activation alone and as the grouped product's epilogue
+    cases["b4 untransposed M=300"] = lambda: nv.quantized_matmul(x512[:300], q4, transpose=False)
+    cases["b4 untransposed M=300 unsplit"] = lambda: nv.quantized_matmul(x512[:300], q4, transpose=False, scratch=False)
+    qs = nv.quantize(wd[:256], nv.Quant.affine(64, 4))
+    for rows in (1, 5, 512):
+        cases[f"b4 N=256 M={rows}"] = lambda rows=rows: nv.quantized_matmul(x512[:rows], qs)
+    cases["glu"] = lambda: nv.glu(x512[:, :2048], x512[:, 2048:], "swiglu_oai")
+    eg = nv.quantize(experts, nv.QuantMode.MXFP4)
+    paired = nv.Quantized(nv.pair_rows(eg.weight[:, :256], eg.weight[:, 256:], 1), nv.pair_rows(eg.scales[:, :256], eg.scales[:, 256:], 1), None, eg.quant)
+    offsets = nv.sorted_offsets(ids.to(torch.int32), 16)
+    tokens = torch.arange(512, device="cuda", dtype=torch.int32)
+    cases["grouped gather with the gated epilogue"] = lambda: nv.gather_qmm_glu(xe.reshape(512, 1024), paired, tokens, ids.to(torch.int32), offsets, "swiglu")
     cases["quantize b4"] = lambda: nv.quantize(wd, nv.Quant.affine(64, 4)).weight
     cases["quantize mxfp4"] = lambda: nv.quantize(wd, nv.QuantMode.MXFP4).weight
     cases["dequantize b4"] = lambda: nv.dequantize(q4)
