@@ -432,9 +432,6 @@ int32_t run_qmd_sized(const ProductArgs &a, hipStream_t s) {
             const double cost = (double)((blocks + slots - 1) / slots) * (2.5 + 1.5 * t);
             if (t == 1 || cost < best) best = cost, tiles = t;
         }
-#ifdef QMD_LAB
-        if (const char *e = getenv("NVQ_LAB_TILES")) tiles = atoi(e);
-#endif
     }
     const dim3 grid((unsigned)((groups + tiles - 1) / tiles), (unsigned)passes, (unsigned)a.batch);
     void (*kernel)(const ProductArgs, int);
