@@ -193,8 +193,8 @@ __global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T
 
 
 // ---- Many rows of x: the same product on the matrix cores ---------------------------------------------------------
-// A block of four wavefronts (2 x 2, each 64 x 64 of y as 2 x 2 tiles of the 32x32x16 instruction) owns 128 x 128 of
-// y and walks K in steps of 64 rows of w through two LDS stages, one barrier per step, two blocks per compute unit.
+// A block of four wavefronts (2 x 2, each 64 x 64 of y as 2 x 2 tiles of the 32x32x16 instruction; for up to 32 rows of
+// x 1 x 4 wavefronts of one tile each, see Shape) owns 128 x 128 of y and walks K in steps of 64 rows of w through two LDS stages, one barrier per step, two blocks per compute unit.
 // The matrix instruction wants eight consecutive k per lane and column, the storage gives eight consecutive columns
 // per row and word, so the weights are turned on the way into LDS: thread (q = t / 16, c = t % 16) loads the codes of
 // columns 8 c .. 8 c + 7 of rows 4 q .. 4 q + 3 of the step (one word per row at 4 bits: sixteen lanes cover the
@@ -213,8 +213,22 @@ namespace qmn {
 
 using namespace qmf;
 
-constexpr int BM = 128, BN = 128, BK = 64, kThreads = 256;
-constexpr int kXBytes = BM * BK * 2, kWBytes = BN * BK * 2, kStageBytes = kXBytes + kWBytes;
+constexpr int BN = 128, BK = 64, kThreads = 256;
+constexpr int kWBytes = BN * BK * 2;
+
+// The four wavefronts of a block as WM x (4 / WM), each TI x TJ tiles of 32 x 32: 128 x 128 of y per block (two blocks
+// per compute unit), or 32 x 128 for up to 32 rows of x (one tile per wavefront, four blocks per compute unit, all of
+// a step's operands read at once).
+template <int WM_, int TI_, int TJ_, int BLOCKS_>
+struct Shape {
+    static constexpr int WM = WM_, WN = 4 / WM_, TI = TI_, TJ = TJ_, kBlocksPerCu = BLOCKS_;
+    static constexpr int BM = WM * TI * 32;
+    static constexpr int kXParts = BM * 8 / kThreads;  // 16-byte pieces of a step of x per thread
+    static constexpr int kXBytes = BM * BK * 2, kStageBytes = kXBytes + kWBytes;
+    static_assert(WN * TJ * 32 == BN && kXParts * kThreads == BM * 8, "the loading assignment below assumes these");
+};
+using Tile128 = Shape<2, 2, 2, 2>;
+using Tile32 = Shape<1, 1, 1, 4>;
 
 __device__ __forceinline__ int x_slot(int row, int ch) { return (row * 8 + (ch ^ ((row >> 1) & 7))) * 16; }
 __device__ __forceinline__ int w_slot(int n, int ch) { return (((n >> 4) * 8 + ch) * 16 + ((n + (n >> 4) + 2 * (ch & 4)) & 15)) * 16; }
@@ -236,12 +250,13 @@ __device__ __forceinline__ void load_run(const unsigned char *p, uint32_t (&d)[B
 }
 
 // EXACT (affine codes): the weights as nuvec's CPU product holds them (qmf::affine_pair).
-template <typename T, int BITS, int FP4, bool EXACT>
-__global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, int splits, float *partial) {
+template <typename T, int BITS, int FP4, bool EXACT, class TL>
+__global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const ProductArgs a, int splits, float *partial) {
     using S = std::conditional_t<FP4 != 0, uint8_t, T>;  // stored scale type
+    constexpr int BM = TL::BM, TI = TL::TI, TJ = TL::TJ, kXParts = TL::kXParts, kXBytes = TL::kXBytes, kStageBytes = TL::kStageBytes;
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kStageBytes];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1, h = lane >> 5, l32 = lane & 31;
+    const int wm = wave / TL::WN, wn = wave % TL::WN, h = lane >> 5, l32 = lane & 31;
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int ngroups = N >> gshift;
@@ -274,10 +289,10 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     for (int j = 0; j < 8; j++) wdst[j] = kXBytes + w_slot(8 * c + j, q >> 1) + 8 * (q & 1);
     // This thread's part of a step of x: 16-byte pieces t + 256 i (piece p: row p / 8, slot p % 8).
     const unsigned char *xbase = (const unsigned char *)(x + (int64_t)m0 * K);
-    uint32_t xoff[4];
-    int xdst[4];
+    uint32_t xoff[kXParts];
+    int xdst[kXParts];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < kXParts; i++) {
         const int p = tid + 256 * i, r = p >> 3, ch = p & 7;
         const int row = m0 + r < M ? r : M - 1 - m0;  // rows past M are computed, not stored
         xoff[i] = ((uint32_t)row * (uint32_t)K + 8u * ch) * 2u;
@@ -285,7 +300,7 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     }
 
     struct Regs {
-        u32x4_t x[4];
+        u32x4_t x[kXParts];
         uint32_t w[4][BITS];
         S s[4], b[4];
     };
@@ -293,7 +308,7 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
         const int64_t k0 = (int64_t)step * BK;
         const unsigned char *xs = xbase + k0 * 2;
 #pragma unroll
-        for (int i = 0; i < 4; i++) r.x[i] = *reinterpret_cast<const u32x4_t *>(xs + xoff[i]);
+        for (int i = 0; i < kXParts; i++) r.x[i] = *reinterpret_cast<const u32x4_t *>(xs + xoff[i]);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             load_run<BITS>(wbase + (k0 + i) * row_bytes + woff, r.w[i]);
@@ -317,7 +332,7 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     auto store = [&](int stage_at, const Regs &r, const uint4 &v0, const uint4 &v1, const uint4 &v2, const uint4 &v3) {
         unsigned char *stage = lds + stage_at * kStageBytes;
 #pragma unroll
-        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4_t *>(stage + xdst[i]) = r.x[i];
+        for (int i = 0; i < kXParts; i++) *reinterpret_cast<u32x4_t *>(stage + xdst[i]) = r.x[i];
         auto turn = [&](uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3, int even_at, int odd_at) {
             const uint2 even = {__builtin_amdgcn_perm(a1, a0, 0x05040100u), __builtin_amdgcn_perm(a3, a2, 0x05040100u)};
             const uint2 odd = {__builtin_amdgcn_perm(a1, a0, 0x07060302u), __builtin_amdgcn_perm(a3, a2, 0x07060302u)};
@@ -330,19 +345,18 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
         turn(v0.w, v1.w, v2.w, v3.w, wdst[6], wdst[7]);
     };
 
-    int xread[2], wread[2];  // of the first slot of the lane's half; the others are an XOR (x) or a constant (w) away
+    int xread[TI], wread[TJ];  // of the first slot of the lane's half; the others are an XOR (x) or a constant (w) away
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        xread[t] = (64 * wm + 32 * t + l32) * 128;
-        wread[t] = kXBytes + w_slot(64 * wn + 32 * t + l32, 4 * h);
-    }
+    for (int t = 0; t < TI; t++) xread[t] = (32 * TI * wm + 32 * t + l32) * 128;
+#pragma unroll
+    for (int t = 0; t < TJ; t++) wread[t] = kXBytes + w_slot(32 * TJ * wn + 32 * t + l32, 4 * h);
     const int xswz = ((l32 >> 1) & 7) ^ (4 * h);  // (the tile bases are multiples of 16 rows) slot s of the lane's half: s ^ xswz
 
-    floatx16_t acc[2][2];
+    floatx16_t acc[TI][TJ];
 #pragma unroll
-    for (int ti = 0; ti < 2; ti++)
+    for (int ti = 0; ti < TI; ti++)
 #pragma unroll
-        for (int tj = 0; tj < 2; tj++)
+        for (int tj = 0; tj < TJ; tj++)
 #pragma unroll
             for (int el = 0; el < 16; el++) acc[ti][tj][el] = 0.0f;
 
@@ -369,24 +383,31 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     auto step = [&](int stage_at, Regs &next, int refill) {
         const unsigned char *stage = lds + stage_at * kStageBytes;
         uint4 v[4];
+        // substep ks takes the eight k of slot ks for the lanes' lower half and of slot 4 + ks for the upper one (any
+        // order of k serves as long as x and w agree): the two halves then never meet in a bank
+        constexpr bool kAllAtOnce = TI * TJ == 1;  // one tile per wavefront: the registers hold the operands of all four substeps
+        uint4 xa[kAllAtOnce ? 4 : 1][TI], wb[kAllAtOnce ? 4 : 1][TJ];
+        auto fragments = [&](int ks) {
+#pragma unroll
+            for (int t = 0; t < TI; t++) xa[kAllAtOnce ? ks : 0][t] = *reinterpret_cast<const uint4 *>(stage + xread[t] + ((ks ^ xswz) << 4));
+#pragma unroll
+            for (int t = 0; t < TJ; t++) wb[kAllAtOnce ? ks : 0][t] = *reinterpret_cast<const uint4 *>(stage + wread[t] + ks * 256);
+        };
+        if constexpr (kAllAtOnce) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) fragments(ks);
+        }
         static_for<4>([&](auto ks_tag) {
             constexpr int ks = decltype(ks_tag)::value;
-            // substep ks takes the eight k of slot ks for the lanes' lower half and of slot 4 + ks for the upper one (any
-            // order of k serves as long as x and w agree): the two halves then never meet in a bank
-            uint4 xa[2], wb[2];
+            if constexpr (!kAllAtOnce) fragments(ks);
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                xa[t] = *reinterpret_cast<const uint4 *>(stage + xread[t] + ((ks ^ xswz) << 4));
-                wb[t] = *reinterpret_cast<const uint4 *>(stage + wread[t] + ks * 256);
-            }
+            for (int ti = 0; ti < TI; ti++)
 #pragma unroll
-            for (int ti = 0; ti < 2; ti++)
-#pragma unroll
-                for (int tj = 0; tj < 2; tj++) acc[ti][tj] = Ops<T>::mfma(xa[ti], wb[tj], acc[ti][tj]);
+                for (int tj = 0; tj < TJ; tj++) acc[ti][tj] = Ops<T>::mfma(xa[kAllAtOnce ? ks : 0][ti], wb[kAllAtOnce ? ks : 0][tj], acc[ti][tj]);
             v[ks] = row(next, ks_tag);
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+            if constexpr (!kAllAtOnce) __builtin_amdgcn_sched_group_barrier(0x100, TI + TJ, 0);
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < TI * TJ; i++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
             }
@@ -407,15 +428,15 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     float *part = partial + ((int64_t)blockIdx.y * splits + blockIdx.z) * M * N;  // (used with a split only)
     const bool biased = a.row_bias != nullptr;
 #pragma unroll
-    for (int tj = 0; tj < 2; tj++) {
-        const int col = n0 + 64 * wn + 32 * tj + l32;
+    for (int tj = 0; tj < TJ; tj++) {
+        const int col = n0 + 32 * TJ * wn + 32 * tj + l32;
         if (col >= N) continue;
         const float bias = biased && splits == 1 ? Elem<T>::load((const T *)a.row_bias, col) : 0.0f;
 #pragma unroll
-        for (int ti = 0; ti < 2; ti++)
+        for (int ti = 0; ti < TI; ti++)
 #pragma unroll
             for (int el = 0; el < 16; el++) {
-                const int m = m0 + 64 * wm + 32 * ti + 8 * (el >> 2) + 4 * h + (el & 3);
+                const int m = m0 + 32 * TI * wm + 32 * ti + 8 * (el >> 2) + 4 * h + (el & 3);
                 if (m >= M) continue;
                 const float v = acc[ti][tj][el];
                 if (splits > 1) part[(int64_t)m * N + col] = v;
@@ -424,33 +445,38 @@ __global__ void __launch_bounds__(kThreads, 2) qmn_kernel(const ProductArgs a, i
     }
 }
 
+inline bool few_rows(const ProductArgs &a) { return a.m <= Tile32::BM; }
+
 // Splits of K for a product whose tiles do not fill the chip: the split with the least estimated time, counted as
-// rounds of resident blocks (two per compute unit) x (3 us to start + 1.2 us per step of the longest split) plus,
-// with a split, the reduction's launch and its float32 traffic at 4 TB/s.
-inline int splits_of(const ProductArgs &a) {
-    const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
-    const int64_t resident = 2 * (int64_t)compute_units();
+// rounds of resident blocks x (3 us to start + 1.2 us per step of the longest split; 0.5 us per step of the 32-row
+// tile) plus, with a split, the reduction's launch and its float32 traffic at 4 TB/s.
+template <class TL>
+int splits_of_shape(const ProductArgs &a) {
+    const int64_t tiles = ((a.m + TL::BM - 1) / TL::BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
+    const int64_t resident = TL::kBlocksPerCu * (int64_t)compute_units();
     if (tiles >= resident || steps < 4) return 1;
+    const double step_us = TL::BM == 32 ? 0.5 : 1.2;
     double best = 0.0;
     int64_t pick = 1;
     for (int64_t splits = 1; splits <= steps / 2 && splits <= 64; splits++) {
         const int64_t per_split = (steps + splits - 1) / splits;
         if ((steps + per_split - 1) / per_split != splits) continue;  // (another count gives the same longest split)
         const int64_t rounds = (tiles * splits + resident - 1) / resident;
-        double us = (double)rounds * (3.0 + 1.2 * (double)per_split);
+        double us = (double)rounds * (3.0 + step_us * (double)per_split);
         if (splits > 1) us += 2.0 + (double)splits * (double)(a.batch * a.m * a.n) * 4.0 / 4.0e6;
         if (splits == 1 || us < best) best = us, pick = splits;
     }
     return (int)pick;
 }
+inline int splits_of(const ProductArgs &a) { return few_rows(a) ? splits_of_shape<Tile32>(a) : splits_of_shape<Tile128>(a); }
 
-template <typename T, int BITS, int FP4>
-int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
-    const int splits = workspace != nullptr ? splits_of(a) : 1;  // without a workspace K is not split
-    const int64_t tiles = ((a.m + BM - 1) / BM) * ((a.n + BN - 1) / BN);
+template <typename T, int BITS, int FP4, class TL>
+int32_t run_shape(const ProductArgs &a, float *workspace, hipStream_t s) {
+    const int splits = workspace != nullptr ? splits_of_shape<TL>(a) : 1;  // without a workspace K is not split
+    const int64_t tiles = ((a.m + TL::BM - 1) / TL::BM) * ((a.n + BN - 1) / BN);
     const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)a.batch, (unsigned)splits);
-    if (FP4 == kAffine && a.exact_weights) hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, FP4 == kAffine>), grid, dim3(kThreads), 0, s, a, splits, workspace);
-    else hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, false>), grid, dim3(kThreads), 0, s, a, splits, workspace);
+    if (FP4 == kAffine && a.exact_weights) hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, FP4 == kAffine, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
+    else hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, false, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     NVQ_LAUNCH_CHECK("qmn");
     if (splits > 1) {
         const int64_t per_batch = a.m * a.n, total = a.batch * per_batch;
@@ -459,6 +485,11 @@ int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
         NVQ_LAUNCH_CHECK("qvm_reduce");
     }
     return NVQ_OK;
+}
+
+template <typename T, int BITS, int FP4>
+int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
+    return few_rows(a) ? run_shape<T, BITS, FP4, Tile32>(a, workspace, s) : run_shape<T, BITS, FP4, Tile128>(a, workspace, s);
 }
 
 template <typename T>
