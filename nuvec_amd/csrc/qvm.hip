@@ -194,7 +194,8 @@ __global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T
 
 // ---- Many rows of x: the same product on the matrix cores ---------------------------------------------------------
 // A block of four wavefronts (2 x 2, each 64 x 64 of y as 2 x 2 tiles of the 32x32x16 instruction; for up to 32 rows of
-// x 1 x 4 wavefronts of one tile each, see Shape) owns 128 x 128 of y and walks K in steps of 64 rows of w through two LDS stages, one barrier per step, two blocks per compute unit.
+// x 1 x 4 wavefronts of one tile each, see Shape) owns 128 x 128 of y and walks K in steps of 64 rows of w through two
+// LDS stages, one barrier per step, two blocks per compute unit.
 // The matrix instruction wants eight consecutive k per lane and column, the storage gives eight consecutive columns
 // per row and word, so the weights are turned on the way into LDS: thread (q = t / 16, c = t % 16) loads the codes of
 // columns 8 c .. 8 c + 7 of rows 4 q .. 4 q + 3 of the step (one word per row at 4 bits: sixteen lanes cover the
