@@ -364,6 +364,7 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
     // This block's steps of K (all of them without a split), loaded two steps ahead into two sets of registers.
     const int all_steps = K / BK, per_split = (all_steps + splits - 1) / splits;
     const int first = (int)blockIdx.z * per_split, steps = all_steps - first < per_split ? all_steps - first : per_split;
+    if (steps <= 0) return;  // (the host gives every split a step; the whole block leaves, before any barrier)
     const int last = first + steps - 1;
     auto at = [&](int step) { return step < last ? step : last; };  // a step past the end loads the last one again
     using I0 = std::integral_constant<int, 0>;
@@ -449,14 +450,15 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
 inline bool few_rows(const ProductArgs &a) { return a.m <= Tile32::BM; }
 
 // Splits of K for a product whose tiles do not fill the chip: the split with the least estimated time, counted as
-// rounds of resident blocks x (3 us to start + 1.2 us per step of the longest split; 0.5 us per step of the 32-row
-// tile) plus, with a split, the reduction's launch and its float32 traffic at 4 TB/s.
+// rounds of resident blocks x (3 us to start + 1.2 us per step of the longest split; 0.64 us per step of the 32-row
+// tile) plus, with a split, the reduction: its launch, 0.38 us per split it adds up in turn and its float32 traffic at
+// 4 TB/s (fitted to w[4096,4096] at 1 to 32 rows: 43 / 26 / 17 / 13 / 15 / 20 us with 1 / 2 / 4 / 8 / 16 / 32 splits).
 template <class TL>
 int splits_of_shape(const ProductArgs &a) {
     const int64_t tiles = ((a.m + TL::BM - 1) / TL::BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
     const int64_t resident = TL::kBlocksPerCu * (int64_t)compute_units();
     if (tiles >= resident || steps < 4) return 1;
-    const double step_us = TL::BM == 32 ? 0.5 : 1.2;
+    const double step_us = TL::BM == 32 ? 0.64 : 1.2;
     double best = 0.0;
     int64_t pick = 1;
     for (int64_t splits = 1; splits <= steps / 2 && splits <= 64; splits++) {
@@ -464,7 +466,7 @@ int splits_of_shape(const ProductArgs &a) {
         if ((steps + per_split - 1) / per_split != splits) continue;  // (another count gives the same longest split)
         const int64_t rounds = (tiles * splits + resident - 1) / resident;
         double us = (double)rounds * (3.0 + step_us * (double)per_split);
-        if (splits > 1) us += 2.0 + (double)splits * (double)(a.batch * a.m * a.n) * 4.0 / 4.0e6;
+        if (splits > 1) us += 2.0 + 0.38 * (double)splits + (double)splits * (double)(a.batch * a.m * a.n) * 4.0 / 4.0e6;
         if (splits == 1 || us < best) best = us, pick = splits;
     }
     return (int)pick;
