@@ -169,13 +169,19 @@ int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose
 using namespace nvq;
 
 // Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row
-// kernel runs a block per pass of 32 rows and 64 weight rows, a round of blocks on the chip taking about 3.2 us
-// per 1024 values of K (never under 4 us).  The counterpart of the reference's device-specific `qmv_batch_limit`
+// kernel runs a block (one per compute unit) per pass of 32 rows and 64 weight rows - 32 weight rows where that leaves
+// fewer than 192 blocks (qmf::row_groups) -, a round of blocks on the chip taking about 5.0 (4.4) us per 1024 values of
+// K, never under 4 us.  Measured at W[2880,2880], 4 bits: 64 / 128 / 256 / 512 rows 13.1 / 25.0 / 32.4 / 48.2 us (180
+// blocks of 32 weight rows in one round; 360 of 32 in two; 360 of 64 in two; 720 in three) against 18.7 / 22.7 / 37.1 us
+// of the tiled kernel at 192 / 384 / 1024 rows.  The counterpart of the reference's device-specific `qmv_batch_limit`
 // (crates/nuvec-core/src/gpu.rs:1506-1538).
 static bool tiled_is_faster(const nvq::ProductArgs &a) {
-    const double blocks = (double)((a.m + 31) / 32) * (double)((a.n + 63) / 64) * (double)a.batch;
-    const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * fmax(4.0, 3.2e-3 * (double)a.k);
-    return nvq::qmm_estimate_us(a) < few_us;
+    const double passes = (double)((a.m + 31) / 32) * (double)a.batch;
+    const double blocks64 = passes * (double)((a.n + 63) / 64);
+    const bool wide = blocks64 >= 192.0;
+    const double blocks = wide ? blocks64 : passes * (double)((a.n + 31) / 32);
+    const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * fmax(4.0, (wide ? 5.0e-3 : 4.4e-3) * (double)a.k);
+    return fmax(4.0, nvq::qmm_estimate_us(a)) < few_us;  // (no launch is under 4 us)
 }
 
 // Whether the 16x16x32 kernel with directly loaded weight operands takes a few-row product, from its measured times
@@ -474,7 +480,7 @@ int32_t nvq_quantized_matmul_supported(const nvq_qmm_desc *d) {
 // (gpu.rs:6975-6981), where its tiles cost less than the passes of the few-row kernel.
 static bool takes_tiled(const nvq_qmm_desc *d, const ProductArgs &a) {
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
-    return item > 32 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a));
+    return item > 16 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a));
 }
 
 size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {

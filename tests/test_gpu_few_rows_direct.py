@@ -37,7 +37,8 @@ def test_routes_of_the_baseline_configurations():
         assert c4(512) == "qmm_kernel"
         assert c4(16, transpose=False) == ("qmn_kernel" if bits == 8 else "qvm_kernel")  # runs of eight codes: 2, 4, 8 bits
         assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
-    assert ops.quantized_matmul_route(24, 1000, 4096, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
+    assert ops.quantized_matmul_route(24, 1000, 1024, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
+    assert ops.quantized_matmul_route(24, 4096, 14336, nv.Quant.affine(64, 4), bf16) == "qmm_kernel"  # (a long K: the tiles split it)
     assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
     assert ops.quantized_matmul_route(64, 2880, 2880, nv.Quant.new(nv.QuantMode.MXFP4), bf16) in ("qmf_kernel", "qmm_kernel")
     # passes of 16 rows where the matrix is small enough to be read again from the caches; the tiles beyond
@@ -45,7 +46,7 @@ def test_routes_of_the_baseline_configurations():
     assert small(64) == "qmd_kernel" and small(192) == "qmd_kernel" and small(512) in ("qmf_kernel", "qmm_kernel")
     assert c2(64) == "qmd_kernel" and c2(96) == "qmm_kernel"
     # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
-    for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (30, 64, 128, 64, 4), (20, 1000, 4096, 64, 6)):
+    for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (30, 64, 128, 64, 4), (20, 1000, 1024, 64, 6)):
         assert ops.quantized_matmul_route(m, n, k, nv.Quant.affine(group, bits), bf16) == "qmf_kernel", (m, n, k, group, bits)
 
 
