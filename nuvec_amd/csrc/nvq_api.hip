@@ -195,8 +195,17 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 // 4 bits g64 W[4096,4096] 64 rows 11.8 / 14.6, 96 rows 18.2 / 18.6; W[14336,4096] 64 rows 33.7 / 35.3, 96 rows 49.3 / 33.9;
 // W[1024,4096] 128 rows 8.2 / 15.5; 8 bits g32 W[4096,4096] 32 rows 13.0 / 16.9, 48 rows 19.5 / 17.1.  The rule below is
 // passes x megabytes of weights, fitted to those tables.
+// Whether a few-row product stays on the decode kernels of the vector units (per-row work there is cheaper than a
+// matrix-core kernel's full dequantization up to these row counts).
+static bool takes_decode(const nvq::ProductArgs &a) {
+    if (a.dtype == NVQ_F32) return false;
+    if (a.mode != NVQ_AFFINE) return nvq::qmv_block_decode_takes(a);
+    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && a.m == 1;
+}
+
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     if (!nvq::qmd_supported(a)) return false;
+    if (a.mode != NVQ_AFFINE && nvq::qmv_block_decode_takes(a)) return false;  // one or two rows (some more): the decode kernel of the vector units
     const int64_t rows = a.n * a.batch;
     // The block formats (bf16, new / the few-row kernel of the 32x32x16 instruction): MXFP4 W[14336,4096] 1 row 11.1 / 13.4,
     // 16 rows 11.3 / 14.6; W[4096,4096] 1 row 5.4 / 6.9, 32 rows 7.0 / 14.2; NVFP4 W[14336,4096] 1 row 13.2 / 17.7;
@@ -507,8 +516,7 @@ static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     // dequantization up to there).  A single row of the other affine widths from 3 bits: the general vector kernel
     // (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against 11.7 us with 8 bits in groups of 32).  Other
     // few-row products share one weight decode on the matrix cores where those kernels take them.
-    const bool decode = a.mode == NVQ_AFFINE && a.dtype != NVQ_F32 && (a.bits == 4 ? a.m <= 4 || qmv_d16_takes(a) : a.bits >= 3 && a.m == 1);
-    if (!decode && qmf_supported(a)) return Route::kFewRows;
+    if (!takes_decode(a) && qmf_supported(a)) return Route::kFewRows;
     return Route::kVector;
 }
 
@@ -799,7 +807,9 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
     if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
-    // weight decoded once.  Otherwise one product per pair, on the few-row kernel where it takes the product.
+    // weight decoded once.  Otherwise one product per pair, on the kernel a single product of that many rows takes:
+    // the few-row matrix-core kernels, or the decode kernels of the vector units (the experts of one decoded token are
+    // pairs of one row each: 32 pairs against 4-bit W[14336,4096] 361 us on the few-row kernel, 221 us there).
     a.offsets = offsets;
     if (glu != nullptr) {
         // (projections of fewer rows take the exact-weights kernels as separate products: the epilogue form would differ)
@@ -815,7 +825,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
     // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
     if (!a.row_exact && takes_few_rows_direct(a)) return launch_qmd(a, (hipStream_t)stream);
-    if (!a.row_exact && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
+    if (!a.row_exact && !takes_decode(a) && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
     return launch_qmv(a, (hipStream_t)stream);
 }
 

@@ -253,38 +253,48 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
     }
 }
 
-// ── 4-bit affine, bf16 / f16: packed-pair dot products ────────────────────────────────────
-// ── 4-bit affine, bf16 / f16, one or two rows of x: the decode kernel ─────────────────────
+// ── 4-bit affine and the block formats, bf16 / f16, one to four rows of x: the decode kernel ───────────
 // A block of WAVES wavefronts shares the x slice of one K step (4096 values) through LDS, stored
-// once in the pair order the nibbles need together with the sums of its 32-value slices, so the
-// per-row work of a wavefront is only: two 128-bit weight loads per lane, the nibble expansion,
-// the packed dot products and one data-parallel-primitive reduction.  Every load of a step is
+// once in the pair order the codes need (affine: together with the sums of its 32-value slices), so the
+// per-row work of a wavefront is only: two 128-bit weight loads per lane (four for 8-bit codes), the code
+// expansion, the packed dot products and one data-parallel-primitive reduction.  Every load of a step is
 // issued before the first use; blocks are small (WAVES*RN weight rows) so that tens of
 // thousands of independent loads are in flight on the chip.
-template <typename T, int RM, int RN, int WAVES, bool BATCHED>
+// MODE: NVQ_AFFINE (4 bits: a code enters as B + c through the constant's mantissa, and the factored form
+// scale (dot - B sum x) + bias sum x never materialises a weight), or NVQ_MXFP4 / NVQ_NVFP4 / NVQ_MXFP8: the
+// conversion instructions give the code values as element pairs (every E2M1 and E4M3 value is exact in bf16 and f16),
+// in memory order, and a lane's 32 values are one group (NVFP4: two), whose float32 scale multiplies the group's sum.
+template <typename T, int RM, int RN, int WAVES, bool BATCHED, int MODE = NVQ_AFFINE>
 __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs a) {
     constexpr int kThreads = WAVES * 64;
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
     static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
-    __shared__ uint4 x_pairs[RM][2][4][64];  // [row][chunk][word][lane]: 4 pairs of a packed word
-    __shared__ float x_sums[RM][2][64];      // [row][chunk][lane]: sum of the lane's 32 values
+    constexpr bool kAffine = MODE == NVQ_AFFINE;
+    constexpr int BITS = MODE == NVQ_MXFP8 ? 8 : 4;
+    constexpr int kQuads = BITS / 4;                    // 16-byte loads of a lane's 32 codes
+    constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
+    __shared__ uint4 x_pairs[RM][2][4][64];               // [row][chunk][word][lane]: 4 pairs of eight values
+    __shared__ float x_sums[kAffine ? RM : 1][2][64];     // [row][chunk][lane]: sum of the lane's 32 values (affine)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // Sizes fit 32 bits (checked on the host); only row bases are 64-bit, and they are uniform.
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
-    const int gshift = a.group == 32 ? 5 : a.group == 64 ? 6 : 7;
+    const int gshift = kAffine ? (a.group == 32 ? 5 : a.group == 64 ? 6 : 7) : (MODE == NVQ_NVFP4 ? 4 : 5);
     const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * WAVES + wave) * RN);
     const int m0 = blockIdx.y * RM;
-    const int kwords = K >> 3, kgroups = K >> gshift;
+    const int kwords = (K * BITS) >> 5, kgroups = K >> gshift;
     // The single-product instantiation carries no batch arithmetic at all.
     const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
-    const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
+    using S = std::conditional_t<kAffine, T, uint8_t>;  // a scale as stored: the element type, or one byte (E8M0; NVFP4: E4M3)
+    const S *scales = (const S *)a.scales + o.s, *biases = kAffine ? (const S *)a.biases + o.s : nullptr;
     T *y = (T *)a.y + o.y;
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     uint32_t mask, magic;
     asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
+    float factor = 1.0f;
+    if constexpr (MODE == NVQ_NVFP4) factor = qmf::nvfp4_factor(a, BATCHED && a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0);
 
     float acc[RN][RM];
 #pragma unroll
@@ -303,8 +313,10 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 xg[i][p] = (kx < K && m0 + i < M) ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + kx)
                                                       : make_uint4(0, 0, 0, 0);  // absent x: contributes nothing
             }
-        uint4 wq[2][RN];
-        T sraw[2][RN], braw[2][RN];
+        uint4 wq[2][RN][kQuads];
+        using SR = std::conditional_t<MODE == NVQ_NVFP4, uint16_t, S>;  // what a lane reads of the scales: NVFP4's two bytes at once
+        SR sraw[2][RN];
+        S braw[2][RN];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const int kb = k0 + u * kStep + lane * 32;
@@ -314,10 +326,11 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const int n = n0 + r < N ? n0 + r : N - 1;  // tail rows are computed, not stored
                 // the codes are read once: a non-temporal load keeps them from displacing x and the scales in the caches
                 // (8.1 -> 7.8 us at W[14336,4096]; the scales, shared by neighbouring lanes and rows, lose by it)
-                wq[u][r] = stream_load(reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 3)));
-                const T *ps = scales + (int64_t)n * kgroups, *pb = biases + (int64_t)n * kgroups;
-                sraw[u][r] = ps[kc >> gshift];
-                braw[u][r] = pb[kc >> gshift];
+                const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
+#pragma unroll
+                for (int c = 0; c < kQuads; c++) wq[u][r][c] = stream_load(pw + c);
+                sraw[u][r] = *reinterpret_cast<const SR *>(scales + (int64_t)n * kgroups + (kc >> gshift));
+                if constexpr (kAffine) braw[u][r] = (biases + (int64_t)n * kgroups)[kc >> gshift];
             }
         }
         if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
@@ -327,19 +340,23 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
             for (int p = 0; p < kXPerThread; p++) {
                 const int idx = tid + p * kThreads;  // 128-bit piece: chunk idx/256, lane (idx%256)/4, word idx%4
                 const uint4 q = xg[i][p];            // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
-                uint4 pr;
-                pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
-                pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
-                pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
-                pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
-                x_pairs[i][idx >> 8][idx & 3][(idx & 255) >> 2] = pr;
-                float sum = Pair<T>::dot2(pr.x, ones, 0.0f);
-                sum = Pair<T>::dot2(pr.y, ones, sum);
-                sum = Pair<T>::dot2(pr.z, ones, sum);
-                sum = Pair<T>::dot2(pr.w, ones, sum);
-                sum += __shfl_xor(sum, 1);  // the four pieces of a lane's slice sit in adjacent threads
-                sum += __shfl_xor(sum, 2);
-                if ((idx & 3) == 0) x_sums[i][idx >> 8][(idx & 255) >> 2] = sum;
+                if constexpr (kAffine) {
+                    uint4 pr;
+                    pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+                    pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+                    pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+                    pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+                    x_pairs[i][idx >> 8][idx & 3][(idx & 255) >> 2] = pr;
+                    float sum = Pair<T>::dot2(pr.x, ones, 0.0f);
+                    sum = Pair<T>::dot2(pr.y, ones, sum);
+                    sum = Pair<T>::dot2(pr.z, ones, sum);
+                    sum = Pair<T>::dot2(pr.w, ones, sum);
+                    sum += __shfl_xor(sum, 1);  // the four pieces of a lane's slice sit in adjacent threads
+                    sum += __shfl_xor(sum, 2);
+                    if ((idx & 3) == 0) x_sums[i][idx >> 8][(idx & 255) >> 2] = sum;
+                } else {
+                    x_pairs[i][idx >> 8][idx & 3][(idx & 255) >> 2] = q;  // (the conversions give the code values in memory order)
+                }
             }
         __syncthreads();
 #pragma unroll
@@ -350,35 +367,85 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
             for (int i = 0; i < RM; i++) {
 #pragma unroll
                 for (int j = 0; j < 4; j++) xp[i][j] = x_pairs[i][u][j][lane];
-                xs[i] = x_sums[i][u][lane];
+                if constexpr (kAffine) xs[i] = x_sums[i][u][lane];
             }
 #pragma unroll
             for (int r = 0; r < RN; r++) {
-                const uint32_t d[4] = {wq[u][r].x, wq[u][r].y, wq[u][r].z, wq[u][r].w};
-                float dot[RM][4];
+                if constexpr (kAffine) {
+                    const uint32_t d[4] = {wq[u][r][0].x, wq[u][r][0].y, wq[u][r][0].z, wq[u][r][0].w};
+                    float dot[RM][4];
 #pragma unroll
-                for (int i = 0; i < RM; i++)
+                    for (int i = 0; i < RM; i++)
 #pragma unroll
-                    for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+                        for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint32_t p0 = and_or(d[j], mask, magic), p1 = and_or(d[j] >> 4, mask, magic);
-                    const uint32_t p2 = and_or(d[j] >> 8, mask, magic), p3 = and_or(d[j] >> 12, mask, magic);
+                    for (int j = 0; j < 4; j++) {
+                        const uint32_t p0 = and_or(d[j], mask, magic), p1 = and_or(d[j] >> 4, mask, magic);
+                        const uint32_t p2 = and_or(d[j] >> 8, mask, magic), p3 = and_or(d[j] >> 12, mask, magic);
+#pragma unroll
+                        for (int i = 0; i < RM; i++) {
+                            dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                            dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                            dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                            dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+                        }
+                    }
+                    // scale * (dot - B * sum x) + bias * sum x
+                    const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
+                    const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
 #pragma unroll
                     for (int i = 0; i < RM; i++) {
-                        dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
-                        dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
-                        dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
-                        dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+                        const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+                        acc[r][i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[r][i]));
                     }
-                }
-                // scale * (dot - B * sum x) + bias * sum x
-                const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
-                const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+                } else {
+                    // piece j of the lane's slice: eight values, the pairs of xp[i][j] in memory order
+                    float dot[RM][kHalves][2];
 #pragma unroll
-                for (int i = 0; i < RM; i++) {
-                    const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
-                    acc[r][i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[r][i]));
+                    for (int i = 0; i < RM; i++)
+#pragma unroll
+                        for (int hf = 0; hf < kHalves; hf++) dot[i][hf][0] = dot[i][hf][1] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        constexpr int kPiecesPerHalf = 4 / kHalves;
+                        const int hf = j / kPiecesPerHalf;
+                        uint32_t p0, p1, p2, p3;
+                        if constexpr (BITS == 4) {
+                            const uint4 q = wq[u][r][0];
+                            const uint32_t d = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+                            p0 = qmf::Ops<T>::template fp4_pair<0>(d, 1.0f);
+                            p1 = qmf::Ops<T>::template fp4_pair<1>(d, 1.0f);
+                            p2 = qmf::Ops<T>::template fp4_pair<2>(d, 1.0f);
+                            p3 = qmf::Ops<T>::template fp4_pair<3>(d, 1.0f);
+                        } else {
+                            const uint4 q = wq[u][r][j >> 1];
+                            const uint32_t d0 = (j & 1) ? q.z : q.x, d1 = (j & 1) ? q.w : q.y;
+                            p0 = qmf::Ops<T>::template fp8_pair<false>(d0, 1.0f);
+                            p1 = qmf::Ops<T>::template fp8_pair<true>(d0, 1.0f);
+                            p2 = qmf::Ops<T>::template fp8_pair<false>(d1, 1.0f);
+                            p3 = qmf::Ops<T>::template fp8_pair<true>(d1, 1.0f);
+                        }
+#pragma unroll
+                        for (int i = 0; i < RM; i++) {
+                            dot[i][hf][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][hf][0]);
+                            dot[i][hf][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][hf][1]);
+                            dot[i][hf][0] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][hf][0]);
+                            dot[i][hf][1] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][hf][1]);
+                        }
+                    }
+                    float sc[2];
+                    if constexpr (MODE == NVQ_NVFP4) {
+                        // both E4M3 scales by one conversion (every E4M3 value is a normal float32 or zero); times the
+                        // global scale's factor as crates/nuvec-core/src/kernels.rs:992-998
+                        const auto two = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8((uint32_t)sraw[u][r], 1.0f, false);
+                        sc[0] = ftz(two[0] * factor), sc[1] = ftz(two[1] * factor);
+                    } else {
+                        sc[0] = sc[1] = ftz(e8m0_to_f32(sraw[u][r]));
+                    }
+#pragma unroll
+                    for (int hf = 0; hf < kHalves; hf++)
+#pragma unroll
+                        for (int i = 0; i < RM; i++) acc[r][i] = __builtin_fmaf(sc[hf], dot[i][hf][0] + dot[i][hf][1], acc[r][i]);
                 }
             }
         }
@@ -906,16 +973,42 @@ int32_t run_mfma4(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
-template <typename T, int RM, int RN, int WAVES>
+template <typename T, int RM, int RN, int WAVES, int MODE = NVQ_AFFINE>
 int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
     const int64_t rows = (int64_t)WAVES * RN;
     dim3 grid((unsigned)((a.n + rows - 1) / rows), (unsigned)((a.m + RM - 1) / RM), (unsigned)a.batch);
     if (a.batch == 1 && a.rhs == nullptr)
-        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, false>), grid, dim3(WAVES * 64), 0, s, a);
+        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, false, MODE>), grid, dim3(WAVES * 64), 0, s, a);
     else
-        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, true>), grid, dim3(WAVES * 64), 0, s, a);
+        hipLaunchKernelGGL((qmv4_lds_kernel<T, RM, RN, WAVES, true, MODE>), grid, dim3(WAVES * 64), 0, s, a);
     NVQ_LAUNCH_CHECK("qmv4_lds");
     return NVQ_OK;
+}
+
+// Whether the decode kernel takes a product of a block format: bf16 / f16, up to kBlockDecodeRows rows of x, whole
+// slices of 32 values (NVFP4 rows may end in half a slice: those stay on the general kernel).  Row-exact products
+// stay on the general kernel at every row count.
+// Measured against the few-row matrix-core kernels (us per launch at 1 / 2 / 3 / 4 rows, bf16; theirs -> this one):
+//   MXFP4 W[14336,4096] 10.2 / 10.3 / 10.3 / 10.3 ->  7.5 /  8.8 / 10.2 / 12.6     W[2880,2880] 5.9 / 6.0 / 6.0 / 6.0 -> 3.7 / 4.2 / 4.8 / 5.4
+//   MXFP4 W[4096,14336] 10.5 / 11.0 / 11.1 / 11.1 ->  8.3 / 10.4 / 12.3 / 14.8     W[4096,4096] 5.2 / 5.3 / 5.3 / 5.4 -> 4.2 / 4.5 / 5.0 / 5.7
+//   NVFP4 W[14336,4096] 13.0 / 13.1 / 13.1 / 13.2 ->  8.9 / 10.3 / 12.3 / 13.9     W[2880,2880] 7.9 / 8.1 / 8.2 / 8.3 -> 4.0 / 4.6 / 5.3 / 6.0
+//   MXFP8 W[14336,4096] 16.8 / 16.0 / 16.1 / 16.1 -> 13.6 / 14.3 / 14.7 / 16.0     W[4096,14336] 16.8 / 16.2 / 16.3 / 16.1 -> 14.6 / 15.5 / 16.6 / 18.8
+// One and two rows: always.  Three rows (MXFP8: and four): up to K = 4096.  Up to four rows where the kernel that
+// loads the weights straight into operand layout does not take the product (K in slices of 512).
+inline bool block_decode_takes(const ProductArgs &a) {
+    if (a.mode == NVQ_AFFINE || a.dtype == NVQ_F32 || a.row_exact) return false;
+    if (a.m < 1 || a.m > 4 || a.k % 32 != 0 || (uintptr_t)a.w % 16 != 0 || (uintptr_t)a.x % 16 != 0) return false;
+    if (a.mode == NVQ_NVFP4 && (uintptr_t)a.scales % 2 != 0) return false;  // (a lane reads its two scales at once)
+    if (a.m <= 2 || !qmd_supported(a)) return true;
+    return a.k <= 4096 && (a.m == 3 || a.mode == NVQ_MXFP8);
+}
+
+template <typename T, int MODE>
+int32_t run_block_decode(const ProductArgs &a, hipStream_t s) {
+    if (a.m == 1) return run_lds4<T, 1, 1, 8, MODE>(a, s);
+    if (a.m == 2) return run_lds4<T, 2, 1, 8, MODE>(a, s);
+    if (a.m == 3) return run_lds4<T, 3, 1, 8, MODE>(a, s);
+    return run_lds4<T, 4, 1, 8, MODE>(a, s);
 }
 
 template <typename T, int BITS, int MODE>
@@ -938,6 +1031,13 @@ int32_t run_general(const ProductArgs &a, hipStream_t s) {
 
 template <typename T>
 int32_t run_typed(const ProductArgs &a, hipStream_t s) {
+    if constexpr (!std::is_same<T, float>::value) {
+        if (block_decode_takes(a)) {
+            if (a.mode == NVQ_MXFP4) return run_block_decode<T, NVQ_MXFP4>(a, s);
+            if (a.mode == NVQ_MXFP8) return run_block_decode<T, NVQ_MXFP8>(a, s);
+            return run_block_decode<T, NVQ_NVFP4>(a, s);
+        }
+    }
     if (a.mode == NVQ_MXFP4) return run_general<T, 4, NVQ_MXFP4>(a, s);
     if (a.mode == NVQ_MXFP8) return run_general<T, 8, NVQ_MXFP8>(a, s);
     if (a.mode == NVQ_NVFP4) return run_general<T, 4, NVQ_NVFP4>(a, s);
@@ -973,6 +1073,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 }  // namespace
 
 bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
+bool qmv_block_decode_takes(const ProductArgs &a) { return block_decode_takes(a); }
 
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
@@ -981,6 +1082,7 @@ const char *qmv_kernel_name(const ProductArgs &a) {
         if (!a.row_exact && a.m >= 4 && mfma_decode_takes<4>(a)) return "qmv4_mfma_kernel";
         return "qmv4_lds_kernel";
     }
+    if (block_decode_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }
 

@@ -140,7 +140,7 @@ def test_direct_few_row_kernel_block_formats(mode, qmode, dtype):
     rng = np.random.default_rng(4300 + 10 * mode + dtype)
     group, bits = ref.FP_PARAMS[mode]
     quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
-    for m, n, k in [(1, 200, 512), (3, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (11, 48, 14336), (23, 64, 1536), (8, 5000, 512),
+    for m, n, k in [(5, 200, 512), (7, 1000, 1024), (16, 130, 4096), (13, 96, 8192), (3, 48, 14336), (23, 64, 1536), (8, 5000, 512),
                     (50, 300, 2048)]:
         assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmd_kernel", (qmode, m, n, k)
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)

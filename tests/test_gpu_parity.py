@@ -582,6 +582,88 @@ def test_block_formats_on_the_matrix_cores(mode, qmode, dtype):
     assert_rows_close(got, want[some], dtype, f"{qmode} gather per pair", exact_weights=True)
 
 
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_block_formats_on_the_decode_kernel(mode, qmode, dtype):
+    """One to four rows of x against MXFP4, MXFP8 and NVFP4 weights on the decode kernel of the vector units (the conversion
+    instructions give the code values, a group's float32 scale multiplies the group's sum): K of one slice, off the
+    kernel's steps and over several, weight rows off the block's eight, a batch, the pairs of an unsorted gather (the
+    experts of a decoded token).  The weights are exact in the element type, so the bar holds for every output."""
+    rng = np.random.default_rng(4700 + 10 * mode + dtype)
+    group, bits = ref.FP_PARAMS[mode]
+    quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
+    for m, n, k in [(1, 203, 32), (1, 1000, 2880), (2, 77, 4096 + 96), (3, 130, 1024), (4, 61, 2880), (1, 48, 14336), (2, 1030, 8192), (4, 96, 224)]:
+        assert nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmv4_lds_kernel", (qmode, m, n, k)
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales = ref.fp_quantize(w, dtype, mode)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, dtype, f"decode kernel {qmode} M={m} N={n} K={k}", exact_weights=True)
+    b, m, n, k = 3, 2, 90, 1056
+    w, x = make_w(rng, b * n, k, dtype), make_x(rng, b * m, k, dtype)
+    packed, scales = ref.fp_quantize(w, dtype, mode)
+    q = nv.Quantized(to_dev(packed.reshape(b, n, -1)), to_dev(scales.reshape(b, n, -1)), None, quant)
+    assert nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype], batch=b) == "qmv4_lds_kernel"
+    got = to_host(nv.quantized_matmul(to_dev(x.reshape(b, m, k)), q))
+    for i in range(b):
+        want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[i * n:(i + 1) * n], scales[i * n:(i + 1) * n], None, mode=mode,
+                                    group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[i], want, dtype, f"decode kernel {qmode} batch item {i}", exact_weights=True)
+    # four experts of one token, unsorted: a product of one row per pair
+    lhs, rhs = np.zeros(4, np.int64), np.array([2, 0, 1, 2], np.int64)
+    xt = make_x(rng, 1, k, dtype)
+    got = to_host(nv.gather_qmm(to_dev(xt.reshape(1, 1, k)), q, torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), nv.GatherQmm()))
+    for z in range(4):
+        e = int(rhs[z])
+        want = ref.quantized_matmul(xt, packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n], None, mode=mode, group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[z], want, dtype, f"decode kernel {qmode} pair {z}", exact_weights=True)
+
+
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+def test_block_formats_at_every_scale_code(mode, qmode):
+    """Every scale code on every product route: weight row n carries scale code n in all its groups (E8M0: 2^(n - 127), zero
+    flushed at code 0; E4M3: both signs, subnormals, 448, NaN at 0x7F and 0xFF), so a conversion that mistook one code
+    fails its column of the output.  Outputs are compared after division by their column's scale, each against the bar of
+    its row.  x is small enough for the large scales to stay finite; the E8M0 codes whose weights overflow float32 (from
+    246; 255 is infinity in the reference, fp8.rs:95-102, and only an infinite weight quantizes to it) or whose products
+    would be float32 subnormals (below 30) are left out; code 0, which flushes to zero, stays."""
+    rng = np.random.default_rng(4800 + mode)
+    dtype = ref.BF16
+    group, bits = ref.FP_PARAMS[mode]
+    quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
+    n, k = 256, 512
+    codes = np.arange(256, dtype=np.uint8)
+    if mode != ref.NVFP4:
+        codes = np.where(((codes > 0) & (codes < 30)) | (codes > 245), 127, codes).astype(np.uint8)
+    w = make_w(rng, n, k, dtype)
+    packed, _ = ref.fp_quantize(w, dtype, mode)
+    scales = np.repeat(codes[:, None], k // group, axis=1)
+    one = np.full(packed.shape, 0x38383838 if mode == ref.MXFP8 else 0x22222222, np.uint32)  # every code 1.0
+    value = ref.fp_dequantize(one, scales, mode, ref.F32)[:, 0].astype(np.float64)  # the scales as the oracle decodes them
+    nan, zero = np.isnan(value), value == 0.0
+    assert (nan[[0x7F, 0xFF]].all() if mode == ref.NVFP4 else zero[0] and not nan.any()) and np.count_nonzero(~nan & ~zero) >= 200
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+    routes = set()
+    for m in (1, 3, 8, 40, 300):
+        x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32) * 2.0 ** -14, dtype)
+        want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8), dtype)
+        got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q)), dtype)
+        routes.add(nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]))
+        assert np.isnan(want[:, nan]).all() and np.isnan(got[:, nan]).all(), f"{qmode} M={m}: NaN scales"
+        # The reference flushes 2^-127 to zero (fp8.rs:95-112).  The vector kernels do; the scaled conversions of the matrix-core
+        # kernels take the code as 2^-127, so an output may hold up to max|code| * 2^-127 * sum|x| there instead of zero.
+        route = nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
+        slack = 0.0 if route in ("qmv4_lds_kernel", "qmv_lds_kernel") else 1.01 * 448.0 * 2.0 ** -127 * float(np.abs(ref.to_f32(x, dtype)).sum(axis=1).max())
+        assert not want[:, zero].any() and float(np.abs(got[:, zero]).max()) <= slack, f"{qmode} M={m}: scales that flush to zero"
+        live = ~nan & ~zero
+        g, r = got[:, live].astype(np.float64) / value[live], want[:, live].astype(np.float64) / value[live]
+        ratio = np.abs(g - r) / (TOL[dtype] * np.max(np.abs(r), axis=1, keepdims=True))
+        worst = np.unravel_index(np.argmax(ratio), ratio.shape)
+        assert ratio[worst] <= 1.0, f"{qmode} M={m} scale code {codes[live][worst[1]]}: {ratio[worst]:.3f} x the bound"
+    assert {"qmv4_lds_kernel", "qmd_kernel"} <= routes and len(routes) >= 3, routes
+
+
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
 def test_nvfp4_global_scale(dtype):
     """NVFP4 with a global scale (MLX's `quantize(..., global_scale=)`): codes, scales and dequantized values bit for
@@ -609,7 +691,7 @@ def test_nvfp4_global_scale(dtype):
         w2 = make_w(rng, n2, k2, dtype)
         p2, s2 = ref.fp_quantize(w2, dtype, ref.NVFP4, g)
         q2 = nv.quantize(to_dev(w2), nv.QuantMode.NVFP4, gs)
-        for m, kernels in ((1, ("qmd_kernel",)), (16, ("qmd_kernel",)), (40, ("qmf_kernel", "qmd_kernel")), (600, ("qmm_kernel", "qmf_kernel"))):
+        for m, kernels in ((1, ("qmv4_lds_kernel",)), (2, ("qmv4_lds_kernel",)), (16, ("qmd_kernel",)), (40, ("qmf_kernel", "qmd_kernel")), (600, ("qmm_kernel", "qmf_kernel"))):
             x = make_x(rng, m, k2, dtype)
             want = ref.fp_quantized_matmul_scaled(x, p2, s2, ref.NVFP4, dtype, g)
             got = to_host(nv.quantized_matmul(to_dev(x), q2))
