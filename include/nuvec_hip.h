@@ -347,10 +347,12 @@ NVQ_API int32_t nvq_weighted_sum(int32_t dtype, const void *x, const void *w, in
  * up[r, c] + up_bias[ids[r], c]), every operation rounded to `dtype` in the reference's order.
  *   NVQ_GLU_SWIGLU      gate * sigmoid(gate) * up                     (crates/nuvec-nn/src/lib.rs:343-345, 513-519)
  *   NVQ_GLU_SWIGLU_OAI  (clip(up, -limit, limit) + 1) * g * sigmoid(alpha * g), g = min(gate, limit)   (lib.rs:564-570)
+ *   NVQ_GLU_GEGLU       0.5 gate (1 + tanh(sqrt(2 / pi) (gate + 0.044715 gate^3))) * up: Gemma's, with the tanh
+ *                       approximation of GELU as MLX's `gelu_approx`                                     (lib.rs:347-357, 581-590)
  *   gate, up dtype[rows, hidden] with `gate_stride` / `up_stride` elements between rows (so the two halves of one
  *   product [rows, 2 * hidden] of fused gate / up weights serve);  out dtype[rows, hidden];  gate_bias, up_bias
  *   dtype[experts, hidden], both or neither, with ids i32[rows] (an id outside is clamped). */
-enum { NVQ_GLU_SWIGLU = 0, NVQ_GLU_SWIGLU_OAI = 1 };
+enum { NVQ_GLU_SWIGLU = 0, NVQ_GLU_SWIGLU_OAI = 1, NVQ_GLU_GEGLU = 2 };
 typedef struct nvq_glu_desc {
     int32_t dtype;       /* NVQ_F32, NVQ_F16 or NVQ_BF16 */
     int32_t activation;  /* NVQ_GLU_* */

@@ -39,8 +39,11 @@ int32_t run_glu(const nvq_glu_desc &d, const void *gate, const void *up, const v
     if (d.activation == NVQ_GLU_SWIGLU)
         hipLaunchKernelGGL((glu_kernel<T, NVQ_GLU_SWIGLU>), grid, block, 0, s, (const T *)gate, (const T *)up, (const T *)gate_bias,
                            (const T *)up_bias, ids, (T *)out, d.rows, d.hidden, d.gate_stride, d.up_stride, d.experts, alpha, limit);
-    else
+    else if (d.activation == NVQ_GLU_SWIGLU_OAI)
         hipLaunchKernelGGL((glu_kernel<T, NVQ_GLU_SWIGLU_OAI>), grid, block, 0, s, (const T *)gate, (const T *)up, (const T *)gate_bias,
+                           (const T *)up_bias, ids, (T *)out, d.rows, d.hidden, d.gate_stride, d.up_stride, d.experts, alpha, limit);
+    else
+        hipLaunchKernelGGL((glu_kernel<T, NVQ_GLU_GEGLU>), grid, block, 0, s, (const T *)gate, (const T *)up, (const T *)gate_bias,
                            (const T *)up_bias, ids, (T *)out, d.rows, d.hidden, d.gate_stride, d.up_stride, d.experts, alpha, limit);
     NVQ_LAUNCH_CHECK("glu");
     return NVQ_OK;

@@ -738,7 +738,7 @@ int32_t nvq_glu(const nvq_glu_desc *d, const void *gate, const void *up, const v
     // model.rs:2139-2143, 2157-2170
     if (d == nullptr) return fail(NVQ_INVALID_ARGUMENT, "glu: null descriptor");
     if (!float_dtype(d->dtype)) return fail(NVQ_INVALID_ARGUMENT, "glu: unsupported dtype %s", dtype_name(d->dtype));
-    if (d->activation != NVQ_GLU_SWIGLU && d->activation != NVQ_GLU_SWIGLU_OAI)
+    if (d->activation < NVQ_GLU_SWIGLU || d->activation > NVQ_GLU_GEGLU)
         return fail(NVQ_INVALID_ARGUMENT, "glu: unknown activation %d", d->activation);
     if (d->rows < 0 || d->hidden < 0 || d->experts < 0) return fail(NVQ_INVALID_ARGUMENT, "glu: negative size");
     if (d->gate_stride < d->hidden || d->up_stride < d->hidden)
@@ -785,7 +785,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(check_aligned("gather_qmm", "rhs", rhs, 4));
     NVQ_TRY(check_aligned("gather_qmm", "offsets", offsets, 4));
     if (glu != nullptr) {
-        if (glu->activation != NVQ_GLU_SWIGLU && glu->activation != NVQ_GLU_SWIGLU_OAI)
+        if (glu->activation < NVQ_GLU_SWIGLU || glu->activation > NVQ_GLU_GEGLU)
             return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: unknown activation %d", glu->activation);
         if (!d->transpose || offsets == nullptr || d->m != 1 || d->k == 0 || d->n % 128 != 0)
             return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue belongs to the grouped product of transposed weights whose "

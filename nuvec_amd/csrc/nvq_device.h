@@ -165,7 +165,7 @@ __device__ __forceinline__ uint32_t e8m0_round_up_code(float x) {
     return c > 254u ? 254u : c;
 }
 
-// ---- The gated activations of the experts' MLPs (crates/nuvec-nn/src/lib.rs:343-345, 513-519, 564-570), every
+// ---- The gated activations of the experts' MLPs (crates/nuvec-nn/src/lib.rs:343-357, 513-519, 564-570, 581-590), every
 // operation rounded to the element type as the reference's element-wise graphs evaluate them.
 // kernels.rs:1539-1543
 __device__ __forceinline__ float sigmoid_f32(float x) {
@@ -188,12 +188,22 @@ __device__ __forceinline__ float glu(float gate, float up, float alpha, float li
     if constexpr (ACT == NVQ_GLU_SWIGLU) {
         const float s = rounded<T>(sigmoid_f32(gate));
         return Elem<T>::mul(Elem<T>::mul(gate, s), up);  // lib.rs:343-345, 516-517
-    } else {
+    } else if constexpr (ACT == NVQ_GLU_SWIGLU_OAI) {
         // lib.rs:565-570
         const float g = nan_min(gate, limit);
         const float x = nan_min(nan_max(up, -limit), limit);
         const float s = rounded<T>(sigmoid_f32(Elem<T>::mul(alpha, g)));
         return Elem<T>::mul(Elem<T>::add(x, 1.0f), Elem<T>::mul(g, s));
+    } else {
+        // lib.rs:350-357, 583-590: gate^3 is one power (powf in float32, kernels.rs:1375, 1594), rounded once; the
+        // constants are weak scalars of the activations' type.  The cube of a 16-bit element is exact in two float32
+        // products but for the last rounding; a float32 gate is cubed in float64 and rounded once.
+        float cube;
+        if constexpr (sizeof(T) == 4) cube = (float)((double)gate * (double)gate * (double)gate);
+        else cube = rounded<T>((gate * gate) * gate);
+        const float inner = Elem<T>::mul(Elem<T>::add(gate, Elem<T>::mul(cube, rounded<T>(0.044715f))), rounded<T>(0.7978845608028654f));
+        const float t = rounded<T>(tanhf(inner));
+        return Elem<T>::mul(Elem<T>::mul(Elem<T>::mul(gate, 0.5f), Elem<T>::add(t, 1.0f)), up);
     }
 }
 

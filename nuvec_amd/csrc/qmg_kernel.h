@@ -331,8 +331,9 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
                         const uint32_t lo = __builtin_amdgcn_readlane(place, m0), hi = __builtin_amdgcn_readlane(place, m0 + 4);
                         if (m < rows) {
                             const float g = value(u, el), up = exchange[(16 * u + el) * 64];
-                            const float out = a.glu == 1 + NVQ_GLU_SWIGLU ? glu<T, NVQ_GLU_SWIGLU>(g, up, a.glu_alpha, a.glu_limit)
-                                                                          : glu<T, NVQ_GLU_SWIGLU_OAI>(g, up, a.glu_alpha, a.glu_limit);
+                            const float out = a.glu == 1 + NVQ_GLU_SWIGLU       ? glu<T, NVQ_GLU_SWIGLU>(g, up, a.glu_alpha, a.glu_limit)
+                                              : a.glu == 1 + NVQ_GLU_SWIGLU_OAI ? glu<T, NVQ_GLU_SWIGLU_OAI>(g, up, a.glu_alpha, a.glu_limit)
+                                                                                : glu<T, NVQ_GLU_GEGLU>(g, up, a.glu_alpha, a.glu_limit);
                             Elem<T>::store(y, (int64_t)(h ? hi : lo) * H + hcol, out);
                         }
                     }

@@ -129,7 +129,7 @@ class SwitchGlu:
     down_proj: SwitchProjection
     gate_up_proj: Optional[SwitchProjection] = None  # `fuse_gate_up`: both projections' rows, gate first
     gate_up_paired: bool = False  # `gate_up_proj` alternates the two projections' rows in runs of 64
-    activation: str = "swiglu"  # or "swiglu_oai" with `alpha` and `limit` (model.rs:2161-2166; gpt-oss: 1.702 and 7)
+    activation: str = "swiglu"  # or "swiglu_oai" with `alpha` and `limit` (model.rs:2161-2166; gpt-oss: 1.702 and 7), or "geglu" (model.rs:2167)
     alpha: float = 1.702
     limit: float = 7.0
 
@@ -178,7 +178,16 @@ class SwitchGlu:
         k = indices.shape[2]
         if indices.numel() < 64:  # model.rs:2189-2192
             xe = x.reshape(b, l, 1, 1, d)
-            up, gate = self.up_proj.forward(xe, indices, add_bias=False), self.gate_proj.forward(xe, indices, add_bias=False)
+            if self.gate_up_proj is not None:  # one gather for both projections (a decoded token's few pairs are launch-bound)
+                both = self.gate_up_proj.forward(xe, indices, add_bias=False)
+                if self.gate_up_paired:
+                    runs = both.reshape(both.shape[:-1] + (-1, 2, 64))
+                    gate, up = runs[..., 0, :].reshape(both.shape[:-1] + (-1,)), runs[..., 1, :].reshape(both.shape[:-1] + (-1,))
+                else:
+                    half = both.shape[-1] // 2
+                    gate, up = both[..., :half], both[..., half:]
+            else:
+                up, gate = self.up_proj.forward(xe, indices, add_bias=False), self.gate_proj.forward(xe, indices, add_bias=False)
             return self.down_proj.forward(self.gated(gate, up, indices), indices).squeeze(-2)
         experts = self.up_proj.weight.shape[0]
         order, restore, sorted_ids, offsets = ops.moe_order(indices, experts)

@@ -78,7 +78,7 @@ def weighted_sum(x: np.ndarray, w: np.ndarray, dtype: int) -> np.ndarray:
     return ref.from_f32(total, dtype)
 
 
-SWIGLU, SWIGLU_OAI = 0, 1
+SWIGLU, SWIGLU_OAI, GEGLU = 0, 1, 2
 
 
 def _sigmoid(x: np.ndarray) -> np.ndarray:
@@ -106,6 +106,13 @@ def glu(gate: np.ndarray, up: np.ndarray, dtype: int, activation: int = SWIGLU, 
         if activation == SWIGLU:
             s = _round(_sigmoid(g), dtype)              # lib.rs:344
             y = _round(_round(g * s, dtype) * x, dtype)  # lib.rs:344, 517
+        elif activation == GEGLU:
+            # lib.rs:350-357, 583-590: x^3 is one power (kernels.rs:1375, 1594), the constants weak scalars of the dtype
+            k1, k2 = _round(np.float32(0.044715), dtype), _round(np.float32(np.sqrt(2.0 / np.pi)), dtype)
+            cube = _round(np.power(g.astype(np.float64), 3.0).astype(np.float32), dtype)
+            inner = _round(_round(g + _round(cube * k1, dtype), dtype) * k2, dtype)
+            t = _round(np.tanh(inner.astype(np.float64)).astype(np.float32), dtype)
+            y = _round(_round(_round(g * np.float32(0.5), dtype) * _round(t + np.float32(1.0), dtype), dtype) * x, dtype)
         else:
             a, l = _round(np.float32(alpha), dtype), _round(np.float32(limit), dtype)  # lib.rs:505-507
             g = _nan_min(g, l)                           # lib.rs:566

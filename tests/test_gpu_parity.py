@@ -1035,6 +1035,13 @@ def test_switch_glu_sorts_gathers_and_restores():
     few = torch.cat([glu(to_dev(x)[:, t:t + 8], torch.from_numpy(idx).cuda()[:, t:t + 8]) for t in range(0, l, 8)], dim=1)
     scale = float(few.float().abs().max())
     assert float((whole.float() - few.float()).abs().max()) <= 2e-2 * scale
+    # the fused gate + up weight on the few-pairs route: one gather for both projections, the same rows of the same weights
+    for fused in (SwitchGlu(gate, up, down).fuse_gate_up(),
+                  SwitchGlu(gate, up, down, SwitchProjection(torch.cat([gate.weight, up.weight], 1), torch.cat([gate.scales, up.scales], 1), None,
+                                                             None, gate.quant))):
+        assert fused.gate_up_proj is not None
+        again = torch.cat([fused(to_dev(x)[:, t:t + 8], torch.from_numpy(idx).cuda()[:, t:t + 8]) for t in range(0, l, 8)], dim=1)
+        assert torch.equal(again, few), "paired" if fused.gate_up_paired else "gate rows first"
 
 
 @pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
@@ -1116,17 +1123,18 @@ def test_moe_block_routes_multiplies_and_sums():
 
 
 @pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
-@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai"])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai", "geglu"])
 def test_gated_activation_against_the_oracle(dtype, activation):
     """`nvq_glu` (SwitchGlu::through between the products, model.rs:2157-2170; the experts' biases of model.rs:2139-2143)
-    against the oracle's operation-by-operation restatement.  The two differ only through `exp` (the device's and
-    numpy's, either within an ulp of float32), which the rounding of the sigmoid to a half type hides except at a tie:
-    there all but a few outputs in ten thousand agree bit for bit and none is off by more than one step of the type;
-    float32 outputs agree within four steps."""
+    against the oracle's operation-by-operation restatement.  The two differ only through `exp` or `tanh` (the device's and
+    the host's, either within a few ulps of float32), which the rounding of the sigmoid or the tanh to a half type hides
+    except at a tie: there all but a few outputs in ten thousand agree bit for bit and none is off by more than one step of
+    the type; float32 outputs agree within four steps.  (geglu: a step of the tanh is a step of 1 + tanh, which cancels
+    for negative gates, so there the step is taken of |gate up / 2| as well as of the output.)"""
     from oracle import moe
     rng = np.random.default_rng(7600 + dtype + len(activation))
     tdtype = {ref.F32: torch.float32, ref.F16: torch.float16, ref.BF16: torch.bfloat16}[dtype]
-    act = moe.SWIGLU if activation == "swiglu" else moe.SWIGLU_OAI
+    act = {"swiglu": moe.SWIGLU, "swiglu_oai": moe.SWIGLU_OAI, "geglu": moe.GEGLU}[activation]
     rows, hidden, experts = 300, 360, 6
     specials = np.array([0.0, -0.0, 7.0, -7.0, 7.5, -9.0, 60.0, -60.0, 100.0, -100.0, np.inf, -np.inf, np.nan, 1e-30, -1e-30], np.float32)
     g = (rng.standard_normal((rows, 2 * hidden)) * 3).astype(np.float32)
@@ -1138,15 +1146,21 @@ def test_gated_activation_against_the_oracle(dtype, activation):
     ub = ref.from_f32(rng.standard_normal((experts, hidden)).astype(np.float32), dtype)
     ids = np.sort(rng.integers(0, experts, rows)).astype(np.int32)
 
-    def check(got, want, what):
+    def check(got, want, what, biased=False):
         got, want = np.asarray(got), np.asarray(want)
         gf, wf = ref.to_f32(got, dtype), ref.to_f32(want, dtype)
         same = (got.view(np.uint8).reshape(got.shape + (-1,)) == want.view(np.uint8).reshape(want.shape + (-1,))).all(-1) | (np.isnan(gf) & np.isnan(wf))
         if dtype != ref.F32:  # (float32 shows the last bits of exp itself: within four steps below)
             assert np.count_nonzero(~same) <= max(1, same.size // 2000), f"{what}: {np.count_nonzero(~same)} of {same.size} outputs differ"
         step = {ref.F32: 4 * 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+        size = np.abs(wf).astype(np.float64)
+        if activation == "geglu":
+            with np.errstate(invalid="ignore", over="ignore"):
+                gv = ref.to_f32(gate, dtype).astype(np.float64) + (ref.to_f32(gb, dtype)[ids] if biased else 0.0)
+                uv = ref.to_f32(up, dtype).astype(np.float64) + (ref.to_f32(ub, dtype)[ids] if biased else 0.0)
+                size = size + np.nan_to_num(np.abs(0.5 * gv * uv), nan=0.0, posinf=0.0)
         off = np.abs(gf[~same].astype(np.float64) - wf[~same].astype(np.float64))
-        assert np.all(off <= step * np.abs(wf[~same]) + 2.0 ** -24), f"{what}: an output off by more than a step"
+        assert np.all(off <= step * size[~same] + 2.0 ** -24), f"{what}: an output off by more than a step"
 
     dboth = to_dev(both)
     dgate, dup = dboth[:, :hidden], dboth[:, hidden:]  # strided views: read in place
@@ -1154,7 +1168,7 @@ def test_gated_activation_against_the_oracle(dtype, activation):
     check(to_host(nv.glu(dgate.contiguous(), dup.contiguous(), activation, alpha=1.5, limit=5.0)),
           moe.glu(gate, up, dtype, act, 1.5, 5.0), f"{activation} {dtype} alpha 1.5 limit 5")
     got = nv.glu(dgate, dup, activation, gate_bias=to_dev(gb), up_bias=to_dev(ub), ids=torch.from_numpy(ids).cuda())
-    check(to_host(got), moe.glu(gate, up, dtype, act, gate_bias=gb, up_bias=ub, ids=ids), f"{activation} {dtype} with biases")
+    check(to_host(got), moe.glu(gate, up, dtype, act, gate_bias=gb, up_bias=ub, ids=ids), f"{activation} {dtype} with biases", biased=True)
     # batched shapes and the composition this library's SwitchGlu replaces: bias added by a separate rounded addition
     lead = nv.glu(dgate.reshape(3, 100, hidden), dup.reshape(3, 100, hidden), activation)
     assert tuple(lead.shape) == (3, 100, hidden) and lead.dtype == tdtype
@@ -1167,7 +1181,7 @@ def test_gated_activation_against_the_oracle(dtype, activation):
     with pytest.raises(nv.InvalidArgument):
         nv.glu(dgate, dup[:, :-1], activation)
     with pytest.raises(nv.InvalidArgument):
-        nv.glu(dgate, dup, "geglu")
+        nv.glu(dgate, dup, "reglu")
     with pytest.raises(nv.InvalidArgument):
         nv.glu(dgate, dup, activation, gate_bias=to_dev(gb))
     with pytest.raises(nv.InvalidArgument):
@@ -1176,8 +1190,25 @@ def test_gated_activation_against_the_oracle(dtype, activation):
         nv.glu(dgate, dup.to(torch.float64), activation)
 
 
+def test_gated_activations_equal_what_mlx_lm_recorded():
+    """The vectors of the reference's own test (crates/nuvec-nn/tests/rope_scaling.rs:150-172: mlx-lm's `swiglu_oai` and
+    `geglu` in float32 and bfloat16) under its own rule (rope_scaling.rs:37-43: 1e-6 and 1e-2 of max(|value|, 1))."""
+    import os
+
+    from safetensors.torch import load_file
+    recorded = load_file(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mlx_lm_activations.safetensors"))
+    for label, tol in (("f32", 1e-6), ("bf16", 1e-2)):
+        gate, x = recorded[f"act_{label}.gate"].cuda(), recorded[f"act_{label}.x"].cuda()
+        for name in ("swiglu_oai", "geglu"):
+            got = nv.glu(gate, x, name, alpha=1.702, limit=7.0).double().cpu()
+            want = recorded[f"act_{label}.{name}"].double()
+            ratio = (got - want).abs() / (tol * want.abs().clamp(min=1.0))
+            record_ratio(f"mlx-lm {label} {name}", float(ratio.max()), ratio.numel())
+            assert float(ratio.max()) <= 1.0, (label, name)
+
+
 @pytest.mark.parametrize("quant", ["MXFP4", "affine4", "affine8", "NVFP4"])
-@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai"])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai", "geglu"])
 def test_grouped_gather_with_the_gated_epilogue(quant, activation):
     """`nvq_gather_qmm_glu`: the gate and up products of the ordered pairs and the activation in one kernel, bit for bit
     the two grouped products (`nvq_gather_qmm`) followed by `nvq_glu`; experts without rows, with one pass of one tile
@@ -1213,7 +1244,7 @@ def test_grouped_gather_with_the_gated_epilogue(quant, activation):
         nv.gather_qmm_glu(x, nv.Quantized(both.weight[:, :320], both.scales[:, :320], None if both.biases is None else both.biases[:, :320], q_of),
                           rows, sorted_ids, offsets, activation)
     with pytest.raises(nv.InvalidArgument):
-        nv.gather_qmm_glu(x, both, rows, sorted_ids, offsets, "geglu")
+        nv.gather_qmm_glu(x, both, rows, sorted_ids, offsets, "reglu")
 
 
 @pytest.mark.parametrize("mode,qmode", [(ref.AFFINE, None), (ref.MXFP4, "MXFP4"), (ref.NVFP4, "NVFP4")])

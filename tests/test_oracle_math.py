@@ -282,3 +282,58 @@ def test_glu_equals_the_closed_forms(dtype):
         slack += np.abs(xc + 1.0) * np.abs(gc) * np.abs(alpha * gc) * eps / 4
         slack += tiny * (np.abs((xc + 1.0) * gc) + np.abs(xc + 1.0) + 1.0)
         assert np.all(np.abs(got - want) <= slack + 1e-30)
+
+
+def test_glu_equals_the_activations_mlx_lm_recorded():
+    """The reference's own test of its gated activations (crates/nuvec-nn/tests/rope_scaling.rs:150-172) holds what
+    mlx-lm computed for `swiglu_oai(gate, x, 1.702, 7)` and `geglu(gate, x)` in float32 and bfloat16 and asks for 1e-6
+    and 1e-2 of max(|value|, 1) for every element (its `close`).  The oracle meets those bounds; how many outputs agree bit for bit is
+    printed (MLX's GPU kernels evaluate the fused graph in float32 and round once, the reference's CPU path and the
+    oracle round after every operation)."""
+    import os
+
+    import torch
+    from safetensors.torch import load_file as load_torch
+
+    from oracle import moe
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mlx_lm_activations.safetensors")
+    recorded = load_torch(path)
+    for label, dtype, tol in (("f32", ref.F32, 1e-6), ("bf16", ref.BF16, 1e-2)):
+        def stored(name):
+            t = recorded[f"act_{label}.{name}"]
+            return t.numpy() if dtype == ref.F32 else t.view(torch.int16).numpy().view(np.uint16)
+        gate, x = stored("gate"), stored("x")
+        assert gate.shape == (4, 33)
+        for name, activation in (("swiglu_oai", moe.SWIGLU_OAI), ("geglu", moe.GEGLU)):
+            got = ref.to_f32(moe.glu(gate, x, dtype, activation, 1.702, 7.0), dtype).astype(np.float64)
+            want = ref.to_f32(stored(name), dtype).astype(np.float64)
+            ratio = np.abs(got - want) / (tol * np.maximum(np.abs(want), 1.0))  # the rule of the reference's `close` (rope_scaling.rs:37-43)
+            print(f"{label} {name}: worst difference {float(ratio.max()):.3f} x the bound, {int(np.count_nonzero(got == want))} of {want.size} equal")
+            assert float(ratio.max()) <= 1.0, (label, name)
+
+
+@pytest.mark.parametrize("dtype", [ref.F32, ref.F16, ref.BF16])
+def test_geglu_equals_the_closed_form(dtype):
+    """0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))) x in float64 with the constants as the element type holds them,
+    within the roundings of the eight operations; the cube of a 16-bit element is the correctly rounded one."""
+    from oracle import moe
+    rng = np.random.default_rng(60 + dtype)
+    eps = {ref.F32: 2.0 ** -23, ref.F16: 2.0 ** -10, ref.BF16: 2.0 ** -7}[dtype]
+    g = ref.from_f32((rng.standard_normal((29, 64)) * 3).astype(np.float32), dtype)
+    x = ref.from_f32((rng.standard_normal((29, 64)) * 3).astype(np.float32), dtype)
+    g64, x64 = ref.to_f32(g, dtype).astype(np.float64), ref.to_f32(x, dtype).astype(np.float64)
+    k1 = float(ref.to_f32(ref.from_f32(np.array([0.044715], np.float32), dtype), dtype)[0])
+    k2 = float(ref.to_f32(ref.from_f32(np.array([np.sqrt(2.0 / np.pi)], np.float32), dtype), dtype)[0])
+    inner = k2 * (g64 + k1 * g64 ** 3)
+    want = 0.5 * g64 * (1.0 + np.tanh(inner)) * x64
+    got = ref.to_f32(moe.glu(g, x, dtype, moe.GEGLU), dtype).astype(np.float64)
+    # the argument of tanh carries about four roundings (slope of tanh at most 1); 1 + tanh cancels for negative gates:
+    # its error is relative to 1, not to the sum
+    slack = 4 * eps * np.abs(want) + np.abs(0.5 * g64 * x64) * (4 * eps * np.abs(inner) * (1.0 - np.tanh(inner) ** 2) + 2 * eps)
+    tiny = 2.0 ** -24 if dtype == ref.F16 else 0.0
+    assert np.all(np.abs(got - want) <= slack + tiny * (np.abs(x64) + 1.0) + 1e-30)
+    if dtype != ref.F32:  # the cube: exact product, one rounding
+        cube = ref.to_f32(ref.from_f32((g64 ** 3).astype(np.float32), dtype), dtype)
+        again = ref.to_f32(ref.from_f32(np.power(ref.to_f32(g, dtype), np.float32(3.0)), dtype), dtype)
+        assert np.array_equal(cube, again)
+    assert np.isnan(ref.to_f32(moe.glu(ref.from_f32(np.array([[np.nan]], np.float32), dtype), x[:1, :1], dtype, moe.GEGLU), dtype)).all()
