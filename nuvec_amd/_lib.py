@@ -104,6 +104,7 @@ SIGNATURES = {
     "nvq_gather_qmm_scaled": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_gather_qmm_scatter": (C.c_int32, [C.c_void_p] * 13),
+    "nvq_gather_qmm_expert_bias": (C.c_int32, [C.c_void_p] * 14),
     "nvq_quantize_dequantize": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_moe_route": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_gather_qmm_glu": (C.c_int32, [C.POINTER(GatherDescC), C.c_int32, C.c_float, C.c_float] + [C.c_void_p] * 10),

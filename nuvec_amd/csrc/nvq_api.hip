@@ -753,7 +753,7 @@ int32_t nvq_glu(const nvq_glu_desc *d, const void *gate, const void *up, const v
     return launch_glu(*d, gate, up, gate_bias, up_bias, ids, out, (hipStream_t)stream);
 }
 
-struct GluEpilogue {
+struct GluEpilogue {  // activation < 0: no activation, only the experts' bias
     int32_t activation;
     float alpha, limit;
     const void *expert_bias;
@@ -784,6 +784,14 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(check_aligned("gather_qmm", "lhs", lhs, 4));
     NVQ_TRY(check_aligned("gather_qmm", "rhs", rhs, 4));
     NVQ_TRY(check_aligned("gather_qmm", "offsets", offsets, 4));
+    const void *expert_bias = nullptr;
+    if (glu != nullptr && glu->activation < 0) {  // the experts' bias alone: the grouped kernel's epilogue
+        expert_bias = glu->expert_bias;
+        glu = nullptr;
+        NVQ_TRY(check_aligned("gather_qmm", "expert bias", expert_bias, (size_t)dtype_size(d->dtype)));
+        if (expert_bias != nullptr && (!d->transpose || offsets == nullptr || d->m != 1 || d->k == 0))
+            return fail(NVQ_UNSUPPORTED, "gather_qmm: the experts' bias belongs to the grouped product of transposed weights");
+    }
     if (glu != nullptr) {
         if (glu->activation < NVQ_GLU_SWIGLU || glu->activation > NVQ_GLU_GEGLU)
             return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: unknown activation %d", glu->activation);
@@ -820,7 +828,9 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
         if (!qmf_supported(a)) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
         return launch_qmf(a, (hipStream_t)stream);
     }
+    a.expert_bias = expert_bias;
     if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
+    if (expert_bias != nullptr) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
     a.offsets = nullptr;
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
     // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
@@ -852,6 +862,15 @@ int32_t nvq_gather_qmm_scatter(const nvq_gather_desc *d, const void *x, const vo
     if (global_scales != nullptr && d != nullptr && d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
     return gather_qmm_any(d, x, w, scales, biases, global_scales, lhs, rhs, offsets, out_rows, y, workspace, stream);
+}
+
+int32_t nvq_gather_qmm_expert_bias(const nvq_gather_desc *d, const void *x, const void *w, const void *scales, const void *biases,
+                                   const float *global_scales, const uint32_t *lhs, const uint32_t *rhs, const int32_t *offsets,
+                                   const uint32_t *out_rows, const void *expert_bias, void *y, void *workspace, void *stream) {
+    if (d != nullptr && global_scales != nullptr && d->quant.mode != NVQ_NVFP4)  // quantized.rs:620-623
+        return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: global scale is only supported for 'nvfp4' quantization mode");
+    const GluEpilogue only_bias{-1, 0.0f, 0.0f, expert_bias};
+    return gather_qmm_any(d, x, w, scales, biases, global_scales, lhs, rhs, offsets, out_rows, y, workspace, stream, &only_bias);
 }
 
 int32_t nvq_gather_qmm_glu(const nvq_gather_desc *d, int32_t activation, float alpha, float limit, const void *x, const void *w,

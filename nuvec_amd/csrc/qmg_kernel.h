@@ -341,13 +341,18 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
             __syncthreads();  // the next pass stores x where the values were exchanged
             continue;
         }
+        // The expert's bias (crates/nuvec-lm/src/model.rs:2139-2143): added to the product as its output holds it, a
+        // separate rounded addition.
+        const bool biased = a.expert_bias != nullptr;
+        const float bias = biased && col < N ? Elem<T>::load((const T *)a.expert_bias, (int64_t)e * N + col) : 0.0f;
 #pragma unroll
         for (int u = 0; u < 2; u++)
 #pragma unroll
             for (int el = 0; el < 16; el++) {
                 const int m0 = 32 * u + 8 * (el >> 2) + (el & 3), m = m0 + 4 * h;
                 const uint32_t lo = __builtin_amdgcn_readlane(place, m0), hi = __builtin_amdgcn_readlane(place, m0 + 4);
-                if (m < rows && col < N) Elem<T>::store(y, (int64_t)(h ? hi : lo) * N + col, acc[u][el]);
+                const float v = biased ? Elem<T>::add(rounded<T>(acc[u][el]), bias) : acc[u][el];
+                if (m < rows && col < N) Elem<T>::store(y, (int64_t)(h ? hi : lo) * N + col, v);
             }
     }
 }

@@ -95,9 +95,10 @@ class SwitchProjection:
     biases: Optional[torch.Tensor]
     bias: Optional[torch.Tensor] = None
     quant: Quant = Quant()
+    global_scale: Optional[torch.Tensor] = None  # NVFP4: one float32 value per expert (model.rs:2095, quantized.rs:620-636)
 
     def quantized(self) -> Quantized:
-        return Quantized(self.weight, self.scales, self.biases, self.quant)
+        return Quantized(self.weight, self.scales, self.biases, self.quant, self.global_scale)
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False, add_bias: bool = True) -> torch.Tensor:
         """model.rs:2113-2146: `x` (`[..., 1, input_dims]` batches) through the experts `indices`."""
@@ -110,10 +111,13 @@ class SwitchProjection:
         `out_rows` (a permutation) result row i is written at row `out_rows[i]`.  `add_bias` False leaves the experts'
         bias to the caller (the gated activation adds it in its own pass)."""
         if rows is None:
-            rows = torch.arange(x.shape[0], dtype=torch.int32, device=x.device)
-        y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows)
+            rows = ops._identity(x.shape[0], x.device)
         if self.bias is None or not add_bias:
-            return y
+            return ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows)
+        try:  # the bias in the grouped kernel's epilogue
+            return ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows, expert_bias=self.bias)
+        except ops.Unsupported:  # (a product the grouped matrix-core kernel does not take: the addition on its own)
+            y = ops.gather_qmm_grouped(x, self.quantized(), rows, sorted_ids, offsets, out_rows)
         if out_rows is None:
             return y + self.bias[sorted_ids.long()]
         ids = torch.empty_like(sorted_ids)
@@ -155,6 +159,8 @@ class SwitchGlu:
         g, u = self.gate_proj, self.up_proj
         if g.quant != u.quant or g.weight.shape != u.weight.shape or (g.bias is None) != (u.bias is None):
             raise ops.InvalidArgument("fuse_gate_up: the gate and up projections differ in shape or quantization")
+        if g.global_scale is not None or u.global_scale is not None:
+            return self  # (NVFP4 with global scales: each projection has its own per expert)
         hidden = g.weight.shape[1]
         if g.quant.mode == ops.QuantMode.AFFINE and 512 <= hidden < 1024:
             # Affine products of fewer than 1024 outputs per row materialise the CPU's doubly rounded weights: one product

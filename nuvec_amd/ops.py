@@ -616,13 +616,16 @@ def _out_rows(op: str, given: Optional[torch.Tensor], pairs: int, device) -> Opt
 
 
 def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor,
-                       offsets: torch.Tensor, out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       offsets: torch.Tensor, out_rows: Optional[torch.Tensor] = None,
+                       expert_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The grouped route of `gather_qmm` (quantized.rs:646-651, 772-782) with the rows of x taken inside the kernel:
     output row i = x[rows[i]] . dequantize(w)[sorted_ids[i]]^T for ids sorted by expert (`offsets` from `moe_order`
     or `sorted_offsets`).  Equal to `gather_qmm(x[rows], q, None, sorted_ids, sorted)`; the gathered copy of x is
     never written.  x is `[T, K]`, the result `[len(rows), N]`.  With `out_rows` (a permutation, e.g. the `order` of
     `moe_order`) result row i is written at row `out_rows[i]`: the ordered product lands in pair order and
-    model.rs:2205-2210's `take(out, inverse)` is not needed."""
+    model.rs:2205-2210's `take(out, inverse)` is not needed.  `expert_bias` `[E, N]` adds each row's expert's bias
+    (model.rs:2139-2143) in the kernel's epilogue (`Unsupported` where the grouped kernel does not take the product).
+    NVFP4 experts carry their global scales (`q.global_scale`, one per expert)."""
     op = "gather_qmm"
     quant = q.quant
     quant.checked(op)
@@ -645,8 +648,23 @@ def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted
     out = torch.empty((rhs.numel(), w.shape[-2]), dtype=dtype, device=x.device)
     d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 0, 0, 1, w.shape[-2], columns, rhs.numel(), x.shape[0], w.shape[0])
     scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
+    gs = q.global_scale
+    if gs is not None:  # quantized.rs:620-636
+        if quant.mode != QuantMode.NVFP4:
+            raise InvalidArgument(f"{op}: global scale is only supported for 'nvfp4' quantization mode")
+        if gs.dtype != torch.float32 or gs.numel() != w.shape[0]:
+            raise InvalidArgument(f"{op}: global scale must be float32 with one entry per expert, got {_name(gs.dtype)} {list(gs.shape)}")
+        gs = gs.to(x.device).contiguous()
+    if expert_bias is not None and (expert_bias.dtype != dtype or tuple(expert_bias.shape) != (w.shape[0], w.shape[-2])):
+        raise InvalidArgument(f"{op}: the experts' bias must be [{w.shape[0]}, {w.shape[-2]}] of {_name(dtype)}")
+    if expert_bias is not None or gs is not None:  # the entry point with every optional operand
+        eb = expert_bias.contiguous() if expert_bias is not None else None
+        _lib.check(_lib.load().nvq_gather_qmm_expert_bias(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs),
+                                                          _ptr(lhs), _ptr(rhs), _ptr(offsets.contiguous()), _ptr(scatter),
+                                                          _ptr(eb), _ptr(out), _ptr(None), _stream()))
+        return out
     if scatter is not None:
-        _lib.check(_lib.load().nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(None),
+        _lib.check(_lib.load().nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs),
                                                       _ptr(lhs), _ptr(rhs), _ptr(offsets.contiguous()), _ptr(scatter),
                                                       _ptr(out), _ptr(None), _stream()))
         return out

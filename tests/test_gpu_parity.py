@@ -440,6 +440,58 @@ def test_grouped_gather_edge_cases():
     assert_rows_close(got, want, ref.BF16, "grouped affine")
 
 
+@pytest.mark.parametrize("quant", ["MXFP4", "affine4", "NVFP4-gs"])
+def test_grouped_gather_with_the_experts_bias(quant):
+    """`SwitchProjection::forward` on ordered pairs (model.rs:2113-2146): the product, then each row's expert's bias.  The
+    grouped kernel adds it in its epilogue (`nvq_gather_qmm_expert_bias`): bit for bit the product followed by the
+    separate rounded addition, with the rows in sorted order and scattered to their pairs' places; NVFP4 experts with a
+    global scale each take the same route.  Where the grouped kernel does not take the product the mirror adds the
+    bias itself."""
+    from nuvec_amd.layers import SwitchProjection
+    rng = np.random.default_rng(8100 + len(quant))
+    experts, n, k, pairs = 6, 1160, 512, 300
+    w = (torch.randn(experts, n, k, device="cuda") * 0.05).to(torch.bfloat16)
+    gs = None
+    if quant == "NVFP4-gs":
+        gs = to_dev(np.array([0.5, 2.0, 7.5, 1.0, 3.25, 0.75], np.float32))
+        parts = [nv.quantize(w[e], nv.QuantMode.NVFP4, gs[e]) for e in range(experts)]
+        q = nv.Quantized(torch.stack([p.weight for p in parts]), torch.stack([p.scales for p in parts]), None, parts[0].quant, gs)
+    else:
+        q = nv.quantize(w, nv.Quant.new(nv.QuantMode.MXFP4) if quant == "MXFP4" else nv.Quant.affine(64, 4))
+    bias = to_dev(make_x(rng, experts, n, ref.BF16))
+    x = to_dev(make_x(rng, 40, k, ref.BF16))
+    ids = torch.from_numpy(rng.integers(0, experts - 1, pairs).astype(np.int32)).cuda()  # (the last expert has no rows)
+    order, restore, sorted_ids, offsets = nv.moe_order(ids.reshape(1, pairs, 1), experts)
+    rows = torch.from_numpy(rng.integers(0, 40, pairs).astype(np.int32)).cuda()
+    plain = nv.gather_qmm_grouped(x, q, rows, sorted_ids, offsets)
+    if gs is not None:  # the grouped route with the experts' global scales equals the sorted gather of ops.gather_qmm
+        same = nv.gather_qmm(x[rows.long()].unsqueeze(1), q, None, sorted_ids, nv.GatherQmm(sorted_indices=True)).squeeze(1)
+        assert torch.equal(plain, same)
+        assert not torch.equal(plain, nv.gather_qmm_grouped(x, nv.Quantized(q.weight, q.scales, None, q.quant), rows, sorted_ids, offsets))
+    want = plain + bias[sorted_ids.long()]
+    got = nv.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, expert_bias=bias)
+    assert torch.equal(got, want), f"{quant}: the bias in the epilogue"
+    scattered = nv.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, out_rows=order, expert_bias=bias)
+    assert torch.equal(scattered[order.long()], want), f"{quant}: scattered rows"
+    proj = SwitchProjection(q.weight, q.scales, q.biases, bias, q.quant, gs)
+    assert torch.equal(proj.forward_sorted_rows(x, rows, sorted_ids, offsets), want)
+    assert torch.equal(proj.forward_sorted_rows(x, rows, sorted_ids, offsets, out_rows=order)[order.long()], want)
+    # the unsorted pairs of the same projection (the route of fewer than 64 pairs) against the ordered ones
+    few = proj.forward(x[rows.long()[:20]].reshape(20, 1, 1, k), sorted_ids[:20].reshape(20, 1)).reshape(20, n)
+    scale = float(want[:20].float().abs().max())
+    assert float((few.float() - want[:20].float()).abs().max()) <= 2e-2 * scale
+    # a product the grouped kernel does not take (K off its steps of 64): refused there, added by the mirror
+    if quant == "MXFP4":
+        q2 = nv.quantize(w[:, :, :96].contiguous(), nv.Quant.new(nv.QuantMode.MXFP4))
+        with pytest.raises(nv.Unsupported):
+            nv.gather_qmm_grouped(x[:, :96].contiguous(), q2, rows, sorted_ids, offsets, expert_bias=bias)
+        proj2 = SwitchProjection(q2.weight, q2.scales, None, bias, q2.quant)
+        y2 = proj2.forward_sorted_rows(x[:, :96].contiguous(), rows, sorted_ids, offsets)
+        assert torch.equal(y2, nv.gather_qmm_grouped(x[:, :96].contiguous(), q2, rows, sorted_ids, offsets) + bias[sorted_ids.long()])
+    with pytest.raises(nv.InvalidArgument):
+        nv.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, expert_bias=bias[:, :-1])
+
+
 @pytest.mark.parametrize("m", [3, 16, 33, 100])
 def test_few_rows_on_matrix_cores(m):
     """3 <= M < 128 of BASELINE's decode weights: one weight decode shared by all rows."""
