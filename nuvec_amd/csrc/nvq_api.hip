@@ -620,10 +620,10 @@ static int32_t check_attention(const nvq_attention_desc *d) {
     if (d->key_heads == 0 || d->query_heads % d->key_heads != 0)
         return fail(NVQ_INVALID_ARGUMENT, "%s: %lld query heads over %lld key heads", op, (long long)d->query_heads, (long long)d->key_heads);
     const int64_t rep = d->query_heads / d->key_heads;
-    if ((d->head_dim != 64 && d->head_dim != 128) || (d->bits != 4 && d->bits != 8) || d->head_dim % d->group_size != 0 ||
+    if ((d->head_dim != 64 && d->head_dim != 128) || (d->bits != 3 && d->bits != 4 && d->bits != 8) || d->head_dim % d->group_size != 0 ||
         !(rep == 1 || rep == 2 || rep == 4 || rep == 8) || d->positions < 1 || d->batch > 65535 ||
         d->batch * d->key_heads * d->positions * d->head_dim >= (1LL << 31))
-        return fail(NVQ_UNSUPPORTED, "%s: the kernel takes head sizes 64 and 128, 4 or 8 bits, 1, 2, 4 or 8 query heads per key head", op);
+        return fail(NVQ_UNSUPPORTED, "%s: the kernel takes head sizes 64 and 128, 3, 4 or 8 bits, 1, 2, 4 or 8 query heads per key head", op);
     return NVQ_OK;
 }
 

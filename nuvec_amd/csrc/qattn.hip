@@ -7,8 +7,8 @@
 // the float bound of the dequantized attention").
 //
 // A block of four wavefronts owns one (batch, query head).  A row of the cache is D bits / 8 bytes = CH chunks of 16
-// bytes; lane l of a wavefront takes chunk l % CH of key l / CH of the wavefront's current tile of 64 / CH keys, so a
-// wavefront-wide load reads 1 KB of consecutive rows.  Per key the lanes of a row form the score from their partial
+// bytes (3 bits: of 12 bytes, 32 codes); lane l of a wavefront takes chunk l % CH of key l / CH of the wavefront's
+// current tile of 64 / CH keys, so a wavefront-wide load reads 1 KB (768 bytes) of consecutive rows.  Per key the lanes of a row form the score from their partial
 // dot products (factored: scale * sum(q * code) + bias * sum(q) per chunk) with cross-lane adds, every lane keeps an
 // online softmax (running maximum, denominator) for the keys it has seen and accumulates its chunk of the output in
 // the same factored form; at the end the (64 / CH) x 4 partial states are merged through LDS.
@@ -21,12 +21,33 @@ namespace {
 
 constexpr int kAttnWaves = 4;
 
-// Code i of a 16-byte chunk (BITS 4: 32 codes, 8: 16 codes) as a float.
+// A lane's chunk of a row: 16 bytes (BITS 4: 32 codes, 8: 16 codes), or the 12 bytes that hold 32 codes of 3 bits.
+template <int BITS> struct Chunk { uint32_t w[BITS == 3 ? 3 : 4]; };
+
 template <int BITS>
-__device__ __forceinline__ float chunk_code(const uint4 &c, int i) {
-    const uint32_t w[4] = {c.x, c.y, c.z, c.w};
-    if constexpr (BITS == 4) return (float)((w[i >> 3] >> (4 * (i & 7))) & 15u);
-    else return (float)((w[i >> 2] >> (8 * (i & 3))) & 255u);
+__device__ __forceinline__ Chunk<BITS> load_chunk(const uint32_t *p) {
+    Chunk<BITS> c;
+    if constexpr (BITS == 3) {
+        c.w[0] = p[0], c.w[1] = p[1], c.w[2] = p[2];  // (rows of 3-bit codes are whole dwords: 4-byte aligned)
+    } else {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        c.w[0] = v.x, c.w[1] = v.y, c.w[2] = v.z, c.w[3] = v.w;
+    }
+    return c;
+}
+
+// Code i of a chunk as a float (i is a constant after unrolling).
+template <int BITS>
+__device__ __forceinline__ float chunk_code(const Chunk<BITS> &c, int i) {
+    if constexpr (BITS == 4) {
+        return (float)((c.w[i >> 3] >> (4 * (i & 7))) & 15u);
+    } else if constexpr (BITS == 8) {
+        return (float)((c.w[i >> 2] >> (8 * (i & 3))) & 255u);
+    } else {
+        const int bit = 3 * i, dw = bit >> 5, sh = bit & 31;
+        const uint32_t v = sh <= 29 ? c.w[dw] >> sh : (c.w[dw] >> sh) | (c.w[dw + 1] << (32 - sh));
+        return (float)(v & 7u);
+    }
 }
 
 // softmax's last step: the weighted sum over a maximum `top` and its denominator, with the head's sink if it has one.
@@ -43,12 +64,13 @@ __host__ __device__ inline int attention_split_keys(int64_t positions, int split
 }
 
 template <typename T, int BITS, int D>
-__global__ void __launch_bounds__(64 * kAttnWaves) qattn_kernel(const nvq_attention_desc d, const T *__restrict__ q, const uint4 *__restrict__ kw,
+__global__ void __launch_bounds__(64 * kAttnWaves) qattn_kernel(const nvq_attention_desc d, const T *__restrict__ q, const uint32_t *__restrict__ kw,
                                                                const T *__restrict__ ks, const T *__restrict__ kb,
-                                                               const uint4 *__restrict__ vw, const T *__restrict__ vs,
+                                                               const uint32_t *__restrict__ vw, const T *__restrict__ vs,
                                                                const T *__restrict__ vb, const T *__restrict__ sinks, T *__restrict__ out,
                                                                float *__restrict__ partials) {
-    constexpr int CPL = 128 / BITS;        // codes (values of D) per lane
+    constexpr int CPL = BITS == 3 ? 32 : 128 / BITS;  // codes (values of D) per lane
+    constexpr int CW = CPL * BITS / 32;               // dwords of a lane's chunk
     constexpr int CH = D / CPL;            // lanes per key: 2, 4 or 8
     constexpr int KPT = 64 / CH;           // keys per wavefront tile
     constexpr int kSlots = KPT * kAttnWaves;
@@ -78,14 +100,14 @@ __global__ void __launch_bounds__(64 * kAttnWaves) qattn_kernel(const nvq_attent
 
     // One tile of keys: everything it reads from memory.  The next tile is requested before the current one is computed.
     struct Tile {
-        uint4 kc, vc;
+        Chunk<BITS> kc, vc;
         T sk, bk, sv, bv;
     };
     auto fetch = [&](int s0) {
         const int s = s0 + j;
         const int64_t r = row0 + (s < s_end ? s : S - 1);  // a key past the end reads the last one and is given no weight
         Tile t;
-        t.kc = kw[r * CH + c], t.vc = vw[r * CH + c];
+        t.kc = load_chunk<BITS>(kw + (r * CH + c) * CW), t.vc = load_chunk<BITS>(vw + (r * CH + c) * CW);
         t.sk = ks[r * groups + gi], t.bk = kb[r * groups + gi], t.sv = vs[r * groups + gi], t.bv = vb[r * groups + gi];
         return t;
     };
@@ -167,8 +189,8 @@ int32_t run_attention_sized(const nvq_attention_desc &d, const void *q, const vo
                             const void *vs, const void *vb, const void *sinks, void *out, void *workspace, hipStream_t s) {
     const int splits = workspace != nullptr ? attention_splits(d) : 1;
     const dim3 grid((unsigned)d.query_heads, (unsigned)d.batch, (unsigned)splits), block(64 * kAttnWaves);
-    hipLaunchKernelGGL((qattn_kernel<T, BITS, D>), grid, block, 0, s, d, (const T *)q, (const uint4 *)kw, (const T *)ks, (const T *)kb,
-                       (const uint4 *)vw, (const T *)vs, (const T *)vb, (const T *)sinks, (T *)out, (float *)workspace);
+    hipLaunchKernelGGL((qattn_kernel<T, BITS, D>), grid, block, 0, s, d, (const T *)q, (const uint32_t *)kw, (const T *)ks, (const T *)kb,
+                       (const uint32_t *)vw, (const T *)vs, (const T *)vb, (const T *)sinks, (T *)out, (float *)workspace);
     NVQ_LAUNCH_CHECK("quantized_attention");
     if (splits > 1) {
         hipLaunchKernelGGL((qattn_merge_kernel<T, D>), dim3((unsigned)d.query_heads, (unsigned)d.batch), dim3(D), 0, s, d,
@@ -188,8 +210,9 @@ int32_t run_attention(const nvq_attention_desc &d, const void *q, const void *kw
 template <typename T>
 int32_t run_attention_bits(const nvq_attention_desc &d, const void *q, const void *kw, const void *ks, const void *kb, const void *vw,
                            const void *vs, const void *vb, const void *sinks, void *out, void *workspace, hipStream_t s) {
-    return d.bits == 4 ? run_attention<T, 4>(d, q, kw, ks, kb, vw, vs, vb, sinks, out, workspace, s)
-                       : run_attention<T, 8>(d, q, kw, ks, kb, vw, vs, vb, sinks, out, workspace, s);
+    return d.bits == 4   ? run_attention<T, 4>(d, q, kw, ks, kb, vw, vs, vb, sinks, out, workspace, s)
+           : d.bits == 3 ? run_attention<T, 3>(d, q, kw, ks, kb, vw, vs, vb, sinks, out, workspace, s)
+                         : run_attention<T, 8>(d, q, kw, ks, kb, vw, vs, vb, sinks, out, workspace, s);
 }
 
 }  // namespace

@@ -453,7 +453,7 @@ def quantized_attention_fits(q: torch.Tensor, k: Quantized, v: Quantized, sinks:
         return False
     b, hq, l, d = q.shape
     group, bits = k.quant.group_size, k.quant.bits
-    if q.dtype not in _FLOATS or l != 1 or d not in (64, 128) or bits not in (4, 8) or group not in (32, 64, 128) or d % group:
+    if q.dtype not in _FLOATS or l != 1 or d not in (64, 128) or bits not in (3, 4, 8) or group not in (32, 64, 128) or d % group:
         return False
     hkv, n = k.weight.shape[1], k.weight.shape[2]
     for t in (k, v):

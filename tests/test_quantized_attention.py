@@ -73,7 +73,8 @@ def test_quantized_attention_matches_the_recorded_outputs(recorded, dt, bits, l)
 @pytest.mark.gpu
 @pytest.mark.parametrize("batch,hq,hkv,s,d,bits,group,with_sinks", [
     (1, 32, 8, 8192, 128, 4, 64, False), (2, 8, 8, 1000, 64, 8, 32, True), (1, 4, 1, 777, 128, 8, 128, True),
-    (3, 16, 2, 2049, 64, 4, 64, False), (1, 2, 2, 513, 128, 4, 32, True)])
+    (3, 16, 2, 2049, 64, 4, 64, False), (1, 2, 2, 513, 128, 4, 32, True), (2, 8, 2, 1500, 128, 3, 64, True),
+    (1, 16, 16, 700, 64, 3, 32, False), (1, 4, 2, 61, 128, 3, 128, True)])
 def test_positions_split_over_the_grid(batch, hq, hkv, s, d, bits, group, with_sinks):
     """Long caches: the positions split over the grid and merged (with the workspace) against one block per head
     (without) and against float32 attention over the dequantized cache; lengths off the tile size, grouped heads,
