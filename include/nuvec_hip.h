@@ -366,10 +366,10 @@ NVQ_API int32_t nvq_glu(const nvq_glu_desc *desc, const void *gate, const void *
 
 /* nvq_gather_qmm_scatter with each row's expert's bias added in the kernel's epilogue (`SwitchProjection::forward`,
  * crates/nuvec-lm/src/model.rs:2139-2143: `y + bias[indices]`): y[z] = round(round(x[lhs[z]] . w[rhs[z]]^T) +
- * expert_bias[rhs[z]]), bit for bit the product followed by the separate addition.  expert_bias dtype[experts, n] or
- * NULL; out_rows and global_scales may be NULL.  The grouped route only (rows sorted by expert with `offsets`, m = 1,
- * transposed weights, a product the grouped matrix-core kernel takes); NVQ_UNSUPPORTED otherwise (the caller then adds
- * the bias after nvq_gather_qmm). */
+ * expert_bias[rhs[z]]), bit for bit the product followed by the separate addition, on the grouped route and on the
+ * routes of one product per pair alike.  expert_bias dtype[experts, n] or NULL; out_rows and global_scales may be
+ * NULL.  Weights stored [N, K] only (transpose = 1); else NVQ_UNSUPPORTED (the caller then adds the bias after
+ * nvq_gather_qmm). */
 NVQ_API int32_t nvq_gather_qmm_expert_bias(const nvq_gather_desc *desc, const void *x, const void *w, const void *scales,
                                    const void *biases, const float *global_scales, const uint32_t *lhs, const uint32_t *rhs,
                                    const int32_t *offsets, const uint32_t *out_rows, const void *expert_bias, void *y,

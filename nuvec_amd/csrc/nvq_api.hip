@@ -789,8 +789,8 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
         expert_bias = glu->expert_bias;
         glu = nullptr;
         NVQ_TRY(check_aligned("gather_qmm", "expert bias", expert_bias, (size_t)dtype_size(d->dtype)));
-        if (expert_bias != nullptr && (!d->transpose || offsets == nullptr || d->m != 1 || d->k == 0))
-            return fail(NVQ_UNSUPPORTED, "gather_qmm: the experts' bias belongs to the grouped product of transposed weights");
+        if (expert_bias != nullptr && (!d->transpose || d->k == 0))
+            return fail(NVQ_UNSUPPORTED, "gather_qmm: the experts' bias takes transposed weights and a reduction that is not empty");
     }
     if (glu != nullptr) {
         if (glu->activation < NVQ_GLU_SWIGLU || glu->activation > NVQ_GLU_GEGLU)
@@ -830,8 +830,12 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     }
     a.expert_bias = expert_bias;
     if (offsets != nullptr && qmf_supported(a)) return launch_qmf(a, (hipStream_t)stream);
-    if (expert_bias != nullptr) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
     a.offsets = nullptr;
+    if (expert_bias != nullptr) {  // one product per pair: the row-bias epilogue of those kernels, pair z taking row rhs[z]
+        a.expert_bias = nullptr;
+        a.row_bias = expert_bias;
+        a.row_bias_per_expert = 1;
+    }
     // Row-exact: every pair on the vector kernels, so that a pair has the bits of its one-row product whether the
     // gather is sorted or not and however many pairs it holds (the few-row contract of gpu.rs:7325-7340).
     if (!a.row_exact && takes_few_rows_direct(a)) return launch_qmd(a, (hipStream_t)stream);

@@ -88,6 +88,7 @@ struct ProductArgs {
     const uint32_t *out_rows;       // gather with the weights stored [N, K]: pair z writes block out_rows[z] of y (NULL: block z)
     const void *row_bias;           // NULL, or one value of the element type per column of y, added to the rounded product
                                     // (QuantizedLinear's bias)
+    int32_t row_bias_per_expert;    // gathered pairs: `row_bias` is [experts, n] and pair z takes row rhs[z] (SwitchProjection's bias)
     int32_t row_exact;              // every row takes the arithmetic of its one-row product: the vector kernels only, K split
                                     // (weights stored [K, N]) by the weight's shape alone
     // Affine codes, 16-bit elements, rows of few outputs: the kernels materialise the weights with the CPU's two roundings

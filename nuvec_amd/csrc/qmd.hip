@@ -168,7 +168,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     float *partial = reinterpret_cast<float *>(lds + (size_t)slices * ((RM * kQmdRowPieces + 1) * 16 + (kBlock ? 0 : SG * 64)));  // [2][RT][slices][RM][16] (chunked: one)
     const int m0 = blockIdx.y * RM;
     const bool batched = !(a.batch == 1 && a.rhs == nullptr);
-    const BatchOffsets o = batched ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
+    const BatchOffsets o = batched ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0, 0};
     const float factor = MODE == NVQ_NVFP4 ? qmf::nvfp4_factor(a, a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0) : 1.0f;
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
@@ -367,7 +367,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
 #pragma unroll 4
             for (int wv = 0; wv < slices; wv++) v += src[wv * RM * 16];
             const int col = (group_of(step) * RT + rt) * 16 + n;
-            if (m0 + m < M && col < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + col, add_row_bias<T>(a.row_bias, v, col));
+            if (m0 + m < M && col < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + col, add_row_bias<T>(a.row_bias, v, o.bias + col));
         }
     };
 

@@ -272,7 +272,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
     const int n0 = blockIdx.x * kRows;
 
     int row_begin, row_end;  // rows of x (and of y) this block multiplies
-    int64_t xo = 0, wo = 0, so = 0, yo = 0;
+    int64_t xo = 0, wo = 0, so = 0, yo = 0, bo = 0;
     row_begin = blockIdx.y * 32;
     row_end = row_begin + 32 < (int)a.m ? row_begin + 32 : (int)a.m;
     if (a.rhs != nullptr) {  // gathered pairs: pair z takes x batch lhs[z] and weight matrix rhs[z]
@@ -281,6 +281,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
         xo = l * a.m * K;
         wo = r * N * row_bytes;
         so = r * N * kgroups;
+        if (a.row_bias_per_expert) bo = r * N;
         yo = (a.out_rows != nullptr ? min((int64_t)a.out_rows[blockIdx.z], a.batch - 1) : (int64_t)blockIdx.z) * a.m * N;
     } else if (a.batch_ndim > 0) {
         xo = (int64_t)blockIdx.z * a.x_strides[0];
@@ -499,7 +500,7 @@ __global__ void __launch_bounds__(kThreads) qmf_kernel(const ProductArgs a) {
             const int l = idx & 63, v = (idx >> 6) % NV, rg = idx / (64 * NV);
             const float sum = ((slot_of(0, rg, v)[l] + slot_of(1, rg, v)[l]) + slot_of(2, rg, v)[l]) + slot_of(3, rg, v)[l];
             const int m = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), col = n0 + 32 * rg + (l & 31);
-            if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, add_row_bias<T>(a.row_bias, sum, col));
+            if (m < rows && col < N) Elem<T>::store(y, (int64_t)(pass + m) * N + col, add_row_bias<T>(a.row_bias, sum, bo + col));
         }
         __syncthreads();
     };

@@ -249,7 +249,7 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 #pragma unroll
     for (int i = 0; i < RM; i++) {
         const float v = wave_sum_lane63(acc[i]);
-        if (lane == 63 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, add_row_bias<T>(a.row_bias, v, n));
+        if (lane == 63 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, add_row_bias<T>(a.row_bias, v, o.bias + n));
     }
 }
 
@@ -283,7 +283,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     const int m0 = blockIdx.y * RM;
     const int kwords = (K * BITS) >> 5, kgroups = K >> gshift;
     // The single-product instantiation carries no batch arithmetic at all.
-    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
     using S = std::conditional_t<kAffine, T, uint8_t>;  // a scale as stored: the element type, or one byte (E8M0; NVFP4: E4M3)
@@ -455,7 +455,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
 #pragma unroll
         for (int i = 0; i < RM; i++) {
             const float v = wave_sum_lane63(acc[r][i]);
-            if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, add_row_bias<T>(a.row_bias, v, n0 + r));
+            if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, add_row_bias<T>(a.row_bias, v, o.bias + n0 + r));
         }
 }
 
@@ -497,7 +497,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
     constexpr int gshift = G128 ? 7 : 6;
     const int kwords = K >> 3, kgroups = K >> gshift, kchunks = K >> 3;  // dwords, groups, 16-byte x chunks per row
     const int n0 = blockIdx.x * kMmRows, m0 = blockIdx.y * RM;
-    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0};
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
     const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
@@ -678,7 +678,7 @@ __global__ void __launch_bounds__(kMmWaves * 64) qmv4_mfma_kernel(const ProductA
         float v = 0.0f;
 #pragma unroll
         for (int wv = 0; wv < kMmWaves; wv++) v += partial[(wv * RM + i) * kMmRows + col];
-        if (m0 + i < M && n0 + col < N) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + col, add_row_bias<T>(a.row_bias, v, n0 + col));
+        if (m0 + i < M && n0 + col < N) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + col, add_row_bias<T>(a.row_bias, v, o.bias + n0 + col));
     }
 }
 
@@ -735,7 +735,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
     const int N = (int)a.n, M = (int)a.m;
     const int kwords = K >> 3;
     const int n0 = blockIdx.x * kD16Rows * RT, m0 = blockIdx.y * RM;
-    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kGroups) : BatchOffsets{0, 0, 0, 0};
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kGroups) : BatchOffsets{0, 0, 0, 0, 0};
     const T *x = (const T *)a.x + o.x;
     const uint32_t *w = (const uint32_t *)a.w + o.w;
     const T *scales = (const T *)a.scales + o.s, *biases = (const T *)a.biases + o.s;
@@ -882,7 +882,7 @@ __global__ void __launch_bounds__(1024) qmv4_mm16_kernel(const ProductArgs a) {
         for (int wv = 0; wv < waves; wv++)
 #pragma unroll
             for (int q = 0; q < kQ; q++) v += src[wv * kMpl * 64 + 16 * q];
-        if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, add_row_bias<T>(a.row_bias, v, n0 + 16 * rt + n));
+        if (m0 + m < M && n0 + 16 * rt + n < N) Elem<T>::store(y, (int64_t)(m0 + m) * N + n0 + 16 * rt + n, add_row_bias<T>(a.row_bias, v, o.bias + n0 + 16 * rt + n));
     }
 }
 

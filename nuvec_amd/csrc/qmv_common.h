@@ -13,10 +13,10 @@ typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 
 // Element offsets of batch `z` for x, w (in packed dwords), scales/biases and y.
-struct BatchOffsets { int64_t x, w, s, y; };
+struct BatchOffsets { int64_t x, w, s, y, bias; };  // elements of x, dwords of w, scales, elements of y, of the row bias
 
 __device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int64_t z, int64_t kwords, int64_t kgroups) {
-    BatchOffsets o{0, 0, 0, z * a.m * a.n};
+    BatchOffsets o{0, 0, 0, z * a.m * a.n, 0};
     if (a.rhs != nullptr) {  // gathered pairs
         // An index outside its operand is the caller's error; it is clamped so that it cannot
         // fault the device.
@@ -24,6 +24,7 @@ __device__ __forceinline__ BatchOffsets batch_offsets(const ProductArgs &a, int6
         o.x = l * a.m * a.k;
         o.w = r * a.n * kwords;
         o.s = r * a.n * kgroups;
+        if (a.row_bias_per_expert) o.bias = r * a.n;
         if (a.out_rows != nullptr) o.y = min((int64_t)a.out_rows[z], a.batch - 1) * a.m * a.n;
         return o;
     }

@@ -102,8 +102,9 @@ class SwitchProjection:
 
     def forward(self, x: torch.Tensor, indices: torch.Tensor, sorted_indices: bool = False, add_bias: bool = True) -> torch.Tensor:
         """model.rs:2113-2146: `x` (`[..., 1, input_dims]` batches) through the experts `indices`."""
-        y = ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices))
-        return y if self.bias is None or not add_bias else y + self.bias[indices.long()].unsqueeze(-2)
+        if self.bias is None or not add_bias:
+            return ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices))
+        return ops.gather_qmm(x, self.quantized(), None, indices, ops.GatherQmm(sorted_indices=sorted_indices), expert_bias=self.bias)
 
     def forward_sorted_rows(self, x: torch.Tensor, rows, sorted_ids: torch.Tensor, offsets: torch.Tensor,
                             out_rows: Optional[torch.Tensor] = None, add_bias: bool = True) -> torch.Tensor:

@@ -755,10 +755,12 @@ def _indices(op: str, a: torch.Tensor, given: Optional[torch.Tensor]) -> torch.T
 
 def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor] = None,
                rhs_indices: Optional[torch.Tensor] = None, options: GatherQmm = GatherQmm(), *,
-               row_exact: bool = False, out_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+               row_exact: bool = False, out_rows: Optional[torch.Tensor] = None,
+               expert_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """ops.rs:1050-1074, quantized.rs:589-673: output batch i = x[lhs[i]] . dequantize(w)[rhs[i]]^T.  `out_rows` (not in
     the reference; one integer per pair, a permutation) writes batch i at position `out_rows[i]` of the flattened
-    batches instead."""
+    batches instead.  `expert_bias` `[E, N]` adds `bias[rhs[i]]` to every row of batch i in the kernels' epilogues
+    (`SwitchProjection::forward`, model.rs:2139-2143; weights stored [N, K] only)."""
     op = "gather_qmm"
     quant = q.quant
     quant.checked(op)
@@ -812,6 +814,13 @@ def gather_qmm(x: torch.Tensor, q: Quantized, lhs_indices: Optional[torch.Tensor
     scatter = _out_rows(op, out_rows, rhs.numel(), x.device)
     if scatter is not None and lhs_indices is None and rhs_indices is None:
         raise InvalidArgument(f"{op}: output rows need indices")
+    if expert_bias is not None:
+        if expert_bias.dtype != dtype or tuple(expert_bias.shape) != (experts, outer):
+            raise InvalidArgument(f"{op}: the experts' bias must be [{experts}, {outer}] of {_name(dtype)}")
+        _lib.check(lib.nvq_gather_qmm_expert_bias(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs), _ptr(lhs),
+                                                  _ptr(rhs), _ptr(offsets), _ptr(scatter), _ptr(expert_bias.contiguous()), _ptr(out),
+                                                  _ptr(workspace), _stream()))
+        return out
     if scatter is not None:
         _lib.check(lib.nvq_gather_qmm_scatter(C.byref(d), _ptr(x), _ptr(w), _ptr(scales), _ptr(biases), _ptr(gs), _ptr(lhs),
                                               _ptr(rhs), _ptr(offsets), _ptr(scatter), _ptr(out), _ptr(workspace), _stream()))

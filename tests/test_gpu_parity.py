@@ -445,8 +445,8 @@ def test_grouped_gather_with_the_experts_bias(quant):
     """`SwitchProjection::forward` on ordered pairs (model.rs:2113-2146): the product, then each row's expert's bias.  The
     grouped kernel adds it in its epilogue (`nvq_gather_qmm_expert_bias`): bit for bit the product followed by the
     separate rounded addition, with the rows in sorted order and scattered to their pairs' places; NVFP4 experts with a
-    global scale each take the same route.  Where the grouped kernel does not take the product the mirror adds the
-    bias itself."""
+    global scale each take the same route.  Unsorted pairs (and products the grouped kernel does not take) run pair by
+    pair with the bias in those kernels' epilogues."""
     from nuvec_amd.layers import SwitchProjection
     rng = np.random.default_rng(8100 + len(quant))
     experts, n, k, pairs = 6, 1160, 512, 300
@@ -477,17 +477,25 @@ def test_grouped_gather_with_the_experts_bias(quant):
     assert torch.equal(proj.forward_sorted_rows(x, rows, sorted_ids, offsets), want)
     assert torch.equal(proj.forward_sorted_rows(x, rows, sorted_ids, offsets, out_rows=order)[order.long()], want)
     # the unsorted pairs of the same projection (the route of fewer than 64 pairs) against the ordered ones
-    few = proj.forward(x[rows.long()[:20]].reshape(20, 1, 1, k), sorted_ids[:20].reshape(20, 1)).reshape(20, n)
+    xf, idf = x[rows.long()[:20]].reshape(20, 1, 1, k), sorted_ids[:20].reshape(20, 1)
+    few = proj.forward(xf, idf)
+    assert torch.equal(few, nv.gather_qmm(xf, q, None, idf) + bias[idf.long()].unsqueeze(-2)), f"{quant}: the bias in the per-pair kernels"
     scale = float(want[:20].float().abs().max())
-    assert float((few.float() - want[:20].float()).abs().max()) <= 2e-2 * scale
-    # a product the grouped kernel does not take (K off its steps of 64): refused there, added by the mirror
+    assert float((few.reshape(20, n).float() - want[:20].float()).abs().max()) <= 2e-2 * scale
+    for m in (3, 12, 40):  # several rows per pair: the few-row matrix-core kernels' epilogues
+        xm = to_dev(make_x(rng, 5 * m, k, ref.BF16)).reshape(5, m, k)
+        lhs, rhs = torch.tensor([4, 0, 2, 2], device="cuda"), torch.tensor([1, 3, 0, 3], device="cuda")
+        got_m = nv.gather_qmm(xm, q, lhs, rhs, expert_bias=bias)
+        assert torch.equal(got_m, nv.gather_qmm(xm, q, lhs, rhs) + bias[rhs].unsqueeze(-2)), f"{quant}: {m} rows per pair"
+    # a product the grouped kernel does not take (K off its steps of 64) runs pair by pair, the bias in those epilogues
     if quant == "MXFP4":
         q2 = nv.quantize(w[:, :, :96].contiguous(), nv.Quant.new(nv.QuantMode.MXFP4))
-        with pytest.raises(nv.Unsupported):
-            nv.gather_qmm_grouped(x[:, :96].contiguous(), q2, rows, sorted_ids, offsets, expert_bias=bias)
         proj2 = SwitchProjection(q2.weight, q2.scales, None, bias, q2.quant)
         y2 = proj2.forward_sorted_rows(x[:, :96].contiguous(), rows, sorted_ids, offsets)
         assert torch.equal(y2, nv.gather_qmm_grouped(x[:, :96].contiguous(), q2, rows, sorted_ids, offsets) + bias[sorted_ids.long()])
+        with pytest.raises(nv.Unsupported):  # weights stored [K, N]
+            nv.gather_qmm(torch.randn(4, 1, n, device="cuda").to(torch.bfloat16), q, None, torch.tensor([0, 1, 2, 3], device="cuda"),
+                          nv.GatherQmm(transpose=False), expert_bias=bias[:, :k].contiguous())
     with pytest.raises(nv.InvalidArgument):
         nv.gather_qmm_grouped(x, q, rows, sorted_ids, offsets, expert_bias=bias[:, :-1])
 
