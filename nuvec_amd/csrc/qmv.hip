@@ -253,6 +253,98 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
     }
 }
 
+// What a lane of the decode kernels reads of the scales of its 32 values: the element (affine), NVFP4's two bytes at
+// once, or one byte.
+template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
+
+// A lane's slice of 32 values of one weight row against the same slice of RM rows of x (xp: the four pieces of eight
+// values as pairs, in the expansion's pair order for affine codes and in memory order for the block formats; xs: the
+// slices' sums, affine only), added to acc.  Affine: scale * (dot - B * sum x) + bias * sum x with the codes entered as
+// B + c.  Block formats: the conversion instructions give the code values, the group's float32 scale (NVFP4: two
+// groups) multiplies the group's sum.
+template <typename T, int RM, int MODE>
+__device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 ? 2 : 1], typename SliceScale<T, MODE>::type sraw, T braw,
+                                          const uint4 (&xp)[RM][4], const float (&xs)[RM], float factor, uint32_t mask, uint32_t magic,
+                                          float (&acc)[RM]) {
+    constexpr int BITS = MODE == NVQ_MXFP8 ? 8 : 4;
+    constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;
+    if constexpr (MODE == NVQ_AFFINE) {
+        const uint32_t d[4] = {wq[0].x, wq[0].y, wq[0].z, wq[0].w};
+        float dot[RM][4];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t p0 = and_or(d[j], mask, magic), p1 = and_or(d[j] >> 4, mask, magic);
+            const uint32_t p2 = and_or(d[j] >> 8, mask, magic), p3 = and_or(d[j] >> 12, mask, magic);
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+            }
+        }
+        const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
+        const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+            acc[i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[i]));
+        }
+    } else {
+        // piece j of the lane's slice: eight values, the pairs of xp[i][j] in memory order
+        float dot[RM][kHalves][2];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int hf = 0; hf < kHalves; hf++) dot[i][hf][0] = dot[i][hf][1] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            constexpr int kPiecesPerHalf = 4 / kHalves;
+            const int hf = j / kPiecesPerHalf;
+            uint32_t p0, p1, p2, p3;
+            if constexpr (BITS == 4) {
+                const uint4 q = wq[0];
+                const uint32_t d = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+                p0 = qmf::Ops<T>::template fp4_pair<0>(d, 1.0f);
+                p1 = qmf::Ops<T>::template fp4_pair<1>(d, 1.0f);
+                p2 = qmf::Ops<T>::template fp4_pair<2>(d, 1.0f);
+                p3 = qmf::Ops<T>::template fp4_pair<3>(d, 1.0f);
+            } else {
+                const uint4 q = wq[j >> 1];
+                const uint32_t d0 = (j & 1) ? q.z : q.x, d1 = (j & 1) ? q.w : q.y;
+                p0 = qmf::Ops<T>::template fp8_pair<false>(d0, 1.0f);
+                p1 = qmf::Ops<T>::template fp8_pair<true>(d0, 1.0f);
+                p2 = qmf::Ops<T>::template fp8_pair<false>(d1, 1.0f);
+                p3 = qmf::Ops<T>::template fp8_pair<true>(d1, 1.0f);
+            }
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][hf][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][hf][0]);
+                dot[i][hf][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][hf][1]);
+                dot[i][hf][0] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][hf][0]);
+                dot[i][hf][1] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][hf][1]);
+            }
+        }
+        float sc[2];
+        if constexpr (MODE == NVQ_NVFP4) {
+            // both E4M3 scales by one conversion (every E4M3 value is a normal float32 or zero); times the
+            // global scale's factor as crates/nuvec-core/src/kernels.rs:992-998
+            const auto two = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8((uint32_t)sraw, 1.0f, false);
+            sc[0] = ftz(two[0] * factor), sc[1] = ftz(two[1] * factor);
+        } else {
+            sc[0] = sc[1] = ftz(e8m0_to_f32(sraw));
+        }
+#pragma unroll
+        for (int hf = 0; hf < kHalves; hf++)
+#pragma unroll
+            for (int i = 0; i < RM; i++) acc[i] = __builtin_fmaf(sc[hf], dot[i][hf][0] + dot[i][hf][1], acc[i]);
+    }
+}
+
 // ── 4-bit affine and the block formats, bf16 / f16, one to four rows of x: the decode kernel ───────────
 // A block of WAVES wavefronts shares the x slice of one K step (4096 values) through LDS, stored
 // once in the pair order the codes need (affine: together with the sums of its 32-value slices), so the
@@ -314,9 +406,9 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                                                       : make_uint4(0, 0, 0, 0);  // absent x: contributes nothing
             }
         uint4 wq[2][RN][kQuads];
-        using SR = std::conditional_t<MODE == NVQ_NVFP4, uint16_t, S>;  // what a lane reads of the scales: NVFP4's two bytes at once
+        using SR = typename SliceScale<T, MODE>::type;
         SR sraw[2][RN];
-        S braw[2][RN];
+        T braw[2][RN];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const int kb = k0 + u * kStep + lane * 32;
@@ -331,6 +423,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 for (int c = 0; c < kQuads; c++) wq[u][r][c] = stream_load(pw + c);
                 sraw[u][r] = *reinterpret_cast<const SR *>(scales + (int64_t)n * kgroups + (kc >> gshift));
                 if constexpr (kAffine) braw[u][r] = (biases + (int64_t)n * kgroups)[kc >> gshift];
+                else braw[u][r] = T{};
             }
         }
         if (k0 != 0) __syncthreads();  // the previous step's readers are done with the LDS
@@ -368,86 +461,10 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
 #pragma unroll
                 for (int j = 0; j < 4; j++) xp[i][j] = x_pairs[i][u][j][lane];
                 if constexpr (kAffine) xs[i] = x_sums[i][u][lane];
+                else xs[i] = 0.0f;
             }
 #pragma unroll
-            for (int r = 0; r < RN; r++) {
-                if constexpr (kAffine) {
-                    const uint32_t d[4] = {wq[u][r][0].x, wq[u][r][0].y, wq[u][r][0].z, wq[u][r][0].w};
-                    float dot[RM][4];
-#pragma unroll
-                    for (int i = 0; i < RM; i++)
-#pragma unroll
-                        for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const uint32_t p0 = and_or(d[j], mask, magic), p1 = and_or(d[j] >> 4, mask, magic);
-                        const uint32_t p2 = and_or(d[j] >> 8, mask, magic), p3 = and_or(d[j] >> 12, mask, magic);
-#pragma unroll
-                        for (int i = 0; i < RM; i++) {
-                            dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
-                            dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
-                            dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
-                            dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
-                        }
-                    }
-                    // scale * (dot - B * sum x) + bias * sum x
-                    const float sc = Elem<T>::load(&sraw[u][r], 0), bi = Elem<T>::load(&braw[u][r], 0);
-                    const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
-#pragma unroll
-                    for (int i = 0; i < RM; i++) {
-                        const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
-                        acc[r][i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[r][i]));
-                    }
-                } else {
-                    // piece j of the lane's slice: eight values, the pairs of xp[i][j] in memory order
-                    float dot[RM][kHalves][2];
-#pragma unroll
-                    for (int i = 0; i < RM; i++)
-#pragma unroll
-                        for (int hf = 0; hf < kHalves; hf++) dot[i][hf][0] = dot[i][hf][1] = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        constexpr int kPiecesPerHalf = 4 / kHalves;
-                        const int hf = j / kPiecesPerHalf;
-                        uint32_t p0, p1, p2, p3;
-                        if constexpr (BITS == 4) {
-                            const uint4 q = wq[u][r][0];
-                            const uint32_t d = j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
-                            p0 = qmf::Ops<T>::template fp4_pair<0>(d, 1.0f);
-                            p1 = qmf::Ops<T>::template fp4_pair<1>(d, 1.0f);
-                            p2 = qmf::Ops<T>::template fp4_pair<2>(d, 1.0f);
-                            p3 = qmf::Ops<T>::template fp4_pair<3>(d, 1.0f);
-                        } else {
-                            const uint4 q = wq[u][r][j >> 1];
-                            const uint32_t d0 = (j & 1) ? q.z : q.x, d1 = (j & 1) ? q.w : q.y;
-                            p0 = qmf::Ops<T>::template fp8_pair<false>(d0, 1.0f);
-                            p1 = qmf::Ops<T>::template fp8_pair<true>(d0, 1.0f);
-                            p2 = qmf::Ops<T>::template fp8_pair<false>(d1, 1.0f);
-                            p3 = qmf::Ops<T>::template fp8_pair<true>(d1, 1.0f);
-                        }
-#pragma unroll
-                        for (int i = 0; i < RM; i++) {
-                            dot[i][hf][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][hf][0]);
-                            dot[i][hf][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][hf][1]);
-                            dot[i][hf][0] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][hf][0]);
-                            dot[i][hf][1] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][hf][1]);
-                        }
-                    }
-                    float sc[2];
-                    if constexpr (MODE == NVQ_NVFP4) {
-                        // both E4M3 scales by one conversion (every E4M3 value is a normal float32 or zero); times the
-                        // global scale's factor as crates/nuvec-core/src/kernels.rs:992-998
-                        const auto two = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8((uint32_t)sraw[u][r], 1.0f, false);
-                        sc[0] = ftz(two[0] * factor), sc[1] = ftz(two[1] * factor);
-                    } else {
-                        sc[0] = sc[1] = ftz(e8m0_to_f32(sraw[u][r]));
-                    }
-#pragma unroll
-                    for (int hf = 0; hf < kHalves; hf++)
-#pragma unroll
-                        for (int i = 0; i < RM; i++) acc[r][i] = __builtin_fmaf(sc[hf], dot[i][hf][0] + dot[i][hf][1], acc[r][i]);
-                }
-            }
+            for (int r = 0; r < RN; r++) slice_dot<T, RM, MODE>(wq[u][r], sraw[u][r], braw[u][r], xp, xs, factor, mask, magic, acc[r]);
         }
     }
 #pragma unroll
@@ -459,6 +476,111 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
         }
 }
 
+
+// ── The same for short rows: K up to 2048 ──────────────────────────────────────────────────────────────
+// The decode kernel above gives a weight row to a wavefront, 32 values a lane: a row of K < 2048 values leaves lanes
+// (and the second of its two loads) without work.  Here a row takes L lanes, L the power of two that covers K / 32
+// (8 to 64), so a wavefront holds 64 / L rows at once and two such sets in flight; x (all of K) is staged once per
+// block, and the L partial sums of a row are added with a butterfly of cross-lane moves inside its L lanes.
+template <typename T, int RM, int L, bool BATCHED, int MODE>
+__global__ void __launch_bounds__(512) qmv4_short_kernel(const ProductArgs a) {
+    constexpr int kWaves = 8;
+    constexpr int kSub = 64 / L;                 // rows of a wavefront's set
+    constexpr int kRowsPerWave = 2 * kSub, kRowsPerBlock = kWaves * kRowsPerWave;
+    constexpr bool kAffine = MODE == NVQ_AFFINE;
+    constexpr int BITS = MODE == NVQ_MXFP8 ? 8 : 4;
+    constexpr int kQuads = BITS / 4;
+    __shared__ uint4 x_pairs[RM][4][L];              // [row][word][slice]: 4 pairs of eight values
+    __shared__ float x_sums[kAffine ? RM : 1][L];    // [row][slice]: sum of the slice's 32 values (affine)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane / L, kl = lane % L;
+    const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
+    const int gshift = kAffine ? (a.group == 32 ? 5 : a.group == 64 ? 6 : 7) : (MODE == NVQ_NVFP4 ? 4 : 5);
+    const int n_base = (blockIdx.x * kWaves + wave) * kRowsPerWave + sub;
+    const int m0 = blockIdx.y * RM;
+    const int kwords = (K * BITS) >> 5, kgroups = K >> gshift;
+    const BatchOffsets o = BATCHED ? batch_offsets(a, blockIdx.z, kwords, kgroups) : BatchOffsets{0, 0, 0, 0, 0};
+    const T *x = (const T *)a.x + o.x;
+    const uint32_t *w = (const uint32_t *)a.w + o.w;
+    using S = std::conditional_t<kAffine, T, uint8_t>;
+    using SR = typename SliceScale<T, MODE>::type;
+    const S *scales = (const S *)a.scales + o.s, *biases = kAffine ? (const S *)a.biases + o.s : nullptr;
+    T *y = (T *)a.y + o.y;
+    constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
+    uint32_t mask, magic;
+    asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
+    float factor = 1.0f;
+    if constexpr (MODE == NVQ_NVFP4) factor = qmf::nvfp4_factor(a, BATCHED && a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0);
+
+    // x first: thread t < 4 L holds piece t (eight values) of every row of x; pieces past K are zero
+    uint4 xg[RM];
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+        xg[i] = (tid * 8 < K && m0 + i < M) ? *reinterpret_cast<const uint4 *>(x + (int64_t)(m0 + i) * K + tid * 8) : make_uint4(0, 0, 0, 0);
+    const int kc = kl * 32 < K ? kl * 32 : 0;  // an absent slice reads valid memory; its x is zero
+    uint4 wq[2][kQuads];
+    SR sraw[2];
+    T braw[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int n = n_base + u * kSub < N ? n_base + u * kSub : N - 1;  // tail rows are computed, not stored
+        const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
+#pragma unroll
+        for (int c = 0; c < kQuads; c++) wq[u][c] = stream_load(pw + c);
+        sraw[u] = *reinterpret_cast<const SR *>(scales + (int64_t)n * kgroups + (kc >> gshift));
+        if constexpr (kAffine) braw[u] = (biases + (int64_t)n * kgroups)[kc >> gshift];
+        else braw[u] = T{};
+    }
+    if (tid < 4 * L) {
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const uint4 q = xg[i];  // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
+            if constexpr (kAffine) {
+                uint4 pr;
+                pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+                pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+                pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+                pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+                x_pairs[i][tid & 3][tid >> 2] = pr;
+                float sum = Pair<T>::dot2(pr.x, ones, 0.0f);
+                sum = Pair<T>::dot2(pr.y, ones, sum);
+                sum = Pair<T>::dot2(pr.z, ones, sum);
+                sum = Pair<T>::dot2(pr.w, ones, sum);
+                sum += __shfl_xor(sum, 1);  // the four pieces of a slice sit in adjacent threads
+                sum += __shfl_xor(sum, 2);
+                if ((tid & 3) == 0) x_sums[i][tid >> 2] = sum;
+            } else {
+                x_pairs[i][tid & 3][tid >> 2] = q;
+            }
+        }
+    }
+    __syncthreads();
+    uint4 xp[RM][4];
+    float xs[RM];
+#pragma unroll
+    for (int i = 0; i < RM; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) xp[i][j] = x_pairs[i][j][kl];
+        if constexpr (kAffine) xs[i] = x_sums[i][kl];
+        else xs[i] = 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        float acc[RM];
+#pragma unroll
+        for (int i = 0; i < RM; i++) acc[i] = 0.0f;
+        slice_dot<T, RM, MODE>(wq[u], sraw[u], braw[u], xp, xs, factor, mask, magic, acc);
+        const int n = n_base + u * kSub;
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            float v = acc[i];
+#pragma unroll
+            for (int off = 1; off < L; off <<= 1) v += __shfl_xor(v, off);  // (inside the row's L lanes)
+            if (kl == 0 && n < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n, add_row_bias<T>(a.row_bias, v, o.bias + n));
+        }
+    }
+}
 
 // ── 4-bit affine, bf16 / f16, up to four rows of x, groups of 64 or 128: decode on the matrix cores ──────
 // The vector units only turn nibbles into elements (one v_and_or_b32 per two codes, the magic-number form
@@ -1003,6 +1125,40 @@ inline bool block_decode_takes(const ProductArgs &a) {
     return a.k <= 4096 && (a.m == 3 || a.mode == NVQ_MXFP8);
 }
 
+// Whether the short-row decode kernel takes the product: the pairs of a gather (the experts of decoded tokens, whose
+// down projections have short rows) with 4-bit affine codes (never materialised: not with exact weights) or a block
+// format the decode kernel takes, bf16 / f16, up to four rows of x, K up to 2048 in whole slices.  Measured, 32 pairs of
+// one row against the kernels above (us): 4-bit g64 W[2048,512] 28.8 -> 8.5, W[2048,768] 29.0 -> 12.1, W[4096,1408]
+// 54.5 -> 34.9; MXFP4 W[2048,768] 24.8 -> 11.3, W[2048,1024] 24.7 -> 11.9, W[2048,2048] 25.4 -> 19.8, W[4096,1408]
+// 46.1 -> 32.3; MXFP8 W[2048,1024] 25.6 -> 18.0.  Where the 16x16x32 decode kernel takes affine pairs it stays ahead
+// (W[2048,1024] 11.2 against 12.7, W[2048,2048] 16.5 against 21.4), and single products gain nothing (a launch either way).
+inline bool short_decode_takes(const ProductArgs &a) {
+    if (a.rhs == nullptr || a.dtype == NVQ_F32 || a.row_exact || a.k > 2048 || a.k % 32 != 0 || a.m < 1 || a.m > 4) return false;
+    if (a.mode != NVQ_AFFINE) return block_decode_takes(a);
+    return a.bits == 4 && !a.exact_weights && !d16_takes(a) && (uintptr_t)a.w % 16 == 0 && (uintptr_t)a.x % 16 == 0;
+}
+
+template <typename T, int MODE, int L>
+int32_t run_short_lanes(const ProductArgs &a, hipStream_t s) {
+    constexpr int kRowsPerBlock = 8 * 2 * (64 / L);
+    const int rm = a.m == 1 ? 1 : a.m == 2 ? 2 : 4;
+    const dim3 grid((unsigned)((a.n + kRowsPerBlock - 1) / kRowsPerBlock), (unsigned)((a.m + rm - 1) / rm), (unsigned)a.batch);
+    void (*kernel)(const ProductArgs) = rm == 1   ? qmv4_short_kernel<T, 1, L, true, MODE>
+                                        : rm == 2 ? qmv4_short_kernel<T, 2, L, true, MODE>
+                                                  : qmv4_short_kernel<T, 4, L, true, MODE>;
+    hipLaunchKernelGGL(kernel, grid, dim3(512), 0, s, a);
+    NVQ_LAUNCH_CHECK("qmv4_short");
+    return NVQ_OK;
+}
+
+template <typename T, int MODE>
+int32_t run_short(const ProductArgs &a, hipStream_t s) {
+    const int slices = (int)(a.k / 32);
+    if (slices <= 16) return run_short_lanes<T, MODE, 16>(a, s);
+    if (slices <= 32) return run_short_lanes<T, MODE, 32>(a, s);
+    return run_short_lanes<T, MODE, 64>(a, s);
+}
+
 template <typename T, int MODE>
 int32_t run_block_decode(const ProductArgs &a, hipStream_t s) {
     if (a.m == 1) return run_lds4<T, 1, 1, 8, MODE>(a, s);
@@ -1032,6 +1188,12 @@ int32_t run_general(const ProductArgs &a, hipStream_t s) {
 template <typename T>
 int32_t run_typed(const ProductArgs &a, hipStream_t s) {
     if constexpr (!std::is_same<T, float>::value) {
+        if (short_decode_takes(a)) {
+            if (a.mode == NVQ_MXFP4) return run_short<T, NVQ_MXFP4>(a, s);
+            if (a.mode == NVQ_MXFP8) return run_short<T, NVQ_MXFP8>(a, s);
+            if (a.mode == NVQ_NVFP4) return run_short<T, NVQ_NVFP4>(a, s);
+            return run_short<T, NVQ_AFFINE>(a, s);
+        }
         if (block_decode_takes(a)) {
             if (a.mode == NVQ_MXFP4) return run_block_decode<T, NVQ_MXFP4>(a, s);
             if (a.mode == NVQ_MXFP8) return run_block_decode<T, NVQ_MXFP8>(a, s);
@@ -1078,10 +1240,12 @@ bool qmv_block_decode_takes(const ProductArgs &a) { return block_decode_takes(a)
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
     if (a.mode == NVQ_AFFINE && a.bits == 4 && a.dtype != NVQ_F32 && !a.exact_weights) {
+        if (short_decode_takes(a)) return "qmv4_short_kernel";
         if (!a.row_exact && d16_takes(a)) return "qmv4_mm16_kernel";
         if (!a.row_exact && a.m >= 4 && mfma_decode_takes<4>(a)) return "qmv4_mfma_kernel";
         return "qmv4_lds_kernel";
     }
+    if (short_decode_takes(a)) return "qmv4_short_kernel";
     if (block_decode_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }

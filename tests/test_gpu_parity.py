@@ -680,6 +680,41 @@ def test_block_formats_on_the_decode_kernel(mode, qmode, dtype):
         assert_rows_close(got[z], want, dtype, f"decode kernel {qmode} pair {z}", exact_weights=True)
 
 
+@pytest.mark.parametrize("quant", ["affine4-g32", "affine4-g64", "affine4-g128", "MXFP4", "MXFP8", "NVFP4"])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_short_rows_of_gathered_pairs(quant, dtype):
+    """Unsorted pairs of one to four rows against weight rows of up to 2048 values (the down projections of a decoded
+    token's experts): the short-row decode kernel, a weight row on 16, 32 or 64 lanes.  K on and off the lanes' powers
+    of two, weight rows off the block's count, every pair against the oracle's product; the experts' bias in the
+    epilogue bit for bit the separate addition."""
+    rng = np.random.default_rng(4900 + len(quant) + dtype)
+    affine = quant.startswith("affine")
+    group = int(quant.split("g")[1]) if affine else None
+    mode = ref.AFFINE if affine else getattr(ref, quant)
+    q_of = nv.Quant.affine(group, 4) if affine else nv.Quant.new(getattr(nv.QuantMode, quant))
+    fgroup, bits = (group, 4) if affine else ref.FP_PARAMS[mode]
+    experts = 5
+    for m, n, k in [(1, 1030, 768), (2, 1061, 384), (3, 1024, 1408), (4, 1100, 2048), (1, 1025, 128), (1, 1040, 1152)]:
+        w = make_w(rng, experts * n, k, dtype)
+        if affine:
+            packed, scales, biases = ref.affine_quantize(w, dtype, group, 4)
+        else:
+            (packed, scales), biases = ref.fp_quantize(w, dtype, mode), None
+        q = nv.Quantized(to_dev(packed.reshape(experts, n, -1)), to_dev(scales.reshape(experts, n, -1)),
+                         None if biases is None else to_dev(biases.reshape(experts, n, -1)), q_of)
+        x = make_x(rng, 3 * m, k, dtype)
+        lhs, rhs = np.array([2, 0, 1, 1, 0, 2, 2], np.int64), np.array([4, 0, 3, 3, 1, 0, 2], np.int64)
+        got = nv.gather_qmm(to_dev(x.reshape(3, m, k)), q, torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda())
+        for z in range(lhs.size):
+            e, i = int(rhs[z]), int(lhs[z])
+            want = ref.quantized_matmul(x[i * m:(i + 1) * m], packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n],
+                                        None if biases is None else biases[e * n:(e + 1) * n], mode=mode, group=fgroup, bits=bits, dtype=dtype)
+            assert_rows_close(to_host(got[z]), want, dtype, f"short rows {quant} M={m} N={n} K={k} pair {z}", exact_weights=not affine)
+        bias = to_dev(make_x(rng, experts, n, dtype))
+        with_bias = nv.gather_qmm(to_dev(x.reshape(3, m, k)), q, torch.from_numpy(lhs).cuda(), torch.from_numpy(rhs).cuda(), expert_bias=bias)
+        assert torch.equal(with_bias, got + bias[torch.from_numpy(rhs).cuda()].unsqueeze(-2))
+
+
 @pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
 def test_block_formats_at_every_scale_code(mode, qmode):
     """Every scale code on every product route: weight row n carries scale code n in all its groups (E8M0: 2^(n - 127), zero
