@@ -813,7 +813,14 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.out_rows = out_rows;
     a.row_exact = d->row_exact != 0;
     a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
-    if (!d->transpose) return launch_qvm(a, workspace, (hipStream_t)stream);  // weights stored [K, N]: one product per pair
+    if (!d->transpose) {
+        // Weights stored [K, N]: rows sorted by expert as groups on the matrix-core kernel (each expert's weights read once
+        // per tile of its rows; the reference's grouped kernel of the block formats, gpu.rs:6786-6812), else one product
+        // per pair.
+        a.offsets = offsets;
+        if (!qvm_takes_grouped(a)) a.offsets = nullptr;
+        return launch_qvm(a, workspace, (hipStream_t)stream);
+    }
     // Grouped route (rows sorted by expert, offsets given): each expert's rows against its weights, every
     // weight decoded once.  Otherwise one product per pair, on the kernel a single product of that many rows takes:
     // the few-row matrix-core kernels, or the decode kernels of the vector units (the experts of one decoded token are

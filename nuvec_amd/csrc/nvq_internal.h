@@ -128,6 +128,7 @@ int32_t launch_calibrate(int32_t kind, const void *buffer, int64_t bytes, int32_
 int qvm_splits(const ProductArgs &a);
 size_t qvm_workspace_bytes(const ProductArgs &a);
 int32_t launch_qvm(const ProductArgs &a, void *workspace, hipStream_t s);
+bool qvm_takes_grouped(const ProductArgs &a);  // whether sorted pairs of one row each run as groups on the matrix-core kernel
 const char *qvm_kernel_name(const ProductArgs &a);  // the matrix-core kernel (many rows of x) or the vector kernel
 
 }  // namespace nvq

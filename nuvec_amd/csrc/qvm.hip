@@ -258,20 +258,44 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kStageBytes];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / TL::WN, wn = wave % TL::WN, h = lane >> 5, l32 = lane & 31;
-    const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
+    const int K = (int)a.k, N = (int)a.n;
     const int gshift = FP4 == kNvfp4 ? 4 : FP4 ? 5 : (a.group == 32 ? 5 : a.group == 64 ? 6 : 7);
     const int ngroups = N >> gshift;
     const int64_t row_bytes = ((int64_t)N * BITS) >> 3;
-    // Blocks are handed to the 8 XCDs (an L2 each) in turn: block p takes item (p % 8) * ceil(items / 8) + p / 8 of the
-    // tile list, whose order walks bands of 8 tiles of rows column tile by column tile, so that an XCD's 64 resident
-    // blocks are 8 x 8 tiles that share 8 tiles of x and 8 of w.
-    const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN, items = mtiles * ntiles, per = (items + 7) >> 3;
-    const int item = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
-    if (item >= items) return;  // the whole block, before any barrier
-    const int band = item / (8 * ntiles), in_band = item - band * 8 * ntiles;
-    const int band_rows = mtiles - 8 * band < 8 ? mtiles - 8 * band : 8;
-    const int m0 = (8 * band + in_band % band_rows) * BM, n0 = (in_band / band_rows) * BN;
-    const Offsets o = batch_offsets(a, blockIdx.y);
+    const int ntiles = (N + BN - 1) / BN;
+    const bool grouped = a.offsets != nullptr;
+    int M = (int)a.m, m0, n0, pair0 = 0;
+    Offsets o;
+    if (grouped) {
+        // Rows of one row of x each, sorted by expert: expert e's rows of x are the pairs [offsets[e], offsets[e + 1]),
+        // taken through `lhs`.  The grid holds ceil(pairs / BM) + experts tiles of rows (every expert adds at most one
+        // partial tile) times the column tiles, in launch order tile of rows by tile of rows (so the work goes round the
+        // XCDs); a block finds its tile's expert by walking the offsets, and the tiles past the last expert's leave.
+        const int tile = (int)blockIdx.x / ntiles;
+        int e = 0, first = 0, rows = 0;
+        for (; e < (int)a.experts; e++) {
+            pair0 = a.offsets[e];
+            rows = (e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch) - pair0;
+            const int tiles = (rows + BM - 1) / BM;
+            if (tile < first + tiles) break;
+            first += tiles;
+        }
+        if (e == (int)a.experts) return;  // the whole block, before any barrier
+        M = rows;
+        m0 = (tile - first) * BM, n0 = ((int)blockIdx.x % ntiles) * BN;
+        o = Offsets{0, (int64_t)e * K * (N * BITS / 32), (int64_t)e * K * ngroups, 0};
+    } else {
+        // Blocks are handed to the 8 XCDs (an L2 each) in turn: block p takes item (p % 8) * ceil(items / 8) + p / 8 of the
+        // tile list, whose order walks bands of 8 tiles of rows column tile by column tile, so that an XCD's 64 resident
+        // blocks are 8 x 8 tiles that share 8 tiles of x and 8 of w.
+        const int mtiles = (M + BM - 1) / BM, items = mtiles * ntiles, per = (items + 7) >> 3;
+        const int item = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+        if (item >= items) return;  // the whole block, before any barrier
+        const int band = item / (8 * ntiles), in_band = item - band * 8 * ntiles;
+        const int band_rows = mtiles - 8 * band < 8 ? mtiles - 8 * band : 8;
+        m0 = (8 * band + in_band % band_rows) * BM, n0 = (in_band / band_rows) * BN;
+        o = batch_offsets(a, blockIdx.y);
+    }
     const T *x = (const T *)a.x + o.x;
 
     // Addresses are a base that is the same for the whole block (scalar registers, advanced per step by scalar
@@ -289,14 +313,16 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
 #pragma unroll
     for (int j = 0; j < 8; j++) wdst[j] = kXBytes + w_slot(8 * c + j, q >> 1) + 8 * (q & 1);
     // This thread's part of a step of x: 16-byte pieces t + 256 i (piece p: row p / 8, slot p % 8).
-    const unsigned char *xbase = (const unsigned char *)(x + (int64_t)m0 * K);
+    const unsigned char *xbase = (const unsigned char *)(x + (grouped ? 0 : (int64_t)m0 * K));
     uint32_t xoff[kXParts];
     int xdst[kXParts];
 #pragma unroll
     for (int i = 0; i < kXParts; i++) {
         const int p = tid + 256 * i, r = p >> 3, ch = p & 7;
         const int row = m0 + r < M ? r : M - 1 - m0;  // rows past M are computed, not stored
-        xoff[i] = ((uint32_t)row * (uint32_t)K + 8u * ch) * 2u;
+        // grouped: the row of x of pair pair0 + m0 + row (an index outside x is the caller's error and is clamped)
+        const uint32_t xrow = grouped ? (uint32_t)min((int64_t)a.lhs[pair0 + m0 + row], a.x_batches - 1) : (uint32_t)row;
+        xoff[i] = (xrow * (uint32_t)K + 8u * ch) * 2u;
         xdst[i] = x_slot(r, ch);
     }
 
@@ -426,8 +452,8 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
     }
 
     // Accumulator element el of lane l is tile row 8 (el / 4) + 4 (l / 32) + el % 4 (a row of x), column l % 32.
-    T *y = (T *)a.y + o.y * M * N;
-    float *part = partial + ((int64_t)blockIdx.y * splits + blockIdx.z) * M * N;  // (used with a split only)
+    T *y = (T *)a.y + (grouped ? (int64_t)pair0 * N : o.y * M * N);
+    float *part = partial + ((int64_t)blockIdx.y * splits + blockIdx.z) * M * N;  // (used with a split only; never grouped)
     const bool biased = a.row_bias != nullptr;
 #pragma unroll
     for (int tj = 0; tj < TJ; tj++) {
@@ -475,9 +501,11 @@ inline int splits_of(const ProductArgs &a) { return few_rows(a) ? splits_of_shap
 
 template <typename T, int BITS, int FP4, class TL>
 int32_t run_shape(const ProductArgs &a, float *workspace, hipStream_t s) {
-    const int splits = workspace != nullptr ? splits_of_shape<TL>(a) : 1;  // without a workspace K is not split
-    const int64_t tiles = ((a.m + TL::BM - 1) / TL::BM) * ((a.n + BN - 1) / BN);
-    const dim3 grid((unsigned)((tiles + 7) / 8 * 8), (unsigned)a.batch, (unsigned)splits);
+    const bool grouped = a.offsets != nullptr;  // ceil(pairs / BM) + experts tiles of rows: every expert adds at most one partial tile
+    const int splits = workspace != nullptr && !grouped ? splits_of_shape<TL>(a) : 1;  // without a workspace K is not split
+    const int64_t row_tiles = grouped ? (a.batch + TL::BM - 1) / TL::BM + a.experts : (a.m + TL::BM - 1) / TL::BM;
+    const int64_t tiles = row_tiles * ((a.n + BN - 1) / BN);
+    const dim3 grid((unsigned)(grouped ? tiles : (tiles + 7) / 8 * 8), (unsigned)(grouped ? 1 : a.batch), (unsigned)splits);
     if (FP4 == kAffine && a.exact_weights) hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, FP4 == kAffine, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     else hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, false, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     NVQ_LAUNCH_CHECK("qmn");
@@ -492,7 +520,9 @@ int32_t run_shape(const ProductArgs &a, float *workspace, hipStream_t s) {
 
 template <typename T, int BITS, int FP4>
 int32_t run(const ProductArgs &a, float *workspace, hipStream_t s) {
-    return few_rows(a) ? run_shape<T, BITS, FP4, Tile32>(a, workspace, s) : run_shape<T, BITS, FP4, Tile128>(a, workspace, s);
+    // (grouped: the tile of 32 rows up to 64 rows per expert on average)
+    const bool few = a.offsets != nullptr ? a.batch <= 2 * (int64_t)Tile32::BM * a.experts : few_rows(a);
+    return few ? run_shape<T, BITS, FP4, Tile32>(a, workspace, s) : run_shape<T, BITS, FP4, Tile128>(a, workspace, s);
 }
 
 template <typename T>
@@ -580,10 +610,18 @@ size_t qvm_workspace_bytes(const ProductArgs &a) {
 bool qvm_takes_tiled(const ProductArgs &a) {
     if (a.dtype == NVQ_F32 || a.row_exact || a.global_scale != nullptr || a.m < 1) return false;
     if (a.mode == NVQ_AFFINE && !(a.bits == 2 || a.bits == 4 || a.bits == 8)) return false;
-    if (a.k < qmn::BK || a.k % qmn::BK != 0 || a.batch > 65535) return false;
+    if (a.k < qmn::BK || a.k % qmn::BK != 0 || (a.batch > 65535 && a.offsets == nullptr)) return false;
     for (int d = 0; d < a.batch_ndim; d++)
         if (a.x_strides[d] % 8 != 0 || a.w_strides[d] % 4 != 0) return false;  // 16-byte pieces of x, 8-byte runs of codes
     return ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
+}
+
+// Whether the tiled kernel takes the pairs of a gather sorted by expert as groups (`a.offsets` set, one row of x per
+// pair): each expert's weights are then read once per tile of its rows instead of once per pair.
+bool qvm_takes_grouped(const ProductArgs &a) {
+    if (a.offsets == nullptr || a.m != 1 || a.rhs == nullptr || a.exact_weights || a.row_bias != nullptr) return false;
+    if (a.experts > 4096 || a.x_batches * a.k >= (1LL << 31) || a.batch >= (1LL << 30)) return false;  // (a block walks the offsets)
+    return qvm_takes_tiled(a);
 }
 
 const char *qvm_kernel_name(const ProductArgs &a) { return qvm_takes_tiled(a) ? "qmn_kernel" : "qvm_kernel"; }

@@ -1367,6 +1367,31 @@ def test_untransposed_gathers(mode, qmode):
         want = ref.gather_qmm(x, packed, scales, biases, lhs.astype(np.uint32), rhs.astype(np.uint32), mode=mode, group=group, bits=bits,
                               dtype=dtype, transpose=False)
         assert_rows_close(got.reshape(pairs * m, n), want.reshape(pairs * m, n), dtype, f"untransposed gather mode {mode} M={m} K={k} N={n}")
+    # Rows sorted by expert (the grouped route: the reference's `_nn` kernel of the block formats, gpu.rs:6786-6812; here for
+    # affine weights too): each expert's weights read once per tile of its rows.  An expert without rows, one with more
+    # rows than a tile of 32 and, with 700 pairs, than a tile of 128; every row against the oracle and close to the
+    # per-pair route's (whose split of K orders the sums differently).
+    experts, k, n = 5, 1088, 1280
+    w = make_w(rng, experts * k, n, dtype).reshape(experts, k, n)
+    if mode == ref.AFFINE:
+        packed, scales, biases = ref.affine_quantize(w, dtype, 64, 4)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(64, 4))
+        group, bits = 64, 4
+    else:
+        group, bits = ref.FP_PARAMS[mode]
+        (packed, scales), biases = ref.fp_quantize(w, dtype, mode), None
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(getattr(nv.QuantMode, qmode)))
+    for counts in ([3, 0, 45, 33, 20], [100, 0, 300, 129, 171]):
+        rhs = np.repeat(np.arange(experts), counts).astype(np.int64)
+        x = make_x(rng, rhs.size, k, dtype).reshape(rhs.size, 1, k)
+        assert nv.GatherQmm.groups(rhs.size, experts)
+        got = nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs).cuda(), nv.GatherQmm(transpose=False, sorted_indices=True))
+        want = ref.gather_qmm(x, packed, scales, biases, np.arange(rhs.size, dtype=np.uint32), rhs.astype(np.uint32), mode=mode,
+                              group=group, bits=bits, dtype=dtype, transpose=False)
+        assert_rows_close(to_host(got).reshape(rhs.size, n), want.reshape(rhs.size, n), dtype,
+                          f"untransposed grouped gather mode {mode}, {rhs.size} rows", exact_weights=mode != ref.AFFINE)
+        pairwise = nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs).cuda(), nv.GatherQmm(transpose=False))
+        assert float((got.float() - pairwise.float()).abs().max()) <= 2e-2 * float(pairwise.float().abs().max())
 
 
 @pytest.mark.parametrize("route", ["grouped-mxfp4", "grouped-affine4", "pairs-affine4-decode", "pairs-affine8-few", "pairs-mxfp8-general",
