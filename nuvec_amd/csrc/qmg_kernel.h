@@ -68,17 +68,69 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
     const int64_t row_bytes = (int64_t)(K >> 3) * BITS;  // of one packed weight row
     const int tstride = table_stride(kgroups, (int)sizeof(S));
     unsigned char *table_b = table_s + kRows * tstride;
-    // Blocks are handed to the 8 XCDs in turn, each with an L2 of its own: block p takes work item
-    // (p % 8) * ceil(items / 8) + p / 8 of the expert-major list, so that the blocks of an expert — which all read
-    // the expert's rows of x — sit on one XCD.
-    const int tiles = (N + kRows - 1) / kRows, items = tiles * (int)a.experts, per = (items + 7) >> 3;
-    const int item = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
-    if (item >= items) return;  // the whole block: no barrier has been reached
-    const int n0 = (item % tiles) * kRows;
-    const int e = item / tiles;
-    const int row_begin = a.offsets[e];
-    const int row_end = e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch;
-    if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
+    // Work items are (pass of up to 64 rows of an expert, 128 weight rows): every item costs the same whatever the
+    // experts' loads, and an expert with many rows has its passes side by side.  The passes are counted from the
+    // offsets by every wavefront on its own (lane l owns a run of experts; a prefix sum over the lanes), and the block
+    // finds the expert and the pass of its item there.  Blocks are handed to the 8 XCDs in turn, each with an L2 of
+    // its own: block p takes item (p % 8) * ceil(items / 8) + p / 8 of the pass-major list, so that the blocks of a
+    // pass, which read the same rows of x and neighbouring pieces of the same cache lines of weights, sit on one XCD.
+    const int tiles = (N + kRows - 1) / kRows, experts = (int)a.experts;
+    const int run = (experts + 63) >> 6, e_first = lane * run;
+    constexpr int kKept = 4;  // experts of a lane whose offsets stay in registers for the walk below (all of them up to 256 experts)
+    int kept_begin[kKept], kept_end[kKept];
+    int mine = 0;  // passes of this lane's experts
+#pragma unroll
+    for (int i = 0; i < kKept; i++) {
+        const int ei = e_first + i;
+        const bool have = i < run && ei < experts;
+        kept_begin[i] = have ? a.offsets[ei] : 0;
+        kept_end[i] = have ? (ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch) : 0;
+        mine += (kept_end[i] - kept_begin[i] + kPassRows - 1) / kPassRows;
+    }
+    for (int i = kKept; i < run; i++) {
+        const int ei = e_first + i;
+        if (ei < experts) {
+            const int rows = (ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch) - a.offsets[ei];
+            mine += (rows + kPassRows - 1) / kPassRows;
+        }
+    }
+    int upto = mine;  // inclusive prefix over the lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int v = __shfl_up(upto, o);
+        if (lane >= o) upto += v;
+    }
+    const int passes = __shfl(upto, 63);
+    const int items = tiles * passes, per = (items + 7) >> 3;
+    const int slot = (int)(blockIdx.x >> 3), item = (int)(blockIdx.x & 7) * per + slot;
+    if (slot >= per || item >= items) return;  // the whole block: no barrier has been reached
+    const int n0 = (item % tiles) * kRows, target = item / tiles;
+    // the lane whose experts hold pass `target` walks them; every lane takes its answer
+    const int owner = __builtin_ctzll(__ballot(upto > target));
+    int found_e = 0, found_begin = 0, found_end = 0;
+    if (lane == owner) {
+        int before = upto - mine;
+        bool found = false;
+        auto look = [&](int ei, int begin, int end) {
+            const int count = (end - begin + kPassRows - 1) / kPassRows;
+            if (!found && target < before + count) {
+                found = true;
+                found_e = ei, found_begin = begin + (target - before) * kPassRows;
+                found_end = found_begin + kPassRows < end ? found_begin + kPassRows : end;
+            }
+            if (!found) before += count;
+        };
+#pragma unroll
+        for (int i = 0; i < kKept; i++) look(e_first + i, kept_begin[i], kept_end[i]);  // (an expert past the lane's run holds no pass)
+        for (int i = kKept; i < run && !found; i++) {
+            const int ei = e_first + i;
+            if (ei >= experts) break;
+            look(ei, a.offsets[ei], ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch);
+        }
+    }
+    const int e = __builtin_amdgcn_readfirstlane(__shfl(found_e, owner));
+    const int row_begin = __builtin_amdgcn_readfirstlane(__shfl(found_begin, owner));
+    const int row_end = __builtin_amdgcn_readfirstlane(__shfl(found_end, owner));
     const int64_t wo = (int64_t)e * N * row_bytes, so = (int64_t)e * N * kgroups;
     const T *x = (const T *)a.x;
     T *y = (T *)a.y;
@@ -371,7 +423,9 @@ int32_t run_kernel(const ProductArgs &a, hipStream_t s) {
                                         G::kFixedLdsBytes + kTableMaxBytes));
         configured = true;
     }
-    const int64_t items = (a.n + kRows - 1) / kRows * a.experts;
+    // every expert with rows adds at most one partial pass: blocks for that many items, the rest leave at once
+    const int64_t passes = a.batch / kPassRows + (a.experts < a.batch ? a.experts : a.batch);
+    const int64_t items = (a.n + kRows - 1) / kRows * passes;
     const dim3 grid((unsigned)((items + 7) / 8 * 8));
     hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds_bytes, s, a);
     NVQ_LAUNCH_CHECK("qmg");

@@ -438,6 +438,22 @@ def test_grouped_gather_edge_cases():
     got = to_host(nv.gather_qmm(to_dev(x), q, None, torch.from_numpy(rhs.astype(np.int64)).cuda(), nv.GatherQmm(sorted_indices=True)))
     want = ref.gather_qmm(x, packed, scales, biases, np.arange(rhs.size, dtype=np.uint32), rhs, group=64, bits=4, dtype=ref.BF16)
     assert_rows_close(got, want, ref.BF16, "grouped affine")
+    # Uneven loads over many experts (the kernel's blocks find their pass of 64 rows in the offsets, every lane walking a
+    # run of experts: more than 256 experts is more than four a lane): one expert with several passes, the last expert
+    # with two, singletons, most experts empty.
+    experts, n, k = 300, 136, 128
+    w = make_w(rng, experts * n, k, ref.BF16).reshape(experts, n, k)
+    packed, scales = ref.fp_quantize(w, ref.BF16, ref.MXFP4)
+    counts = np.zeros(experts, np.int64)
+    counts[[7, 299, 0, 64, 128, 255, 256, 257, 298]] = [200, 70, 1, 1, 65, 1, 3, 64, 1]
+    rhs = np.repeat(np.arange(experts), counts).astype(np.uint32)
+    x = make_x(rng, rhs.size, k, ref.BF16).reshape(-1, 1, k)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, nv.Quant.new(nv.QuantMode.MXFP4))
+    ids = torch.from_numpy(rhs.astype(np.int32)).cuda()
+    rows = torch.arange(rhs.size, dtype=torch.int32, device="cuda")
+    got = to_host(nv.gather_qmm_grouped(to_dev(x).reshape(-1, k), q, rows, ids, nv.sorted_offsets(ids, experts)))  # (the grouped kernel whatever the rows per expert)
+    want = ref.gather_qmm(x, packed, scales, None, np.arange(rhs.size, dtype=np.uint32), rhs, mode=ref.MXFP4, group=32, bits=4, dtype=ref.BF16)
+    assert_rows_close(got, want.reshape(rhs.size, n), ref.BF16, "grouped MXFP4, 300 experts with uneven loads", exact_weights=True)
 
 
 @pytest.mark.parametrize("quant", ["MXFP4", "affine4", "NVFP4-gs"])
