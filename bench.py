@@ -81,9 +81,11 @@ class Product:
 
 
 class GatherProduct:
-    """One prepared grouped nvq_gather_qmm call (sorted pairs, one row of x per pair)."""
+    """One prepared nvq_gather_qmm call with one row of x per pair: sorted pairs with their offsets (the grouped route) or
+    unsorted ones."""
 
     def __init__(self, lib, x, q, lhs, rhs, offsets, y, n, k, experts):
+        """`offsets` None: unsorted pairs, one product per pair."""
         from nuvec_amd import _lib
         pairs = rhs.numel()
         self.d = _lib.GatherDescC(q.quant._c(), _lib.BF16, 1, 0, 0, 1, n, k, pairs, x.shape[0], experts)
@@ -91,7 +93,8 @@ class GatherProduct:
         biases = q.biases.data_ptr() if q.biases is not None else None
         self.args = (C.byref(self.d), C.c_void_p(x.data_ptr()), C.c_void_p(q.weight.data_ptr()),
                      C.c_void_p(q.scales.data_ptr()), C.c_void_p(biases), C.c_void_p(lhs.data_ptr()),
-                     C.c_void_p(rhs.data_ptr()), C.c_void_p(offsets.data_ptr()), C.c_void_p(y.data_ptr()), C.c_void_p(None))
+                     C.c_void_p(rhs.data_ptr()), C.c_void_p(None if offsets is None else offsets.data_ptr()), C.c_void_p(y.data_ptr()),
+                     C.c_void_p(None))
         self.keep = (x, q, lhs, rhs, offsets, y)
 
     def __call__(self, stream):
@@ -280,6 +283,16 @@ def all_configs(lib, device, qs):
                 "us_per_launch": ms * 1e3, "weight_gbps": 141_004_800 / (ms * 1e-3) / 1e9,
                 "tflops": 16_986_931_200 / (ms * 1e-3) / 1e12, "frac_of_peak": 141_004_800 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                 "bound": "hbm"})
+    # Beside the configurations: the same experts at decode, one token's four experts as unsorted pairs (one product
+    # per pair on the decode kernel), and 32 such pairs
+    for pairs in (top, 32):
+        ids = torch.from_numpy(rng.permutation(experts)[:pairs].astype(np.int32)).to(device)
+        calls = [GatherProduct(lib, x[:pairs], q, lhs[:pairs], ids, None, y[:pairs], n, k, experts) for q in weights]
+        ms = best_of(calls * 4, 320)
+        moved = pairs * (n * k // 2 + n * k // 32)
+        out.append({"config": f"C5's experts at decode: {pairs} unsorted rows, one expert each", "m": pairs, "kernel": "qmv4_lds_kernel",
+                    "us_per_launch": ms * 1e3, "weight_gbps": moved / (ms * 1e-3) / 1e9, "tflops": 2.0 * pairs * n * k / (ms * 1e-3) / 1e12,
+                    "frac_of_peak": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "bound": "hbm"})
     del weights, calls
 
     # The weights' own kernels at the same shapes: quantize (dense in, packed out) and dequantize (packed in, dense out),
