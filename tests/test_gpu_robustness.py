@@ -145,6 +145,24 @@ def determinism_cases():
     offsets = nv.sorted_offsets(ids.to(torch.int32), 16)
     tokens = torch.arange(512, device="cuda", dtype=torch.int32)
     cases["grouped gather with the gated epilogue"] = lambda: nv.gather_qmm_glu(xe.reshape(512, 1024), paired, tokens, ids.to(torch.int32), offsets, "swiglu")
+    # the decode kernel on the block formats, unsorted pairs on the decode and the short-row kernels, the experts' bias in
+    # the grouped and the per-pair epilogues, sorted pairs against weights stored [K, N], the fused attention at 3 bits
+    em4 = nv.quantize(experts, nv.QuantMode.MXFP4)
+    bias = to_dev(make_x(rng, 16, 512, ref.BF16))
+    for mode in ("MXFP4", "MXFP8", "NVFP4"):
+        qm = nv.quantize(wd[:1024], nv.QuantMode[mode])
+        for rows in (1, 2):
+            cases[f"{mode} decode M={rows}"] = lambda qm=qm, rows=rows: nv.quantized_matmul(x512[:rows], qm)
+    cases["pair gather MXFP4, short rows"] = lambda: nv.gather_qmm(xe[:24], em4, None, ids[:24].flip(0), nv.GatherQmm())
+    cases["pair gather b4, long rows"] = lambda: nv.gather_qmm(x512[:6].reshape(6, 1, 4096), nv.Quantized(q4.weight[None], q4.scales[None], q4.biases[None], q4.quant),
+                                                               None, torch.zeros(6, dtype=torch.int64, device="cuda"), nv.GatherQmm())
+    cases["grouped gather with the experts' bias"] = lambda: nv.gather_qmm_grouped(xe.reshape(512, 1024), em4, tokens, ids.to(torch.int32), offsets, expert_bias=bias)
+    cases["pair gather with the experts' bias"] = lambda: nv.gather_qmm(xe[:24], em4, None, ids[:24].flip(0), nv.GatherQmm(), expert_bias=bias)
+    ekn = nv.quantize(experts.transpose(1, 2).contiguous(), nv.QuantMode.MXFP4)  # stored [K, N] = [1024, 512]
+    cases["grouped gather, weights stored [K, N]"] = lambda: nv.gather_qmm(xe, ekn, None, ids, nv.GatherQmm(transpose=False, sorted_indices=True))
+    kv = nv.quantize(to_dev(make_x(rng, 2 * 700, 128, ref.BF16)).reshape(1, 2, 700, 128), nv.Quant.affine(64, 3))
+    qh = to_dev(make_x(rng, 8, 128, ref.BF16)).reshape(1, 8, 1, 128)
+    cases["attention, 3-bit cache"] = lambda: nv.ops.quantized_attention(qh, kv, kv, 0.088)
     cases["quantize b4"] = lambda: nv.quantize(wd, nv.Quant.affine(64, 4)).weight
     cases["quantize mxfp4"] = lambda: nv.quantize(wd, nv.QuantMode.MXFP4).weight
     cases["dequantize b4"] = lambda: nv.dequantize(q4)
