@@ -9,7 +9,7 @@ the CPU: 2.5e-3 * max|row|.
 
 How the half-precision bar is applied.  EVERY output of every product is held to the bar against the
 CPU oracle (`assert_rows_close`), and the worst ratio error / bar of each case is printed and appended to
-`gpurun_out/parity_ratios.txt` so that a run's record holds the margin.  The kernels compute in the
+a `parity_ratios.txt` in the run's output folder so that a run's record holds the margin.  The kernels compute in the
 arithmetic of the reference's device kernels (weights dequantized with one rounding of
 fma(code, scale, bias), or not rounded at all in the decode kernels) while the reference's CPU path rounds
 the dequantized weights twice in the element type; a second check (`assert_device_arithmetic`) holds every
