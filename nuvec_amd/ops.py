@@ -45,6 +45,11 @@ class QuantMode(IntEnum):
 _DEFAULTS = {QuantMode.AFFINE: (64, 4), QuantMode.MXFP4: (32, 4), QuantMode.MXFP8: (32, 8), QuantMode.NVFP4: (16, 4)}
 
 
+_VALID: set = set()     # quantizations the library has accepted
+_QUANT_C: dict = {}     # their C descriptors (read-only: descriptors that embed one copy it)
+_READY: set = set()     # devices nvq_init has answered for
+
+
 @dataclass(frozen=True)
 class Quant:
     """quantized.rs:93-168: a mode, a group size and a bit width."""
@@ -62,12 +67,18 @@ class Quant:
         return Quant(QuantMode.AFFINE, group_size, bits)
 
     def checked(self, op: str):
-        """Quant::checked: raises InvalidArgument with the reference's message."""
-        _lib.check(_lib.load().nvq_quant_check(C.byref(self._c()), op.encode()))
+        """Quant::checked: raises InvalidArgument with the reference's message.  (A quantization that has passed is not
+        asked about again: the library's answer depends on its three numbers alone.)"""
+        if self not in _VALID:
+            _lib.check(_lib.load().nvq_quant_check(C.byref(self._c()), op.encode()))
+            _VALID.add(self)
         return self.group_size, self.bits
 
     def _c(self) -> _lib.QuantC:
-        return _lib.QuantC(int(self.mode), int(self.group_size), int(self.bits))
+        c = _QUANT_C.get(self)
+        if c is None:
+            c = _QUANT_C[self] = _lib.QuantC(int(self.mode), int(self.group_size), int(self.bits))
+        return c
 
 
 @dataclass
@@ -113,7 +124,10 @@ _FLOATS = tuple(_CODE)
 def _init(t: torch.Tensor) -> None:
     if not t.is_cuda:
         raise _lib.NoDevice("operands must live on the GPU: this backend has no CPU path")
-    _lib.check(_lib.load().nvq_init(t.device.index or 0))
+    index = t.device.index or 0
+    if index not in _READY:
+        _lib.check(_lib.load().nvq_init(index))
+        _READY.add(index)
 
 
 def _stream() -> C.c_void_p:
