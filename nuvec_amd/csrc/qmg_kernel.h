@@ -76,22 +76,29 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
     // pass, which read the same rows of x and neighbouring pieces of the same cache lines of weights, sit on one XCD.
     const int tiles = (N + kRows - 1) / kRows, experts = (int)a.experts;
     const int run = (experts + 63) >> 6, e_first = lane * run;
+    // Rows [begin, end) of expert ei, as the offsets give them; offsets that do not ascend within the rows are the
+    // caller's error and are clamped so that they cannot fault the device.
+    auto rows_of = [&](int ei, int &begin, int &end) {
+        const int rows_all = (int)a.batch;
+        begin = min(max(a.offsets[ei], 0), rows_all);
+        end = ei + 1 < experts ? min(max(a.offsets[ei + 1], begin), rows_all) : rows_all;
+    };
     constexpr int kKept = 4;  // experts of a lane whose offsets stay in registers for the walk below (all of them up to 256 experts)
     int kept_begin[kKept], kept_end[kKept];
     int mine = 0;  // passes of this lane's experts
 #pragma unroll
     for (int i = 0; i < kKept; i++) {
         const int ei = e_first + i;
-        const bool have = i < run && ei < experts;
-        kept_begin[i] = have ? a.offsets[ei] : 0;
-        kept_end[i] = have ? (ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch) : 0;
+        kept_begin[i] = kept_end[i] = 0;
+        if (i < run && ei < experts) rows_of(ei, kept_begin[i], kept_end[i]);
         mine += (kept_end[i] - kept_begin[i] + kPassRows - 1) / kPassRows;
     }
     for (int i = kKept; i < run; i++) {
         const int ei = e_first + i;
         if (ei < experts) {
-            const int rows = (ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch) - a.offsets[ei];
-            mine += (rows + kPassRows - 1) / kPassRows;
+            int begin, end;
+            rows_of(ei, begin, end);
+            mine += (end - begin + kPassRows - 1) / kPassRows;
         }
     }
     int upto = mine;  // inclusive prefix over the lanes
@@ -125,12 +132,15 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3
         for (int i = kKept; i < run && !found; i++) {
             const int ei = e_first + i;
             if (ei >= experts) break;
-            look(ei, a.offsets[ei], ei + 1 < experts ? a.offsets[ei + 1] : (int)a.batch);
+            int begin, end;
+            rows_of(ei, begin, end);
+            look(ei, begin, end);
         }
     }
     const int e = __builtin_amdgcn_readfirstlane(__shfl(found_e, owner));
     const int row_begin = __builtin_amdgcn_readfirstlane(__shfl(found_begin, owner));
     const int row_end = __builtin_amdgcn_readfirstlane(__shfl(found_end, owner));
+    if (row_begin >= row_end) return;  // the whole block: no barrier has been reached
     const int64_t wo = (int64_t)e * N * row_bytes, so = (int64_t)e * N * kgroups;
     const T *x = (const T *)a.x;
     T *y = (T *)a.y;

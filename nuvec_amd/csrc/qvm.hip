@@ -274,8 +274,9 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
         const int tile = (int)blockIdx.x / ntiles;
         int e = 0, first = 0, rows = 0;
         for (; e < (int)a.experts; e++) {
-            pair0 = a.offsets[e];
-            rows = (e + 1 < (int)a.experts ? a.offsets[e + 1] : (int)a.batch) - pair0;
+            // (offsets that do not ascend within the pairs are the caller's error: clamped, so that they cannot fault the device)
+            pair0 = min(max(a.offsets[e], 0), (int)a.batch);
+            rows = (e + 1 < (int)a.experts ? min(max(a.offsets[e + 1], pair0), (int)a.batch) : (int)a.batch) - pair0;
             const int tiles = (rows + BM - 1) / BM;
             if (tile < first + tiles) break;
             first += tiles;

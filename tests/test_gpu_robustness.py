@@ -209,3 +209,41 @@ def test_eight_host_threads_on_their_own_streams():
     for th in threads:
         th.join()
     assert not failures, failures[:5]
+
+
+@pytest.mark.parametrize("transpose", [True, False])
+def test_indices_and_offsets_outside_their_operands_are_clamped(transpose):
+    """A caller's error must not reach the device as an access outside an operand (the reference's contract for
+    primitives built with bad parameters, tests/primitive_fuzz.rs:97-131, 423-431: an error or a result, never a
+    crash): expert ids beyond the experts, rows of x beyond x, offsets that do not ascend or leave the pairs.  The
+    kernels clamp them; rows whose indices were valid keep their values."""
+    rng = np.random.default_rng(77)
+    experts, n, k, pairs = 6, 1152, 256, 96
+    w = to_dev(make_w(rng, experts * n, k, ref.BF16)).reshape(experts, n, k)
+    q = nv.quantize(w if transpose else w.transpose(1, 2).contiguous(), nv.QuantMode.MXFP4)
+    x = to_dev(make_x(rng, pairs, k, ref.BF16))
+    ids = torch.sort(torch.from_numpy(rng.integers(0, experts, pairs).astype(np.int32)).cuda())[0]
+    rows = torch.arange(pairs, dtype=torch.int32, device="cuda")
+    offsets = nv.sorted_offsets(ids, experts)
+    options = nv.GatherQmm(transpose=transpose)
+    good = nv.gather_qmm(x.reshape(pairs, 1, k), q, rows, ids, options)
+    # unsorted pairs with indices out of range
+    bad_ids, bad_rows = ids.clone(), rows.clone()
+    bad_ids[::7] = 1000
+    bad_rows[::5] = 5000
+    got = nv.gather_qmm(x.reshape(pairs, 1, k), q, bad_rows, bad_ids, options)
+    keep = torch.ones(pairs, dtype=torch.bool, device="cuda")
+    keep[::7] = False
+    keep[::5] = False
+    assert torch.isfinite(got.float()).all() and torch.equal(got[keep], good[keep])
+    # grouped, with offsets that descend, are negative or leave the pairs
+    if transpose:
+        for broken in ([5, 3, 900, -4, 50, 20], [0, 0, 0, 0, 0, 0], [96, 96, 96, 96, 96, 96], [-1, -1, 200, 200, 10, 10 ** 6]):
+            out = nv.gather_qmm_grouped(x, q, bad_rows, ids, torch.tensor(broken, dtype=torch.int32, device="cuda"))
+            torch.cuda.synchronize()
+            assert tuple(out.shape) == (pairs, n)
+        whole = nv.gather_qmm_grouped(x, q, rows, ids, offsets)
+        assert torch.isfinite(whole.float()).all()
+    else:
+        sorted_out = nv.gather_qmm(x.reshape(pairs, 1, k), q, None, ids, nv.GatherQmm(transpose=False, sorted_indices=True))
+        assert torch.isfinite(sorted_out.float()).all()
