@@ -382,8 +382,10 @@ NVQ_API int32_t nvq_gather_qmm_expert_bias(const nvq_gather_desc *desc, const vo
  * their total (a multiple of 128), desc->m is 1, rows sorted by expert with `offsets` as for nvq_gather_qmm.
  *   y dtype[pairs, n / 2] = act(x[lhs] . gate^T + bias_gate[rhs], x[lhs] . up^T + bias_up[rhs]), the products rounded
  *   to `dtype` as nvq_gather_qmm returns them, then nvq_glu's arithmetic: bit for bit that composition.
- *   expert_bias dtype[experts, n] or NULL.  NVQ_UNSUPPORTED where the grouped matrix-core kernel does not take the
- *   product (the caller then composes nvq_gather_qmm and nvq_glu). */
+ *   expert_bias dtype[experts, n] or NULL.  With offsets = NULL the pairs are unsorted (the experts of decoded tokens,
+ *   up to four rows of x each: desc->m) and run on the decode kernel with the same epilogue: y dtype[pairs, m, n / 2].
+ *   NVQ_UNSUPPORTED where the grouped matrix-core kernel (the decode kernel) does not take the product (the caller
+ *   then composes nvq_gather_qmm and nvq_glu). */
 NVQ_API int32_t nvq_gather_qmm_glu(const nvq_gather_desc *desc, int32_t activation, float alpha, float limit, const void *x,
                            const void *w, const void *scales, const void *biases, const uint32_t *lhs, const uint32_t *rhs,
                            const int32_t *offsets, const void *expert_bias, void *y, void *stream);

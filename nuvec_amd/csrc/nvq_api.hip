@@ -795,9 +795,9 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     if (glu != nullptr) {
         if (glu->activation < NVQ_GLU_SWIGLU || glu->activation > NVQ_GLU_GEGLU)
             return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: unknown activation %d", glu->activation);
-        if (!d->transpose || offsets == nullptr || d->m != 1 || d->k == 0 || d->n % 128 != 0)
-            return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue belongs to the grouped product of transposed weights whose "
-                                         "gate and up rows alternate in runs of 64");
+        if (!d->transpose || (offsets != nullptr && d->m != 1) || d->k == 0 || d->n % 128 != 0)
+            return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue belongs to products of transposed weights whose gate and up "
+                                         "rows alternate in runs of 64 (sorted pairs: of one row each)");
     }
     if (d->k == 0) {
         return launch_fill_zero(y, d->pairs * d->m * d->n * dtype_size(d->dtype), (hipStream_t)stream);
@@ -831,7 +831,14 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
         if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2))
             return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue takes affine projections of 1024 rows or more each");
         a.exact_weights = 0;
-        a.glu = 1 + glu->activation; a.glu_alpha = glu->alpha; a.glu_limit = glu->limit; a.expert_bias = glu->expert_bias;
+        a.glu = 1 + glu->activation; a.glu_alpha = glu->alpha; a.glu_limit = glu->limit;
+        if (offsets == nullptr) {  // unsorted pairs (the experts of decoded tokens): the decode kernel's epilogue
+            a.row_bias = glu->expert_bias;
+            a.row_bias_per_expert = 1;
+            if (!qmv_glu_pairs_take(a)) return fail(NVQ_UNSUPPORTED, "gather_qmm: the decode kernel does not take these pairs with the gated epilogue");
+            return launch_qmv_glu_pairs(a, (hipStream_t)stream);
+        }
+        a.expert_bias = glu->expert_bias;
         if (!qmf_supported(a)) return fail(NVQ_UNSUPPORTED, "gather_qmm: the grouped matrix-core kernel does not take this product");
         return launch_qmf(a, (hipStream_t)stream);
     }

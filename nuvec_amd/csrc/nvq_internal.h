@@ -106,6 +106,8 @@ int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 const char *qmv_kernel_name(const ProductArgs &a);  // which of the vector / decode kernels launch_qmv runs for `a`
 // Whether the 16x16x32 matrix-core decode kernel takes the product (4-bit affine, groups of 64, K = 4096).
 bool qmv_d16_takes(const ProductArgs &a);
+bool qmv_glu_pairs_take(const ProductArgs &a);      // whether the decode kernel takes unsorted pairs with the gated epilogue
+int32_t launch_qmv_glu_pairs(const ProductArgs &a, hipStream_t s);
 bool qmv_block_decode_takes(const ProductArgs &a);  // whether the decode kernel takes a product of a block format
 // The 16x16x32 matrix-core kernel for passes of up to 16 rows of x (affine 2, 3, 4 and 8 bits, every group size).
 bool qmd_supported(const ProductArgs &a);

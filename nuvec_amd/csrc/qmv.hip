@@ -356,7 +356,11 @@ __device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 ? 
 // scale (dot - B sum x) + bias sum x never materialises a weight), or NVQ_MXFP4 / NVQ_NVFP4 / NVQ_MXFP8: the
 // conversion instructions give the code values as element pairs (every E2M1 and E4M3 value is exact in bf16 and f16),
 // in memory order, and a lane's 32 values are one group (NVFP4: two), whose float32 scale multiplies the group's sum.
-template <typename T, int RM, int RN, int WAVES, bool BATCHED, int MODE = NVQ_AFFINE>
+// GLU (the pairs of a gather whose weights hold the experts' gate and up projections in alternating runs of 64 rows,
+// RN = 2): a wavefront takes output column c of [pairs, N / 2], i.e. weight rows 128 (c / 64) + c % 64 (gate) and that
+// + 64 (up), and stores the gated activation of the two rounded products (each with its expert's bias first), bit for
+// bit what the product followed by the activation kernel gives.
+template <typename T, int RM, int RN, int WAVES, bool BATCHED, int MODE = NVQ_AFFINE, bool GLU = false>
 __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs a) {
     constexpr int kThreads = WAVES * 64;
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
@@ -371,7 +375,10 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     // Sizes fit 32 bits (checked on the host); only row bases are 64-bit, and they are uniform.
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = kAffine ? (a.group == 32 ? 5 : a.group == 64 ? 6 : 7) : (MODE == NVQ_NVFP4 ? 4 : 5);
-    const int n0 = __builtin_amdgcn_readfirstlane((blockIdx.x * WAVES + wave) * RN);
+    static_assert(!GLU || (RN == 2 && BATCHED), "the gated epilogue: a gate and an up row per wavefront, pairs of a gather");
+    const int column = __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES + wave);  // (GLU: of the output)
+    const int n0 = GLU ? 128 * (column >> 6) + (column & 63) : column * RN;
+    constexpr int kRowStep = GLU ? 64 : 1;  // between a wavefront's rows
     const int m0 = blockIdx.y * RM;
     const int kwords = (K * BITS) >> 5, kgroups = K >> gshift;
     // The single-product instantiation carries no batch arithmetic at all.
@@ -415,7 +422,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
             const int kc = kb < K ? kb : 0;  // an absent slice reads valid memory; its x is zero
 #pragma unroll
             for (int r = 0; r < RN; r++) {
-                const int n = n0 + r < N ? n0 + r : N - 1;  // tail rows are computed, not stored
+                const int n = n0 + r * kRowStep < N ? n0 + r * kRowStep : N - 1;  // tail rows are computed, not stored
                 // the codes are read once: a non-temporal load keeps them from displacing x and the scales in the caches
                 // (8.1 -> 7.8 us at W[14336,4096]; the scales, shared by neighbouring lanes and rows, lose by it)
                 const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
@@ -467,6 +474,23 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
             for (int r = 0; r < RN; r++) slice_dot<T, RM, MODE>(wq[u][r], sraw[u][r], braw[u][r], xp, xs, factor, mask, magic, acc[r]);
         }
     }
+    if constexpr (GLU) {
+        const int H = N >> 1;
+        T *out = (T *)a.y + (int64_t)blockIdx.z * M * H;  // (no scattered rows on this route)
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float g = wave_sum_lane63(acc[0][i]), u = wave_sum_lane63(acc[1][i]);
+            if (lane == 63 && column < H && m0 + i < M) {
+                // the products as their outputs hold them, the expert's bias by a separate rounded addition
+                const float gate = add_row_bias<T>(a.row_bias, rounded<T>(g), o.bias + n0), up = add_row_bias<T>(a.row_bias, rounded<T>(u), o.bias + n0 + 64);
+                const float v = a.glu == 1 + NVQ_GLU_SWIGLU       ? glu<T, NVQ_GLU_SWIGLU>(gate, up, a.glu_alpha, a.glu_limit)
+                                : a.glu == 1 + NVQ_GLU_SWIGLU_OAI ? glu<T, NVQ_GLU_SWIGLU_OAI>(gate, up, a.glu_alpha, a.glu_limit)
+                                                                  : glu<T, NVQ_GLU_GEGLU>(gate, up, a.glu_alpha, a.glu_limit);
+                Elem<T>::store(out, (int64_t)(m0 + i) * H + column, v);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < RN; r++)
 #pragma unroll
@@ -475,6 +499,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
             if (lane == 63 && n0 + r < N && m0 + i < M) Elem<T>::store(y, (int64_t)(m0 + i) * N + n0 + r, add_row_bias<T>(a.row_bias, v, o.bias + n0 + r));
         }
 }
+
 
 
 // ── The same for short rows: K up to 2048 ──────────────────────────────────────────────────────────────
@@ -1107,6 +1132,39 @@ int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
+// The pairs of a gather with the gated activation as the epilogue: whether the decode kernel takes them (4-bit affine
+// codes that are never materialised, or a block format; bf16 / f16; up to four rows of x per pair; K in whole slices;
+// the two projections' rows in whole runs of 64) ...
+bool glu_pairs_take(const ProductArgs &a) {
+    if (a.rhs == nullptr || a.dtype == NVQ_F32 || a.row_exact || a.exact_weights || a.out_rows != nullptr) return false;
+    if (a.m < 1 || a.m > 4 || a.k % 32 != 0 || a.n % 128 != 0 || ((uintptr_t)a.w | (uintptr_t)a.x) % 16 != 0) return false;
+    if (a.mode == NVQ_AFFINE) return a.bits == 4;
+    return a.mode != NVQ_NVFP4 || (uintptr_t)a.scales % 2 == 0;
+}
+
+// ... and their launch: a wavefront per output column.
+template <typename T, int MODE>
+int32_t run_glu_pairs_mode(const ProductArgs &a, hipStream_t s) {
+    const int rm = a.m == 1 ? 1 : a.m == 2 ? 2 : 4;
+    const dim3 grid((unsigned)((a.n / 2 + 7) / 8), (unsigned)((a.m + rm - 1) / rm), (unsigned)a.batch);
+    void (*kernel)(const ProductArgs) = rm == 1   ? qmv4_lds_kernel<T, 1, 2, 8, true, MODE, true>
+                                        : rm == 2 ? qmv4_lds_kernel<T, 2, 2, 8, true, MODE, true>
+                                                  : qmv4_lds_kernel<T, 4, 2, 8, true, MODE, true>;
+    hipLaunchKernelGGL(kernel, grid, dim3(512), 0, s, a);
+    NVQ_LAUNCH_CHECK("qmv4_lds with the gated epilogue");
+    return NVQ_OK;
+}
+
+template <typename T>
+int32_t run_glu_pairs(const ProductArgs &a, hipStream_t s) {
+    switch (a.mode) {
+    case NVQ_MXFP4: return run_glu_pairs_mode<T, NVQ_MXFP4>(a, s);
+    case NVQ_MXFP8: return run_glu_pairs_mode<T, NVQ_MXFP8>(a, s);
+    case NVQ_NVFP4: return run_glu_pairs_mode<T, NVQ_NVFP4>(a, s);
+    default: return run_glu_pairs_mode<T, NVQ_AFFINE>(a, s);
+    }
+}
+
 // Whether the decode kernel takes a product of a block format: bf16 / f16, up to kBlockDecodeRows rows of x, whole
 // slices of 32 values (NVFP4 rows may end in half a slice: those stay on the general kernel).  Row-exact products
 // stay on the general kernel at every row count.
@@ -1248,6 +1306,14 @@ const char *qmv_kernel_name(const ProductArgs &a) {
     if (short_decode_takes(a)) return "qmv4_short_kernel";
     if (block_decode_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
+}
+
+bool qmv_glu_pairs_take(const ProductArgs &a) { return glu_pairs_take(a); }
+
+int32_t launch_qmv_glu_pairs(const ProductArgs &a, hipStream_t s) {
+    if (!glu_pairs_take(a) || a.glu == 0) return fail(NVQ_UNSUPPORTED, "gather_qmm: the decode kernel does not take these pairs with the gated epilogue");
+    if (a.batch > 65535) return fail(NVQ_UNSUPPORTED, "gather_qmm: %lld pairs exceed the grid limit", (long long)a.batch);
+    return a.dtype == NVQ_BF16 ? run_glu_pairs<bf16_t>(a, s) : run_glu_pairs<f16_t>(a, s);
 }
 
 int32_t launch_qmv(const ProductArgs &a, hipStream_t s) {

@@ -185,6 +185,17 @@ class SwitchGlu:
         k = indices.shape[2]
         if indices.numel() < 64:  # model.rs:2189-2192
             xe = x.reshape(b, l, 1, 1, d)
+            hidden = None
+            if self.gate_up_proj is not None and self.gate_up_paired:
+                try:  # one kernel: both products of every pair on the decode kernel, the activation as its epilogue
+                    tokens = ops._pair_tokens(b * l, k, x.device)
+                    hidden = ops.gather_qmm_glu(x.reshape(b * l, d), self.gate_up_proj.quantized(), tokens, indices.reshape(-1), None,
+                                                self.activation, alpha=self.alpha, limit=self.limit, expert_bias=self.gate_up_proj.bias)
+                    hidden = hidden.reshape(b, l, k, 1, -1)
+                except ops.Unsupported:
+                    hidden = None
+            if hidden is not None:
+                return self.down_proj.forward(hidden, indices).squeeze(-2)
             if self.gate_up_proj is not None:  # one gather for both projections (a decoded token's few pairs are launch-bound)
                 both = self.gate_up_proj.forward(xe, indices, add_bias=False)
                 if self.gate_up_paired:

@@ -687,13 +687,15 @@ def gather_qmm_grouped(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted
     return out
 
 
-def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor, offsets: torch.Tensor,
+def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids: torch.Tensor, offsets: Optional[torch.Tensor],
                    activation: str = "swiglu", *, alpha: float = 1.702, limit: float = 7.0,
                    expert_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`gather_qmm_grouped` of the experts' gate and up projections with `glu` as the kernel's epilogue
     (`SwitchGlu::through` up to the down projection, model.rs:2157-2169): `q` (and `expert_bias` `[E, N]`) hold both
     projections in alternating runs of 64 rows (`pair_rows`), the result is `[len(rows), N / 2]`, bit for bit
-    `glu(gate, up, ...)` of the two products.  Raises `Unsupported` where the grouped kernel does not take the product."""
+    `glu(gate, up, ...)` of the two products.  `offsets` None: the ids are in any order (the few pairs of decoded
+    tokens) and every pair runs on the decode kernel, with the same epilogue.  Raises `Unsupported` where the grouped
+    kernel (the decode kernel) does not take the product."""
     op = "gather_qmm"
     if activation not in GLU_ACTIVATIONS:
         raise InvalidArgument(f"{op}: unknown activation {activation!r}")
@@ -716,14 +718,14 @@ def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids
         raise InvalidArgument(f"{op}: the experts' bias must be [{w.shape[0]}, {n}] of {dtype}")
     _init(x)
     lhs, rhs = _indices(op, x, rows.reshape(-1)).contiguous(), _indices(op, w, sorted_ids.reshape(-1)).contiguous()
-    if lhs.numel() != rhs.numel() or offsets.numel() != w.shape[0] or offsets.dtype != torch.int32:
+    if lhs.numel() != rhs.numel() or (offsets is not None and (offsets.numel() != w.shape[0] or offsets.dtype != torch.int32)):
         raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
     out = torch.empty((rhs.numel(), n // 2), dtype=dtype, device=x.device)
     d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 0, 0, 1, n, columns, rhs.numel(), x.shape[0], w.shape[0])
     eb = None if expert_bias is None else expert_bias.contiguous()
     _lib.check(_lib.load().nvq_gather_qmm_glu(C.byref(d), GLU_ACTIVATIONS[activation], float(alpha), float(limit), _ptr(x), _ptr(w),
-                                              _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs), _ptr(offsets.contiguous()), _ptr(eb),
-                                              _ptr(out), _stream()))
+                                              _ptr(scales), _ptr(biases), _ptr(lhs), _ptr(rhs),
+                                              _ptr(None if offsets is None else offsets.contiguous()), _ptr(eb), _ptr(out), _stream()))
     return out
 
 
@@ -751,6 +753,17 @@ def _identity(n: int, device: torch.device) -> torch.Tensor:
         if len(_IDENTITY) >= 64:
             _IDENTITY.clear()
         t = _IDENTITY[key] = torch.arange(n, dtype=torch.int32, device=device)
+    return t
+
+
+def _pair_tokens(tokens: int, k: int, device: torch.device) -> torch.Tensor:
+    """The token of each of `tokens * k` pairs (pair t * k + j belongs to token t) as int32, kept between calls."""
+    key = ("pairs", tokens, k, device)
+    t = _IDENTITY.get(key)
+    if t is None:
+        if len(_IDENTITY) >= 64:
+            _IDENTITY.clear()
+        t = _IDENTITY[key] = torch.arange(tokens, dtype=torch.int32, device=device).repeat_interleave(k)
     return t
 
 

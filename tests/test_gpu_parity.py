@@ -1318,6 +1318,61 @@ def test_gated_activations_equal_what_mlx_lm_recorded():
             assert float(ratio.max()) <= 1.0, (label, name)
 
 
+@pytest.mark.parametrize("quant", ["MXFP4", "MXFP8", "NVFP4", "affine4-g64", "affine4-g32"])
+@pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai", "geglu"])
+def test_unsorted_pairs_with_the_gated_epilogue(quant, activation):
+    """`nvq_gather_qmm_glu` without offsets: the experts of decoded tokens, pairs in any order, on the decode kernel with
+    the gated activation as its epilogue (a wavefront takes a gate row and its up row).  Bit for bit the per-pair
+    product of the paired weights followed by `nvq_glu` where that product runs on the same decode kernel (K beyond
+    2048 off the 16x16x32 kernel's shapes), and within a step of the type elsewhere; with the experts' biases; through
+    `SwitchGlu`'s route of fewer than 64 pairs."""
+    from nuvec_amd.layers import SwitchGlu, SwitchProjection
+    rng = np.random.default_rng(7800 + len(quant) + len(activation))
+    q_of = {"MXFP4": nv.Quant.new(nv.QuantMode.MXFP4), "MXFP8": nv.Quant.new(nv.QuantMode.MXFP8), "NVFP4": nv.Quant.new(nv.QuantMode.NVFP4),
+            "affine4-g64": nv.Quant.affine(64, 4), "affine4-g32": nv.Quant.affine(32, 4)}[quant]
+    experts, hidden = 5, 1088  # (affine projections below 1024 rows stay apart)
+    for dtype, k in ((ref.BF16, 2880), (ref.F16, 2304), (ref.BF16, 768)):
+        gate = nv.quantize(to_dev(make_w(rng, experts * hidden, k, dtype).reshape(experts, hidden, k)), q_of)
+        up = nv.quantize(to_dev(make_w(rng, experts * hidden, k, dtype).reshape(experts, hidden, k)), q_of)
+        down = nv.quantize(to_dev(make_w(rng, experts * 1024, hidden, dtype).reshape(experts, 1024, hidden)), q_of)
+        pair = lambda a, b: None if a is None else nv.pair_rows(a, b, 1)
+        both = nv.Quantized(pair(gate.weight, up.weight), pair(gate.scales, up.scales), pair(gate.biases, up.biases), q_of)
+        tokens, top = 3, 4
+        x = to_dev(make_x(rng, tokens, k, dtype))
+        ids = torch.from_numpy(np.stack([rng.permutation(experts)[:top] for _ in range(tokens)]).astype(np.int32)).cuda()
+        rows = torch.arange(tokens, dtype=torch.int32, device="cuda").repeat_interleave(top)
+        gb, ub = to_dev(make_x(rng, experts, hidden, dtype)), to_dev(make_x(rng, experts, hidden, dtype))
+        xe = x[rows.long()].unsqueeze(1)
+        g = nv.gather_qmm(xe, gate, None, ids.reshape(-1)).squeeze(1)
+        u = nv.gather_qmm(xe, up, None, ids.reshape(-1)).squeeze(1)
+        for biased in (False, True):
+            kw = dict(gate_bias=gb, up_bias=ub, ids=ids.reshape(-1)) if biased else {}
+            want = nv.glu(g, u, activation, alpha=1.702, limit=7.0, **kw)
+            got = nv.gather_qmm_glu(x, both, rows, ids.reshape(-1), None, activation, alpha=1.702, limit=7.0,
+                                    expert_bias=nv.pair_rows(gb, ub, 1) if biased else None)
+            assert tuple(got.shape) == (tokens * top, hidden)
+            if k > 2048 and not (quant == "affine4-g64" and k % 512 == 0):  # the same kernel both ways
+                assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"{quant} {activation} K={k} biased {biased}"
+            else:
+                scale = float(want.float().abs().max())
+                assert float((got.float() - want.float()).abs().max()) <= 2e-2 * scale, f"{quant} {activation} K={k} biased {biased}"
+        block = SwitchGlu(SwitchProjection(gate.weight, gate.scales, gate.biases, gb, q_of), SwitchProjection(up.weight, up.scales, up.biases, ub, q_of),
+                          SwitchProjection(down.weight, down.scales, down.biases, None, q_of), activation=activation)
+        apart = block(x.reshape(1, tokens, k), ids.reshape(1, tokens, top))
+        fused = block.fuse_gate_up()
+        assert fused.gate_up_paired
+        together = fused(x.reshape(1, tokens, k), ids.reshape(1, tokens, top))
+        scale = float(apart.float().abs().max())
+        assert tuple(together.shape) == (1, tokens, top, 1024) and float((together.float() - apart.float()).abs().max()) <= 2e-2 * scale
+    with pytest.raises(nv.Unsupported):  # five rows of x per pair are beyond the decode kernel
+        from nuvec_amd import _lib
+        import ctypes as C
+        d = _lib.GatherDescC(q_of._c(), _lib.BF16, 1, 0, 0, 5, 2 * hidden, k, 2, 2, experts)
+        p = lambda t: C.c_void_p(None if t is None else t.data_ptr())
+        _lib.check(_lib.load().nvq_gather_qmm_glu(C.byref(d), 0, 1.702, 7.0, p(x), p(both.weight), p(both.scales), p(both.biases), p(rows), p(rows),
+                                                  None, None, p(x), None))
+
+
 @pytest.mark.parametrize("quant", ["MXFP4", "affine4", "affine8", "NVFP4"])
 @pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai", "geglu"])
 def test_grouped_gather_with_the_gated_epilogue(quant, activation):

@@ -163,6 +163,7 @@ def determinism_cases():
     kv = nv.quantize(to_dev(make_x(rng, 2 * 700, 128, ref.BF16)).reshape(1, 2, 700, 128), nv.Quant.affine(64, 3))
     qh = to_dev(make_x(rng, 8, 128, ref.BF16)).reshape(1, 8, 1, 128)
     cases["attention, 3-bit cache"] = lambda: nv.ops.quantized_attention(qh, kv, kv, 0.088)
+    cases["unsorted pairs with the gated epilogue"] = lambda: nv.gather_qmm_glu(xe.reshape(512, 1024)[:24], paired, tokens[:24], ids.to(torch.int32)[:24].flip(0), None, "geglu")
     cases["quantize b4"] = lambda: nv.quantize(wd, nv.Quant.affine(64, 4)).weight
     cases["quantize mxfp4"] = lambda: nv.quantize(wd, nv.QuantMode.MXFP4).weight
     cases["dequantize b4"] = lambda: nv.dequantize(q4)
