@@ -375,6 +375,16 @@ NVQ_API int32_t nvq_gather_qmm_expert_bias(const nvq_gather_desc *desc, const vo
                                    const int32_t *offsets, const uint32_t *out_rows, const void *expert_bias, void *y,
                                    void *workspace, void *stream);
 
+/* `Mlp::forward` up to its down projection (crates/nuvec-lm/src/model.rs:2066-2074: `swiglu(gate(x), up(x))`, Gemma's
+ * `geglu`) for up to four rows of x in one kernel: w, scales, biases (and bias, dtype[n] or NULL: the two
+ * projections' biases, layers.rs:155-162) hold the gate and up projections in alternating runs of 64 rows as for
+ * nvq_gather_qmm_glu, desc->n is their total, y dtype[m, n / 2] = act(x . gate^T + bias_gate, x . up^T + bias_up) with
+ * the products rounded to `dtype` first: bit for bit nvq_quantized_linear on the decode kernel followed by nvq_glu.
+ * NVQ_UNSUPPORTED beyond four rows, for float32, batches, untransposed weights and affine widths other than 4 bits
+ * (the caller then composes the products and nvq_glu). */
+NVQ_API int32_t nvq_quantized_matmul_glu(const nvq_qmm_desc *desc, int32_t activation, float alpha, float limit, const void *x,
+                                 const void *w, const void *scales, const void *biases, const void *bias, void *y, void *stream);
+
 /* The grouped gathered product of the experts' gate and up projections with the gated activation as its epilogue:
  * `SwitchGlu::through` up to its down projection (crates/nuvec-lm/src/model.rs:2157-2169) in one kernel.  w, scales,
  * biases and expert_bias hold both projections in alternating runs of 64 rows (rows 128 b .. 128 b + 63: rows

@@ -8,4 +8,4 @@ into `Quantized` operands in device memory.
 """
 from .ops import (GatherQmm, InvalidArgument, Quant, QuantMode, Quantized, Unsupported, dequantize, embedding,  # noqa: F401
                   gather_qmm, gather_qmm_glu, gather_qmm_grouped, gather_qqmm, glu, moe_order, pair_rows, moe_route, qqmm, quantize, quantize_dequantize,
-                  quantized_matmul, quantized_matmul_route, sorted_offsets, weighted_sum)
+                  quantized_matmul, quantized_matmul_glu, quantized_matmul_route, sorted_offsets, weighted_sum)

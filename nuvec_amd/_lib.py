@@ -107,6 +107,7 @@ SIGNATURES = {
     "nvq_gather_qmm_expert_bias": (C.c_int32, [C.c_void_p] * 14),
     "nvq_quantize_dequantize": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_moe_route": (C.c_int32, [C.c_int32, C.c_void_p, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "nvq_quantized_matmul_glu": (C.c_int32, [C.POINTER(QmmDescC), C.c_int32, C.c_float, C.c_float] + [C.c_void_p] * 7),
     "nvq_gather_qmm_glu": (C.c_int32, [C.POINTER(GatherDescC), C.c_int32, C.c_float, C.c_float] + [C.c_void_p] * 10),
     "nvq_glu": (C.c_int32, [C.POINTER(GluDescC), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "nvq_weighted_sum": (C.c_int32, [C.c_int32, C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_int64, C.c_void_p, C.c_void_p]),

@@ -582,6 +582,37 @@ int32_t nvq_quantized_linear(const nvq_qmm_desc *d, const void *x, const void *w
     return quantized_matmul_any(d, x, w, scales, biases, nullptr, y, workspace, stream, bias);
 }
 
+// `Mlp::forward` up to its down projection (crates/nuvec-lm/src/model.rs:2066-2074) for a few rows of x: the gate and up
+// products and the gated activation in one kernel.
+int32_t nvq_quantized_matmul_glu(const nvq_qmm_desc *d, int32_t activation, float alpha, float limit, const void *x, const void *w,
+                                 const void *scales, const void *biases, const void *bias, void *y, void *stream) {
+    const char *op = "quantized_matmul";
+    NVQ_TRY(check_qmm(d, op));
+    NVQ_TRY(check_groups(op, d->quant.mode, biases));
+    if (activation < NVQ_GLU_SWIGLU || activation > NVQ_GLU_GEGLU) return fail(NVQ_INVALID_ARGUMENT, "%s: unknown activation %d", op, activation);
+    if (d->m == 0 || d->n == 0) return NVQ_OK;
+    if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null operand", op);
+    if (!d->transpose || d->batch_ndim != 0 || d->k == 0 || d->n % 128 != 0 || d->row_exact || d->rows)
+        return fail(NVQ_UNSUPPORTED, "%s: the gated epilogue takes x [M, K] times transposed weights whose gate and up rows alternate in runs of 64", op);
+    if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2))
+        return fail(NVQ_UNSUPPORTED, "%s: the gated epilogue takes affine projections of 1024 rows or more each", op);
+    NVQ_TRY(require_device());
+    NVQ_TRY(check_aligned(op, "x", x));
+    NVQ_TRY(check_aligned(op, "w", w));
+    NVQ_TRY(check_aligned(op, "y", y));
+    NVQ_TRY(check_groups_aligned(op, d->quant, d->dtype, scales, biases));
+    NVQ_TRY(check_aligned(op, "bias", bias, (size_t)dtype_size(d->dtype)));
+    ProductArgs a{};
+    a.x = x; a.w = w; a.scales = scales; a.biases = biases; a.y = y;
+    a.mode = d->quant.mode; a.group = d->quant.group_size; a.bits = d->quant.bits; a.dtype = d->dtype;
+    a.m = d->m; a.n = d->n; a.k = d->k;
+    a.batch = 1;
+    a.row_bias = bias;
+    a.glu = 1 + activation; a.glu_alpha = alpha; a.glu_limit = limit;
+    if (!qmv_glu_pairs_take(a)) return fail(NVQ_UNSUPPORTED, "%s: the decode kernel does not take this product with the gated epilogue", op);
+    return launch_qmv_glu_pairs(a, (hipStream_t)stream);
+}
+
 int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *d, const void *x, const void *w, const void *scales, const void *biases,
                                     void *y, void *stream) {
     NVQ_TRY(check_qmm(d, "quantized_matmul"));

@@ -1135,8 +1135,8 @@ int32_t run_lds4(const ProductArgs &a, hipStream_t s) {
 // The pairs of a gather with the gated activation as the epilogue: whether the decode kernel takes them (4-bit affine
 // codes that are never materialised, or a block format; bf16 / f16; up to four rows of x per pair; K in whole slices;
 // the two projections' rows in whole runs of 64) ...
-bool glu_pairs_take(const ProductArgs &a) {
-    if (a.rhs == nullptr || a.dtype == NVQ_F32 || a.row_exact || a.exact_weights || a.out_rows != nullptr) return false;
+bool glu_pairs_take(const ProductArgs &a) {  // (also a single product, without pairs: batch 1)
+    if ((a.rhs == nullptr && a.batch != 1) || a.dtype == NVQ_F32 || a.row_exact || a.exact_weights || a.out_rows != nullptr) return false;
     if (a.m < 1 || a.m > 4 || a.k % 32 != 0 || a.n % 128 != 0 || ((uintptr_t)a.w | (uintptr_t)a.x) % 16 != 0) return false;
     if (a.mode == NVQ_AFFINE) return a.bits == 4;
     return a.mode != NVQ_NVFP4 || (uintptr_t)a.scales % 2 == 0;

@@ -729,6 +729,48 @@ def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids
     return out
 
 
+def quantized_matmul_glu(x: torch.Tensor, q: Quantized, activation: str = "swiglu", *, alpha: float = 1.702, limit: float = 7.0,
+                         bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`Mlp::forward` up to the down projection (model.rs:2066-2074) for a few rows of x in one kernel: `q` (and `bias`
+    `[N]`) hold the gate and up projections in alternating runs of 64 rows (`pair_rows`); the result is `[..., N / 2]`, bit
+    for bit `glu(gate(x), up(x))` of the two rounded products.  Raises `Unsupported` beyond four rows of x and where the
+    decode kernel does not take the product (the caller then composes the products and `glu`)."""
+    op = "quantized_matmul"
+    if activation not in GLU_ACTIVATIONS:
+        raise InvalidArgument(f"{op}: unknown activation {activation!r}")
+    quant = q.quant
+    quant.checked(op)
+    _check_groups(op, quant.mode, q.scales, q.biases)
+    if q.global_scale is not None:
+        raise Unsupported(f"{op}: the gated epilogue takes no global scale")
+    affine = quant.mode == QuantMode.AFFINE
+    dtype = _promoted(op, x, q.scales, q.biases)
+    w = _u32(q.weight)
+    if x.ndim < 1 or w.ndim != 2:
+        raise Unsupported(f"{op}: the gated epilogue takes x [..., K] and one weight matrix, got {list(x.shape)} and {list(w.shape)}")
+    x = x.to(dtype).contiguous()
+    w = w.contiguous()
+    scales = (q.scales.to(dtype) if affine else q.scales).contiguous()
+    biases = q.biases.to(dtype).contiguous() if affine else None
+    columns = _quantized_columns(op, w, scales, biases, quant)
+    n = w.shape[0]
+    if x.shape[-1] != columns:
+        raise InvalidArgument(f"{op}: shapes {list(x.shape)} and {list(w.shape)} do not match")
+    if bias is not None and (bias.dtype != dtype or tuple(bias.shape) != (n,)):
+        raise InvalidArgument(f"{op}: the fused bias must be [{n}] of {_name(dtype)}")
+    _init(x)
+    rows = x.numel() // columns if columns else 0
+    out = torch.empty(x.shape[:-1] + (n // 2,), dtype=dtype, device=x.device)
+    d = _lib.QmmDescC()
+    d.quant, d.dtype, d.transpose = quant._c(), _CODE[dtype], 1
+    d.m = d.item_rows = rows
+    d.n, d.k, d.batch_ndim = n, columns, 0
+    _lib.check(_lib.load().nvq_quantized_matmul_glu(C.byref(d), GLU_ACTIVATIONS[activation], float(alpha), float(limit), _ptr(x), _ptr(w),
+                                                    _ptr(scales), _ptr(biases), _ptr(None if bias is None else bias.contiguous()),
+                                                    _ptr(out), _stream()))
+    return out
+
+
 def pair_rows(gate: torch.Tensor, up: torch.Tensor, dim: int) -> torch.Tensor:
     """The gate and up projections' rows (along `dim`, a multiple of 64 long) in alternating runs of 64: the layout
     `gather_qmm_glu` reads.  A copy, made once at load time."""

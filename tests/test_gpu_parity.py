@@ -1318,6 +1318,63 @@ def test_gated_activations_equal_what_mlx_lm_recorded():
             assert float(ratio.max()) <= 1.0, (label, name)
 
 
+@pytest.mark.parametrize("quant", ["MXFP4", "NVFP4", "affine4-g64", "affine4-g128"])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_dense_mlp_with_the_gated_epilogue(quant, dtype):
+    """`Mlp::forward` (model.rs:2044-2075) over the library: the composition (two products with their biases, the
+    activation, the down projection) against the oracle's products and activation, and — with the gate and up
+    projections stored as one weight — up to four rows of x through `nvq_quantized_matmul_glu`: bit for bit the
+    composition where its products run on the same decode kernel (K = 2880), within a step of the type elsewhere."""
+    from nuvec_amd.layers import Mlp, QuantizedLinear
+    from oracle import moe
+    rng = np.random.default_rng(7900 + len(quant) + dtype)
+    affine = quant.startswith("affine")
+    q_of = nv.Quant.affine(int(quant.split("g")[1]), 4) if affine else nv.Quant.new(getattr(nv.QuantMode, quant))
+    hidden = 1152
+    for k, geglu, biased in ((2880, False, True), (2880, True, False), (4096, False, False)):
+        def linear(n, kk, with_bias):
+            q = nv.quantize(to_dev(make_w(rng, n, kk, dtype)), q_of)
+            return QuantizedLinear(q.weight, q.scales, q.biases, to_dev(make_x(rng, 1, n, dtype)[0]) if with_bias else None, q.quant)
+        if quant == "affine4-g128" and k % 128:
+            k = 2944
+        gate, up, down = linear(hidden, k, biased), linear(hidden, k, biased), linear(1024, hidden, biased)
+        apart = Mlp(gate, up, down, geglu)
+        fused = Mlp(gate, up, down, geglu).fuse_gate_up()
+        assert fused.gate_up_proj is not None
+        for rows in (1, 2, 3, 4, 5):
+            x = to_dev(make_x(rng, rows, k, dtype))
+            want = apart(x)
+            got = fused(x)
+            assert tuple(got.shape) == (rows, 1024)
+            if k % 512:  # (both ways on the decode kernel)
+                assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"{quant} K={k} rows={rows}"
+            else:
+                assert float((got.float() - want.float()).abs().max()) <= 2e-2 * float(want.float().abs().max())
+        # the hidden activations against the oracle: products, biases, activation
+        x = to_dev(make_x(rng, 2, k, dtype))
+        p = fused.gate_up_proj
+        hid = to_host(nv.quantized_matmul_glu(x, p.quantized(), "geglu" if geglu else "swiglu", bias=p.bias))
+        def product(lin):
+            args = (to_host(lin.weight), to_host(lin.scales), None if lin.biases is None else to_host(lin.biases))
+            if affine:
+                y = ref.quantized_matmul(to_host(x), *args, group=q_of.group_size, bits=4, dtype=dtype)
+            else:
+                mode = getattr(ref, quant)
+                group, bits = ref.FP_PARAMS[mode]
+                y = ref.quantized_matmul(to_host(x), args[0], args[1], None, mode=mode, group=group, bits=bits, dtype=dtype)
+            if lin.bias is not None:
+                y = ref.from_f32(ref.to_f32(ref.from_f32(ref.to_f32(y, dtype), dtype), dtype) + ref.to_f32(to_host(lin.bias), dtype), dtype)
+            return y
+        want_hid = moe.glu(product(gate), product(up), dtype, moe.GEGLU if geglu else moe.SWIGLU)
+        wf, gf = ref.to_f32(want_hid, dtype), ref.to_f32(hid, dtype)
+        bound = (4e-2 if dtype == ref.BF16 else 1e-2) * np.abs(wf).max()  # (the activation of two outputs that each carry the product's bar)
+        assert float(np.abs(gf - wf).max()) <= bound, f"{quant} K={k}: hidden activations against the oracle"
+    with pytest.raises(nv.Unsupported):
+        nv.quantized_matmul_glu(to_dev(make_x(rng, 5, k, dtype)), fused.gate_up_proj.quantized())
+    with pytest.raises(nv.InvalidArgument):
+        nv.quantized_matmul_glu(x, fused.gate_up_proj.quantized(), "reglu")
+
+
 @pytest.mark.parametrize("quant", ["MXFP4", "MXFP8", "NVFP4", "affine4-g64", "affine4-g32"])
 @pytest.mark.parametrize("activation", ["swiglu", "swiglu_oai", "geglu"])
 def test_unsorted_pairs_with_the_gated_epilogue(quant, activation):

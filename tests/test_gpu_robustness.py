@@ -164,6 +164,9 @@ def determinism_cases():
     qh = to_dev(make_x(rng, 8, 128, ref.BF16)).reshape(1, 8, 1, 128)
     cases["attention, 3-bit cache"] = lambda: nv.ops.quantized_attention(qh, kv, kv, 0.088)
     cases["unsorted pairs with the gated epilogue"] = lambda: nv.gather_qmm_glu(xe.reshape(512, 1024)[:24], paired, tokens[:24], ids.to(torch.int32)[:24].flip(0), None, "geglu")
+    q4p = nv.Quantized(nv.pair_rows(q4.weight[:2048], q4.weight[2048:], 0), nv.pair_rows(q4.scales[:2048], q4.scales[2048:], 0),
+                       nv.pair_rows(q4.biases[:2048], q4.biases[2048:], 0), q4.quant)
+    cases["two rows with the gated epilogue"] = lambda: nv.quantized_matmul_glu(x512[:2], q4p, "swiglu")
     cases["quantize b4"] = lambda: nv.quantize(wd, nv.Quant.affine(64, 4)).weight
     cases["quantize mxfp4"] = lambda: nv.quantize(wd, nv.QuantMode.MXFP4).weight
     cases["dequantize b4"] = lambda: nv.dequantize(q4)
