@@ -255,7 +255,8 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 
 // What a lane of the decode kernels reads of the scales of its 32 values: the element (affine), NVFP4's two bytes at
 // once, or one byte.
-template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
+constexpr int kAffine8 = 64;  // as a MODE of the decode kernels: affine codes of 8 bits (NVQ_AFFINE there means 4 bits)
+template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE || MODE == kAffine8, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
 
 // A lane's slice of 32 values of one weight row against the same slice of RM rows of x (xp: the four pieces of eight
 // values as pairs, in the expansion's pair order for affine codes and in memory order for the block formats; xs: the
@@ -263,12 +264,37 @@ template <typename T, int MODE> struct SliceScale { using type = std::conditiona
 // B + c.  Block formats: the conversion instructions give the code values, the group's float32 scale (NVFP4: two
 // groups) multiplies the group's sum.
 template <typename T, int RM, int MODE>
-__device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 ? 2 : 1], typename SliceScale<T, MODE>::type sraw, T braw,
+__device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 || MODE == kAffine8 ? 2 : 1], typename SliceScale<T, MODE>::type sraw, T braw,
                                           const uint4 (&xp)[RM][4], const float (&xs)[RM], float factor, uint32_t mask, uint32_t magic,
                                           float (&acc)[RM]) {
-    constexpr int BITS = MODE == NVQ_MXFP8 ? 8 : 4;
+    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : 4;
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;
-    if constexpr (MODE == NVQ_AFFINE) {
+    if constexpr (MODE == kAffine8) {
+        // 8-bit codes: converted (a bf16 mantissa has no room for them), paired in memory order; the slice is inside one
+        // group (groups of 32 and more): scale * dot + bias * sum x
+        float dot[RM][2];
+#pragma unroll
+        for (int i = 0; i < RM; i++) dot[i][0] = dot[i][1] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint4 q = wq[j >> 1];
+            const uint32_t d0 = (j & 1) ? q.z : q.x, d1 = (j & 1) ? q.w : q.y;
+            const uint32_t p0 = qmf::Ops<T>::pack(qmf::ubyte_to_float<0>(d0), qmf::ubyte_to_float<1>(d0));
+            const uint32_t p1 = qmf::Ops<T>::pack(qmf::ubyte_to_float<2>(d0), qmf::ubyte_to_float<3>(d0));
+            const uint32_t p2 = qmf::Ops<T>::pack(qmf::ubyte_to_float<0>(d1), qmf::ubyte_to_float<1>(d1));
+            const uint32_t p3 = qmf::Ops<T>::pack(qmf::ubyte_to_float<2>(d1), qmf::ubyte_to_float<3>(d1));
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                dot[i][0] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][1]);
+            }
+        }
+        const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
+#pragma unroll
+        for (int i = 0; i < RM; i++) acc[i] = __builtin_fmaf(sc, dot[i][0] + dot[i][1], __builtin_fmaf(bi, xs[i], acc[i]));
+    } else if constexpr (MODE == NVQ_AFFINE) {
         const uint32_t d[4] = {wq[0].x, wq[0].y, wq[0].z, wq[0].w};
         float dot[RM][4];
 #pragma unroll
@@ -365,8 +391,8 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     constexpr int kThreads = WAVES * 64;
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
     static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
-    constexpr bool kAffine = MODE == NVQ_AFFINE;
-    constexpr int BITS = MODE == NVQ_MXFP8 ? 8 : 4;
+    constexpr bool kAffine = MODE == NVQ_AFFINE || MODE == kAffine8;
+    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : 4;
     constexpr int kQuads = BITS / 4;                    // 16-byte loads of a lane's 32 codes
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
     __shared__ uint4 x_pairs[RM][2][4][64];               // [row][chunk][word][lane]: 4 pairs of eight values
@@ -441,11 +467,13 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const int idx = tid + p * kThreads;  // 128-bit piece: chunk idx/256, lane (idx%256)/4, word idx%4
                 const uint4 q = xg[i][p];            // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
                 if constexpr (kAffine) {
-                    uint4 pr;
-                    pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
-                    pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
-                    pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
-                    pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+                    uint4 pr = q;
+                    if constexpr (MODE == NVQ_AFFINE) {  // (8-bit codes are converted in memory order)
+                        pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
+                        pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
+                        pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
+                        pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);  // (x3, x7)
+                    }
                     x_pairs[i][idx >> 8][idx & 3][(idx & 255) >> 2] = pr;
                     float sum = Pair<T>::dot2(pr.x, ones, 0.0f);
                     sum = Pair<T>::dot2(pr.y, ones, sum);
@@ -1217,6 +1245,12 @@ int32_t run_short(const ProductArgs &a, hipStream_t s) {
     return run_short_lanes<T, MODE, 64>(a, s);
 }
 
+// Whether the decode kernel takes a row against 8-bit affine codes.
+inline bool decode8_takes(const ProductArgs &a) {
+    return a.mode == NVQ_AFFINE && a.bits == 8 && a.dtype != NVQ_F32 && a.m == 1 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
+           ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
+}
+
 template <typename T, int MODE>
 int32_t run_block_decode(const ProductArgs &a, hipStream_t s) {
     if (a.m == 1) return run_lds4<T, 1, 1, 8, MODE>(a, s);
@@ -1262,6 +1296,10 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
     if (a.mode == NVQ_MXFP8) return run_general<T, 8, NVQ_MXFP8>(a, s);
     if (a.mode == NVQ_NVFP4) return run_general<T, 4, NVQ_NVFP4>(a, s);
     if constexpr (!std::is_same<T, float>::value) {
+        // A single row against 8-bit codes (groups of 32 and more hold a lane's 32 values): the decode kernel.  Against
+        // the general kernel below (us): W[4096,4096] g32 6.90 -> 5.80, g64 6.68 -> 5.35; W[14336,4096] g64 15.87 ->
+        // 14.25; W[2880,2880] g32 5.99 -> 4.80; W[4096,14336] g128 15.69 -> 15.62.
+        if (decode8_takes(a)) return run_lds4<T, 1, 1, 8, kAffine8>(a, s);
         if (a.bits == 4 && !a.exact_weights) {  // (the decode kernels never materialise a weight)
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
@@ -1304,7 +1342,7 @@ const char *qmv_kernel_name(const ProductArgs &a) {
         return "qmv4_lds_kernel";
     }
     if (short_decode_takes(a)) return "qmv4_short_kernel";
-    if (block_decode_takes(a)) return "qmv4_lds_kernel";
+    if (block_decode_takes(a) || decode8_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }
 
