@@ -218,6 +218,10 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
         if (a.group == 32) return passes * mb <= 30.0;
         return passes * mb <= 50.0 || (passes <= 4.0 && mb <= 32.0);
     }
+    // A single row of 3- or 8-bit codes with K beyond 2048: the decode kernel of the vector units (3 bits, us: W[4096,4096]
+    // g128 4.91 -> 4.07, W[14336,4096] g128 9.16 -> 7.75, W[32768,4096] g64 20.1 -> 15.0; with K up to 2048 and many
+    // weight rows this kernel stays ahead: W[65536,2048] 17.7 against 24.6).
+    if (a.m == 1 && (a.bits == 3 || a.bits == 8) && a.k > 2048 && nvq::qmv_decode_takes_width(a)) return false;
     switch (a.bits) {
     case 2: return true;
     case 3: return a.group == 128 || a.m >= 2 || rows >= 16384;

@@ -256,7 +256,8 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 // What a lane of the decode kernels reads of the scales of its 32 values: the element (affine), NVFP4's two bytes at
 // once, or one byte.
 constexpr int kAffine8 = 64;  // as a MODE of the decode kernels: affine codes of 8 bits (NVQ_AFFINE there means 4 bits)
-template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE || MODE == kAffine8, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
+constexpr int kAffine3 = 65;  // ... and of 3 bits: a lane's 32 codes are three dwords, carried in a uint4
+template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE || MODE == kAffine8 || MODE == kAffine3, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
 
 // A lane's slice of 32 values of one weight row against the same slice of RM rows of x (xp: the four pieces of eight
 // values as pairs, in the expansion's pair order for affine codes and in memory order for the block formats; xs: the
@@ -294,6 +295,36 @@ __device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 ||
         const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
 #pragma unroll
         for (int i = 0; i < RM; i++) acc[i] = __builtin_fmaf(sc, dot[i][0] + dot[i][1], __builtin_fmaf(bi, xs[i], acc[i]));
+    } else if constexpr (MODE == kAffine3) {
+        // 3-bit codes: piece j is the 24 bits from bit 24 j of the lane's 96; codes 0..3 stay in the low half, codes 4..7
+        // move to the high half, and the pairs (c0, c4) (c1, c5) (c2, c6) (c3, c7) enter as B + c like the 4-bit ones
+        const uint32_t d0 = wq[0].x, d1 = wq[0].y, d2 = wq[0].z;
+        const uint32_t piece[4] = {d0, __builtin_amdgcn_alignbit(d1, d0, 24), __builtin_amdgcn_alignbit(d2, d1, 16), d2 >> 8};
+        float dot[RM][4];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t z = (piece[j] & 0xFFFu) | ((piece[j] << 4) & 0x0FFF0000u);
+            const uint32_t p0 = and_or(z, mask, magic), p1 = and_or(z >> 3, mask, magic);
+            const uint32_t p2 = and_or(z >> 6, mask, magic), p3 = and_or(z >> 9, mask, magic);
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+            }
+        }
+        const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
+        const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+            acc[i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[i]));
+        }
     } else if constexpr (MODE == NVQ_AFFINE) {
         const uint32_t d[4] = {wq[0].x, wq[0].y, wq[0].z, wq[0].w};
         float dot[RM][4];
@@ -391,9 +422,9 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     constexpr int kThreads = WAVES * 64;
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
     static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
-    constexpr bool kAffine = MODE == NVQ_AFFINE || MODE == kAffine8;
-    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : 4;
-    constexpr int kQuads = BITS / 4;                    // 16-byte loads of a lane's 32 codes
+    constexpr bool kAffine = MODE == NVQ_AFFINE || MODE == kAffine8 || MODE == kAffine3;
+    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : MODE == kAffine3 ? 3 : 4;
+    constexpr int kQuads = BITS == 8 ? 2 : 1;           // 16-byte loads of a lane's 32 codes (3 bits: one of 12 bytes)
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
     __shared__ uint4 x_pairs[RM][2][4][64];               // [row][chunk][word][lane]: 4 pairs of eight values
     __shared__ float x_sums[kAffine ? RM : 1][2][64];     // [row][chunk][lane]: sum of the lane's 32 values (affine)
@@ -416,7 +447,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     T *y = (T *)a.y + o.y;
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     uint32_t mask, magic;
-    asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(mask));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 3 ? 0x00070007 : 0x000F000F));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
     float factor = 1.0f;
     if constexpr (MODE == NVQ_NVFP4) factor = qmf::nvfp4_factor(a, BATCHED && a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0);
@@ -451,9 +482,15 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const int n = n0 + r * kRowStep < N ? n0 + r * kRowStep : N - 1;  // tail rows are computed, not stored
                 // the codes are read once: a non-temporal load keeps them from displacing x and the scales in the caches
                 // (8.1 -> 7.8 us at W[14336,4096]; the scales, shared by neighbouring lanes and rows, lose by it)
-                const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
+                if constexpr (BITS == 3) {  // three dwords, dword-aligned
+                    typedef uint32_t u32x3_a4_t __attribute__((ext_vector_type(3), aligned(4)));
+                    const u32x3_a4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4_t *>(w + (int64_t)n * kwords + (kc >> 5) * 3));
+                    wq[u][r][0] = make_uint4(v.x, v.y, v.z, 0u);
+                } else {
+                    const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
 #pragma unroll
-                for (int c = 0; c < kQuads; c++) wq[u][r][c] = stream_load(pw + c);
+                    for (int c = 0; c < kQuads; c++) wq[u][r][c] = stream_load(pw + c);
+                }
                 sraw[u][r] = *reinterpret_cast<const SR *>(scales + (int64_t)n * kgroups + (kc >> gshift));
                 if constexpr (kAffine) braw[u][r] = (biases + (int64_t)n * kgroups)[kc >> gshift];
                 else braw[u][r] = T{};
@@ -468,7 +505,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const uint4 q = xg[i][p];            // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
                 if constexpr (kAffine) {
                     uint4 pr = q;
-                    if constexpr (MODE == NVQ_AFFINE) {  // (8-bit codes are converted in memory order)
+                    if constexpr (MODE != kAffine8) {  // (8-bit codes are converted in memory order)
                         pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
                         pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
                         pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
@@ -1251,6 +1288,12 @@ inline bool decode8_takes(const ProductArgs &a) {
            ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
 }
 
+// ... and against 3-bit ones.
+inline bool decode3_takes(const ProductArgs &a) {
+    return a.mode == NVQ_AFFINE && a.bits == 3 && a.dtype != NVQ_F32 && a.m == 1 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
+           (uintptr_t)a.x % 16 == 0;
+}
+
 template <typename T, int MODE>
 int32_t run_block_decode(const ProductArgs &a, hipStream_t s) {
     if (a.m == 1) return run_lds4<T, 1, 1, 8, MODE>(a, s);
@@ -1300,6 +1343,8 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
         // the general kernel below (us): W[4096,4096] g32 6.90 -> 5.80, g64 6.68 -> 5.35; W[14336,4096] g64 15.87 ->
         // 14.25; W[2880,2880] g32 5.99 -> 4.80; W[4096,14336] g128 15.69 -> 15.62.
         if (decode8_takes(a)) return run_lds4<T, 1, 1, 8, kAffine8>(a, s);
+        // (3 bits, against the general kernel: W[4096,4096] g64 5.47 -> 4.01, W[14336,4096] 12.2 -> 8.2, W[2880,2880] g32 5.39 -> 3.78)
+        if (decode3_takes(a)) return run_lds4<T, 1, 1, 8, kAffine3>(a, s);
         if (a.bits == 4 && !a.exact_weights) {  // (the decode kernels never materialise a weight)
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
@@ -1332,6 +1377,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 
 bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
 bool qmv_block_decode_takes(const ProductArgs &a) { return block_decode_takes(a); }
+bool qmv_decode_takes_width(const ProductArgs &a) { return decode8_takes(a) || decode3_takes(a); }
 
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
@@ -1342,7 +1388,7 @@ const char *qmv_kernel_name(const ProductArgs &a) {
         return "qmv4_lds_kernel";
     }
     if (short_decode_takes(a)) return "qmv4_short_kernel";
-    if (block_decode_takes(a) || decode8_takes(a)) return "qmv4_lds_kernel";
+    if (block_decode_takes(a) || decode8_takes(a) || decode3_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }
 
