@@ -200,7 +200,7 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 static bool takes_decode(const nvq::ProductArgs &a) {
     if (a.dtype == NVQ_F32) return false;
     if (a.mode != NVQ_AFFINE) return nvq::qmv_block_decode_takes(a);
-    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && a.m == 1;
+    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || (a.k > 2048 && nvq::qmv_decode_takes_width(a)));
 }
 
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
@@ -218,10 +218,10 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
         if (a.group == 32) return passes * mb <= 30.0;
         return passes * mb <= 50.0 || (passes <= 4.0 && mb <= 32.0);
     }
-    // A single row of 3- or 8-bit codes with K beyond 2048: the decode kernel of the vector units (3 bits, us: W[4096,4096]
+    // One or two rows of 3-bit, up to three or four of 8-bit codes with K beyond 2048: the decode kernel of the vector units (3 bits, us: W[4096,4096]
     // g128 4.91 -> 4.07, W[14336,4096] g128 9.16 -> 7.75, W[32768,4096] g64 20.1 -> 15.0; with K up to 2048 and many
     // weight rows this kernel stays ahead: W[65536,2048] 17.7 against 24.6).
-    if (a.m == 1 && (a.bits == 3 || a.bits == 8) && a.k > 2048 && nvq::qmv_decode_takes_width(a)) return false;
+    if ((a.bits == 3 || a.bits == 8) && a.k > 2048 && nvq::qmv_decode_takes_width(a)) return false;
     switch (a.bits) {
     case 2: return true;
     case 3: return a.group == 128 || a.m >= 2 || rows >= 16384;

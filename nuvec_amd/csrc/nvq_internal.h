@@ -108,8 +108,8 @@ const char *qmv_kernel_name(const ProductArgs &a);  // which of the vector / dec
 bool qmv_d16_takes(const ProductArgs &a);
 bool qmv_glu_pairs_take(const ProductArgs &a);      // whether the decode kernel takes unsorted pairs with the gated epilogue
 int32_t launch_qmv_glu_pairs(const ProductArgs &a, hipStream_t s);
-bool qmv_block_decode_takes(const ProductArgs &a);
-bool qmv_decode_takes_width(const ProductArgs &a);  // whether the decode kernel takes a single row of these 3- or 8-bit affine codes  // whether the decode kernel takes a product of a block format
+bool qmv_block_decode_takes(const ProductArgs &a);  // whether the decode kernel takes a product of a block format
+bool qmv_decode_takes_width(const ProductArgs &a);  // whether the decode kernel takes these few rows of 3- or 8-bit affine codes
 // The 16x16x32 matrix-core kernel for passes of up to 16 rows of x (affine 2, 3, 4 and 8 bits, every group size).
 bool qmd_supported(const ProductArgs &a);
 int32_t launch_qmd(const ProductArgs &a, hipStream_t s);

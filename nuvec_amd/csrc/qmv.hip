@@ -1282,15 +1282,19 @@ int32_t run_short(const ProductArgs &a, hipStream_t s) {
     return run_short_lanes<T, MODE, 64>(a, s);
 }
 
-// Whether the decode kernel takes a row against 8-bit affine codes.
+// Whether the decode kernel takes a few rows against 8-bit affine codes: up to three, four with groups of 32 (against
+// the kernel that loads the weights straight into operand layout, 2 / 3 / 4 rows, us: W[4096,4096] g32 9.6 / 9.6 / 9.7 ->
+// 6.4 / 7.0 / 7.3, g64 8.2 / 8.2 / 8.2 -> 6.3 / 6.9 / 7.2; W[14336,4096] g32 20.6 / 20.5 / 20.7 -> 14.7 / 17.1 / 17.6, g64
+// 17.8 / 17.7 / 17.8 -> 15.5 / 16.9 / 17.9; W[4096,14336] g64 19.7 / 19.8 / 20.0 -> 17.0 / 20.3 / 21.3).
 inline bool decode8_takes(const ProductArgs &a) {
-    return a.mode == NVQ_AFFINE && a.bits == 8 && a.dtype != NVQ_F32 && a.m == 1 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
+    return a.mode == NVQ_AFFINE && a.bits == 8 && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= (a.group == 32 ? 4 : 3) && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
            ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
 }
 
-// ... and against 3-bit ones.
+// ... and one or two rows against 3-bit ones (two rows: W[4096,4096] 5.95 -> 4.78 us, W[4096,14336] 15.7 -> 12.8 us,
+// W[14336,4096] 11.2 -> 11.3 us; three rows and more are the other kernel's: 5.8 against 6.2, 11.1 against 14.4).
 inline bool decode3_takes(const ProductArgs &a) {
-    return a.mode == NVQ_AFFINE && a.bits == 3 && a.dtype != NVQ_F32 && a.m == 1 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
+    return a.mode == NVQ_AFFINE && a.bits == 3 && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= 2 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
            (uintptr_t)a.x % 16 == 0;
 }
 
@@ -1342,9 +1346,9 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
         // A single row against 8-bit codes (groups of 32 and more hold a lane's 32 values): the decode kernel.  Against
         // the general kernel below (us): W[4096,4096] g32 6.90 -> 5.80, g64 6.68 -> 5.35; W[14336,4096] g64 15.87 ->
         // 14.25; W[2880,2880] g32 5.99 -> 4.80; W[4096,14336] g128 15.69 -> 15.62.
-        if (decode8_takes(a)) return run_lds4<T, 1, 1, 8, kAffine8>(a, s);
+        if (decode8_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine8>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine8>(a, s) : run_lds4<T, 4, 1, 8, kAffine8>(a, s);
         // (3 bits, against the general kernel: W[4096,4096] g64 5.47 -> 4.01, W[14336,4096] 12.2 -> 8.2, W[2880,2880] g32 5.39 -> 3.78)
-        if (decode3_takes(a)) return run_lds4<T, 1, 1, 8, kAffine3>(a, s);
+        if (decode3_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine3>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine3>(a, s) : run_lds4<T, 4, 1, 8, kAffine3>(a, s);
         if (a.bits == 4 && !a.exact_weights) {  // (the decode kernels never materialise a weight)
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against

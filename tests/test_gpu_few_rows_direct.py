@@ -33,7 +33,7 @@ def test_routes_of_the_baseline_configurations():
     for group, bits in ((64, 3), (32, 8)):
         c4 = lambda m, **kw: ops.quantized_matmul_route(m, 4096, 4096, nv.Quant.affine(group, bits), bf16, **kw)
         assert c4(1) == "qmv4_lds_kernel"  # (the decode kernel takes a row of 3- and of 8-bit codes too)
-        assert c4(16) == "qmd_kernel" and c4(2) == "qmd_kernel"
+        assert c4(16) == "qmd_kernel" and c4(5) == "qmd_kernel" and c4(2) == "qmv4_lds_kernel"  # (K = 4096: two rows stay on the decode kernel)
         assert c4(512) == "qmm_kernel"
         assert c4(16, transpose=False) == ("qmn_kernel" if bits == 8 else "qvm_kernel")  # runs of eight codes: 2, 4, 8 bits
         assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
