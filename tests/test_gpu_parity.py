@@ -696,6 +696,42 @@ def test_block_formats_on_the_decode_kernel(mode, qmode, dtype):
         assert_rows_close(got[z], want, dtype, f"decode kernel {qmode} pair {z}", exact_weights=True)
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("bits,group", [(3, 32), (3, 64), (3, 128), (8, 32), (8, 64), (8, 128)])
+def test_decode_kernel_three_and_eight_bits(dtype, bits, group):
+    """The decode kernel's 3-bit and 8-bit variants (a lane's 32 codes: three dwords split 24 bits at a time into two
+    halves of four codes; eight dwords converted in memory order): one row at any K, up to two (3 bits), three or four
+    (8 bits) where K is beyond 2048; K off the kernel's steps, weight rows off the block's eight; a batch and the pairs
+    of a gather.  Against the CPU oracle within the bar and the device arithmetic within half of it."""
+    rng = np.random.default_rng(5200 + 10 * bits + group + dtype)
+    most = 2 if bits == 3 else 4 if group == 32 else 3
+    quant = nv.Quant.affine(group, bits)
+    for m, n, k in [(1, 1030, 4096), (1, 1100, 2944), (1, 2053, 128), (1, 1025, 1024), (2, 1061, 4096 + 128), (most, 1030, 2944), (most, 1024, 8192)]:
+        route = nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
+        # (a single row of 3-bit codes in groups of 128 with K a multiple of 512 up to 2048 stays on the direct kernel)
+        assert route == "qmv4_lds_kernel" or (bits == 3 and group == 128 and k <= 2048 and k % 512 == 0 and route == "qmd_kernel"), (bits, group, m, n, k, route)
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=bits, dtype=dtype, threads=8)
+        assert_rows_close(got, want, dtype, f"decode kernel b{bits} g{group} M={m} N={n} K={k}")
+        assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, f"decode kernel b{bits} g{group} M={m} N={n} K={k}")
+    assert nv.quantized_matmul_route(most + 1, 1030, 4096, quant, TORCH[dtype]) != "qmv4_lds_kernel"
+    # the pairs of a gather, one row each
+    experts, n, k = 3, 1040, 2304
+    w = make_w(rng, experts * n, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
+    q = nv.Quantized(to_dev(packed.reshape(experts, n, -1)), to_dev(scales.reshape(experts, n, -1)), to_dev(biases.reshape(experts, n, -1)), quant)
+    x = make_x(rng, 4, k, dtype)
+    rhs = np.array([2, 0, 2, 1], np.int64)
+    got = to_host(nv.gather_qmm(to_dev(x.reshape(4, 1, k)), q, None, torch.from_numpy(rhs).cuda()))
+    for z in range(4):
+        e = int(rhs[z])
+        want = ref.quantized_matmul(x[z:z + 1], packed[e * n:(e + 1) * n], scales[e * n:(e + 1) * n], biases[e * n:(e + 1) * n], group=group, bits=bits, dtype=dtype)
+        assert_rows_close(got[z], want, dtype, f"decode kernel b{bits} g{group} pair {z}")
+
+
 @pytest.mark.parametrize("quant", ["affine4-g32", "affine4-g64", "affine4-g128", "MXFP4", "MXFP8", "NVFP4"])
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 def test_short_rows_of_gathered_pairs(quant, dtype):
