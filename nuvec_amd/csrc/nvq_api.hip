@@ -200,7 +200,7 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 static bool takes_decode(const nvq::ProductArgs &a) {
     if (a.dtype == NVQ_F32) return false;
     if (a.mode != NVQ_AFFINE) return nvq::qmv_block_decode_takes(a);
-    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || (a.k > 2048 && nvq::qmv_decode_takes_width(a)));
+    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || ((a.k > 2048 || (a.k == 2048 && a.m <= 2 && (a.bits == 5 || a.bits == 6))) && nvq::qmv_decode_takes_width(a)));
 }
 
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {

@@ -257,7 +257,11 @@ __global__ void __launch_bounds__(512) qmv_lds_kernel(const ProductArgs a) {
 // once, or one byte.
 constexpr int kAffine8 = 64;  // as a MODE of the decode kernels: affine codes of 8 bits (NVQ_AFFINE there means 4 bits)
 constexpr int kAffine3 = 65;  // ... and of 3 bits: a lane's 32 codes are three dwords, carried in a uint4
-template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<MODE == NVQ_AFFINE || MODE == kAffine8 || MODE == kAffine3, T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
+constexpr int kAffine6 = 66;  // ... of 6 bits: six dwords, three to a uint4
+constexpr int kAffine5 = 67;  // ... of 5 bits: five dwords, three and two
+constexpr bool is_affine_mode(int mode) { return mode == NVQ_AFFINE || mode == kAffine8 || mode == kAffine3 || mode == kAffine6 || mode == kAffine5; }
+constexpr int slice_quads(int mode) { return mode == NVQ_MXFP8 || mode == kAffine8 || mode == kAffine6 || mode == kAffine5 ? 2 : 1; }  // uint4 that carry a lane's 32 codes
+template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<is_affine_mode(MODE), T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
 
 // A lane's slice of 32 values of one weight row against the same slice of RM rows of x (xp: the four pieces of eight
 // values as pairs, in the expansion's pair order for affine codes and in memory order for the block formats; xs: the
@@ -265,7 +269,7 @@ template <typename T, int MODE> struct SliceScale { using type = std::conditiona
 // B + c.  Block formats: the conversion instructions give the code values, the group's float32 scale (NVFP4: two
 // groups) multiplies the group's sum.
 template <typename T, int RM, int MODE>
-__device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 || MODE == kAffine8 ? 2 : 1], typename SliceScale<T, MODE>::type sraw, T braw,
+__device__ __forceinline__ void slice_dot(const uint4 (&wq)[slice_quads(MODE)], typename SliceScale<T, MODE>::type sraw, T braw,
                                           const uint4 (&xp)[RM][4], const float (&xs)[RM], float factor, uint32_t mask, uint32_t magic,
                                           float (&acc)[RM]) {
     constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : 4;
@@ -310,6 +314,46 @@ __device__ __forceinline__ void slice_dot(const uint4 (&wq)[MODE == NVQ_MXFP8 ||
             const uint32_t z = (piece[j] & 0xFFFu) | ((piece[j] << 4) & 0x0FFF0000u);
             const uint32_t p0 = and_or(z, mask, magic), p1 = and_or(z >> 3, mask, magic);
             const uint32_t p2 = and_or(z >> 6, mask, magic), p3 = and_or(z >> 9, mask, magic);
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+            }
+        }
+        const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
+        const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+            acc[i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[i]));
+        }
+    } else if constexpr (MODE == kAffine6 || MODE == kAffine5) {
+        // 6- and 5-bit codes: piece t is the four codes (24 or 20 bits) from bit 24 t or 20 t of the lane's 192 or 160;
+        // its codes 0, 1 stay in the low half, 2, 3 move to the high half, and the pairs (c0, c2) (c1, c3) enter as B + c
+        constexpr int W = MODE == kAffine6 ? 6 : 5;
+        const uint32_t d0 = wq[0].x, d1 = wq[0].y, d2 = wq[0].z, d3 = wq[1].x, d4 = wq[1].y, d5 = wq[1].z;
+        uint32_t piece[8];
+        if constexpr (W == 6) {
+            piece[0] = d0, piece[1] = __builtin_amdgcn_alignbit(d1, d0, 24), piece[2] = __builtin_amdgcn_alignbit(d2, d1, 16), piece[3] = d2 >> 8;
+            piece[4] = d3, piece[5] = __builtin_amdgcn_alignbit(d4, d3, 24), piece[6] = __builtin_amdgcn_alignbit(d5, d4, 16), piece[7] = d5 >> 8;
+        } else {
+            piece[0] = d0, piece[1] = __builtin_amdgcn_alignbit(d1, d0, 20), piece[2] = __builtin_amdgcn_alignbit(d2, d1, 8), piece[3] = __builtin_amdgcn_alignbit(d2, d1, 28);
+            piece[4] = __builtin_amdgcn_alignbit(d3, d2, 16), piece[5] = d3 >> 4, piece[6] = __builtin_amdgcn_alignbit(d4, d3, 24), piece[7] = d4 >> 12;
+        }
+        constexpr uint32_t kLow = (1u << (2 * W)) - 1;
+        float dot[RM][4];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t za = (piece[2 * j] & kLow) | ((piece[2 * j] << (16 - 2 * W)) & (kLow << 16));
+            const uint32_t zb = (piece[2 * j + 1] & kLow) | ((piece[2 * j + 1] << (16 - 2 * W)) & (kLow << 16));
+            const uint32_t p0 = and_or(za, mask, magic), p1 = and_or(za >> W, mask, magic);
+            const uint32_t p2 = and_or(zb, mask, magic), p3 = and_or(zb >> W, mask, magic);
 #pragma unroll
             for (int i = 0; i < RM; i++) {
                 dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
@@ -422,9 +466,9 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     constexpr int kThreads = WAVES * 64;
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
     static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
-    constexpr bool kAffine = MODE == NVQ_AFFINE || MODE == kAffine8 || MODE == kAffine3;
-    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : MODE == kAffine3 ? 3 : 4;
-    constexpr int kQuads = BITS == 8 ? 2 : 1;           // 16-byte loads of a lane's 32 codes (3 bits: one of 12 bytes)
+    constexpr bool kAffine = is_affine_mode(MODE);
+    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : MODE == kAffine3 ? 3 : MODE == kAffine6 ? 6 : MODE == kAffine5 ? 5 : 4;
+    constexpr int kQuads = slice_quads(MODE);           // loads of a lane's 32 codes (16 bytes each; 3, 5 and 6 bits: 12 and 8)
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
     __shared__ uint4 x_pairs[RM][2][4][64];               // [row][chunk][word][lane]: 4 pairs of eight values
     __shared__ float x_sums[kAffine ? RM : 1][2][64];     // [row][chunk][lane]: sum of the lane's 32 values (affine)
@@ -447,7 +491,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     T *y = (T *)a.y + o.y;
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     uint32_t mask, magic;
-    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 3 ? 0x00070007 : 0x000F000F));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 3 ? 0x00070007 : BITS == 6 ? 0x003F003F : BITS == 5 ? 0x001F001F : 0x000F000F));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
     float factor = 1.0f;
     if constexpr (MODE == NVQ_NVFP4) factor = qmf::nvfp4_factor(a, BATCHED && a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0);
@@ -486,6 +530,19 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                     typedef uint32_t u32x3_a4_t __attribute__((ext_vector_type(3), aligned(4)));
                     const u32x3_a4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4_t *>(w + (int64_t)n * kwords + (kc >> 5) * 3));
                     wq[u][r][0] = make_uint4(v.x, v.y, v.z, 0u);
+                } else if constexpr (BITS == 6 || BITS == 5) {  // three dwords and three (5 bits: two), dword-aligned
+                    typedef uint32_t u32x3_a4_t __attribute__((ext_vector_type(3), aligned(4)));
+                    typedef uint32_t u32x2_a4_t __attribute__((ext_vector_type(2), aligned(4)));
+                    const uint32_t *pw = w + (int64_t)n * kwords + (kc >> 5) * BITS;
+                    const u32x3_a4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4_t *>(pw));
+                    wq[u][r][0] = make_uint4(v.x, v.y, v.z, 0u);
+                    if constexpr (BITS == 6) {
+                        const u32x3_a4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4_t *>(pw + 3));
+                        wq[u][r][1] = make_uint4(t.x, t.y, t.z, 0u);
+                    } else {
+                        const u32x2_a4_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_a4_t *>(pw + 3));
+                        wq[u][r][1] = make_uint4(t.x, t.y, 0u, 0u);
+                    }
                 } else {
                     const uint4 *pw = reinterpret_cast<const uint4 *>(w + (int64_t)n * kwords + (kc >> 5) * BITS);
 #pragma unroll
@@ -505,7 +562,12 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const uint4 q = xg[i][p];            // q.x = (x0,x1) q.y = (x2,x3) q.z = (x4,x5) q.w = (x6,x7)
                 if constexpr (kAffine) {
                     uint4 pr = q;
-                    if constexpr (MODE != kAffine8) {  // (8-bit codes are converted in memory order)
+                    if constexpr (MODE == kAffine6 || MODE == kAffine5) {
+                        pr.x = __builtin_amdgcn_perm(q.y, q.x, 0x05040100u);  // (x0, x2)
+                        pr.y = __builtin_amdgcn_perm(q.y, q.x, 0x07060302u);  // (x1, x3)
+                        pr.z = __builtin_amdgcn_perm(q.w, q.z, 0x05040100u);  // (x4, x6)
+                        pr.w = __builtin_amdgcn_perm(q.w, q.z, 0x07060302u);  // (x5, x7)
+                    } else if constexpr (MODE != kAffine8) {  // (8-bit codes are converted in memory order)
                         pr.x = __builtin_amdgcn_perm(q.z, q.x, 0x05040100u);  // (x0, x4)
                         pr.y = __builtin_amdgcn_perm(q.z, q.x, 0x07060302u);  // (x1, x5)
                         pr.z = __builtin_amdgcn_perm(q.w, q.y, 0x05040100u);  // (x2, x6)
@@ -1293,6 +1355,17 @@ inline bool decode8_takes(const ProductArgs &a) {
 
 // ... and one or two rows against 3-bit ones (two rows: W[4096,4096] 5.95 -> 4.78 us, W[4096,14336] 15.7 -> 12.8 us,
 // W[14336,4096] 11.2 -> 11.3 us; three rows and more are the other kernel's: 5.8 against 6.2, 11.1 against 14.4).
+// ... and up to four rows against 6- and 5-bit ones (us, against the general kernel at one row and the matrix-core kernel
+// of few rows beyond: 6 bits W[4096,4096] g64 1 / 2 / 3 / 4 rows 6.5 / 11.9 / 12.0 / 12.1 -> 4.9 / 5.6 / 6.4 / 7.7, W[14336,4096]
+// 14.5 / 20.6 / 20.8 / 20.8 -> 11.2 / 13.5 / 14.9 / 17.5, W[4096,14336] g128 14.7 / 24.8 / 25.0 / 25.2 -> 14.1 / 15.3 / 18.3 / 20.4;
+// 5 bits W[4096,4096] 6.2 / 11.9 / 12.0 / 12.0 -> 4.7 / 5.3 / 6.5 / 7.5, W[14336,4096] 13.3 / 19.4 / 19.5 / 19.5 -> 10.2 / 12.5 / 14.2 /
+// 16.8.  Rows of K = 2048 and less leave lanes idle: W[8192,2048] 6 bits 2 / 4 rows 8.7 / 8.7 -> 7.3 / 10.3, W[16384,1024]
+// 9.2 / 9.2 -> 10.8 / 16.8, so the callers send those only with one row, or two at K = 2048.)
+inline bool decode56_takes(const ProductArgs &a) {
+    return a.mode == NVQ_AFFINE && (a.bits == 6 || a.bits == 5) && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= 4 && !a.exact_weights && !a.row_exact &&
+           a.k % 32 == 0 && (uintptr_t)a.x % 16 == 0;
+}
+
 inline bool decode3_takes(const ProductArgs &a) {
     return a.mode == NVQ_AFFINE && a.bits == 3 && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= 2 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
            (uintptr_t)a.x % 16 == 0;
@@ -1349,6 +1422,10 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
         if (decode8_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine8>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine8>(a, s) : run_lds4<T, 4, 1, 8, kAffine8>(a, s);
         // (3 bits, against the general kernel: W[4096,4096] g64 5.47 -> 4.01, W[14336,4096] 12.2 -> 8.2, W[2880,2880] g32 5.39 -> 3.78)
         if (decode3_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine3>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine3>(a, s) : run_lds4<T, 4, 1, 8, kAffine3>(a, s);
+        if (decode56_takes(a)) {
+            if (a.bits == 6) return run_block_decode<T, kAffine6>(a, s);
+            return run_block_decode<T, kAffine5>(a, s);
+        }
         if (a.bits == 4 && !a.exact_weights) {  // (the decode kernels never materialise a weight)
             // Four rows at a time run faster on the matrix cores (measured at W[14336,4096]: 14.0 against 15.3 us);
             // one to three rows stay on the vector kernel, whose blocks are smaller and start sooner (7.8 against
@@ -1381,7 +1458,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 
 bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
 bool qmv_block_decode_takes(const ProductArgs &a) { return block_decode_takes(a); }
-bool qmv_decode_takes_width(const ProductArgs &a) { return decode8_takes(a) || decode3_takes(a); }
+bool qmv_decode_takes_width(const ProductArgs &a) { return decode8_takes(a) || decode3_takes(a) || decode56_takes(a); }
 
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
@@ -1392,7 +1469,7 @@ const char *qmv_kernel_name(const ProductArgs &a) {
         return "qmv4_lds_kernel";
     }
     if (short_decode_takes(a)) return "qmv4_short_kernel";
-    if (block_decode_takes(a) || decode8_takes(a) || decode3_takes(a)) return "qmv4_lds_kernel";
+    if (block_decode_takes(a) || decode8_takes(a) || decode3_takes(a) || decode56_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }
 
