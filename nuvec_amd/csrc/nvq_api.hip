@@ -197,10 +197,16 @@ static bool tiled_is_faster(const nvq::ProductArgs &a) {
 // passes x megabytes of weights, fitted to those tables.
 // Whether a few-row product stays on the decode kernels of the vector units (per-row work there is cheaper than a
 // matrix-core kernel's full dequantization up to these row counts).
+// A few rows of 3-, 5-, 6- or 8-bit codes that the decode kernel's variants take ahead of the matrix-core kernels: K
+// beyond 2048 (shorter rows leave its lanes idle), for 5 and 6 bits also two rows at K = 2048.
+static bool wide_decode_takes(const nvq::ProductArgs &a) {
+    return (a.k > 2048 || (a.k == 2048 && a.m <= 2 && (a.bits == 5 || a.bits == 6))) && nvq::qmv_decode_takes_width(a);
+}
+
 static bool takes_decode(const nvq::ProductArgs &a) {
     if (a.dtype == NVQ_F32) return false;
     if (a.mode != NVQ_AFFINE) return nvq::qmv_block_decode_takes(a);
-    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || ((a.k > 2048 || (a.k == 2048 && a.m <= 2 && (a.bits == 5 || a.bits == 6))) && nvq::qmv_decode_takes_width(a)));
+    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || wide_decode_takes(a));
 }
 
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
@@ -212,7 +218,9 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     // MXFP8 W[4096,14336] 16 rows 18.8 / 29.4: every row count up to 16, 32 where K or the matrix is short.
     if (a.mode != NVQ_AFFINE && a.m <= 32) return a.m <= 16 || a.k <= 4096 || rows <= 4096;
     if (a.m > 16) {
-        if (a.k > 4096 || a.m > 192) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
+        // (5 and 6 bits: the passes' never-rounded weights put one of 139360 half-precision outputs of a 130-row product of
+        // 6-bit codes in groups of 128 at 1.06 x the bar against the CPU's doubly rounded ones; the tiles round once)
+        if (a.k > 4096 || a.m > 192 || a.bits == 5 || a.bits == 6) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
         const double passes = (double)((a.m + 15) / 16), mb = (double)rows * (double)a.k * a.bits / 8.0 / 1048576.0;
         if (a.bits == 8) return passes * mb <= (a.group == 32 ? 34.0 : 40.0);
         if (a.group == 32) return passes * mb <= 30.0;
@@ -221,9 +229,14 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     // One or two rows of 3-bit, up to three or four of 8-bit codes with K beyond 2048: the decode kernel of the vector units (3 bits, us: W[4096,4096]
     // g128 4.91 -> 4.07, W[14336,4096] g128 9.16 -> 7.75, W[32768,4096] g64 20.1 -> 15.0; with K up to 2048 and many
     // weight rows this kernel stays ahead: W[65536,2048] 17.7 against 24.6).
-    if ((a.bits == 3 || a.bits == 8) && a.k > 2048 && nvq::qmv_decode_takes_width(a)) return false;
+    if (a.bits != 4 && a.bits != 2 && wide_decode_takes(a)) return false;
     switch (a.bits) {
     case 2: return true;
+    case 5:  // beside the decode kernel's rows, against the few-row kernel of the 32x32x16 instruction (us): 6 bits W[4096,4096] g64
+    case 6:  // 5 / 16 rows 12.2 / 12.4 -> 7.8 / 8.7, W[14336,4096] 8 / 16 rows 21.2 / 21.9 -> 16.6 / 17.2, W[4096,14336] g128 16 rows
+             // 31.0 -> 20.0, W[8192,2048] 4 / 16 rows 8.8 / 10.6 -> 6.4 / 7.2, W[2048,1024] 3 / 16 rows 6.4 / 9.2 -> 4.4 / 5.1; 32 / 64 rows of
+             // W[4096,4096] stay on the tiles (16.9 / 18.2 against 10.5 / 15.5: see above); 5 bits alike
+        return a.m >= 2;
     case 3: return a.group == 128 || a.m >= 2 || rows >= 16384;
     case 8: return a.m >= 2 || rows >= (a.group == 128 ? 32768 : 65536);
     default:  // 4 bits: beside the 4-bit decode kernels

@@ -1,8 +1,8 @@
-// Few rows of x (passes of up to 16) times affine weights of 2, 3, 4 or 8 bits in groups of 32, 64 or 128, bf16 / f16,
+// Few rows of x (passes of up to 16) times affine weights of 2, 3, 4, 5, 6 or 8 bits in groups of 32, 64 or 128, bf16 / f16,
 // on the 16x16x32 matrix instruction with the weights loaded straight into the instruction's operand layout: the
 // counterpart of the reference's few-row matrix-unit kernel affine_qmv_mma (crates/nuvec-kernels/src/metal/quantized.h:1722-1905:
 // 1 to 16 rows, 4 and 8 bits, groups of 32, 64 and 128; routed at crates/nuvec-core/src/gpu.rs:6978-7024), here also
-// for 2 and 3 bits.
+// for 2, 3, 5 and 6 bits.
 //
 // A block of W wavefronts owns 16 RT weight rows and walks K in chunks of W slices of 512 values; wavefront v owns
 // slice v of the chunk.  A slice is cut into spans of 4 C values.  Lane (column n = lane % 16, quarter q = lane / 16)
@@ -41,11 +41,11 @@ template <int MODE, int BITS, int GROUP> constexpr int qmd_chunk() {
 template <typename T, int BITS> constexpr bool qmd_magic() { return !(BITS == 8 && std::is_same<T, bf16_t>::value); }
 
 // The eight values of a piece of x in the order of the expansion's pairs: (0,4)(1,5)(2,6)(3,7) for 2, 3 and 4 bits,
-// (0,2)(1,3)(4,6)(5,7) for 8 bits.
+// (0,2)(1,3)(4,6)(5,7) for 5, 6 and 8 bits.
 template <int BITS>
 __device__ __forceinline__ uint4 qmd_pair_order(const uint4 q) {
     uint4 pr;
-    if constexpr (BITS == 8) {
+    if constexpr (BITS == 8 || BITS == 6 || BITS == 5) {
         pr.x = __builtin_amdgcn_perm(q.y, q.x, 0x05040100u);
         pr.y = __builtin_amdgcn_perm(q.y, q.x, 0x07060302u);
         pr.z = __builtin_amdgcn_perm(q.w, q.z, 0x05040100u);
@@ -57,6 +57,16 @@ __device__ __forceinline__ uint4 qmd_pair_order(const uint4 q) {
         pr.w = __builtin_amdgcn_perm(q.w, q.y, 0x07060302u);
     }
     return pr;
+}
+
+// The LEN bits (up to 32) from bit OFF of the lane's chunk, in the low bits of the result (the bits above them are the
+// chunk's next ones or zeros).
+template <int OFF, int LEN, int DW>
+__device__ __forceinline__ uint32_t qmd_bits(const uint32_t (&dw)[DW]) {
+    constexpr int i = OFF / 32, sh = OFF % 32;
+    if constexpr (sh == 0) return dw[i];
+    else if constexpr (sh + LEN <= 32) return dw[i] >> sh;
+    else return __builtin_amdgcn_alignbit(dw[i + 1], dw[i], sh);
 }
 
 // The weight operand of matrix instruction J from the lane's chunk of a span (DW dwords).  Written in C so that the
@@ -95,8 +105,17 @@ __device__ __forceinline__ uint4 qmd_operand(const uint32_t (&dw)[DW], uint32_t 
         b.y = ((z >> 3) & mask) | magic;
         b.z = ((z >> 6) & mask) | magic;
         b.w = ((z >> 9) & mask) | magic;
+    } else if constexpr (BITS == 6 || BITS == 5) {
+        // four codes (24 or 20 bits) at a time: codes 0, 1 stay in the low half, codes 2, 3 move to the high half
+        constexpr uint32_t kLow = (1u << (2 * BITS)) - 1;
+        const uint32_t va = qmd_bits<8 * BITS * J, 4 * BITS>(dw), vb = qmd_bits<8 * BITS * J + 4 * BITS, 4 * BITS>(dw);
+        const uint32_t za = (va & kLow) | ((va << (16 - 2 * BITS)) & (kLow << 16)), zb = (vb & kLow) | ((vb << (16 - 2 * BITS)) & (kLow << 16));
+        b.x = (za & mask) | magic;
+        b.y = ((za >> BITS) & mask) | magic;
+        b.z = (zb & mask) | magic;
+        b.w = ((zb >> BITS) & mask) | magic;
     } else {
-        static_assert(BITS == 2, "2, 3, 4 and 8 bits");
+        static_assert(BITS == 2, "2, 3, 4, 5, 6 and 8 bits");
         const uint32_t v = dw[J >> 1] >> (16 * (J & 1));
         const uint32_t z = (v & 0xFFu) | ((v << 8) & 0x00FF0000u);
         b.x = (z & mask) | magic;
@@ -112,6 +131,8 @@ template <> struct QmdWords<1> { typedef uint32_t type; };
 template <> struct QmdWords<2> { typedef uint2 type; };
 template <> struct QmdWords<3> { struct __attribute__((aligned(4))) type { uint32_t x, y, z; }; };
 template <> struct QmdWords<4> { typedef uint4 type; };
+template <> struct QmdWords<5> { struct __attribute__((aligned(4))) type { uint32_t x, y, z, w, v; }; };
+template <> struct QmdWords<6> { struct __attribute__((aligned(4))) type { uint32_t x, y, z, w, v, u; }; };
 
 // DW dwords from p (whole-dword aligned; 16-byte aligned where DW is 4 or 8).
 template <int DW>
@@ -178,7 +199,7 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     constexpr float base = qmd_magic<T, BITS>() ? Pair<T>::base : 0.0f;
     uint32_t mask, magic;
-    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 8 ? 0x00FF00FF : BITS == 4 ? 0x000F000F : BITS == 3 ? 0x00070007 : 0x00030003));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 8 ? 0x00FF00FF : BITS == 6 ? 0x003F003F : BITS == 5 ? 0x001F001F : BITS == 4 ? 0x000F000F : BITS == 3 ? 0x00070007 : 0x00030003));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
 
     if (lane == 0) xs[RM * kQmdRowPieces] = make_uint4(0, 0, 0, 0);
@@ -462,7 +483,7 @@ int32_t run_qmd_rows(const ProductArgs &a, hipStream_t s) {
 
 template <typename T, int BITS>
 int32_t run_qmd_group(const ProductArgs &a, hipStream_t s) {
-    if constexpr (BITS == 4 || BITS == 8) {
+    if constexpr (BITS == 4 || BITS == 6 || BITS == 8) {
         if (a.group == 32) return run_qmd_rows<T, NVQ_AFFINE, BITS, 32>(a, s);
     }
     return a.group == 64 ? run_qmd_rows<T, NVQ_AFFINE, BITS, 64>(a, s) : run_qmd_rows<T, NVQ_AFFINE, BITS, 128>(a, s);
@@ -477,19 +498,21 @@ int32_t run_qmd(const ProductArgs &a, hipStream_t s) {
     case 2: return run_qmd_group<T, 2>(a, s);
     case 3: return run_qmd_group<T, 3>(a, s);
     case 4: return run_qmd_group<T, 4>(a, s);
+    case 5: return run_qmd_group<T, 5>(a, s);
+    case 6: return run_qmd_group<T, 6>(a, s);
     default: return run_qmd_group<T, 8>(a, s);
     }
 }
 
 }  // namespace
 
-// Whether the kernel takes the product: bf16 / f16, affine 2, 3, 4 or 8 bits, K in slices of 512, 16-byte aligned
+// Whether the kernel takes the product: bf16 / f16, affine 2, 3, 4, 5, 6 or 8 bits, K in slices of 512, 16-byte aligned
 // scale and bias rows (a lane reads the scales of its slice with vector loads).
 bool qmd_supported(const ProductArgs &a) {
     if (a.dtype == NVQ_F32 || a.row_exact || a.exact_weights) return false;  // (the factored form never materialises a weight)
     if (a.mode == NVQ_AFFINE) {
-        if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 8)) return false;
-        if (!(a.group == 64 || a.group == 128 || (a.group == 32 && a.bits >= 4))) return false;  // 2 and 3 bits in groups of 32: four groups per span
+        if (!(a.bits == 2 || a.bits == 3 || a.bits == 4 || a.bits == 5 || a.bits == 6 || a.bits == 8)) return false;
+        if (!(a.group == 64 || a.group == 128 || (a.group == 32 && (a.bits == 4 || a.bits == 6 || a.bits == 8)))) return false;  // 2, 3 and 5 bits in groups of 32: four groups per span
     }
     if (a.k < kQmdSlice || a.k % kQmdSlice != 0 || a.m < 1) return false;
     if ((a.m + 15) / 16 > 65535 || a.batch > 65535) return false;

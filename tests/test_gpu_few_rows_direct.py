@@ -17,7 +17,7 @@ from tests.test_gpu_parity import assert_device_arithmetic, assert_rows_close, m
 
 pytestmark = pytest.mark.gpu
 
-WIDTHS = [(2, 64), (2, 128), (3, 64), (3, 128), (4, 32), (4, 64), (4, 128), (8, 32), (8, 64), (8, 128)]
+WIDTHS = [(2, 64), (2, 128), (3, 64), (3, 128), (4, 32), (4, 64), (4, 128), (5, 64), (5, 128), (6, 32), (6, 64), (6, 128), (8, 32), (8, 64), (8, 128)]
 
 
 def test_routes_of_the_baseline_configurations():
@@ -66,6 +66,8 @@ def test_direct_few_row_kernel_every_width(dtype, bits, group):
         route = ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
         if bits == 4 and m <= 8:
             continue  # the 4-bit decode kernels' rows
+        if bits in (5, 6) and m > 16:
+            continue  # passes of rows of 5- and 6-bit codes stay on the kernels that round a weight once
         assert route == "qmd_kernel", f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
         packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
@@ -95,7 +97,7 @@ def test_direct_few_row_kernel_batched_with_bias(bits, group):
         assert_rows_close(got[i], want, ref.BF16, f"direct few rows batched b{bits} item {i}")
     # two batch dimensions of dense operands are one to the kernels (not the vector kernels' business)
     assert ops.quantized_matmul_route(m, n, k, quant, torch.bfloat16, batch=(3, 1)) == "qmd_kernel"
-    assert ops.quantized_matmul_route(40, n, k, nv.Quant.affine(64, 6), torch.bfloat16, batch=(2, 3)) == "qmf_kernel"
+    assert ops.quantized_matmul_route(40, n, k, nv.Quant.affine(32, 5), torch.bfloat16, batch=(2, 3)) == "qmf_kernel"  # (5 bits in groups of 32: not the direct kernel's)
     w2, x2 = make_w(rng, 6 * n, k, ref.BF16), make_x(rng, 6 * m, k, ref.BF16)
     p2, s2, b2 = ref.affine_quantize(w2, ref.BF16, group, bits)
     q2 = nv.Quantized(to_dev(p2.reshape(2, 3, n, -1)), to_dev(s2.reshape(2, 3, n, -1)), to_dev(b2.reshape(2, 3, n, -1)), quant)
