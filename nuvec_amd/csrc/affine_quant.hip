@@ -306,8 +306,8 @@ affine_quantize_kernel(const T *__restrict__ w, int64_t rows, int lanes_log2, ui
 // kernels.rs:835-859: round(round(code * scale) + bias), both roundings in T.  With `ids`, output row r is
 // table row ids[r] (the rows of a quantized embedding, crates/nuvec-nn/src/layers.rs:245-255): `row_chunks` chunks
 // per row, ids clamped to the table's `table_rows`.
-// Chunks per thread, a block apart: all their loads are requested before the first conversion.  Four for the 16-bit
-// types; a float32 chunk already moves 32 bytes out and was slower unrolled (70.6 against 57.6 us at [14336,4096], 6 bits).
+// Chunks per thread, a block apart: all their loads are requested before the first conversion.  (The 16-bit types;
+// float32 has the kernel below.)
 template <typename T> constexpr int kUnrollOf = sizeof(T) == 4 ? 1 : 4;
 template <typename T, int BITS>
 __global__ void __launch_bounds__(kBlock)
@@ -361,6 +361,48 @@ affine_dequantize_kernel(const uint8_t *__restrict__ packed, const T *__restrict
     }
 }
 
+// float32 out: a lane's eight values would leave as two 16-byte stores 32 bytes apart.  Here a lane takes four values, one
+// half of a chunk, of two chunks that lie 32 chunks apart, so that each of a wavefront's two stores writes 1 KB of
+// consecutive bytes; the two lanes of a chunk read the same codes, scale and bias.  The arithmetic of a value is the same.
+// [4096,4096] at 4 bits in groups of 64: 18.9 us with the eight-value lanes, 16.3 us with these stores, 12.0-15.1 us with
+// them non-temporal; 3 bits in groups of 128: 20.8 -> 11.8 us.
+template <int BITS>
+__global__ void __launch_bounds__(kBlock)
+affine_dequantize_f32_kernel(const uint8_t *__restrict__ packed, const float *__restrict__ scales, const float *__restrict__ biases,
+                             uint32_t chunks, int lanes_log2, float *__restrict__ out, const uint32_t *__restrict__ ids,
+                             uint32_t row_chunks, int64_t table_rows) {
+    const uint32_t lane = threadIdx.x & 63u, half = lane & 1u;
+    const uint32_t base = blockIdx.x * kBlock + (threadIdx.x & ~63u);  // the wavefront's 64 chunks
+    uint64_t stream_[2];
+    float s_[2], b_[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint32_t at = base + 32 * j + (lane >> 1);
+        const uint32_t chunk = at < chunks ? at : chunks - 1;  // past the end: the last chunk again, never stored
+        int64_t src = chunk;
+        if (ids != nullptr) {
+            const uint32_t r = chunk / row_chunks;
+            const int64_t row = min((int64_t)ids[r], table_rows - 1);
+            src = row * row_chunks + (chunk - r * row_chunks);
+        }
+        stream_[j] = load_codes<BITS>(packed, src) >> (half * 4 * BITS);
+        const int64_t g = src >> lanes_log2;
+        s_[j] = scales[g];
+        b_[j] = biases[g];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint32_t chunk = base + 32 * j + (lane >> 1);
+        if (chunk >= chunks) continue;
+        constexpr uint32_t mask = (1u << BITS) - 1u;
+        float r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[i] = Elem<float>::add(Elem<float>::mul((float)((uint32_t)(stream_[j] >> (i * BITS)) & mask), s_[j]), b_[j]);
+        // written once and not read here again: a non-temporal store
+        stream_store(reinterpret_cast<uint4 *>(out + (int64_t)chunk * 8 + half * 4), make_uint4(f2u(r[0]), f2u(r[1]), f2u(r[2]), f2u(r[3])));
+    }
+}
+
 template <typename T, int BITS>
 int32_t quantize_t(int group, const void *w, int64_t n, void *packed, void *scales, void *biases, hipStream_t s) {
     const int64_t rows = n / 32;  // a lane's 32 values; the group is 1, 2 or 4 of them
@@ -374,6 +416,13 @@ template <typename T, int BITS>
 int32_t dequantize_t(int group, const void *packed, const void *scales, const void *biases, int64_t n, void *out,
                      const uint32_t *ids, int64_t cols, int64_t table_rows, hipStream_t s) {
     const int64_t chunks = n / 8;
+    if constexpr (std::is_same<T, float>::value) {
+        hipLaunchKernelGGL((affine_dequantize_f32_kernel<BITS>), dim3((unsigned)((chunks + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                           (const uint8_t *)packed, (const float *)scales, (const float *)biases, (uint32_t)chunks,
+                           group == 32 ? 2 : group == 64 ? 3 : 4, (float *)out, ids, (uint32_t)(cols / 8), table_rows);
+        NVQ_LAUNCH_CHECK("affine_dequantize");
+        return NVQ_OK;
+    }
     const unsigned blocks = (unsigned)((chunks + kBlock * kUnrollOf<T> - 1) / (kBlock * kUnrollOf<T>));
     hipLaunchKernelGGL((affine_dequantize_kernel<T, BITS>), dim3(blocks), dim3(kBlock), 0, s,
                        (const uint8_t *)packed, (const T *)scales, (const T *)biases, (uint32_t)chunks,
