@@ -33,8 +33,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_216_700   # rocprofv3 FETCH_SIZE + WRITE_SIZE per launch, scaled by a plain 1 GiB copy (profiles/)
-QMM_TRAFFIC_BYTES = 297_185_596  # the same for the tiled kernel at configs[2]
+QMV_TRAFFIC_BYTES = 33_213_631
+QMM_TRAFFIC_BYTES = 297_185_816
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -263,7 +263,10 @@ def all_configs(lib, device, qs):
              7_340_032)
     products("C4 bf16 8-bit g32 W[4096,4096]", 4096, 4096, nv.Quant.affine(32, 8), torch.bfloat16, _lib.BF16, [1, 16, 512], 32,
              18_874_368)
-    # Beside the BASELINE configurations: C2's product with the weights stored [K, N] (transpose = false)
+    # Beside the BASELINE configurations: 6-bit codes, the width mixed-precision checkpoints give their sensitive layers
+    products("beside C4: bf16 6-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 6), torch.bfloat16, _lib.BF16, [1, 4, 16], 32,
+             13_631_488)
+    # ... and C2's product with the weights stored [K, N] (transpose = false)
     products("bf16 4-bit g64 w[4096,14336] stored [K, N]", N, K, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1, 16, 2048], 24,
              WEIGHT_BYTES, transpose=False)
     # C5: 32 MXFP4 experts [2880,2880], 256 tokens x 4 distinct experts, pairs sorted by expert
