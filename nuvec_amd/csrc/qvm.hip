@@ -75,11 +75,16 @@ __device__ __forceinline__ Offsets batch_offsets(const ProductArgs &a, int64_t z
 }
 
 // MODE: NVQ_AFFINE, NVQ_MXFP4, NVQ_MXFP8 or NVQ_NVFP4.  grid = (ceil(N / 2048), splits, batch * passes of RM rows).
-template <typename T, int BITS, int MODE, int RM>
-__global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits, float *partial) {
+// A block's kQvmWaves wavefronts own the same 2048 columns and consecutive pieces of the split's rows of w; their sums
+// meet in LDS in wavefront order, so that the grid's splits (and the reduction kernel's serial additions) stay few
+// while enough wavefronts stream the weights.
+constexpr int kQvmWaves = 8;
+template <typename T, int BITS, int MODE, int RM, bool EXACT = false>
+__global__ void __launch_bounds__(64 * kQvmWaves) qvm_kernel(const ProductArgs a, int splits, float *partial) {
     constexpr bool kAffine = MODE == NVQ_AFFINE;
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane
-    const int lane = threadIdx.x;
+    __shared__ float sums[kQvmWaves - 1][32][64];  // [wavefront - 1][column of the lane][lane]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int K = (int)a.k, N = (int)a.n, M = (int)a.m;
     const int gshift = kAffine ? (a.group == 32 ? 5 : a.group == 64 ? 6 : 7) : (MODE == NVQ_NVFP4 ? 4 : 5);
     const int passes = (M + RM - 1) / RM;
@@ -94,8 +99,10 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
     const uint32_t *w = (const uint32_t *)a.w + o.w + (nc >> 5) * BITS;
     const int64_t s_at = o.s + (nc >> gshift);
     const int per = (K + splits - 1) / splits;
-    const int k_begin = blockIdx.y * per, k_end = k_begin + per < K ? k_begin + per : K;
-    const bool exact = kAffine && a.exact_weights != 0;  // (the same for the whole launch)
+    const int s_begin = blockIdx.y * per, s_end = s_begin + per < K ? s_begin + per : K;  // the split's rows of w
+    const int sub = (s_end - s_begin + kQvmWaves - 1) / kQvmWaves;                          // ... and the wavefront's
+    const int k_begin = s_begin + wave * sub < s_end ? s_begin + wave * sub : s_end, k_end = k_begin + sub < s_end ? k_begin + sub : s_end;
+    constexpr bool exact = kAffine && EXACT;  // the weights as the CPU holds them (rows of few outputs)
 
     float acc[RM][32], accb[RM];
 #pragma unroll
@@ -133,13 +140,17 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
     };
 
     if (k_begin < k_end) {
-        Row ring[2];
-        load_row(k_begin, ring[0]);
-        for (int k = k_begin; k < k_end; k += 2) {
+        // D rows of the weights in flight per lane: a wavefront's row is 1 KB (4 bits), and a split's few wavefronts
+        // need tens of KB each under way to cover the memory latency
+        constexpr int D = RM == 1 ? 8 : 4;
+        Row ring[D];
 #pragma unroll
-            for (int d = 0; d < 2; d++) {
-                load_row(k + d + 1, ring[(d + 1) & 1]);
-                const Row &r = ring[d];
+        for (int d = 0; d < D; d++) load_row(k_begin + d, ring[d]);
+        for (int k = k_begin; k < k_end; k += D) {
+#pragma unroll
+            for (int d = 0; d < D; d++) {
+                const Row r = ring[d];
+                load_row(k + d + D, ring[d]);
                 if (k + d < k_end) {
                     float xs[RM][kHalves];
 #pragma unroll
@@ -161,10 +172,24 @@ __global__ void __launch_bounds__(64) qvm_kernel(const ProductArgs a, int splits
             }
         }
     }
-    if (!live) return;
 #pragma unroll
     for (int i = 0; i < RM; i++) {
-        if (m0 + i >= M) break;
+        if (i > 0) __syncthreads();  // the previous row's sums are read
+        if (wave > 0) {
+#pragma unroll
+            for (int j = 0; j < 32; j++) sums[wave - 1][j][lane] = acc[i][j] + accb[i];
+        }
+        __syncthreads();
+        if (wave > 0) continue;
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            float v = acc[i][j] + accb[i];
+#pragma unroll
+            for (int wv = 0; wv < kQvmWaves - 1; wv++) v += sums[wv][j][lane];
+            acc[i][j] = v;
+        }
+        accb[i] = 0.0f;
+        if (!live || m0 + i >= M) continue;
         if (splits == 1) {
             T *out = (T *)a.y + (o.y * M + m0 + i) * N + n0;
 #pragma unroll
@@ -186,8 +211,17 @@ __global__ void __launch_bounds__(256) qvm_reduce_kernel(const float *partial, T
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     const int64_t b = idx / per_batch, rest = idx - b * per_batch;
+    const float *p = partial + b * splits * per_batch + rest;
     float sum = 0.0f;
-    for (int s = 0; s < splits; s++) sum += partial[(b * splits + s) * per_batch + rest];
+    int s = 0;
+    for (; s + 8 <= splits; s += 8) {  // eight loads under way at a time; the additions keep the splits' order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = p[(int64_t)(s + u) * per_batch];
+#pragma unroll
+        for (int u = 0; u < 8; u++) sum += v[u];
+    }
+    for (; s < splits; s++) sum += p[(int64_t)s * per_batch];
     Elem<T>::store(y, idx, add_row_bias<T>(row_bias, sum, idx % n));
 }
 
@@ -549,8 +583,15 @@ int32_t run_qvm(const ProductArgs &a, void *workspace, hipStream_t s) {
     const int64_t z = a.batch * ((a.m + rm - 1) / rm);
     if (z > 65535) return fail(NVQ_UNSUPPORTED, "quantized_matmul: %lld row passes exceed the grid limit", (long long)z);
     const dim3 grid(tiles, (unsigned)splits, (unsigned)z);
-    if (rm == 1) hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 1>), grid, dim3(64), 0, s, a, splits, (float *)workspace);
-    else hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 4>), grid, dim3(64), 0, s, a, splits, (float *)workspace);
+    constexpr bool kCanBeExact = MODE == NVQ_AFFINE && !std::is_same<T, float>::value;
+    if (kCanBeExact && a.exact_weights) {
+        if (rm == 1) hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 1, kCanBeExact>), grid, dim3(64 * kQvmWaves), 0, s, a, splits, (float *)workspace);
+        else hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 4, kCanBeExact>), grid, dim3(64 * kQvmWaves), 0, s, a, splits, (float *)workspace);
+    } else if (rm == 1) {
+        hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 1>), grid, dim3(64 * kQvmWaves), 0, s, a, splits, (float *)workspace);
+    } else {
+        hipLaunchKernelGGL((qvm_kernel<T, BITS, MODE, 4>), grid, dim3(64 * kQvmWaves), 0, s, a, splits, (float *)workspace);
+    }
     NVQ_LAUNCH_CHECK("qvm");
     if (splits > 1) {
         const int64_t per_batch = a.m * a.n, total = a.batch * per_batch;
@@ -583,15 +624,16 @@ int32_t run_qvm_typed(const ProductArgs &a, void *workspace, hipStream_t s) {
 
 }  // namespace
 
-// Splits of K: enough blocks for about four wavefronts per compute unit, at least 32 rows per split.
+// Splits of K: about a block (of eight wavefronts) per compute unit, at least 16 rows of w per wavefront, at most 32
+// splits (the reduction kernel adds them one after the other).
 int qvm_splits(const ProductArgs &a) {
     const int rm = a.m == 1 ? 1 : 4;
     // row-exact: the split is the one-row product's, whatever the rows and batches, so that every row keeps its bits
     const int64_t base = ((a.n + 2047) / 2048) * (a.row_exact ? 1 : a.batch * ((a.m + rm - 1) / rm));
-    const int64_t want = ((int64_t)compute_units() * 4 + base - 1) / base;
-    const int64_t most = a.k / 32 > 1 ? a.k / 32 : 1;
+    const int64_t want = ((int64_t)compute_units() + base - 1) / base;
+    const int64_t most = a.k / (16 * kQvmWaves) > 1 ? a.k / (16 * kQvmWaves) : 1;
     const int64_t splits = want < 1 ? 1 : (want > most ? most : want);
-    return (int)(splits > 1024 ? 1024 : splits);
+    return (int)(splits > 32 ? 32 : splits);
 }
 
 size_t qvm_workspace_bytes(const ProductArgs &a) {
@@ -603,6 +645,9 @@ size_t qvm_workspace_bytes(const ProductArgs &a) {
     return splits > 1 ? (size_t)splits * (size_t)a.batch * (size_t)a.m * (size_t)a.n * sizeof(float) : 0;
 }
 
+// (With eight wavefronts a block, eight rows of w in flight per lane and at most 32 splits the vector kernel above went,
+// at bf16 4-bit g64 and one row of x, kernel and reduction: w[4096,14336] 67 -> 23 us, w[14336,4096] 143 -> 52 us,
+// w[4096,4096] 65 -> 19 us; the matrix-core kernel: 23 / 26 / 12 us, and flat up to 16 rows where this one adds 8 us a row.)
 // The matrix-core kernel takes the 16-bit products whose codes come in whole runs of eight columns (2, 4 and 8 bits,
 // the block formats without a global scale) and whose K is whole steps of 64, whatever the rows of x: measured
 // against the vector kernel above (bf16, 4-bit g64, both with their split of K and its reduction, us per call of the
