@@ -206,7 +206,9 @@ static bool wide_decode_takes(const nvq::ProductArgs &a) {
 static bool takes_decode(const nvq::ProductArgs &a) {
     if (a.dtype == NVQ_F32) return false;
     if (a.mode != NVQ_AFFINE) return nvq::qmv_block_decode_takes(a);
-    return a.bits == 4 ? a.m <= 4 || nvq::qmv_d16_takes(a) : a.bits >= 3 && (a.m == 1 || wide_decode_takes(a));
+    if (a.bits == 4) return a.m <= 4 || nvq::qmv_d16_takes(a);
+    if (a.bits == 2) return nvq::qmv_decode_takes_width(a) && (a.m == 1 || a.k > 2048);
+    return a.bits >= 3 && (a.m == 1 || wide_decode_takes(a));
 }
 
 static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
@@ -231,7 +233,7 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     // weight rows this kernel stays ahead: W[65536,2048] 17.7 against 24.6).
     if (a.bits != 4 && a.bits != 2 && wide_decode_takes(a)) return false;
     switch (a.bits) {
-    case 2: return true;
+    case 2: return !(nvq::qmv_decode_takes_width(a) && (a.m == 1 || a.k > 2048));
     case 5:  // beside the decode kernel's rows, against the few-row kernel of the 32x32x16 instruction (us): 6 bits W[4096,4096] g64
     case 6:  // 5 / 16 rows 12.2 / 12.4 -> 7.8 / 8.7, W[14336,4096] 8 / 16 rows 21.2 / 21.9 -> 16.6 / 17.2, W[4096,14336] g128 16 rows
              // 31.0 -> 20.0, W[8192,2048] 4 / 16 rows 8.8 / 10.6 -> 6.4 / 7.2, W[2048,1024] 3 / 16 rows 6.4 / 9.2 -> 4.4 / 5.1; 32 / 64 rows of
@@ -530,9 +532,10 @@ static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     if (takes_tiled(d, a)) return Route::kTiled;
     // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the
     // decode kernels (per-row work on the vector units, which is cheaper than the matrix-core kernel's full
-    // dequantization up to there).  A single row of the other affine widths from 3 bits: the general vector kernel
-    // (5.5 against 10.1 us at 4096 x 4096 with 3 bits, 6.6 against 11.7 us with 8 bits in groups of 32).  Other
-    // few-row products share one weight decode on the matrix cores where those kernels take them.
+    // dequantization up to there).  A single row of the other affine widths from 3 bits, and the few rows the decode
+    // kernel's 3-, 5-, 6- and 8-bit variants take (wide_decode_takes): the vector kernels too (a row of 3-bit codes at
+    // 4096 x 4096: 4.0 us against 10.1 us on the matrix cores, of 8-bit codes in groups of 32 5.8 against 11.7 us).
+    // Other few-row products share one weight decode on the matrix cores where those kernels take them.
     if (!takes_decode(a) && qmf_supported(a)) return Route::kFewRows;
     return Route::kVector;
 }

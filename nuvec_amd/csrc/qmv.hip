@@ -259,7 +259,8 @@ constexpr int kAffine8 = 64;  // as a MODE of the decode kernels: affine codes o
 constexpr int kAffine3 = 65;  // ... and of 3 bits: a lane's 32 codes are three dwords, carried in a uint4
 constexpr int kAffine6 = 66;  // ... of 6 bits: six dwords, three to a uint4
 constexpr int kAffine5 = 67;  // ... of 5 bits: five dwords, three and two
-constexpr bool is_affine_mode(int mode) { return mode == NVQ_AFFINE || mode == kAffine8 || mode == kAffine3 || mode == kAffine6 || mode == kAffine5; }
+constexpr int kAffine2 = 68;  // ... of 2 bits: two dwords
+constexpr bool is_affine_mode(int mode) { return mode == NVQ_AFFINE || mode == kAffine8 || mode == kAffine3 || mode == kAffine6 || mode == kAffine5 || mode == kAffine2; }
 constexpr int slice_quads(int mode) { return mode == NVQ_MXFP8 || mode == kAffine8 || mode == kAffine6 || mode == kAffine5 ? 2 : 1; }  // uint4 that carry a lane's 32 codes
 template <typename T, int MODE> struct SliceScale { using type = std::conditional_t<is_affine_mode(MODE), T, std::conditional_t<MODE == NVQ_NVFP4, uint16_t, uint8_t>>; };
 
@@ -314,6 +315,36 @@ __device__ __forceinline__ void slice_dot(const uint4 (&wq)[slice_quads(MODE)], 
             const uint32_t z = (piece[j] & 0xFFFu) | ((piece[j] << 4) & 0x0FFF0000u);
             const uint32_t p0 = and_or(z, mask, magic), p1 = and_or(z >> 3, mask, magic);
             const uint32_t p2 = and_or(z >> 6, mask, magic), p3 = and_or(z >> 9, mask, magic);
+#pragma unroll
+            for (int i = 0; i < RM; i++) {
+                dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
+                dot[i][1] = Pair<T>::dot2(xp[i][j].y, p1, dot[i][1]);
+                dot[i][2] = Pair<T>::dot2(xp[i][j].z, p2, dot[i][2]);
+                dot[i][3] = Pair<T>::dot2(xp[i][j].w, p3, dot[i][3]);
+            }
+        }
+        const float sc = Elem<T>::load(&sraw, 0), bi = Elem<T>::load(&braw, 0);
+        const float bb = __builtin_fmaf(-Pair<T>::base, sc, bi);
+#pragma unroll
+        for (int i = 0; i < RM; i++) {
+            const float dsum = (dot[i][0] + dot[i][1]) + (dot[i][2] + dot[i][3]);
+            acc[i] = __builtin_fmaf(sc, dsum, __builtin_fmaf(bb, xs[i], acc[i]));
+        }
+    } else if constexpr (MODE == kAffine2) {
+        // 2-bit codes: piece j is the 16 bits from bit 16 j of the lane's 64; codes 0..3 stay in the low half, codes 4..7
+        // move to the high half, and the pairs (c0, c4) (c1, c5) (c2, c6) (c3, c7) enter as B + c like the 4-bit ones
+        const uint32_t d[2] = {wq[0].x, wq[0].y};
+        float dot[RM][4];
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) dot[i][t] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t v = d[j >> 1] >> (16 * (j & 1));
+            const uint32_t z = (v & 0xFFu) | ((v << 8) & 0x00FF0000u);
+            const uint32_t p0 = and_or(z, mask, magic), p1 = and_or(z >> 2, mask, magic);
+            const uint32_t p2 = and_or(z >> 4, mask, magic), p3 = and_or(z >> 6, mask, magic);
 #pragma unroll
             for (int i = 0; i < RM; i++) {
                 dot[i][0] = Pair<T>::dot2(xp[i][j].x, p0, dot[i][0]);
@@ -457,6 +488,7 @@ __device__ __forceinline__ void slice_dot(const uint4 (&wq)[slice_quads(MODE)], 
 // scale (dot - B sum x) + bias sum x never materialises a weight), or NVQ_MXFP4 / NVQ_NVFP4 / NVQ_MXFP8: the
 // conversion instructions give the code values as element pairs (every E2M1 and E4M3 value is exact in bf16 and f16),
 // in memory order, and a lane's 32 values are one group (NVFP4: two), whose float32 scale multiplies the group's sum.
+// kAffine2 / kAffine3 / kAffine5 / kAffine6 / kAffine8: affine codes of those widths (2, 3, 5, 6 or 8 dwords a lane; see slice_dot).
 // GLU (the pairs of a gather whose weights hold the experts' gate and up projections in alternating runs of 64 rows,
 // RN = 2): a wavefront takes output column c of [pairs, N / 2], i.e. weight rows 128 (c / 64) + c % 64 (gate) and that
 // + 64 (up), and stores the gated activation of the two rounded products (each with its expert's bias first), bit for
@@ -467,7 +499,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     constexpr int kXPerThread = 512 / kThreads;  // 128-bit pieces of one x row per thread and step
     static_assert(512 % kThreads == 0, "a step of x must split evenly over the block");
     constexpr bool kAffine = is_affine_mode(MODE);
-    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : MODE == kAffine3 ? 3 : MODE == kAffine6 ? 6 : MODE == kAffine5 ? 5 : 4;
+    constexpr int BITS = MODE == NVQ_MXFP8 || MODE == kAffine8 ? 8 : MODE == kAffine3 ? 3 : MODE == kAffine6 ? 6 : MODE == kAffine5 ? 5 : MODE == kAffine2 ? 2 : 4;
     constexpr int kQuads = slice_quads(MODE);           // loads of a lane's 32 codes (16 bytes each; 3, 5 and 6 bits: 12 and 8)
     constexpr int kHalves = MODE == NVQ_NVFP4 ? 2 : 1;  // groups per lane slice
     __shared__ uint4 x_pairs[RM][2][4][64];               // [row][chunk][word][lane]: 4 pairs of eight values
@@ -491,7 +523,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
     T *y = (T *)a.y + o.y;
     constexpr uint32_t ones = std::is_same<T, bf16_t>::value ? 0x3F803F80u : 0x3C003C00u;
     uint32_t mask, magic;
-    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 3 ? 0x00070007 : BITS == 6 ? 0x003F003F : BITS == 5 ? 0x001F001F : 0x000F000F));
+    asm volatile("s_mov_b32 %0, %1" : "=s"(mask) : "i"(BITS == 3 ? 0x00070007 : BITS == 6 ? 0x003F003F : BITS == 5 ? 0x001F001F : BITS == 2 ? 0x00030003 : 0x000F000F));
     asm volatile("v_mov_b32 %0, %1" : "=v"(magic) : "s"(Pair<T>::magic));
     float factor = 1.0f;
     if constexpr (MODE == NVQ_NVFP4) factor = qmf::nvfp4_factor(a, BATCHED && a.rhs != nullptr ? (int64_t)a.rhs[blockIdx.z] : 0);
@@ -526,7 +558,10 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
                 const int n = n0 + r * kRowStep < N ? n0 + r * kRowStep : N - 1;  // tail rows are computed, not stored
                 // the codes are read once: a non-temporal load keeps them from displacing x and the scales in the caches
                 // (8.1 -> 7.8 us at W[14336,4096]; the scales, shared by neighbouring lanes and rows, lose by it)
-                if constexpr (BITS == 3) {  // three dwords, dword-aligned
+                if constexpr (BITS == 2) {  // two dwords (rows are whole multiples of 8 bytes: K % 32 == 0)
+                    const uint2 v = stream_load(reinterpret_cast<const uint2 *>(w + (int64_t)n * kwords + (kc >> 5) * 2));
+                    wq[u][r][0] = make_uint4(v.x, v.y, 0u, 0u);
+                } else if constexpr (BITS == 3) {  // three dwords, dword-aligned
                     typedef uint32_t u32x3_a4_t __attribute__((ext_vector_type(3), aligned(4)));
                     const u32x3_a4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x3_a4_t *>(w + (int64_t)n * kwords + (kc >> 5) * 3));
                     wq[u][r][0] = make_uint4(v.x, v.y, v.z, 0u);
@@ -1361,6 +1396,14 @@ inline bool decode8_takes(const ProductArgs &a) {
 // 5 bits W[4096,4096] 6.2 / 11.9 / 12.0 / 12.0 -> 4.7 / 5.3 / 6.5 / 7.5, W[14336,4096] 13.3 / 19.4 / 19.5 / 19.5 -> 10.2 / 12.5 / 14.2 /
 // 16.8.  Rows of K = 2048 and less leave lanes idle: W[8192,2048] 6 bits 2 / 4 rows 8.7 / 8.7 -> 7.3 / 10.3, W[16384,1024]
 // 9.2 / 9.2 -> 10.8 / 16.8, so the callers send those only with one row, or two at K = 2048.)
+// ... and one or two rows against 2-bit ones (us, against the kernel that loads the weights straight into operand layout:
+// W[4096,4096] g64 1 / 2 rows 5.3 / 5.3 -> 3.9 / 4.5, W[14336,4096] 10.1 / 10.1 -> 7.8 / 10.0, W[4096,14336] g128 one row
+// 12.3 -> 9.1, W[2880,2880] g32 one row 7.7 -> 3.8; three rows and more are the other kernel's: 10.1 against 12.2).
+inline bool decode2_takes(const ProductArgs &a) {
+    return a.mode == NVQ_AFFINE && a.bits == 2 && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= 2 && !a.exact_weights && !a.row_exact && a.k % 32 == 0 &&
+           ((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 8 == 0);
+}
+
 inline bool decode56_takes(const ProductArgs &a) {
     return a.mode == NVQ_AFFINE && (a.bits == 6 || a.bits == 5) && a.dtype != NVQ_F32 && a.m >= 1 && a.m <= 4 && !a.exact_weights && !a.row_exact &&
            a.k % 32 == 0 && (uintptr_t)a.x % 16 == 0;
@@ -1422,6 +1465,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
         if (decode8_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine8>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine8>(a, s) : run_lds4<T, 4, 1, 8, kAffine8>(a, s);
         // (3 bits, against the general kernel: W[4096,4096] g64 5.47 -> 4.01, W[14336,4096] 12.2 -> 8.2, W[2880,2880] g32 5.39 -> 3.78)
         if (decode3_takes(a)) return a.m == 1 ? run_lds4<T, 1, 1, 8, kAffine3>(a, s) : a.m == 2 ? run_lds4<T, 2, 1, 8, kAffine3>(a, s) : run_lds4<T, 4, 1, 8, kAffine3>(a, s);
+        if (decode2_takes(a)) return run_block_decode<T, kAffine2>(a, s);
         if (decode56_takes(a)) {
             if (a.bits == 6) return run_block_decode<T, kAffine6>(a, s);
             return run_block_decode<T, kAffine5>(a, s);
@@ -1458,7 +1502,7 @@ int32_t run_typed(const ProductArgs &a, hipStream_t s) {
 
 bool qmv_d16_takes(const ProductArgs &a) { return !a.row_exact && d16_takes(a); }
 bool qmv_block_decode_takes(const ProductArgs &a) { return block_decode_takes(a); }
-bool qmv_decode_takes_width(const ProductArgs &a) { return decode8_takes(a) || decode3_takes(a) || decode56_takes(a); }
+bool qmv_decode_takes_width(const ProductArgs &a) { return decode8_takes(a) || decode3_takes(a) || decode56_takes(a) || decode2_takes(a); }
 
 // Mirrors run_typed.
 const char *qmv_kernel_name(const ProductArgs &a) {
@@ -1469,7 +1513,7 @@ const char *qmv_kernel_name(const ProductArgs &a) {
         return "qmv4_lds_kernel";
     }
     if (short_decode_takes(a)) return "qmv4_short_kernel";
-    if (block_decode_takes(a) || decode8_takes(a) || decode3_takes(a) || decode56_takes(a)) return "qmv4_lds_kernel";
+    if (block_decode_takes(a) || decode8_takes(a) || decode3_takes(a) || decode56_takes(a) || decode2_takes(a)) return "qmv4_lds_kernel";
     return "qmv_lds_kernel";
 }
 

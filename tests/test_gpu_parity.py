@@ -697,15 +697,16 @@ def test_block_formats_on_the_decode_kernel(mode, qmode, dtype):
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("bits,group", [(3, 32), (3, 64), (3, 128), (5, 32), (5, 64), (5, 128), (6, 32), (6, 64), (6, 128), (8, 32), (8, 64), (8, 128)])
-def test_decode_kernel_three_and_eight_bits(dtype, bits, group):
-    """The decode kernel's 3-, 5-, 6- and 8-bit variants (a lane's 32 codes: three dwords split 24 bits at a time into two
-    halves of four codes; five or six dwords split 20 or 24 bits at a time into two halves of two codes; eight dwords
-    converted in memory order): one row at any K, up to two (3 bits), three or four (8 bits), four (5 and 6 bits) where K
+@pytest.mark.parametrize("bits,group", [(2, 32), (2, 64), (2, 128), (3, 32), (3, 64), (3, 128), (5, 32), (5, 64), (5, 128), (6, 32), (6, 64), (6, 128), (8, 32), (8, 64), (8, 128)])
+def test_decode_kernel_other_affine_widths(dtype, bits, group):
+    """The decode kernel's 2-, 3-, 5-, 6- and 8-bit variants (a lane's 32 codes: two dwords split 16 bits, three dwords
+    split 24 bits at a time into two halves of four codes; five or six dwords split 20 or 24 bits at a time into two halves
+    of two codes; eight dwords converted in memory order): one row at any K, up to two (2 and 3 bits), three or four (8
+    bits), four (5 and 6 bits) where K
     is beyond 2048; K off the kernel's steps, weight rows off the block's eight; a batch and the pairs of a gather.
     Against the CPU oracle within the bar and the device arithmetic within half of it."""
     rng = np.random.default_rng(5200 + 10 * bits + group + dtype)
-    most = 2 if bits == 3 else 4 if group == 32 or bits in (5, 6) else 3
+    most = 2 if bits in (2, 3) else 4 if group == 32 or bits in (5, 6) else 3
     quant = nv.Quant.affine(group, bits)
     for m, n, k in [(1, 1030, 4096), (1, 1100, 2944), (1, 2053, 128), (1, 1025, 1024), (2, 1061, 4096 + 128), (most, 1030, 2944), (most, 1024, 8192)]:
         route = nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
