@@ -135,7 +135,7 @@ typedef struct nvq_gather_desc {
  *   out dtype [batch, query_heads, 1, head_dim], all contiguous. */
 typedef struct nvq_attention_desc {
     int32_t dtype;      /* NVQ_F16 / NVQ_BF16 / NVQ_F32: q, scales, biases, sinks, out */
-    int32_t bits;       /* 4 or 8 (3 bits: NVQ_UNSUPPORTED, the caller's composition) */
+    int32_t bits;       /* 3, 4 or 8 (3 bits: a row's chunks of 32 codes are 12 bytes, rows 4-byte aligned) */
     int32_t group_size; /* 32, 64 or 128, dividing head_dim */
     int32_t head_dim;   /* 64 or 128 */
     int64_t batch, query_heads, key_heads, positions;
@@ -249,8 +249,9 @@ NVQ_API int32_t nvq_quantized_matmul_static(const nvq_qmm_desc *desc, const void
 
 /* GpuEval::quantized_attention (gpu.rs:4969-5040): softmax(scale * q . K^T [, sinks]) . V in one kernel, the codes
  * dequantized in registers (never rounded), float32 products and sums; within the float bound of the dequantized
- * attention, as the reference's kernel.  What the fit rule excludes (several query rows, a mask, other head sizes,
- * 3 bits, query heads that are not 1, 2, 4 or 8 per key head) answers NVQ_UNSUPPORTED: the caller then records the
+ * attention, as the reference's kernel.  Caches of 3, 4 and 8 bits are taken.  What the fit rule excludes (several query
+ * rows, a mask, other head sizes or widths, query heads that are not 1, 2, 4 or 8 per key head, more than 65535 batches or
+ * 2^31 cache values) answers NVQ_UNSUPPORTED: the caller then records the
  * composition of two quantized products and a softmax, as the reference does (fast/imp.rs:3996-4035).
  * With the workspace the size query names (float32 states of the splits: maximum, denominator and weighted sum per
  * split and head) the positions are split over the grid and a second kernel merges the splits; with NULL one block

@@ -820,6 +820,10 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     NVQ_TRY(check_product_dims("gather_qmm", d->quant, d->transpose, d->m, d->n, d->k));
     if (d->pairs < 0 || d->x_batches < 0 || d->experts < 0) return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: negative size");
     if (d->pairs == 0 || d->m == 0 || d->n == 0) return NVQ_OK;
+    // Indices are clamped into [0, x_batches) and [0, experts) on the device: an empty operand leaves nothing to clamp to.
+    if (d->x_batches < 1 || d->experts < 1)
+        return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: %lld pairs index %lld batches of x and %lld experts", (long long)d->pairs,
+                    (long long)d->x_batches, (long long)d->experts);
     if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr || lhs == nullptr || rhs == nullptr)
         return fail(NVQ_INVALID_ARGUMENT, "gather_qmm: null operand");
     NVQ_TRY(require_device());

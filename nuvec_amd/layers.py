@@ -309,7 +309,7 @@ def quantized_attention(q: torch.Tensor, k: ops.Quantized, v: ops.Quantized, sca
     queries `q [B, Hq, L, D]` over affine-quantized keys and values (codes `[B, Hkv, S, D * bits / 32]`, scales and
     biases `[B, Hkv, S, D / group]`), grouped query heads, optional per-head `sinks [Hq]`, optionally causal (query i
     of L sees keys up to S - L + i, nuvec-lm's `quantized_attention`, model.rs:3646-3700):
-    `softmax(scale * q k^T [, sinks]) v`.  One query row per head that fits the kernel (head size 64 or 128, 4 or 8 bits)
+    `softmax(scale * q k^T [, sinks]) v`.  One query row per head that fits the kernel (head size 64 or 128, 3, 4 or 8 bits)
     takes the library's fused kernel; the rest is the reference's composition (the one it runs wherever its fused
     kernel does not fit): both products are the library's quantized products, transposed for the keys and
     untransposed for the values; the softmax (float32 inside, one rounding) is an elementwise step outside the path."""
@@ -317,7 +317,8 @@ def quantized_attention(q: torch.Tensor, k: ops.Quantized, v: ops.Quantized, sca
         raise ops.InvalidArgument("quantized_attention: keys and values need one affine quantization")
     if k.biases is None or v.biases is None:
         raise ops.InvalidArgument("quantized_attention: affine biases missing")
-    if fused and not causal and q.is_cuda and ops.quantized_attention_fits(q, k, v, sinks):
+    # (a single causal query row sees every key: the mask is empty)
+    if fused and (not causal or q.shape[-2] == 1) and q.is_cuda and ops.quantized_attention_fits(q, k, v, sinks):
         return ops.quantized_attention(q, k, v, scale, sinks)  # one kernel (the reference's FastOp::QuantizedAttention)
     b, hq, l, d = q.shape
     hkv = k.weight.shape[1]

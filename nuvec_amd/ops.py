@@ -479,6 +479,8 @@ def quantized_attention_fits(q: torch.Tensor, k: Quantized, v: Quantized, sinks:
             return False
     if hkv == 0 or n < 1 or hq % hkv or hq // hkv not in (1, 2, 4, 8):
         return False
+    if b > 65535 or b * hkv * n * d >= 1 << 31:  # the kernel's grid and 32-bit cache offsets
+        return False
     return sinks is None or (sinks.ndim == 1 and sinks.numel() == hq and sinks.dtype == q.dtype)
 
 
@@ -716,10 +718,11 @@ def gather_qmm_glu(x: torch.Tensor, q: Quantized, rows: torch.Tensor, sorted_ids
     n = w.shape[-2]
     if expert_bias is not None and (tuple(expert_bias.shape) != (w.shape[0], n) or expert_bias.dtype != dtype):
         raise InvalidArgument(f"{op}: the experts' bias must be [{w.shape[0]}, {n}] of {dtype}")
-    _init(x)
     lhs, rhs = _indices(op, x, rows.reshape(-1)).contiguous(), _indices(op, w, sorted_ids.reshape(-1)).contiguous()
     if lhs.numel() != rhs.numel() or (offsets is not None and (offsets.numel() != w.shape[0] or offsets.dtype != torch.int32)):
-        raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, {offsets.numel()} offsets for {w.shape[0]} experts")
+        raise InvalidArgument(f"{op}: {lhs.numel()} rows, {rhs.numel()} expert ids, "
+                              f"{'no' if offsets is None else offsets.numel()} offsets for {w.shape[0]} experts")
+    _init(x)
     out = torch.empty((rhs.numel(), n // 2), dtype=dtype, device=x.device)
     d = _lib.GatherDescC(quant._c(), _CODE[dtype], 1, 0, 0, 1, n, columns, rhs.numel(), x.shape[0], w.shape[0])
     eb = None if expert_bias is None else expert_bias.contiguous()

@@ -88,6 +88,27 @@ def _quant(mode, group, bits):
     return _lib.QuantC(mode, group, bits)
 
 
+def test_gather_with_an_empty_operand_is_refused():
+    """The device clamps indices into [0, x_batches) and [0, experts): pairs against an empty x or no experts have
+    nothing to clamp to and are refused on the host, before the device is asked for."""
+    lib = _lib.load()
+    one = C.c_void_p(16)
+    for x_batches, experts in ((0, 2), (2, 0), (0, 0)):
+        g = _lib.GatherDescC(_quant(0, 64, 4), _lib.BF16, 1, 0, 0, 1, 8, 64, 3, x_batches, experts)
+        assert lib.nvq_gather_qmm(C.byref(g), one, one, one, one, one, one, None, one, None, None) == _lib.INVALID_ARGUMENT
+        assert "experts" in _lib.last_error()
+        assert lib.nvq_gather_qmm_glu(C.byref(g), 0, 1.0, 7.0, one, one, one, one, one, one, None, one, None, None) == _lib.INVALID_ARGUMENT
+    empty = _lib.GatherDescC(_quant(0, 64, 4), _lib.BF16, 1, 0, 0, 1, 8, 64, 0, 0, 0)  # no pairs: nothing to do
+    assert lib.nvq_gather_qmm(C.byref(empty), one, one, one, one, one, one, None, one, None, None) == _lib.OK
+
+
+def test_gated_gather_counts_rows_and_ids_without_offsets():
+    """The unsorted route (no offsets) answers a row / id count mismatch with InvalidArgument, like the sorted one."""
+    q = nv.Quantized(torch.zeros(2, 128, 8, dtype=torch.uint32), torch.ones(2, 128, 1), torch.zeros(2, 128, 1), nv.Quant.affine(64, 4))
+    with pytest.raises(nv.InvalidArgument, match="no offsets"):
+        nv.gather_qmm_glu(torch.ones(3, 64), q, torch.tensor([0, 1, 2], dtype=torch.int32), torch.tensor([0, 1], dtype=torch.int32), None)
+
+
 def test_quantization_parameters_are_validated_by_the_library():
     """primitive_fuzz.rs:97-131 at the C boundary: each bad `Quant` is refused by every entry point that takes one,
     with NVQ_INVALID_ARGUMENT and before the device is asked for (none is bound in this process)."""
