@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(HERE, "..", "include")
 LIB = os.path.join(HERE, "libnuvec_hip.so")
-SOURCES = ["qmf_b8.hip", "qmf_fp8.hip", "qmf_b6.hip", "qmf_b5.hip", "qmf_b4.hip", "qmf_fp4.hip", "qmf_nvfp4.hip", "qmf_b3.hip", "qmf_b2.hip", "qmf_b1.hip", "qmm.hip", "qmv.hip",
+SOURCES = ["qmf_b8.hip", "qmf_fp8.hip", "qmf_b6.hip", "qmf_b5.hip", "qmf_b4.hip", "qmf_fp4.hip", "qmf_nvfp4.hip", "qmf_b3.hip", "qmf_b2.hip", "qmf_b1.hip", "qmm.hip", "qmv.hip", "qmv_dot8.hip",
            "qvm.hip", "nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmf.hip", "gather.hip", "repack.hip", "calib.hip", "qattn.hip", "qmd.hip", "glu.hip"]  # slowest to compile first
 
 # -ffp-contract=off: the quantizers must round every operation as the CPU does; fused
@@ -37,13 +37,19 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose: bool = False, jobs: int = 8) -> str:
+def build(verbose: bool = False, jobs: int = 8, changed_only: bool = False) -> str:
+    """Compiles every source and links the library.  `changed_only` (a development aid, `--changed` on the command line):
+    sources older than their object files are not compiled again, unless a header is newer than the object."""
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
+    headers = [os.path.join(d, f) for d in (CSRC, INCLUDE) for f in os.listdir(d) if f.endswith(".h")]
+    newest_header = max(os.path.getmtime(h) for h in headers)
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        if changed_only and os.path.exists(obj) and os.path.getmtime(obj) > max(newest_header, os.path.getmtime(os.path.join(CSRC, src))):
+            return obj
         cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -67,4 +73,4 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, changed_only="--changed" in sys.argv))

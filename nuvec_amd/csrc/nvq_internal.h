@@ -106,6 +106,10 @@ int32_t launch_qmv(const ProductArgs &a, hipStream_t s);
 const char *qmv_kernel_name(const ProductArgs &a);  // which of the vector / decode kernels launch_qmv runs for `a`
 // Whether the 16x16x32 matrix-core decode kernel takes the product (4-bit affine, groups of 64, K = 4096).
 bool qmv_d16_takes(const ProductArgs &a);
+// The integer dot-product decode kernel: one row of x (or the rows of a row-exact product) against 4-bit affine weights.
+bool qmv_dot8_takes(const ProductArgs &a);
+int32_t launch_qmv_dot8(const ProductArgs &a, hipStream_t s);
+int qmv_dot8_rows_per_wave(int64_t n, int cus);  // rows a wavefront takes, by the weight's rows and the chip's compute units
 bool qmv_glu_pairs_take(const ProductArgs &a);      // whether the decode kernel takes unsorted pairs with the gated epilogue
 int32_t launch_qmv_glu_pairs(const ProductArgs &a, hipStream_t s);
 bool qmv_block_decode_takes(const ProductArgs &a);  // whether the decode kernel takes a product of a block format
