@@ -33,8 +33,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_206_466
-QMM_TRAFFIC_BYTES = 297_180_045
+QMV_TRAFFIC_BYTES = 33_235_167
+QMM_TRAFFIC_BYTES = 297_179_760
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -390,7 +390,8 @@ def main():
                        "weight_copies_rotated": args.copies,
                        "submission": "one C-ABI call per launch, back to back on one stream"},
             "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": gbps / HBM_PEAK_GBPS, "traffic": QMV_TRAFFIC_BYTES, "kernel": "qmv4_lds_kernel",
+                         "frac": gbps / HBM_PEAK_GBPS, "traffic": QMV_TRAFFIC_BYTES,
+                         "kernel": lib.nvq_quantized_matmul_route(C.byref(calls[0].d)).decode(),
                          "bytes_per_launch": WEIGHT_BYTES, "us_per_launch": ms * 1e3},
         })
         if only is None:

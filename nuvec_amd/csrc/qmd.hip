@@ -304,13 +304,13 @@ __global__ void __launch_bounds__(64 * kQmdSlices) qmd_kernel(const ProductArgs 
                     for (int j = 0; j < J; j++) {
                         uint4 b;
                         if constexpr (MODE == NVQ_MXFP8) {
-                            const uint32_t w0 = t.w[rt][sp][2 * j], w1 = t.w[rt][sp][2 * j + 1];
+                            const uint32_t w0 = qmf::Ops<T>::mx_codes(t.w[rt][sp][2 * j], sc0), w1 = qmf::Ops<T>::mx_codes(t.w[rt][sp][2 * j + 1], sc0);
                             b.x = qmf::Ops<T>::template fp8_pair<false>(w0, sc0);
                             b.y = qmf::Ops<T>::template fp8_pair<true>(w0, sc0);
                             b.z = qmf::Ops<T>::template fp8_pair<false>(w1, sc0);
                             b.w = qmf::Ops<T>::template fp8_pair<true>(w1, sc0);
                         } else if constexpr (MODE == NVQ_MXFP4) {
-                            const uint32_t w0 = t.w[rt][sp][j];
+                            const uint32_t w0 = qmf::Ops<T>::mx_codes(t.w[rt][sp][j], sc0);
                             b.x = qmf::Ops<T>::template fp4_pair<0>(w0, sc0);
                             b.y = qmf::Ops<T>::template fp4_pair<1>(w0, sc0);
                             b.z = qmf::Ops<T>::template fp4_pair<2>(w0, sc0);

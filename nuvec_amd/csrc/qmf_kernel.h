@@ -111,6 +111,10 @@ template <> struct Ops<bf16_t> {
     template <bool HIGH> __device__ static __forceinline__ uint32_t fp8_pair(uint32_t word, float scale) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(word, scale, HIGH));
     }
+    // The codes of a group for the scaled conversions above, which take the exponent field of `scale` alone: an E8M0
+    // scale of 2^-127 is zero once flushed (crates/nuvec-core/src/fp8.rs:95-112) but reads as 2^-127 there, and bf16
+    // holds 448 x 2^-127, so such a group's codes become code 0 (+0 in E2M1 and in E4M3).
+    __device__ static __forceinline__ uint32_t mx_codes(uint32_t word, float scale) { return scale != 0.0f ? word : 0u; }
 };
 template <> struct Ops<f16_t> {
     __device__ static __forceinline__ floatx16_t mfma(uint4 a, uint4 b, floatx16_t c) {
@@ -126,6 +130,8 @@ template <> struct Ops<f16_t> {
     template <bool HIGH> __device__ static __forceinline__ uint32_t fp8_pair(uint32_t word, float scale) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, scale, HIGH));
     }
+    // (448 x 2^-127 is far below half of f16's smallest subnormal: the conversion itself gives the zero of a flushed scale)
+    __device__ static __forceinline__ uint32_t mx_codes(uint32_t word, float) { return word; }
 };
 
 // Low / high 16 bits of a word as element-type values.
@@ -187,7 +193,7 @@ template <typename T, int BITS, int FP4, int KK, bool EXACT = false>
 __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float s, float b) {
     uint4 r;
     if constexpr (FP4 == kMxfp8) {
-        const uint32_t w0 = dw[2 * KK], w1 = dw[2 * KK + 1];
+        const uint32_t w0 = Ops<T>::mx_codes(dw[2 * KK], s), w1 = Ops<T>::mx_codes(dw[2 * KK + 1], s);
         r.x = Ops<T>::template fp8_pair<false>(w0, s);
         r.y = Ops<T>::template fp8_pair<true>(w0, s);
         r.z = Ops<T>::template fp8_pair<false>(w1, s);
@@ -199,7 +205,7 @@ __device__ __forceinline__ uint4 expand_piece(const uint32_t (&dw)[BITS], float 
         r.z = fp4_pair_times<T, 2>(word, s);
         r.w = fp4_pair_times<T, 3>(word, s);
     } else if constexpr (FP4) {
-        const uint32_t word = dw[KK];
+        const uint32_t word = Ops<T>::mx_codes(dw[KK], s);
         r.x = Ops<T>::template fp4_pair<0>(word, s);
         r.y = Ops<T>::template fp4_pair<1>(word, s);
         r.z = Ops<T>::template fp4_pair<2>(word, s);

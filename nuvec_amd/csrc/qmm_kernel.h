@@ -122,11 +122,11 @@ __device__ __forceinline__ void keep(const uint4 &v) { asm volatile("" : : "v"(v
 template <typename T, int BITS, int FP4, int KK, int D, bool EXACT = false>
 __device__ __forceinline__ uint32_t expand_dword(const uint32_t (&dw)[BITS], float s, float b) {
     if constexpr (FP4 == kMxfp8) {
-        return Ops<T>::template fp8_pair<(D & 1) != 0>(dw[2 * KK + D / 2], s);
+        return Ops<T>::template fp8_pair<(D & 1) != 0>(Ops<T>::mx_codes(dw[2 * KK + D / 2], s), s);
     } else if constexpr (FP4 == kNvfp4) {
         return fp4_pair_times<T, D>(dw[KK], s);
     } else if constexpr (FP4) {
-        return Ops<T>::template fp4_pair<D>(dw[KK], s);
+        return Ops<T>::template fp4_pair<D>(Ops<T>::mx_codes(dw[KK], s), s);
     } else if constexpr (BITS == 4) {
         const uint32_t word = dw[KK];
         const uint32_t even = opaque(word & 0x0F0F0F0Fu), odd = opaque((word >> 4) & 0x0F0F0F0Fu);

@@ -769,48 +769,71 @@ def test_short_rows_of_gathered_pairs(quant, dtype):
         assert torch.equal(with_bias, got + bias[torch.from_numpy(rhs).cuda()].unsqueeze(-2))
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 @pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
-def test_block_formats_at_every_scale_code(mode, qmode):
-    """Every scale code on every product route: weight row n carries scale code n in all its groups (E8M0: 2^(n - 127), zero
-    flushed at code 0; E4M3: both signs, subnormals, 448, NaN at 0x7F and 0xFF), so a conversion that mistook one code
-    fails its column of the output.  Outputs are compared after division by their column's scale, each against the bar of
-    its row.  x is small enough for the large scales to stay finite; the E8M0 codes whose weights overflow float32 (from
-    246; 255 is infinity in the reference, fp8.rs:95-102, and only an infinite weight quantizes to it) or whose products
-    would be float32 subnormals (below 30) are left out; code 0, which flushes to zero, stays."""
-    rng = np.random.default_rng(4800 + mode)
-    dtype = ref.BF16
+def test_block_formats_at_every_scale_code(mode, qmode, dtype):
+    """Every scale code on every product route, weights stored [N, K] and [K, N]: output column n carries scale code n in all
+    its groups (E8M0: 2^(n - 127), zero flushed at code 0; E4M3: both signs, subnormals, 448, NaN at 0x7F and 0xFF), so a
+    conversion that mistook one code fails its column of the output.  Outputs are compared after division by their
+    column's scale, each against the bar of its row.  x is small enough for the large scales to stay finite; the E8M0
+    codes whose weights overflow float32 (from 246; 255 is infinity in the reference, fp8.rs:95-102, and only an infinite
+    weight quantizes to it) or whose products would be float32 subnormals (below 30) are left out; code 0, which
+    flushes to zero (fp8.rs:95-112), stays, and its columns are zero on every route.  float16 keeps the E8M0 codes whose
+    outputs are normal float16 values, and code 0."""
+    rng = np.random.default_rng(4800 + mode + 10 * dtype)
     group, bits = ref.FP_PARAMS[mode]
     quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
     n, k = 256, 512
     codes = np.arange(256, dtype=np.uint8)
     if mode != ref.NVFP4:
-        codes = np.where(((codes > 0) & (codes < 30)) | (codes > 245), 127, codes).astype(np.uint8)
-    w = make_w(rng, n, k, dtype)
-    packed, _ = ref.fp_quantize(w, dtype, mode)
-    scales = np.repeat(codes[:, None], k // group, axis=1)
-    one = np.full(packed.shape, 0x38383838 if mode == ref.MXFP8 else 0x22222222, np.uint32)  # every code 1.0
-    value = ref.fp_dequantize(one, scales, mode, ref.F32)[:, 0].astype(np.float64)  # the scales as the oracle decodes them
+        keep = (codes == 0) | ((codes >= 120) & (codes <= 134) if dtype == ref.F16 else (codes >= 30) & (codes <= 245))
+        codes = np.where(keep, codes, 127).astype(np.uint8)
+    x_scale = 2.0 ** -6 if dtype == ref.F16 else 2.0 ** -14
+    one = np.full((n, k * bits // 32), 0x38383838 if mode == ref.MXFP8 else 0x22222222, np.uint32)  # every code 1.0
+    value = ref.fp_dequantize(one, np.repeat(codes[:, None], k // group, axis=1), mode, ref.F32)[:, 0].astype(np.float64)  # the scales as the oracle decodes them
     nan, zero = np.isnan(value), value == 0.0
-    assert (nan[[0x7F, 0xFF]].all() if mode == ref.NVFP4 else zero[0] and not nan.any()) and np.count_nonzero(~nan & ~zero) >= 200
-    q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+    assert (nan[[0x7F, 0xFF]].all() if mode == ref.NVFP4 else zero[0] and not nan.any())
+    assert np.count_nonzero(~nan & ~zero) >= (15 if dtype == ref.F16 and mode != ref.NVFP4 else 200)
+    live = ~nan & ~zero
     routes = set()
-    for m in (1, 3, 8, 40, 300):
-        x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32) * 2.0 ** -14, dtype)
-        want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8), dtype)
-        got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q)), dtype)
-        routes.add(nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]))
-        assert np.isnan(want[:, nan]).all() and np.isnan(got[:, nan]).all(), f"{qmode} M={m}: NaN scales"
-        # The reference flushes 2^-127 to zero (fp8.rs:95-112).  The vector kernels do; the scaled conversions of the matrix-core
-        # kernels take the code as 2^-127, so an output may hold up to max|code| * 2^-127 * sum|x| there instead of zero.
-        route = nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype])
-        slack = 0.0 if route in ("qmv4_lds_kernel", "qmv_lds_kernel") else 1.01 * 448.0 * 2.0 ** -127 * float(np.abs(ref.to_f32(x, dtype)).sum(axis=1).max())
-        assert not want[:, zero].any() and float(np.abs(got[:, zero]).max()) <= slack, f"{qmode} M={m}: scales that flush to zero"
-        live = ~nan & ~zero
+
+    def compare(got, want, what):
+        assert np.isnan(want[:, nan]).all() and np.isnan(got[:, nan]).all(), f"{what}: NaN scales"
+        assert not want[:, zero].any() and not got[:, zero].any(), f"{what}: scales that flush to zero"
         g, r = got[:, live].astype(np.float64) / value[live], want[:, live].astype(np.float64) / value[live]
         ratio = np.abs(g - r) / (TOL[dtype] * np.max(np.abs(r), axis=1, keepdims=True))
         worst = np.unravel_index(np.argmax(ratio), ratio.shape)
-        assert ratio[worst] <= 1.0, f"{qmode} M={m} scale code {codes[live][worst[1]]}: {ratio[worst]:.3f} x the bound"
+        assert ratio[worst] <= 1.0, f"{what} scale code {codes[live][worst[1]]}: {ratio[worst]:.3f} x the bound"
+
+    # weights stored [N, K]: row n of the weight carries code n
+    w = make_w(rng, n, k, dtype)
+    packed, _ = ref.fp_quantize(w, dtype, mode)
+    scales = np.repeat(codes[:, None], k // group, axis=1)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+    for m in (1, 3, 8, 40, 300):
+        x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32) * x_scale, dtype)
+        want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8), dtype)
+        got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q)), dtype)
+        routes.add(nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]))
+        compare(got, want, f"{qmode} M={m}")
     assert {"qmv4_lds_kernel", "qmd_kernel"} <= routes and len(routes) >= 3, routes
+
+    # weights stored [K, N]: the groups run along N, so every column of group n carries code n; the matrix-core kernel
+    # and the kernel of few rows
+    k2, n2 = 256, 256 * group
+    w = make_w(rng, k2, n2, dtype)
+    packed, _ = ref.fp_quantize(w, dtype, mode)
+    scales = np.repeat(codes[None, :], k2, axis=0)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+    nan, zero, live, value, codes = (np.repeat(v, group) for v in (nan, zero, live, value, codes))
+    routes = set()
+    for m in (1, 40, 300):
+        x = ref.from_f32(rng.standard_normal((m, k2)).astype(np.float32) * x_scale, dtype)
+        want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, transpose=False, threads=8), dtype)
+        got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q, transpose=False)), dtype)
+        routes.add(nv.quantized_matmul_route(m, n2, k2, quant, TORCH[dtype], transpose=False))
+        compare(got, want, f"{qmode} stored [K, N] M={m}")
+    assert "qmn_kernel" in routes, routes
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
