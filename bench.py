@@ -219,6 +219,17 @@ def measured_peaks(lib, device, qs):
     ms = best_of([lambda stream: torch.matmul(a, b.t(), out=c)], 20)
     out["vendor_dense_gemm"] = {"us_per_launch": ms * 1e3, "tflops": 2.0 * 2048 * N * K / (ms * 1e-3) / 1e12,
                                 "note": "torch.matmul bf16 [2048,4096] x [4096,14336] (hipBLASLt, nothing to dequantize): baseline only"}
+    # The same two launches on operands that are all zero: the same instruction streams with no bit toggling in the
+    # operand paths.  What they gain over random data is what the chip's power management takes from a kernel at this
+    # occupancy of the matrix cores, whatever its schedule.
+    a.zero_(), b.zero_()
+    ms = best_of([lambda stream: torch.matmul(a, b.t(), out=c)], 20)
+    out["vendor_dense_gemm_zero_operands"] = {"us_per_launch": ms * 1e3, "tflops": 2.0 * 2048 * N * K / (ms * 1e-3) / 1e12}
+    import nuvec_amd as nv
+    zq = nv.Quantized(torch.zeros_like(qs[0].weight), torch.zeros_like(qs[0].scales), torch.zeros_like(qs[0].biases), qs[0].quant)
+    ms = best_of([Product(lib, 2048, a, zq, c)], 20)
+    out["prefill_zero_operands"] = {"us_per_launch": ms * 1e3, "tflops": 2.0 * 2048 * N * K / (ms * 1e-3) / 1e12,
+                                    "note": "configs[2]'s own kernel on all-zero x, codes, scales and biases"}
     return out
 
 

@@ -249,11 +249,18 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 }
 
 // The kernels' view of a product descriptor.
-// Rows of few outputs: the bar of a product (a fraction of the row's largest output) is then so tight that the one
-// rounding the device kernels give a dequantized affine weight, against the CPU's two (kernels.rs:835-859), shows in
-// the worst output; such products materialise the CPU's weights instead, bit for bit.
-static bool wants_exact_weights(int32_t mode, int32_t dtype, int64_t n) {
-    return mode == NVQ_AFFINE && dtype != NVQ_F32 && n < 1024;
+// Which half-precision affine products materialise the CPU's weights, round(round(code * scale) + bias)
+// (kernels.rs:835-859), bit for bit, instead of the one rounding of fma(code, scale, bias) the device kernels give a
+// weight.  The CPU's first rounding is a noise of about 0.7 % of a bfloat16 weight; over a product it is the same
+// fraction of an output's deviation, and the worst of M x N outputs against the bar of a product (1e-2 of a row's
+// largest output) grows with the rows of x and falls with the outputs of a row: measured over 100 seeds each, one-
+// rounding products of 130 rows and 1024..2048 outputs exceed the bar for one seed in five, of 12 rows for none, of
+// 2048 rows and 14336 outputs stay at 0.8 of it.  So: every row of fewer than 1024 outputs, and bfloat16 products of
+// more than 16 rows up to 8192 outputs (float16 stays under 0.65 of its bar from 1024 outputs on).  With the CPU's
+// weights only the order of the float32 sums differs: at most one rounding step of an output, 0.78 of the bar.
+static bool wants_exact_weights(int32_t mode, int32_t dtype, int64_t n, int64_t m) {
+    if (mode != NVQ_AFFINE || dtype == NVQ_F32) return false;
+    return n < 1024 || (dtype == NVQ_BF16 && m > 16 && n < 8192);
 }
 
 static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
@@ -266,7 +273,7 @@ static nvq::ProductArgs product_args(const nvq_qmm_desc *d, int64_t batch) {
     // gpu.rs:6956-6981, primitive.rs:489-493).
     const int64_t item = d->item_rows > 0 ? d->item_rows : d->m;
     a.row_exact = d->rows != 0 || (d->row_exact != 0 && item <= 8);
-    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
+    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n, a.row_exact ? 1 : d->m);  // (row-exact: one-row products)
     // Batch dimensions that one stride per operand describes together are merged (dimension i with i + 1 where every
     // operand's stride of i is its stride of i + 1 times the extent of i + 1; extents of 1 vanish): a [B, H] batch of
     // dense operands is one dimension, which the matrix-core kernels take.
@@ -614,7 +621,7 @@ int32_t nvq_quantized_matmul_glu(const nvq_qmm_desc *d, int32_t activation, floa
     if (x == nullptr || w == nullptr || scales == nullptr || y == nullptr) return fail(NVQ_INVALID_ARGUMENT, "%s: null operand", op);
     if (!d->transpose || d->batch_ndim != 0 || d->k == 0 || d->n % 128 != 0 || d->row_exact || d->rows)
         return fail(NVQ_UNSUPPORTED, "%s: the gated epilogue takes x [M, K] times transposed weights whose gate and up rows alternate in runs of 64", op);
-    if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2))
+    if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2, d->m))
         return fail(NVQ_UNSUPPORTED, "%s: the gated epilogue takes affine projections of 1024 rows or more each", op);
     NVQ_TRY(require_device());
     NVQ_TRY(check_aligned(op, "x", x));
@@ -867,7 +874,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.global_scale = global_scale;
     a.out_rows = out_rows;
     a.row_exact = d->row_exact != 0;
-    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n);
+    a.exact_weights = wants_exact_weights(d->quant.mode, d->dtype, d->n, a.row_exact ? 1 : d->m);
     if (!d->transpose) {
         // Weights stored [K, N]: rows sorted by expert as groups on the matrix-core kernel (each expert's weights read once
         // per tile of its rows; the reference's grouped kernel of the block formats, gpu.rs:6786-6812), else one product
@@ -883,7 +890,7 @@ static int32_t gather_qmm_any(const nvq_gather_desc *d, const void *x, const voi
     a.offsets = offsets;
     if (glu != nullptr) {
         // (projections of fewer rows take the exact-weights kernels as separate products: the epilogue form would differ)
-        if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2))
+        if (wants_exact_weights(d->quant.mode, d->dtype, d->n / 2, d->m))
             return fail(NVQ_UNSUPPORTED, "gather_qmm: the gated epilogue takes affine projections of 1024 rows or more each");
         a.exact_weights = 0;
         a.glu = 1 + glu->activation; a.glu_alpha = glu->alpha; a.glu_limit = glu->limit;

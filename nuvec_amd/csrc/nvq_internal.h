@@ -7,6 +7,7 @@
 #include <atomic>
 
 #include "nuvec_hip.h"
+#include "nvq_splits.h"
 
 namespace nvq {
 

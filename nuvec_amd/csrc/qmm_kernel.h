@@ -464,51 +464,19 @@ __global__ void __launch_bounds__(256) qmm_reduce_kernel(const float *__restrict
     }
 }
 
-// Estimated microseconds of `tiles` tiles of TL walking `steps` steps of 64 values on `cus` compute units, from
-// the kernel's measured behaviour: about 1.7 us per step for the big tile (one block per compute unit); the small
-// tile takes 0.8 us per step alone on a compute unit and 1.2 us when two share it.
-template <class TL>
-inline double tiles_us(double tiles, double steps, int cus) {
-    if (TL::BM == 256) return ceil(tiles / cus) * steps * 1.7;
-    if (tiles <= cus) return steps * 0.8;
-    return ceil(tiles / (2.0 * cus)) * steps * 1.2;
+// Tile choice and the split of K over the grid: the host rules of nvq_splits.h, here bound to this kernel's constants.
+static_assert(BK == splits::kQmmStep && BigTile::BM == splits::kQmmBigTile && BigTile::BN == splits::kQmmBigTile &&
+              SmallTile::BM == splits::kQmmSmallTile && SmallTile::BN == splits::kQmmSmallTile, "nvq_splits.h describes these tiles");
+inline splits::Product split_product(const ProductArgs &a) {
+    return splits::Product{a.m, a.n, a.k, a.batch, a.row_exact != 0, a.exact_weights != 0};
 }
-template <class TL>
-inline double estimate_us(const ProductArgs &a, int cus) {
-    const double tiles = (double)((a.m + TL::BM - 1) / TL::BM) * (double)((a.n + TL::BN - 1) / TL::BN) * (double)a.batch;
-    return tiles_us<TL>(tiles, (double)(a.k / BK), cus);
-}
-inline bool small_tile_is_faster(const ProductArgs &a, int cus) {
-    return a.exact_weights || estimate_us<SmallTile>(a, cus) < estimate_us<BigTile>(a, cus);
-}
-
-// How many ways a single product splits K over the grid, by estimate: the splits fill the chip's block slots
-// with its (few) tiles, and cost a second kernel that reads their float32 partial sums (about 3 us to launch and
-// 4 bytes per microsecond and compute unit... in all: 4 TB/s).  Each split has at least eight steps, in whole table
-// periods; at most eight splits.  1: no split.
+inline bool small_tile_is_faster(const ProductArgs &a, int cus) { return splits::qmm_small_tile_is_faster(split_product(a), cus); }
+// How many ways a single product splits K over the grid (1: no split), the steps of a split, the estimated duration.
 inline int k_splits(const ProductArgs &a, int cus, int *steps_per_split = nullptr, double *estimate = nullptr) {
-    const int64_t steps = a.k / BK;
-    if (steps_per_split != nullptr) *steps_per_split = (int)steps;
-    const bool small = small_tile_is_faster(a, cus);
-    if (estimate != nullptr) *estimate = small ? estimate_us<SmallTile>(a, cus) : estimate_us<BigTile>(a, cus);
-    if (a.batch != 1) return 1;
-    const int64_t bm = small ? SmallTile::BM : BigTile::BM, bn = small ? SmallTile::BN : BigTile::BN;
-    const double tiles = (double)(((a.m + bm - 1) / bm) * ((a.n + bn - 1) / bn));
-    auto walk_us = [&](double t, double st) { return small ? tiles_us<SmallTile>(t, st, cus) : tiles_us<BigTile>(t, st, cus); };
-    double best_us = walk_us(tiles, (double)steps);
-    int best = 1;
-    int64_t best_per = steps;
-    for (int want = 2; want <= 8 && want <= steps / 8; want++) {
-        const int64_t per = (((steps + want - 1) / want) + 3) & ~(int64_t)3;  // whole table periods
-        const int splits = (int)((steps + per - 1) / per);                    // every split has a step
-        if (splits < 2) continue;
-        const double reduce_us = 3.0 + ((double)splits * 4.0 + 2.0) * (double)a.m * (double)a.n * 2.0 / 4.0e6;  // written, then read
-        const double us = walk_us(tiles * splits, (double)per) + reduce_us;
-        if (us < 0.9 * best_us) best_us = us, best = splits, best_per = per;
-    }
-    if (steps_per_split != nullptr) *steps_per_split = (int)best_per;
-    if (estimate != nullptr) *estimate = best_us;
-    return best;
+    const splits::Plan p = splits::qmm_plan(split_product(a), cus);
+    if (steps_per_split != nullptr) *steps_per_split = (int)p.per_split;
+    if (estimate != nullptr) *estimate = p.estimate_us;
+    return p.splits;
 }
 
 template <typename T, int BITS, int FP4, class TL, bool EXACT = false>
@@ -523,6 +491,8 @@ int32_t run_tile(ProductArgs a, void *workspace, hipStream_t s) {
     }
     int per = 0;
     const int splits = workspace != nullptr ? k_splits(a, compute_units(), &per) : 1;
+    if (splits > 1 && (int64_t)(splits - 1) * per >= a.k / BK)  // (a block of such a split would leave its partial sums unwritten)
+        return fail(NVQ_BACKEND, "quantized_matmul: %d splits of %d steps leave one without a step of K = %lld", splits, per, (long long)a.k);
     a.k_splits = splits;
     a.k_split_steps = per;
     a.partials = splits > 1 ? static_cast<float *>(workspace) : nullptr;

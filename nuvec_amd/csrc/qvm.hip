@@ -510,27 +510,16 @@ __global__ void __launch_bounds__(kThreads, TL::kBlocksPerCu) qmn_kernel(const P
 
 inline bool few_rows(const ProductArgs &a) { return a.m <= Tile32::BM; }
 
-// Splits of K for a product whose tiles do not fill the chip: the split with the least estimated time, counted as
-// rounds of resident blocks x (3 us to start + 1.2 us per step of the longest split; 0.64 us per step of the 32-row
-// tile) plus, with a split, the reduction: its launch, 0.38 us per split it adds up in turn and its float32 traffic at
-// 4 TB/s (fitted to w[4096,4096] at 1 to 32 rows: 43 / 26 / 17 / 13 / 15 / 20 us with 1 / 2 / 4 / 8 / 16 / 32 splits).
+// Splits of K for a product whose tiles do not fill the chip: the host rule of nvq_splits.h, bound to these tiles.
+static_assert(BK == splits::kQmnStep && BN == splits::kQmnTileCols && Tile32::BM == splits::kQmnFewRows &&
+              Tile128::BM == splits::kQmnManyRows && Tile32::kBlocksPerCu == splits::kQmnFewBlocksPerCu &&
+              Tile128::kBlocksPerCu == splits::kQmnManyBlocksPerCu, "nvq_splits.h describes these tiles");
+inline splits::Product split_product(const ProductArgs &a) {
+    return splits::Product{a.m, a.n, a.k, a.batch, a.row_exact != 0, a.exact_weights != 0};
+}
 template <class TL>
 int splits_of_shape(const ProductArgs &a) {
-    const int64_t tiles = ((a.m + TL::BM - 1) / TL::BM) * ((a.n + BN - 1) / BN) * a.batch, steps = a.k / BK;
-    const int64_t resident = TL::kBlocksPerCu * (int64_t)compute_units();
-    if (tiles >= resident || steps < 4) return 1;
-    const double step_us = TL::BM == 32 ? 0.64 : 1.2;
-    double best = 0.0;
-    int64_t pick = 1;
-    for (int64_t splits = 1; splits <= steps / 2 && splits <= 64; splits++) {
-        const int64_t per_split = (steps + splits - 1) / splits;
-        if ((steps + per_split - 1) / per_split != splits) continue;  // (another count gives the same longest split)
-        const int64_t rounds = (tiles * splits + resident - 1) / resident;
-        double us = (double)rounds * (3.0 + step_us * (double)per_split);
-        if (splits > 1) us += 2.0 + 0.38 * (double)splits + (double)splits * (double)(a.batch * a.m * a.n) * 4.0 / 4.0e6;
-        if (splits == 1 || us < best) best = us, pick = splits;
-    }
-    return (int)pick;
+    return splits::qmn_plan(split_product(a), compute_units(), TL::BM == Tile32::BM).splits;
 }
 inline int splits_of(const ProductArgs &a) { return few_rows(a) ? splits_of_shape<Tile32>(a) : splits_of_shape<Tile128>(a); }
 
@@ -541,6 +530,11 @@ int32_t run_shape(const ProductArgs &a, float *workspace, hipStream_t s) {
     const int64_t row_tiles = grouped ? (a.batch + TL::BM - 1) / TL::BM + a.experts : (a.m + TL::BM - 1) / TL::BM;
     const int64_t tiles = row_tiles * ((a.n + BN - 1) / BN);
     const dim3 grid((unsigned)(grouped ? tiles : (tiles + 7) / 8 * 8), (unsigned)(grouped ? 1 : a.batch), (unsigned)splits);
+    {  // (the kernel's split of the steps; a block of a split without a step would leave its partial sums unwritten)
+        const int64_t steps = a.k / BK, per_split = (steps + splits - 1) / splits;
+        if (splits > 1 && (int64_t)(splits - 1) * per_split >= steps)
+            return fail(NVQ_BACKEND, "quantized_matmul: %d splits leave one without a step of K = %lld", splits, (long long)a.k);
+    }
     if (FP4 == kAffine && a.exact_weights) hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, FP4 == kAffine, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     else hipLaunchKernelGGL((qmn_kernel<T, BITS, FP4, false, TL>), grid, dim3(kThreads), 0, s, a, splits, workspace);
     NVQ_LAUNCH_CHECK("qmn");
@@ -624,16 +618,10 @@ int32_t run_qvm_typed(const ProductArgs &a, void *workspace, hipStream_t s) {
 
 }  // namespace
 
-// Splits of K: about a block (of eight wavefronts) per compute unit, at least 16 rows of w per wavefront, at most 32
-// splits (the reduction kernel adds them one after the other).
+// Splits of K of the vector kernel: the host rule of nvq_splits.h.
+static_assert(kQvmWaves == splits::kQvmWaves, "nvq_splits.h describes this block");
 int qvm_splits(const ProductArgs &a) {
-    const int rm = a.m == 1 ? 1 : 4;
-    // row-exact: the split is the one-row product's, whatever the rows and batches, so that every row keeps its bits
-    const int64_t base = ((a.n + 2047) / 2048) * (a.row_exact ? 1 : a.batch * ((a.m + rm - 1) / rm));
-    const int64_t want = ((int64_t)compute_units() + base - 1) / base;
-    const int64_t most = a.k / (16 * kQvmWaves) > 1 ? a.k / (16 * kQvmWaves) : 1;
-    const int64_t splits = want < 1 ? 1 : (want > most ? most : want);
-    return (int)(splits > 32 ? 32 : splits);
+    return splits::qvm_plan(splits::Product{a.m, a.n, a.k, a.batch, a.row_exact != 0, a.exact_weights != 0}, compute_units()).splits;
 }
 
 size_t qvm_workspace_bytes(const ProductArgs &a) {

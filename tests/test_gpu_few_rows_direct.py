@@ -44,8 +44,11 @@ def test_routes_of_the_baseline_configurations():
     assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
     assert ops.quantized_matmul_route(64, 2880, 2880, nv.Quant.new(nv.QuantMode.MXFP4), bf16) in ("qmf_kernel", "qmm_kernel")
     # passes of 16 rows where the matrix is small enough to be read again from the caches; the tiles beyond
-    small = lambda m: ops.quantized_matmul_route(m, 1024, 4096, nv.Quant.affine(64, 4), bf16)
+    # (bfloat16 products of more than 16 rows and fewer than 8192 outputs per row take the kernels that hold the CPU's weights)
+    small = lambda m, t=torch.float16: ops.quantized_matmul_route(m, 1024, 4096, nv.Quant.affine(64, 4), t)
     assert small(64) == "qmd_kernel" and small(192) == "qmd_kernel" and small(512) in ("qmf_kernel", "qmm_kernel")
+    assert small(16, bf16) == "qmd_kernel" and small(64, bf16) in ("qmf_kernel", "qmm_kernel") and small(192, bf16) in ("qmf_kernel", "qmm_kernel")
+    assert ops.quantized_matmul_route(64, 8192, 4096, nv.Quant.affine(64, 4), bf16) == "qmd_kernel"
     assert c2(64) == "qmd_kernel" and c2(96) == "qmm_kernel"
     # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
     for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (30, 64, 128, 64, 4), (20, 1000, 1024, 64, 6)):
@@ -54,7 +57,7 @@ def test_routes_of_the_baseline_configurations():
 
 # (rows of 1024 outputs or more: affine products of shorter rows take the kernels that materialise the CPU's weights)
 SHAPES = [(2, 1224, 512), (9, 2024, 1024), (16, 1154, 4096), (13, 1120, 8192), (11, 1072, 14336), (23, 1088, 1536), (16, 5000, 512),
-          (12, 1064, 7168), (77, 1324, 2048), (130, 1072, 512)]
+          (12, 1064, 7168), (77, 1324, 2048), (130, 1072, 512), (23, 8200, 512)]
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
@@ -70,6 +73,9 @@ def test_direct_few_row_kernel_every_width(dtype, bits, group):
             continue  # the 4-bit decode kernels' rows
         if bits in (5, 6) and m > 16:
             continue  # passes of rows of 5- and 6-bit codes stay on the kernels that round a weight once
+        if dtype == ref.BF16 and m > 16 and n < 8192:  # the CPU's weights: not this kernel's, which never materialises one
+            assert route in ("qmf_kernel", "qmm_kernel"), f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
+            continue
         assert route == "qmd_kernel", f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
         packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
