@@ -1668,7 +1668,7 @@ def test_quantize_dequantize_bit_exact(mode, qmode, dtype):
         nv.quantize_dequantize(to_dev(x), nv.Quant.affine(64, 4))
 
 
-@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32])
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F32, ref.F16])
 @pytest.mark.parametrize("group,bits,d", [(64, 4, 128), (32, 8, 64), (64, 3, 128)])
 def test_quantized_attention_composition(dtype, group, bits, d):
     """`quantized_attention` (fast.rs:694-718) as the reference composes it over the library's products: one query row
@@ -1690,7 +1690,7 @@ def test_quantized_attention_composition(dtype, group, bits, d):
     vf = ref.to_f32(ref.affine_dequantize(*vq, dtype, group, bits), dtype).astype(np.float64)
     qf = ref.to_f32(q, dtype).astype(np.float64).reshape(b, hkv, rep, d)
     logits = scale * np.einsum("bhrd,bhsd->bhrs", qf, kf)
-    tol = {ref.BF16: 2e-2, ref.F32: 2e-5}[dtype]
+    tol = {ref.BF16: 2e-2, ref.F32: 2e-5, ref.F16: 2.5e-3}[dtype]
     from nuvec_amd import ops as nv_ops
     fits = nv_ops.quantized_attention_fits(to_dev(q), K, V)
     assert fits == (bits in (3, 4, 8) and d in (64, 128))  # the fused kernel's rule (fast/imp.rs:3944-3992)

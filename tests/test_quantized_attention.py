@@ -75,28 +75,33 @@ def test_quantized_attention_matches_the_recorded_outputs(recorded, dt, bits, l)
     (1, 32, 8, 8192, 128, 4, 64, False), (2, 8, 8, 1000, 64, 8, 32, True), (1, 4, 1, 777, 128, 8, 128, True),
     (3, 16, 2, 2049, 64, 4, 64, False), (1, 2, 2, 513, 128, 4, 32, True), (2, 8, 2, 1500, 128, 3, 64, True),
     (1, 16, 16, 700, 64, 3, 32, False), (1, 4, 2, 61, 128, 3, 128, True)])
-def test_positions_split_over_the_grid(batch, hq, hkv, s, d, bits, group, with_sinks):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_positions_split_over_the_grid(batch, hq, hkv, s, d, bits, group, with_sinks, dtype):
     """Long caches: the positions split over the grid and merged (with the workspace) against one block per head
     (without) and against float32 attention over the dequantized cache; lengths off the tile size, grouped heads,
-    sinks.  Bound: 2e-3 of the largest output, far under the bfloat16 step of the recorded cases' tolerance."""
+    sinks; queries, scales, biases and outputs in float32, bfloat16 and float16.  Bound: 2e-3 of the largest output
+    in float32 (far under the bfloat16 step of the recorded cases' tolerance); in the 16-bit types one and a half
+    rounding steps of the largest output (1.2e-2 bfloat16, inside the reference's 2e-2; 1.5e-3 float16), the output
+    being rounded once from float32 sums."""
     from nuvec_amd import ops
     torch.manual_seed(s)
-    kd, vd = torch.randn(batch, hkv, s, d, device="cuda"), torch.randn(batch, hkv, s, d, device="cuda")
+    kd, vd = torch.randn(batch, hkv, s, d, device="cuda").to(dtype), torch.randn(batch, hkv, s, d, device="cuda").to(dtype)
     quant = nv.Quant.affine(group, bits)
     k, v = nv.quantize(kd, quant), nv.quantize(vd, quant)
-    q = torch.randn(batch, hq, 1, d, device="cuda")
-    sinks = torch.randn(hq, device="cuda") if with_sinks else None
+    q = torch.randn(batch, hq, 1, d, device="cuda").to(dtype)
+    sinks = torch.randn(hq, device="cuda").to(dtype) if with_sinks else None
     scale = d ** -0.5
-    assert ops.quantized_attention_fits(q, k, v)
+    assert ops.quantized_attention_fits(q, k, v, sinks)
     split = ops.quantized_attention(q, k, v, scale, sinks)
     whole = ops.quantized_attention(q, k, v, scale, sinks, scratch=False)
-    kf = nv.dequantize(k).repeat_interleave(hq // hkv, dim=1)
-    vf = nv.dequantize(v).repeat_interleave(hq // hkv, dim=1)
-    scores = scale * q @ kf.transpose(-1, -2)
+    assert split.dtype == dtype and whole.dtype == dtype
+    kf = nv.dequantize(k).float().repeat_interleave(hq // hkv, dim=1)
+    vf = nv.dequantize(v).float().repeat_interleave(hq // hkv, dim=1)
+    scores = scale * q.float() @ kf.transpose(-1, -2)
     if with_sinks:
-        scores = torch.cat([scores, sinks.view(1, hq, 1, 1).expand(batch, hq, 1, 1)], dim=-1)
+        scores = torch.cat([scores, sinks.float().view(1, hq, 1, 1).expand(batch, hq, 1, 1)], dim=-1)
     p = torch.softmax(scores, dim=-1)[..., :s]
     want = p @ vf
-    bound = 2e-3 * want.abs().max().item()
-    assert (split - want).abs().max().item() <= bound, "split"
-    assert (whole - want).abs().max().item() <= bound, "one block per head"
+    bound = {torch.float32: 2e-3, torch.bfloat16: 1.2e-2, torch.float16: 1.5e-3}[dtype] * want.abs().max().item()
+    assert (split.float() - want).abs().max().item() <= bound, "split"
+    assert (whole.float() - want).abs().max().item() <= bound, "one block per head"
