@@ -69,7 +69,7 @@ class Mlp:
         """Stores the gate and up projections as one weight whose rows alternate in runs of 64 (a copy made once, at load
         time), so that a few rows of x (decoding) take both products and the activation in one kernel
         (`ops.quantized_matmul_glu`).  Left apart: projections that differ in shape or quantization, hidden sizes off
-        whole runs, affine projections of fewer than 1024 rows (they take the kernels with the CPU's weights)."""
+        whole runs, affine projections of fewer than 1024 rows (they take the kernels with the CPU's weights at every row count)."""
         g, u = self.gate_proj, self.up_proj
         hidden = g.weight.shape[0]
         if g.quant != u.quant or g.weight.shape != u.weight.shape or (g.bias is None) != (u.bias is None) or hidden % 64 != 0:
