@@ -21,6 +21,11 @@
 // keeps the limbs in registers for all of its rows; from then on every wavefront requests two rows ahead of the one it
 // works on and shares nothing, so the loads never wait for arithmetic.  The R row sums of a wavefront are folded across its
 // lanes in one pass (half-wavefront and 16-lane-row swaps, then moves inside a row).
+//
+// Several rows of x.  A block may carry the limbs of up to four rows of x (MX; 16 registers per lane, row and chunk) and
+// multiply every weight row with each of them: the codes, their sum and the scale and bias are fetched once.  The rows
+// share nothing else, so each has the bits of its one-row product whatever MX is: a row-exact product of many rows walks
+// the weights once per four rows, and two to four ordinary rows take one pass.
 #include <type_traits>
 #include <utility>
 
@@ -105,30 +110,34 @@ __device__ __forceinline__ void to_limbs(const uint4 piece, uint4 &limbs, float 
     limbs.w = squeeze((ha >> 4) & k, (hb >> 4) & k);
 }
 
-// S: chunks of 2048 values of K.  R: rows per wavefront.  Grid: (blocks of 8 R rows, rows of x).
-template <typename T, int S, int R>
+// S: chunks of 2048 values of K.  R: weight rows per wavefront.  MX: rows of x per block.
+// Grid: (blocks of 8 R weight rows, groups of MX rows of x).
+template <typename T, int S, int R, int MX>
 __global__ void __launch_bounds__(kWaves * 64) qmv4_dot8_kernel(const ProductArgs a) {
-    static_assert(R >= 1 && R <= 8 && S >= 1, "one batched reduction of up to eight rows");
-    constexpr int kPieces = S * 256;                       // 16-byte pieces of x
+    static_assert(R >= 1 && R <= 8 && S >= 1 && MX >= 1 && MX <= 4, "one batched reduction of up to eight rows per row of x");
+    constexpr int kRowPieces = S * 256;                    // 16-byte pieces of a row of x
+    constexpr int kPieces = MX * kRowPieces;
     constexpr int kPerThread = (kPieces + 511) / 512;
     constexpr int kRowQuads = S * 64;                      // 16-byte pieces of a row of codes
-    __shared__ uint4 x_limbs[S][4][64];                    // [chunk][dword t of the slice][lane]: limbs 0..3 of values 8 t .. 8 t + 7
-    __shared__ float2 x_meta[S][64];                       // [chunk][lane]: (2^(e-14), sum of the slice's x)
+    __shared__ uint4 x_limbs[MX][S][4][64];                // [row][chunk][dword t of the slice][lane]: limbs 0..3 of values 8 t .. 8 t + 7
+    __shared__ float2 x_meta[MX][S][64];                   // [row][chunk][lane]: (2^(e-14), sum of the slice's x)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int N = (int)a.n;
+    const int N = (int)a.n, M = (int)a.m;
     const int gshift = a.group == 32 ? 5 : a.group == 64 ? 6 : 7;
     const int kgroups = (S * 2048) >> gshift;
-    const T *x = (const T *)a.x + (int64_t)blockIdx.y * (S * 2048);
-    T *y = (T *)a.y + (int64_t)blockIdx.y * N;
+    const int m0 = blockIdx.y * MX;                        // this block's first row of x
+    const T *x = (const T *)a.x;
+    T *y = (T *)a.y;
     const T *scales = (const T *)a.scales, *biases = (const T *)a.biases;
 
-    // x first: it is needed first
+    // x first: it is needed first (a row past M reads row M - 1 and is not stored)
     uint4 xg[kPerThread];
 #pragma unroll
     for (int p = 0; p < kPerThread; p++) {
-        const int piece = tid + p * 512;
-        xg[p] = reinterpret_cast<const uint4 *>(x)[piece < kPieces ? piece : kPieces - 1];
+        const int piece = tid + p * 512, pc = piece < kPieces ? piece : kPieces - 1;
+        const int mr = m0 + pc / kRowPieces < M ? m0 + pc / kRowPieces : M - 1;
+        xg[p] = reinterpret_cast<const uint4 *>(x + (int64_t)mr * (S * 2048))[pc % kRowPieces];
     }
     __builtin_amdgcn_sched_barrier(0);
     // Row j of this wavefront: its codes (one 16-byte load per chunk, read once: non-temporal), and the scale and bias of
@@ -159,91 +168,113 @@ __global__ void __launch_bounds__(kWaves * 64) qmv4_dot8_kernel(const ProductArg
         float down, sum;
         to_limbs<T>(xg[p], limbs, down, sum);
         if (piece < kPieces) {
-            x_limbs[piece >> 8][piece & 3][(piece & 255) >> 2] = limbs;
-            if ((piece & 3) == 0) x_meta[piece >> 8][(piece & 255) >> 2] = make_float2(down, sum);
+            const int mr = piece / kRowPieces, q = piece % kRowPieces;
+            x_limbs[mr][q >> 8][q & 3][(q & 255) >> 2] = limbs;
+            if ((q & 3) == 0) x_meta[mr][q >> 8][(q & 255) >> 2] = make_float2(down, sum);
         }
     }
     __syncthreads();
-    uint4 xr[S][4];
-    float2 xm[S];
+    uint4 xr[MX][S][4];
+    float2 xm[MX][S];
 #pragma unroll
-    for (int u = 0; u < S; u++) {
+    for (int mr = 0; mr < MX; mr++)
 #pragma unroll
-        for (int t = 0; t < 4; t++) xr[u][t] = x_limbs[u][t][lane];
-        xm[u] = x_meta[u][lane];
-    }
+        for (int u = 0; u < S; u++) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) xr[mr][u][t] = x_limbs[mr][u][t][lane];
+            xm[mr][u] = x_meta[mr][u][lane];
+        }
     uint32_t ones;
     asm volatile("s_mov_b32 %0, 0x11111111" : "=s"(ones));  // (held in a scalar register: a literal would be re-materialised per use)
 
-    float sums[8];
+    float sums[MX][8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) sums[j] = 0.0f;
+    for (int mr = 0; mr < MX; mr++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) sums[mr][j] = 0.0f;
     auto row = [&](auto jt) {
         constexpr int j = decltype(jt)::value;
         request(std::integral_constant<int, j + kAhead>{});
-        float acc = 0.0f;
+        float acc[MX];
+#pragma unroll
+        for (int mr = 0; mr < MX; mr++) acc[mr] = 0.0f;
 #pragma unroll
         for (int u = 0; u < S; u++) {
             const uint32_t d[4] = {wq[j][u].x, wq[j][u].y, wq[j][u].z, wq[j][u].w};
-            uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0, cs = 0;
+            uint32_t cs = 0;
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                a0 = __builtin_amdgcn_udot8(d[t], xr[u][t].x, a0, false);
-                a1 = __builtin_amdgcn_udot8(d[t], xr[u][t].y, a1, false);
-                a2 = __builtin_amdgcn_udot8(d[t], xr[u][t].z, a2, false);
-                a3 = __builtin_amdgcn_udot8(d[t], xr[u][t].w, a3, false);
-                cs = __builtin_amdgcn_udot8(d[t], ones, cs, false);
-            }
-            uint32_t h = (a3 << 4) + a2;
-            h = (h << 4) + a1;
-            h = (h << 4) + a0;
-            const int total = (int)h - (int)(cs << (kLimbBits - 1));  // sum code * round(x * up): below 2^25 in magnitude
+            for (int t = 0; t < 4; t++) cs = __builtin_amdgcn_udot8(d[t], ones, cs, false);
             const float sc = Elem<T>::load(&sr[j][u], 0), bi = Elem<T>::load(&br[j][u], 0);
-            acc = __builtin_fmaf(sc * xm[u].x, (float)total, __builtin_fmaf(bi, xm[u].y, acc));
+#pragma unroll
+            for (int mr = 0; mr < MX; mr++) {
+                uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    a0 = __builtin_amdgcn_udot8(d[t], xr[mr][u][t].x, a0, false);
+                    a1 = __builtin_amdgcn_udot8(d[t], xr[mr][u][t].y, a1, false);
+                    a2 = __builtin_amdgcn_udot8(d[t], xr[mr][u][t].z, a2, false);
+                    a3 = __builtin_amdgcn_udot8(d[t], xr[mr][u][t].w, a3, false);
+                }
+                uint32_t h = (a3 << 4) + a2;
+                h = (h << 4) + a1;
+                h = (h << 4) + a0;
+                const int total = (int)h - (int)(cs << (kLimbBits - 1));  // sum code * round(x * up): below 2^25 in magnitude
+                acc[mr] = __builtin_fmaf(sc * xm[mr][u].x, (float)total, __builtin_fmaf(bi, xm[mr][u].y, acc[mr]));
+            }
         }
-        sums[j] = acc;
+#pragma unroll
+        for (int mr = 0; mr < MX; mr++) sums[mr][j] = acc[mr];
     };
     static_for<R>(row);
 
-    // Eight rows' sums at once: after the two swaps and the select, lane l carries row (l >> 3) & 7, and three moves
-    // inside its eight lanes finish the sum.
-    float s4[4], s2[2];
+    // Eight rows' sums at once, per row of x: after the two swaps and the select, lane l carries row (l >> 3) & 7, and
+    // three moves inside its eight lanes finish the sum.
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        float p = sums[j], q = sums[j + 4];
-        swap_halves(p, q);
-        s4[j] = p + q;
-    }
+    for (int mr = 0; mr < MX; mr++) {
+        float s4[4], s2[2];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        float p = s4[j], q = s4[j + 2];
-        swap_rows(p, q);
-        s2[j] = p + q;
+        for (int j = 0; j < 4; j++) {
+            float p = sums[mr][j], q = sums[mr][j + 4];
+            swap_halves(p, q);
+            s4[j] = p + q;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            float p = s4[j], q = s4[j + 2];
+            swap_rows(p, q);
+            s2[j] = p + q;
+        }
+        const float u0 = dpp_add<0x128>(s2[0]), u1 = dpp_add<0x128>(s2[1]);  // row_ror:8
+        float total = (lane & 8) ? u1 : u0;
+        total = dpp_add<0x141>(total);  // row_half_mirror
+        total = dpp_add<0xB1>(total);   // quad_perm [1,0,3,2]
+        total = dpp_add<0x4E>(total);   // quad_perm [2,3,0,1]
+        const int j = (lane >> 3) & 7, n = row0 + j * kWaves;
+        if ((lane & 7) == 0 && j < R && n < N && m0 + mr < M)
+            Elem<T>::store(y, (int64_t)(m0 + mr) * N + n, add_row_bias<T>(a.row_bias, total, n));
     }
-    const float u0 = dpp_add<0x128>(s2[0]), u1 = dpp_add<0x128>(s2[1]);  // row_ror:8
-    float total = (lane & 8) ? u1 : u0;
-    total = dpp_add<0x141>(total);  // row_half_mirror
-    total = dpp_add<0xB1>(total);   // quad_perm [1,0,3,2]
-    total = dpp_add<0x4E>(total);   // quad_perm [2,3,0,1]
-    const int j = (lane >> 3) & 7, n = row0 + j * kWaves;
-    if ((lane & 7) == 0 && j < R && n < N) Elem<T>::store(y, n, add_row_bias<T>(a.row_bias, total, n));
 }
 
-template <typename T, int S>
+template <typename T, int S, int MX>
 int32_t run_rows(const ProductArgs &a, int r, hipStream_t s) {
-    const dim3 grid((unsigned)((a.n + kWaves * r - 1) / (kWaves * r)), (unsigned)a.m), block(kWaves * 64);
+    const dim3 grid((unsigned)((a.n + kWaves * r - 1) / (kWaves * r)), (unsigned)((a.m + MX - 1) / MX)), block(kWaves * 64);
     switch (r) {
-    case 1: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 1>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 2>), grid, block, 0, s, a); break;
-    case 3: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 3>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 4>), grid, block, 0, s, a); break;
-    case 5: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 5>), grid, block, 0, s, a); break;
-    case 6: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 6>), grid, block, 0, s, a); break;
-    case 7: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 7>), grid, block, 0, s, a); break;
-    default: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 8>), grid, block, 0, s, a); break;
+    case 1: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 1, MX>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 2, MX>), grid, block, 0, s, a); break;
+    case 3: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 3, MX>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 4, MX>), grid, block, 0, s, a); break;
+    case 5: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 5, MX>), grid, block, 0, s, a); break;
+    case 6: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 6, MX>), grid, block, 0, s, a); break;
+    case 7: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 7, MX>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((qmv4_dot8_kernel<T, S, 8, MX>), grid, block, 0, s, a); break;
     }
     NVQ_LAUNCH_CHECK("qmv4_dot8");
     return NVQ_OK;
+}
+template <typename T, int S>
+int32_t run_x_rows(const ProductArgs &a, int r, hipStream_t s) {
+    const int mx = a.m >= 4 ? 4 : (int)a.m;  // rows of x per block (more rows: groups of four)
+    return mx == 1 ? run_rows<T, S, 1>(a, r, s) : mx == 2 ? run_rows<T, S, 2>(a, r, s) : mx == 3 ? run_rows<T, S, 3>(a, r, s) : run_rows<T, S, 4>(a, r, s);
 }
 
 }  // namespace
@@ -256,23 +287,25 @@ int qmv_dot8_rows_per_wave(int64_t n, int cus) {
 
 // What the kernel takes: single products (no batch, no gathered pairs, no gated epilogue) of 4-bit affine weights stored
 // [N, K] with K = 2048 or 4096, bf16 / f16, 1024 outputs and more (rows of fewer outputs materialise the CPU's weights
-// elsewhere), operands 16-byte aligned.  One row of x, or the rows of a row-exact product, each as its own pass over the
-// weights, so that every row has the bits of its one-row product.
+// elsewhere), operands 16-byte aligned.  One row of x (two against 8192 weight rows and more) in one pass over the
+// weights, or the rows of a row-exact product four per pass: every row has the bits of its one-row product either way.
 bool qmv_dot8_takes(const ProductArgs &a) {
     if (a.mode != NVQ_AFFINE || a.bits != 4 || (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16)) return false;
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.glu != 0 || a.exact_weights) return false;
     if (a.k != 2048 && a.k != 4096) return false;
     if (a.group != 32 && a.group != 64 && a.group != 128) return false;
     if (a.n < 1024 || a.n > 0x7FFFFFFF / 128 || a.m < 1 || a.m > 65535) return false;
-    if (!(a.m == 1 || a.row_exact)) return false;
+    // two rows where the matrix is large (W[14336,4096]: 8.7 us against 9.8 on the 16x16x32 decode kernel; three and four rows
+    // cost 1.7 us each here and stay there: 10.4 / 12.3 against 9.8 / 9.9 us); a row-exact product any number, four per pass
+    if (!(a.m == 1 || (a.m == 2 && a.n >= 8192) || a.row_exact)) return false;  // up to four rows in one pass; a row-exact product any number, four per pass
     return ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
 }
 
 int32_t launch_qmv_dot8(const ProductArgs &a, hipStream_t s) {
     if (!qmv_dot8_takes(a)) return fail(NVQ_UNSUPPORTED, "quantized_matmul: the integer decode kernel does not take this product");
     const int r = qmv_dot8_rows_per_wave(a.n, compute_units());
-    if (a.dtype == NVQ_BF16) return a.k == 4096 ? run_rows<bf16_t, 2>(a, r, s) : run_rows<bf16_t, 1>(a, r, s);
-    return a.k == 4096 ? run_rows<f16_t, 2>(a, r, s) : run_rows<f16_t, 1>(a, r, s);
+    if (a.dtype == NVQ_BF16) return a.k == 4096 ? run_x_rows<bf16_t, 2>(a, r, s) : run_x_rows<bf16_t, 1>(a, r, s);
+    return a.k == 4096 ? run_x_rows<f16_t, 2>(a, r, s) : run_x_rows<f16_t, 1>(a, r, s);
 }
 
 }  // namespace nvq

@@ -99,6 +99,26 @@ def test_row_exact_rows_have_the_bits_of_the_one_row_product(dtype):
         assert np.array_equal(one[0], both[r]) and np.array_equal(one[0], wide[r]) and np.array_equal(one[0], wide[2 * m + r])
 
 
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+def test_two_rows_in_one_pass(dtype):
+    """Two rows of x against 8192 weight rows and more share one pass over the weights (the limbs of both rows in
+    registers, the codes fetched once); each row keeps the bits of its one-row product, so the pair is row-exact as it is."""
+    rng = np.random.default_rng(23)
+    n, k = 8200, 4096
+    quant = nv.Quant.affine(64, 4)
+    assert ops.quantized_matmul_route(2, n, k, quant, TORCH[dtype]) == "qmv4_dot8_kernel"
+    assert ops.quantized_matmul_route(2, 4096, k, quant, TORCH[dtype]) != "qmv4_dot8_kernel"  # (small matrices: the other decode kernels)
+    assert ops.quantized_matmul_route(3, n, k, quant, TORCH[dtype]) != "qmv4_dot8_kernel"
+    w, x = make_w(rng, n, k, dtype), make_x(rng, 2, k, dtype)
+    got, (packed, scales, biases) = product(x, w, dtype, 64)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=dtype, threads=8)
+    assert_rows_close(got, want, dtype, "integer decode, two rows")
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+    for r in range(2):
+        one = to_host(nv.quantized_matmul(to_dev(x[r:r + 1]), q))
+        assert np.array_equal(one.view(np.uint8)[0], got.view(np.uint8)[r])
+
+
 def test_bias_epilogue_and_repeatability():
     """QuantizedLinear's bias (crates/nuvec-nn/src/layers.rs:155-162): the rounded product plus the bias, rounded again, bit
     for bit; and two launches give the same bits."""

@@ -26,7 +26,8 @@ def test_routes_of_the_baseline_configurations():
     c2 = lambda m, **kw: ops.quantized_matmul_route(m, 14336, 4096, nv.Quant.affine(64, 4), bf16, **kw)
     assert ops.quantized_matmul_route(1, 4096, 4096, nv.Quant.affine(64, 4), torch.float32) == "qmv_lds_kernel"
     assert c2(1) == "qmv4_dot8_kernel"  # (one row, K = 4096: the integer dot-product decode kernel)
-    assert c2(4) == "qmv4_mm16_kernel" and c2(8) == "qmv4_mm16_kernel"
+    assert c2(2) == "qmv4_dot8_kernel"  # (two rows share a pass over a matrix this large)
+    assert c2(3) == "qmv4_mm16_kernel" and c2(4) == "qmv4_mm16_kernel" and c2(8) == "qmv4_mm16_kernel"
     assert c2(12) == "qmd_kernel" and c2(16) == "qmd_kernel"
     assert c2(2048) == "qmm_kernel"
     # row-exact rows take the kernel of the one-row product, each row as its own pass
