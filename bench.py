@@ -280,6 +280,9 @@ def all_configs(lib, device, qs):
     # ... and C2's product with the weights stored [K, N] (transpose = false)
     products("bf16 4-bit g64 w[4096,14336] stored [K, N]", N, K, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1, 16, 2048], 24,
              WEIGHT_BYTES, transpose=False)
+    # ... and with 6-bit codes (a run of eight columns is six bytes): the widths other than 2, 4 and 8 bits on the same kernel
+    products("bf16 6-bit g64 w[4096,14336] stored [K, N]", N, K, nv.Quant.affine(64, 6), torch.bfloat16, _lib.BF16, [16, 512], 12,
+             K * N * 6 // 8 + 2 * (K * (N // 64) * 2), transpose=False)
     # C5: 32 MXFP4 experts [2880,2880], 256 tokens x 4 distinct experts, pairs sorted by expert
     experts, n, k, tokens, top = 32, 2880, 2880, 256, 4
     weights = [nv.quantize((torch.randn(experts, n, k, device=device) * 0.02).to(torch.bfloat16), nv.QuantMode.MXFP4)

@@ -278,9 +278,11 @@ __device__ __forceinline__ void load_run(const unsigned char *p, uint32_t (&d)[B
         d[0] = v.x, d[1] = v.y;
     } else if constexpr (BITS == 4) {
         d[0] = *reinterpret_cast<const uint32_t *>(p);
-    } else {
-        static_assert(BITS == 2, "runs of eight codes of 2, 4 or 8 bits");
+    } else if constexpr (BITS == 2) {
         d[0] = *reinterpret_cast<const uint16_t *>(p);
+    } else {  // 1, 3, 5 and 6 bits: a run is BITS bytes at any byte offset of the row
+#pragma unroll
+        for (int i = 0; i < BITS; i++) d[i >> 2] |= (uint32_t)p[i] << (8 * (i & 3));
     }
 }
 
@@ -562,7 +564,15 @@ int32_t run_typed(const ProductArgs &a, float *ws, hipStream_t s) {
     case NVQ_NVFP4: return run<T, 4, kNvfp4>(a, ws, s);
     default: break;
     }
-    return a.bits == 2 ? run<T, 2, kAffine>(a, ws, s) : a.bits == 4 ? run<T, 4, kAffine>(a, ws, s) : run<T, 8, kAffine>(a, ws, s);
+    switch (a.bits) {
+    case 1: return run<T, 1, kAffine>(a, ws, s);
+    case 2: return run<T, 2, kAffine>(a, ws, s);
+    case 3: return run<T, 3, kAffine>(a, ws, s);
+    case 4: return run<T, 4, kAffine>(a, ws, s);
+    case 5: return run<T, 5, kAffine>(a, ws, s);
+    case 6: return run<T, 6, kAffine>(a, ws, s);
+    default: return run<T, 8, kAffine>(a, ws, s);
+    }
 }
 
 }  // namespace qmn
@@ -636,14 +646,18 @@ size_t qvm_workspace_bytes(const ProductArgs &a) {
 // (With eight wavefronts a block, eight rows of w in flight per lane and at most 32 splits the vector kernel above went,
 // at bf16 4-bit g64 and one row of x, kernel and reduction: w[4096,14336] 67 -> 23 us, w[14336,4096] 143 -> 52 us,
 // w[4096,4096] 65 -> 19 us; the matrix-core kernel: 23 / 26 / 12 us, and flat up to 16 rows where this one adds 8 us a row.)
-// The matrix-core kernel takes the 16-bit products whose codes come in whole runs of eight columns (2, 4 and 8 bits,
+// The matrix-core kernel takes the 16-bit products whose codes come in whole runs of eight columns (every affine width,
 // the block formats without a global scale) and whose K is whole steps of 64, whatever the rows of x: measured
 // against the vector kernel above (bf16, 4-bit g64, both with their split of K and its reduction, us per call of the
 // Python wrapper) w[4096,14336] 1 row 42 / 55, 8 rows 42 / 91, 32 rows 45 / 246, 512 rows 128 / 1890; w[14336,4096]
 // 1 row 35 / 131; w[1024,1024] 1 row 24 / 24, 32 rows 24 / 37; MXFP4 w[4096,4096] 1 row 22 / 94, 128 rows 26 / 588.
 bool qvm_takes_tiled(const ProductArgs &a) {
     if (a.dtype == NVQ_F32 || a.row_exact || a.global_scale != nullptr || a.m < 1) return false;
-    if (a.mode == NVQ_AFFINE && !(a.bits == 2 || a.bits == 4 || a.bits == 8)) return false;
+    // 1, 3, 5 and 6 bits: a run of eight codes is 1, 3, 5 or 6 bytes, fetched byte by byte.  bf16, us, vector kernel ->
+    // this one: w[4096,4096] 3 bits at 1 / 16 / 512 rows 17.9 / 31.6 / 961 -> 14.9 / 13.4 / 52.5; w[4096,14336] 6 bits at
+    // 2 / 16 / 512 rows 32.0 / 152 / 2324 -> 29.5 / 31.8 / 115; only a single row against many columns stays behind
+    // (w[4096,14336] 3 bits 18.7 against 23.4, 6 bits 24.6 against 29.3).
+    if (a.mode == NVQ_AFFINE && !(a.bits == 2 || a.bits == 4 || a.bits == 8) && a.m == 1 && a.offsets == nullptr && a.n > 8192) return false;
     if (a.k < qmn::BK || a.k % qmn::BK != 0 || (a.batch > 65535 && a.offsets == nullptr)) return false;
     for (int d = 0; d < a.batch_ndim; d++)
         if (a.x_strides[d] % 8 != 0 || a.w_strides[d] % 4 != 0) return false;  // 16-byte pieces of x, 8-byte runs of codes

@@ -38,7 +38,8 @@ def test_routes_of_the_baseline_configurations():
         assert c4(1) == "qmv4_lds_kernel"  # (the decode kernel takes a row of 3- and of 8-bit codes too)
         assert c4(16) == "qmd_kernel" and c4(5) == "qmd_kernel" and c4(2) == "qmv4_lds_kernel"  # (K = 4096: two rows stay on the decode kernel)
         assert c4(512) == "qmm_kernel"
-        assert c4(16, transpose=False) == ("qmn_kernel" if bits == 8 else "qvm_kernel")  # runs of eight codes: 2, 4, 8 bits
+        assert c4(16, transpose=False) == "qmn_kernel" and c4(1, transpose=False) == "qmn_kernel"  # runs of eight codes: every width
+        assert ops.quantized_matmul_route(1, 14336, 4096, nv.Quant.affine(group, bits), bf16, transpose=False) == ("qmn_kernel" if bits == 8 else "qvm_kernel")
         assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
     assert ops.quantized_matmul_route(24, 1000, 1024, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
     assert ops.quantized_matmul_route(24, 4096, 14336, nv.Quant.affine(64, 4), bf16) == "qmm_kernel"  # (a long K: the tiles split it)

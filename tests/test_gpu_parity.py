@@ -950,7 +950,7 @@ def test_untransposed_products_batched():
 
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
-@pytest.mark.parametrize("group,bits", [(64, 4), (32, 4), (128, 8), (32, 8), (64, 2), (128, 2)])
+@pytest.mark.parametrize("group,bits", [(64, 4), (32, 4), (128, 8), (32, 8), (64, 2), (128, 2), (64, 3), (32, 5), (64, 6), (128, 1), (128, 3), (32, 6)])
 def test_untransposed_products_on_the_matrix_cores(dtype, group, bits):
     """Weights stored [K, N] with K in whole steps of 64 and codes in runs of eight columns: the tiled matrix-core
     kernel, for one row of x and for several tiles of rows, ragged M and N, K split over the grid (through the
