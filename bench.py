@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor figure
+MFMA_F32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 MFMA, vendor figure
 N, K = 14336, 4096
 GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
@@ -246,7 +247,7 @@ def all_configs(lib, device, qs):
     def best_of(calls, steps):
         return min(time_launches(calls, steps, len(calls), graph=False)[0] for _ in range(3))
 
-    def products(label, n, k, quant, tdtype, code, ms_list, copies, wbytes, weights=None, transpose=True):
+    def products(label, n, k, quant, tdtype, code, ms_list, copies, wbytes, weights=None, transpose=True, matrix_peak=MFMA_BF16_PEAK_TFLOPS):
         if weights is None:
             gen = torch.Generator(device=device)
             weights = []
@@ -264,10 +265,12 @@ def all_configs(lib, device, qs):
             out.append({"config": label, "m": m, "kernel": kernel.decode() if kernel else None, "us_per_launch": ms * 1e3,
                         "weight_gbps": gbps, "tflops": tflops,
                         # the roof that bounds the row: weight bytes over HBM for few rows, the bf16 matrix peak for many
-                        "frac_of_peak": gbps / HBM_PEAK_GBPS if m <= 64 else tflops / MFMA_BF16_PEAK_TFLOPS,
+                        "frac_of_peak": gbps / HBM_PEAK_GBPS if m <= 64 else tflops / matrix_peak,
                         "bound": "hbm" if m <= 64 else "mfma"})
 
-    products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1], 48, 10_485_760)
+    # (C1 is one row; 512 rows beside it: float32 on the matrix cores, against the 157.3 TFLOP/s of the float32 matrix instruction)
+    products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1, 512], 48, 10_485_760,
+             matrix_peak=MFMA_F32_PEAK_TFLOPS)
     products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 2048], 0, WEIGHT_BYTES,
              weights=qs)
     products("C4 bf16 3-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 3), torch.bfloat16, _lib.BF16, [1, 16, 512], 48,

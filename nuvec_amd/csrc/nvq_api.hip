@@ -530,11 +530,12 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
 }
 
 // The kernel family of a product (the counterpart of the routing in GpuEval::quantized_matmul, gpu.rs:6934-7168).
-enum class Route { kUntransposed, kVector, kTiled, kFewRowsDirect, kFewRows };
+enum class Route { kUntransposed, kVector, kTiled, kTiledF32, kFewRowsDirect, kFewRows };
 
 static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     if (!d->transpose) return Route::kUntransposed;        // weights stored [K, N]
     if (a.row_exact) return Route::kVector;                // the vector kernels: a row's bits do not depend on its neighbours
+    if (qmm_f32_takes(a)) return Route::kTiledF32;         // float32, many rows: the float32 matrix instruction
     if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;  // (also passes of 16 rows of small matrices, ahead of the tiles)
     if (takes_tiled(d, a)) return Route::kTiled;
     // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the
@@ -573,6 +574,7 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     switch (pick_route(d, a)) {
     case Route::kUntransposed: return launch_qvm(a, workspace, (hipStream_t)stream);
     case Route::kTiled: return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
+    case Route::kTiledF32: return launch_qmm_f32(a, (hipStream_t)stream);
     case Route::kFewRowsDirect: return launch_qmd(a, (hipStream_t)stream);
     case Route::kFewRows: return launch_qmf(a, (hipStream_t)stream);
     default: return launch_qmv(a, (hipStream_t)stream);
@@ -589,6 +591,7 @@ const char *nvq_quantized_matmul_route(const nvq_qmm_desc *d) {
     switch (pick_route(d, a)) {
     case Route::kUntransposed: return qvm_kernel_name(a);
     case Route::kTiled: return "qmm_kernel";
+    case Route::kTiledF32: return "qmm_f32_kernel";
     case Route::kFewRowsDirect: return "qmd_kernel";
     case Route::kFewRows: return "qmf_kernel";
     default: return qmv_kernel_name(a);

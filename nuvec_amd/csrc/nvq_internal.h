@@ -123,6 +123,9 @@ bool qmm_supported(const ProductArgs &a);
 size_t qmm_workspace_bytes(const ProductArgs &a);  // float32 partial sums when K is split over the grid, else 0
 int32_t launch_qmm(const ProductArgs &a, void *workspace, hipStream_t s);  // workspace NULL: no split
 double qmm_estimate_us(const ProductArgs &a);  // estimated duration of the tiled kernel with its better tile
+// float32 products of many rows on v_mfma_f32_32x32x2_f32 (affine codes, weights stored [N, K]).
+bool qmm_f32_takes(const ProductArgs &a);
+int32_t launch_qmm_f32(const ProductArgs &a, hipStream_t s);
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).
 bool qmf_supported(const ProductArgs &a);
 int32_t launch_qmf(const ProductArgs &a, hipStream_t s);

@@ -309,7 +309,7 @@ def test_rows_of_few_outputs_take_the_cpu_weights(dtype):
     cases = [(5, 200, 1024, 4, 64, True, "qmf_kernel"), (1, 100, 4096, 4, 64, True, "qmv_lds_kernel"), (3, 64, 480, 8, 32, True, "qmv_lds_kernel"),
              (2048, 768, 512, 4, 64, True, "qmm_kernel"), (300, 640, 1024, 4, 64, True, None), (260, 257, 192, 3, 64, True, None), (16, 48, 1536, 8, 128, True, "qmf_kernel"),
              (40, 384, 256, 4, 64, False, "qmn_kernel"), (130, 992, 192, 8, 32, False, "qmn_kernel"), (7, 256, 200, 4, 64, False, "qvm_kernel"),
-             (9, 128, 320, 6, 64, False, "qvm_kernel")]
+             (9, 128, 320, 6, 64, False, "qmn_kernel")]
     for m, n, k, bits, group, transpose, kernel in cases:
         w = make_w(rng, n, k, dtype) if transpose else make_w(rng, k, n, dtype)
         x = make_x(rng, m, k, dtype)
