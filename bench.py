@@ -273,6 +273,8 @@ def all_configs(lib, device, qs):
              matrix_peak=MFMA_F32_PEAK_TFLOPS)
     products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 2048], 0, WEIGHT_BYTES,
              weights=qs)
+    # Beside C2: the same layer's down projection, whose rows are K = 14336 long
+    products("beside C2: bf16 4-bit g64 W[4096,14336]", 4096, 14336, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1], 24, WEIGHT_BYTES)
     products("C4 bf16 3-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 3), torch.bfloat16, _lib.BF16, [1, 16, 512], 48,
              7_340_032)
     products("C4 bf16 8-bit g32 W[4096,4096]", 4096, 4096, nv.Quant.affine(32, 8), torch.bfloat16, _lib.BF16, [1, 16, 512], 32,

@@ -1,4 +1,4 @@
-// One row of x against 4-bit affine weights, bf16 / f16, K = 2048 or 4096: the decode product y[1,N] = x . dequantize(w)^T
+// One row of x against 4-bit affine weights, bf16 / f16, K in whole chunks of 2048 up to 14336: the decode product y[1,N] = x . dequantize(w)^T
 // with the integer dot-product instruction.  Values follow nuvec's CPU product (reference:
 // crates/nuvec-core/src/kernels.rs:1091-1142) within the stated tolerance, in the factored form of the reference's device
 // kernels, scale * sum(x * code) + bias * sum(x) per group (crates/nuvec-kernels/src/metal/quantized.h:247-360, 876-988).
@@ -36,7 +36,6 @@ namespace nvq {
 namespace {
 
 constexpr int kWaves = 8;       // wavefronts of a block
-constexpr int kAhead = 2;       // rows whose loads run ahead of the arithmetic
 constexpr int kLimbBits = 16;   // x in fixed point: four nibbles, offset 2^15
 
 template <int... I, class F>
@@ -114,7 +113,10 @@ __device__ __forceinline__ void to_limbs(const uint4 piece, uint4 &limbs, float 
 // Grid: (blocks of 8 R weight rows, groups of MX rows of x).
 template <typename T, int S, int R, int MX>
 __global__ void __launch_bounds__(kWaves * 64) qmv4_dot8_kernel(const ProductArgs a) {
-    static_assert(R >= 1 && R <= 8 && S >= 1 && MX >= 1 && MX <= 4, "one batched reduction of up to eight rows per row of x");
+    static_assert(R >= 1 && R <= 8 && S >= 1 && S <= 7 && MX >= 1 && MX <= 4, "one batched reduction of up to eight rows per row of x");
+    // Rows whose loads run ahead of the arithmetic: two; one where a row is 4 KB and more per wavefront (a row ahead then
+    // already keeps 8 x 4 KB per compute unit under way, and the registers hold the limbs of a long x).
+    constexpr int kAhead = S >= 4 ? 1 : 2;
     constexpr int kRowPieces = S * 256;                    // 16-byte pieces of a row of x
     constexpr int kPieces = MX * kRowPieces;
     constexpr int kPerThread = (kPieces + 511) / 512;
@@ -286,13 +288,16 @@ int qmv_dot8_rows_per_wave(int64_t n, int cus) {
 }
 
 // What the kernel takes: single products (no batch, no gathered pairs, no gated epilogue) of 4-bit affine weights stored
-// [N, K] with K = 2048 or 4096, bf16 / f16, 1024 outputs and more (rows of fewer outputs materialise the CPU's weights
+// [N, K] with K = 2048, 4096 (several rows of x) or 6144 .. 14336 (one row), bf16 / f16, 1024 outputs and more (rows of fewer outputs materialise the CPU's weights
 // elsewhere), operands 16-byte aligned.  One row of x (two against 8192 weight rows and more) in one pass over the
 // weights, or the rows of a row-exact product four per pass: every row has the bits of its one-row product either way.
 bool qmv_dot8_takes(const ProductArgs &a) {
     if (a.mode != NVQ_AFFINE || a.bits != 4 || (a.dtype != NVQ_BF16 && a.dtype != NVQ_F16)) return false;
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.glu != 0 || a.exact_weights) return false;
-    if (a.k != 2048 && a.k != 4096) return false;
+    // K in whole chunks of 2048 up to 14336 (us against the float decode kernel: W[4096,14336] 8.85 -> 8.26, W[14336,8192]
+    // 13.6 -> 12.1, W[8192,6144] 7.9 -> 6.3; at K = 16384 the limbs no longer fit the registers: 10.5 -> 12.4, not taken)
+    if (a.k < 2048 || a.k > 14336 || a.k % 2048 != 0) return false;
+    if (a.k > 4096 && a.m != 1) return false;  // (the limbs of one long row of x fill the registers)
     if (a.group != 32 && a.group != 64 && a.group != 128) return false;
     if (a.n < 1024 || a.n > 0x7FFFFFFF / 128 || a.m < 1 || a.m > 65535) return false;
     // two rows where the matrix is large (W[14336,4096]: 8.7 us against 9.8 on the 16x16x32 decode kernel; three and four rows
@@ -301,11 +306,24 @@ bool qmv_dot8_takes(const ProductArgs &a) {
     return ((uintptr_t)a.w | (uintptr_t)a.x) % 16 == 0;
 }
 
+template <typename T>
+int32_t run_chunks(const ProductArgs &a, int r, hipStream_t s) {
+    switch (a.k / 2048) {
+    case 1: return run_x_rows<T, 1>(a, r, s);
+    case 2: return run_x_rows<T, 2>(a, r, s);
+    // longer rows (K = 6144 .. 14336): one row of x per pass
+    case 3: return run_rows<T, 3, 1>(a, r, s);
+    case 4: return run_rows<T, 4, 1>(a, r, s);
+    case 5: return run_rows<T, 5, 1>(a, r, s);
+    case 6: return run_rows<T, 6, 1>(a, r, s);
+    default: return run_rows<T, 7, 1>(a, r, s);
+    }
+}
+
 int32_t launch_qmv_dot8(const ProductArgs &a, hipStream_t s) {
     if (!qmv_dot8_takes(a)) return fail(NVQ_UNSUPPORTED, "quantized_matmul: the integer decode kernel does not take this product");
     const int r = qmv_dot8_rows_per_wave(a.n, compute_units());
-    if (a.dtype == NVQ_BF16) return a.k == 4096 ? run_x_rows<bf16_t, 2>(a, r, s) : run_x_rows<bf16_t, 1>(a, r, s);
-    return a.k == 4096 ? run_x_rows<f16_t, 2>(a, r, s) : run_x_rows<f16_t, 1>(a, r, s);
+    return a.dtype == NVQ_BF16 ? run_chunks<bf16_t>(a, r, s) : run_chunks<f16_t>(a, r, s);
 }
 
 }  // namespace nvq

@@ -1,5 +1,5 @@
-"""The integer dot-product decode kernel (`qmv4_dot8_kernel`): one row of x against 4-bit affine weights with K = 2048 or
-4096, the reference's `qmv_fast` shape (crates/nuvec-kernels/src/metal/quantized.h:876-988, routed at
+"""The integer dot-product decode kernel (`qmv4_dot8_kernel`): one row of x against 4-bit affine weights with K in whole
+chunks of 2048 up to 14336, the reference's `qmv_fast` shape (crates/nuvec-kernels/src/metal/quantized.h:876-988, routed at
 crates/nuvec-core/src/gpu.rs:7025-7060).  x enters as 16-bit fixed point per slice of 32 values, so the tests hold the
 values to the CPU's product like every other kernel's (every output within the bar of its row, and within half of it
 against the device arithmetic) and then press on what fixed point could break: slices whose values span many binades,
@@ -26,7 +26,8 @@ def product(x, w, dtype, group, **kw):
 
 @pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
 @pytest.mark.parametrize("n,k,group", [(14336, 4096, 64), (4096, 4096, 64), (4096, 2048, 64), (1024, 4096, 32), (11008, 4096, 128),
-                                       (2049, 2048, 128), (1031, 4096, 64), (5000, 2048, 32), (28672, 4096, 64), (16400, 2048, 64)])
+                                       (2049, 2048, 128), (1031, 4096, 64), (5000, 2048, 32), (28672, 4096, 64), (16400, 2048, 64),
+                                       (4096, 14336, 64), (4096, 8192, 64), (1032, 6144, 128), (5120, 12288, 32), (2048, 10240, 64)])
 def test_values_against_the_cpu_product(dtype, n, k, group):
     """Rows that fill the blocks and rows that do not (N off 8 R for every R the host picks), both K, the three groups."""
     rng = np.random.default_rng(n + k + group)

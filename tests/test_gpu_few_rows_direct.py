@@ -32,7 +32,9 @@ def test_routes_of_the_baseline_configurations():
     assert c2(2048) == "qmm_kernel"
     # row-exact rows take the kernel of the one-row product, each row as its own pass
     assert c2(8, row_exact=True) == "qmv4_dot8_kernel" and c2(300, rows=True) == "qmv4_dot8_kernel"
-    assert ops.quantized_matmul_route(1, 14336, 8192, nv.Quant.affine(64, 4), bf16) == "qmv4_lds_kernel"  # (K beyond 4096)
+    assert ops.quantized_matmul_route(1, 14336, 8192, nv.Quant.affine(64, 4), bf16) == "qmv4_dot8_kernel"  # (K in chunks of 2048 up to 14336)
+    assert ops.quantized_matmul_route(1, 14336, 16384, nv.Quant.affine(64, 4), bf16) == "qmv4_lds_kernel"
+    assert ops.quantized_matmul_route(2, 14336, 8192, nv.Quant.affine(64, 4), bf16) != "qmv4_dot8_kernel"  # (one row of x only beyond 4096)
     for group, bits in ((64, 3), (32, 8)):
         c4 = lambda m, **kw: ops.quantized_matmul_route(m, 4096, 4096, nv.Quant.affine(group, bits), bf16, **kw)
         assert c4(1) == "qmv4_lds_kernel"  # (the decode kernel takes a row of 3- and of 8-bit codes too)
