@@ -30,6 +30,33 @@ def test_every_width_against_the_cpu_product(bits, group):
         assert_rows_close(got, want, ref.F32, f"float32 rows b{bits} g{group} M={m} N={n} K={k}")
 
 
+@pytest.mark.parametrize("mode,qmode", [(ref.MXFP4, "MXFP4"), (ref.MXFP8, "MXFP8"), (ref.NVFP4, "NVFP4")])
+def test_block_formats_against_the_cpu_product(mode, qmode):
+    """The block formats (the reference instantiates them for float32 as well, crates/nuvec-kernels/src/metal/fp_quantized.metal:105-107):
+    decoded code times decoded scale in float32; NVFP4 also with a global scale (kernels.rs:992-998)."""
+    rng = np.random.default_rng(5400 + mode)
+    group, bits = ref.FP_PARAMS[mode]
+    quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
+    for m, n, k in ((300, 1000, 1024), (70, 4100, 512), (2048, 320, 256)):
+        assert ops.quantized_matmul_route(m, n, k, quant, torch.float32) == "qmm_f32_kernel", (m, n, k)
+        w, x = make_w(rng, n, k, ref.F32), make_x(rng, m, k, ref.F32)
+        packed, scales = ref.fp_quantize(w, ref.F32, mode)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+        want = ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=ref.F32, threads=8)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, ref.F32, f"float32 rows {qmode} M={m} N={n} K={k}", exact_weights=True)
+    if mode == ref.NVFP4:
+        m, n, k, g = 300, 1000, 1024, 3.25
+        w, x = make_w(rng, n, k, ref.F32), make_x(rng, m, k, ref.F32)
+        gs = torch.tensor(g, dtype=torch.float32, device="cuda")
+        q = nv.quantize(to_dev(w), nv.QuantMode.NVFP4, gs)
+        packed, scales = ref.fp_quantize(w, ref.F32, ref.NVFP4, g)
+        assert np.array_equal(to_host(q.weight), packed) and np.array_equal(to_host(q.scales), scales)
+        want = ref.fp_quantized_matmul_scaled(x, packed, scales, ref.NVFP4, ref.F32, g)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        assert_rows_close(got, want, ref.F32, "float32 rows NVFP4 with a global scale", exact_weights=True)
+
+
 def test_routes_and_what_stays_on_the_vector_kernel():
     """The rule is an estimate of both kernels: few rows, row-exact products, K off whole steps of 64 and batches stay
     where they were."""
@@ -41,7 +68,8 @@ def test_routes_and_what_stays_on_the_vector_kernel():
     assert route(512, 4096, 4096, rows=True) == "qmv_lds_kernel"
     assert ops.quantized_matmul_route(512, 4096, 4096 + 32, nv.Quant.affine(32, 4), torch.float32) == "qmv_lds_kernel"
     assert route(512, 4096, 4096, batch=2) == "qmv_lds_kernel"
-    assert ops.quantized_matmul_route(512, 4096, 4096, nv.Quant.new(nv.QuantMode.MXFP4), torch.float32) == "qmv_lds_kernel"
+    assert ops.quantized_matmul_route(512, 4096, 4096, nv.Quant.new(nv.QuantMode.MXFP4), torch.float32) == "qmm_f32_kernel"
+    assert ops.quantized_matmul_route(4, 4096, 4096, nv.Quant.new(nv.QuantMode.MXFP4), torch.float32) == "qmv_lds_kernel"
 
 
 def test_bias_epilogue_determinism_and_the_vector_kernel():
