@@ -667,7 +667,7 @@ __global__ void __launch_bounds__(WAVES * 64) qmv4_lds_kernel(const ProductArgs 
 // ── The same for short rows: K up to 2048 ──────────────────────────────────────────────────────────────
 // The decode kernel above gives a weight row to a wavefront, 32 values a lane: a row of K < 2048 values leaves lanes
 // (and the second of its two loads) without work.  Here a row takes L lanes, L the power of two that covers K / 32
-// (8 to 64), so a wavefront holds 64 / L rows at once and two such sets in flight; x (all of K) is staged once per
+// (2 to 64), so a wavefront holds 64 / L rows at once and two such sets in flight; x (all of K) is staged once per
 // block, and the L partial sums of a row are added with a butterfly of cross-lane moves inside its L lanes.
 template <typename T, int RM, int L, bool BATCHED, int MODE>
 __global__ void __launch_bounds__(512) qmv4_short_kernel(const ProductArgs a) {
@@ -1352,8 +1352,13 @@ inline bool block_decode_takes(const ProductArgs &a) {
 // 54.5 -> 34.9; MXFP4 W[2048,768] 24.8 -> 11.3, W[2048,1024] 24.7 -> 11.9, W[2048,2048] 25.4 -> 19.8, W[4096,1408]
 // 46.1 -> 32.3; MXFP8 W[2048,1024] 25.6 -> 18.0.  Where the 16x16x32 decode kernel takes affine pairs it stays ahead
 // (W[2048,1024] 11.2 against 12.7, W[2048,2048] 16.5 against 21.4), and single products gain nothing (a launch either way).
+// Single products take it too where a row is at most 512 values (the reference's qmv_quad shapes, K = 64 and 128,
+// crates/nuvec-kernels/src/metal/quantized.h:819-874, and up to 16 lanes a row): a wavefront per row leaves 48 to 62
+// of its lanes idle there (us, one / four rows of x, 4-bit g64 bf16: W[32768,128] 10.9 / 24.8, W[131072,128] 38.7 / 90.2
+// on the decode kernel).
 inline bool short_decode_takes(const ProductArgs &a) {
-    if (a.rhs == nullptr || a.dtype == NVQ_F32 || a.row_exact || a.k > 2048 || a.k % 32 != 0 || a.m < 1 || a.m > 4) return false;
+    if (a.dtype == NVQ_F32 || a.row_exact || a.k > 2048 || a.k % 32 != 0 || a.m < 1 || a.m > 4) return false;
+    if (a.rhs == nullptr && (a.k > 512 || a.batch != 1 || a.batch_ndim != 0 || a.glu != 0)) return false;
     if (a.mode != NVQ_AFFINE) return block_decode_takes(a);
     return a.bits == 4 && !a.exact_weights && !d16_takes(a) && (uintptr_t)a.w % 16 == 0 && (uintptr_t)a.x % 16 == 0;
 }
@@ -1374,6 +1379,9 @@ int32_t run_short_lanes(const ProductArgs &a, hipStream_t s) {
 template <typename T, int MODE>
 int32_t run_short(const ProductArgs &a, hipStream_t s) {
     const int slices = (int)(a.k / 32);
+    if (slices <= 2) return run_short_lanes<T, MODE, 2>(a, s);
+    if (slices <= 4) return run_short_lanes<T, MODE, 4>(a, s);
+    if (slices <= 8) return run_short_lanes<T, MODE, 8>(a, s);
     if (slices <= 16) return run_short_lanes<T, MODE, 16>(a, s);
     if (slices <= 32) return run_short_lanes<T, MODE, 32>(a, s);
     return run_short_lanes<T, MODE, 64>(a, s);

@@ -134,3 +134,22 @@ def test_bias_epilogue_and_repeatability():
     from nuvec_amd.layers import QuantizedLinear
     layer = QuantizedLinear(q.weight, q.scales, q.biases, bias, q.quant)
     assert torch.equal(layer(xd), plain + bias)
+
+
+@pytest.mark.parametrize("dtype", [ref.BF16, ref.F16])
+@pytest.mark.parametrize("k,group", [(64, 64), (128, 32), (128, 128), (256, 64), (512, 64), (96, 32)])
+def test_short_rows_of_single_products(dtype, k, group):
+    """Rows of at most 512 values (the reference's `qmv_quad` shapes K = 64 and 128,
+    crates/nuvec-kernels/src/metal/quantized.h:819-874, and up to sixteen lanes a row): single products take the short-row
+    decode kernel, 2 to 16 lanes a weight row, one to four rows of x; rows off the block size."""
+    rng = np.random.default_rng(600 + k + group)
+    quant = nv.Quant.affine(group, 4)
+    for m, n in ((1, 32768), (4, 5000), (3, 1031), (2, 2048)):
+        assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmv4_short_kernel", (m, n, k)
+        w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+        got, (packed, scales, biases) = product(x, w, dtype, group)
+        want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=4, dtype=dtype, threads=8)
+        what = f"short rows g{group} M={m} N={n} K={k}"
+        assert_rows_close(got, want, dtype, what)
+        assert_device_arithmetic(got, x, packed, scales, biases, group, 4, dtype, what, limit=0.8)
+    assert ops.quantized_matmul_route(1, 32768, 1024, quant, TORCH[dtype]) != "qmv4_short_kernel" or group != 64  # (longer rows: the other decode kernels)

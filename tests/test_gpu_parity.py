@@ -671,7 +671,8 @@ def test_block_formats_on_the_decode_kernel(mode, qmode, dtype):
     group, bits = ref.FP_PARAMS[mode]
     quant = nv.Quant.new(getattr(nv.QuantMode, qmode))
     for m, n, k in [(1, 203, 32), (1, 1000, 2880), (2, 77, 4096 + 96), (3, 130, 1024), (4, 61, 2880), (1, 48, 14336), (2, 1030, 8192), (4, 96, 224)]:
-        assert nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmv4_lds_kernel", (qmode, m, n, k)
+        # (rows of at most 512 values take the short-row form of the same arithmetic: several weight rows a wavefront)
+        assert nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == ("qmv4_short_kernel" if k <= 512 else "qmv4_lds_kernel"), (qmode, m, n, k)
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
         packed, scales = ref.fp_quantize(w, dtype, mode)
         q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
@@ -807,18 +808,20 @@ def test_block_formats_at_every_scale_code(mode, qmode, dtype):
         worst = np.unravel_index(np.argmax(ratio), ratio.shape)
         assert ratio[worst] <= 1.0, f"{what} scale code {codes[live][worst[1]]}: {ratio[worst]:.3f} x the bound"
 
-    # weights stored [N, K]: row n of the weight carries code n
-    w = make_w(rng, n, k, dtype)
-    packed, _ = ref.fp_quantize(w, dtype, mode)
-    scales = np.repeat(codes[:, None], k // group, axis=1)
-    q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
-    for m in (1, 3, 8, 40, 300):
-        x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32) * x_scale, dtype)
-        want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8), dtype)
-        got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q)), dtype)
-        routes.add(nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]))
-        compare(got, want, f"{qmode} M={m}")
-    assert {"qmv4_lds_kernel", "qmd_kernel"} <= routes and len(routes) >= 3, routes
+    # weights stored [N, K]: row n of the weight carries code n (rows of 512 values: the short-row decode kernel at one
+    # and three rows of x; rows of 1024: the decode kernel)
+    for k in (512, 1024):
+        w = make_w(rng, n, k, dtype)
+        packed, _ = ref.fp_quantize(w, dtype, mode)
+        scales = np.repeat(codes[:, None], k // group, axis=1)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), None, quant)
+        for m in ((1, 3, 8, 40, 300) if k == 512 else (1, 2)):
+            x = ref.from_f32(rng.standard_normal((m, k)).astype(np.float32) * x_scale, dtype)
+            want = ref.to_f32(ref.quantized_matmul(x, packed, scales, None, mode=mode, group=group, bits=bits, dtype=dtype, threads=8), dtype)
+            got = ref.to_f32(to_host(nv.quantized_matmul(to_dev(x), q)), dtype)
+            routes.add(nv.quantized_matmul_route(m, n, k, quant, TORCH[dtype]))
+            compare(got, want, f"{qmode} M={m} K={k}")
+    assert {"qmv4_lds_kernel", "qmv4_short_kernel", "qmd_kernel"} <= routes and len(routes) >= 4, routes
 
     # weights stored [K, N]: the groups run along N, so every column of group n carries code n; the matrix-core kernel
     # and the kernel of few rows
