@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(HERE, "..", "include")
 LIB = os.path.join(HERE, "libnuvec_hip.so")
-SOURCES = ["qmf_b8.hip", "qmf_fp8.hip", "qmf_b6.hip", "qmf_b5.hip", "qmf_b4.hip", "qmf_fp4.hip", "qmf_nvfp4.hip", "qmf_b3.hip", "qmf_b2.hip", "qmf_b1.hip", "qmm.hip", "qmv.hip", "qmv_dot8.hip", "qmm_f32.hip",
+SOURCES = ["qmf_b8.hip", "qmf_fp8.hip", "qmf_b6.hip", "qmf_b5.hip", "qmf_b4.hip", "qmf_fp4.hip", "qmf_nvfp4.hip", "qmf_b3.hip", "qmf_b2.hip", "qmf_b1.hip", "qmm.hip", "qmv.hip", "qmv_dot8.hip", "qmm_f32.hip", "qmr.hip",
            "qvm.hip", "nvq_api.hip", "affine_quant.hip", "fp_quant.hip", "qmf.hip", "gather.hip", "repack.hip", "calib.hip", "qattn.hip", "qmd.hip", "glu.hip"]  # slowest to compile first
 
 # -ffp-contract=off: the quantizers must round every operation as the CPU does; fused

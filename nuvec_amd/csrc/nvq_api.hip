@@ -248,6 +248,17 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     }
 }
 
+// Whether a product takes the batched-decode kernel: 33 to 64 rows of x against at least 11008 weight rows and K from
+// 4096, where its one pass over the weights beats the passes of 16 rows of the few-row kernel and the tiles of the
+// tiled one.  Measured (bf16, 4 bits in groups of 64, us, new / old): W[14336,4096] 48 rows 24.1 / 30.5, 64 rows 24.0 / 34.1
+// (f16: 33 rows 22.9 / 28.9); W[11008,4096] 40 / 64 rows 23.2 / 26.8, 23.3 / 29.8; W[16384,4096] 23.3 / 31.7, 23.7 / 35.1;
+// W[22016,4096] 43.4 / 46.6; W[32768,4096] 47.6 / 52.9; W[14336,8192] 40.9 / 50.1, 42.6 / 51.9; W[28672,8192] 83.8 / 93.3.  It
+// loses below: W[8192,4096] 23.0 against 18.7, W[8192,8192] 36.0 / 30.4, W[14336,4096] at 32 rows 20.2 / 18.7, at 128 rows
+// (two passes) 44.2 / 35.0, W[14336,2048] a tie.
+static bool takes_batched_decode(const nvq::ProductArgs &a) {
+    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.k >= 4096 && nvq::qmr_supported(a);
+}
+
 // The kernels' view of a product descriptor.
 // Which half-precision affine products materialise the CPU's weights, round(round(code * scale) + bias)
 // (kernels.rs:835-859), bit for bit, instead of the one rounding of fma(code, scale, bias) the device kernels give a
@@ -518,6 +529,10 @@ static bool takes_tiled(const nvq_qmm_desc *d, const ProductArgs &a) {
     return item > 16 && qmm_supported(a) && (!qmf_supported(a) || tiled_is_faster(a));
 }
 
+// The kernel family of a product (the counterpart of the routing in GpuEval::quantized_matmul, gpu.rs:6934-7168).
+enum class Route { kUntransposed, kVector, kTiled, kTiledF32, kBatchedDecode, kFewRowsDirect, kFewRows };
+static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a);
+
 size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
     if (check_qmm(d, "quantized_matmul") != NVQ_OK) return 0;
     int64_t batch = 1;
@@ -526,16 +541,14 @@ size_t nvq_quantized_matmul_workspace_bytes(const nvq_qmm_desc *d) {
     const ProductArgs a = product_args(d, batch);
     // float32 partial sums of the splits of K: weights stored [K, N], or few tiles of a long K
     if (!d->transpose) return qvm_workspace_bytes(a);
-    return !a.row_exact && takes_tiled(d, a) ? qmm_workspace_bytes(a) : 0;
+    return pick_route(d, a) == Route::kTiled ? qmm_workspace_bytes(a) : 0;
 }
-
-// The kernel family of a product (the counterpart of the routing in GpuEval::quantized_matmul, gpu.rs:6934-7168).
-enum class Route { kUntransposed, kVector, kTiled, kTiledF32, kFewRowsDirect, kFewRows };
 
 static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     if (!d->transpose) return Route::kUntransposed;        // weights stored [K, N]
     if (a.row_exact) return Route::kVector;                // the vector kernels: a row's bits do not depend on its neighbours
     if (qmm_f32_takes(a)) return Route::kTiledF32;         // float32, many rows: the float32 matrix instruction
+    if (takes_batched_decode(a)) return Route::kBatchedDecode;
     if (takes_few_rows_direct(a)) return Route::kFewRowsDirect;  // (also passes of 16 rows of small matrices, ahead of the tiles)
     if (takes_tiled(d, a)) return Route::kTiled;
     // Up to four rows of 4-bit affine weights (up to eight where the 16x16x32 decode kernel takes the product): the
@@ -575,6 +588,7 @@ static int32_t quantized_matmul_any(const nvq_qmm_desc *d, const void *x, const 
     case Route::kUntransposed: return launch_qvm(a, workspace, (hipStream_t)stream);
     case Route::kTiled: return launch_qmm(a, workspace, (hipStream_t)stream);  // without a workspace: K is not split
     case Route::kTiledF32: return launch_qmm_f32(a, (hipStream_t)stream);
+    case Route::kBatchedDecode: return launch_qmr(a, (hipStream_t)stream);
     case Route::kFewRowsDirect: return launch_qmd(a, (hipStream_t)stream);
     case Route::kFewRows: return launch_qmf(a, (hipStream_t)stream);
     default: return launch_qmv(a, (hipStream_t)stream);
@@ -592,6 +606,7 @@ const char *nvq_quantized_matmul_route(const nvq_qmm_desc *d) {
     case Route::kUntransposed: return qvm_kernel_name(a);
     case Route::kTiled: return "qmm_kernel";
     case Route::kTiledF32: return "qmm_f32_kernel";
+    case Route::kBatchedDecode: return "qmr_kernel";
     case Route::kFewRowsDirect: return "qmd_kernel";
     case Route::kFewRows: return "qmf_kernel";
     default: return qmv_kernel_name(a);

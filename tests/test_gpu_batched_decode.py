@@ -1,0 +1,75 @@
+"""Batched decode (`qmr_kernel`): 33 to 64 rows of x against 4-bit affine weights stored [N, K] with many rows, every
+weight fetched and dequantized once.  The reference takes these row counts on its tiled kernel
+(crates/nuvec-core/src/gpu.rs:6975-7060, crates/nuvec-kernels/src/metal/quantized.h:1358-1485); the values are held to the
+CPU product (crates/nuvec-core/src/kernels.rs:1091-1142) at the bar of the element type (1e-2 of a row's largest output
+in bfloat16, 1e-3 in float16) and to the device arithmetic of a once-rounded weight at half of it."""
+import numpy as np
+import pytest
+import torch
+
+import nuvec_amd as nv
+from nuvec_amd import ops
+from oracle import ref
+from tests.hip_backend import to_dev, to_host
+from tests.test_gpu_parity import assert_device_arithmetic, assert_rows_close, make_w, make_x
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {ref.BF16: torch.bfloat16, ref.F16: torch.float16}
+
+
+# Whole tiles and tails: rows of x off the pass of 64, weight rows off the block of 64 and off the 16-byte stores of y,
+# K whose chunks of 512 do not divide among the four wavefronts (9 and 10 chunks), every group size, both element types.
+@pytest.mark.parametrize("dtype,group,m,n,k", [
+    (ref.BF16, 64, 64, 11008, 4096),
+    (ref.BF16, 64, 33, 11017, 4096),
+    (ref.F16, 32, 50, 11040, 4608),
+    (ref.BF16, 128, 47, 11072, 5120),
+    (ref.F16, 128, 64, 12288, 4096),
+])
+def test_against_the_cpu_product(dtype, group, m, n, k):
+    rng = np.random.default_rng(6100 + group + m)
+    quant = nv.Quant.affine(group, 4)
+    assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmr_kernel"
+    w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, 4)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=4, dtype=dtype, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    what = f"batched decode g{group} M={m} N={n} K={k}"
+    assert_rows_close(got, want, dtype, what)
+    assert_device_arithmetic(got, x, packed, scales, biases, group, 4, dtype, what)
+
+
+def test_routes():
+    """The rule is measured: 33 to 64 rows, at least 11008 weight rows, K from 4096 in chunks of 512, 4 bits, one
+    product; everything else stays where it was."""
+    q4 = nv.Quant.affine(64, 4)
+    route = lambda m, n, k, quant=q4, dtype=torch.bfloat16, **kw: ops.quantized_matmul_route(m, n, k, quant, dtype, **kw)
+    assert route(33, 14336, 4096) == "qmr_kernel" and route(64, 14336, 4096) == "qmr_kernel"
+    assert route(64, 14336, 4096, dtype=torch.float16) == "qmr_kernel" and route(48, 28672, 8192) == "qmr_kernel"
+    assert route(32, 14336, 4096) != "qmr_kernel" and route(65, 14336, 4096) != "qmr_kernel"
+    assert route(64, 8192, 4096) != "qmr_kernel" and route(64, 14336, 2048) != "qmr_kernel"
+    assert route(64, 14336, 4096 + 256) != "qmr_kernel"  # K off the chunks of 512
+    assert route(64, 14336, 4096, nv.Quant.affine(64, 8)) != "qmr_kernel"
+    assert route(64, 14336, 4096, nv.Quant.new(nv.QuantMode.MXFP4)) != "qmr_kernel"
+    assert route(64, 14336, 4096, dtype=torch.float32) != "qmr_kernel"
+    assert route(64, 14336, 4096, batch=2) != "qmr_kernel"
+    assert route(64, 14336, 4096, rows=True) != "qmr_kernel"
+
+
+def test_bias_epilogue_and_determinism():
+    """QuantizedLinear's bias in the epilogue is the separate addition bit for bit (crates/nuvec-nn/src/layers.rs:155-162),
+    and two launches give the same bits (the wavefronts' partial tiles are added in a fixed order)."""
+    rng = np.random.default_rng(6200)
+    m, n, k = 40, 11008, 4096
+    quant = nv.Quant.affine(64, 4)
+    w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+    q = nv.quantize(to_dev(w), quant)
+    xd = to_dev(x)
+    bias = (torch.randn(n, device="cuda") * 0.5).to(torch.bfloat16)
+    plain = nv.quantized_matmul(xd, q)
+    again = nv.quantized_matmul(xd, q)
+    assert torch.equal(plain.view(torch.int16), again.view(torch.int16))
+    fused = nv.quantized_matmul(xd, q, bias=bias)
+    assert torch.equal(fused.view(torch.int16), (plain + bias).view(torch.int16))

@@ -53,7 +53,8 @@ def test_routes_of_the_baseline_configurations():
     assert small(64) == "qmd_kernel" and small(192) == "qmd_kernel" and small(512) in ("qmf_kernel", "qmm_kernel")
     assert small(16, bf16) == "qmd_kernel" and small(64, bf16) in ("qmf_kernel", "qmm_kernel") and small(192, bf16) in ("qmf_kernel", "qmm_kernel")
     assert ops.quantized_matmul_route(64, 8192, 4096, nv.Quant.affine(64, 4), bf16) == "qmd_kernel"
-    assert c2(64) == "qmd_kernel" and c2(96) == "qmm_kernel"
+    assert c2(32) == "qmd_kernel" and c2(96) == "qmm_kernel"
+    assert c2(33) == "qmr_kernel" and c2(64) == "qmr_kernel"  # (one pass over this many weight rows: the batched-decode kernel)
     # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
     for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (30, 64, 128, 64, 4), (20, 1000, 1024, 64, 6)):
         assert ops.quantized_matmul_route(m, n, k, nv.Quant.affine(group, bits), bf16) == "qmf_kernel", (m, n, k, group, bits)
