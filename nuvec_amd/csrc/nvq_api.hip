@@ -168,20 +168,26 @@ int32_t check_product_dims(const char *op, const nvq_quant &q, int32_t transpose
 
 using namespace nvq;
 
-// Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row
-// kernel runs a block (one per compute unit) per pass of 32 rows and 64 weight rows - 32 weight rows where that leaves
-// fewer than 192 blocks (qmf::row_groups) -, a round of blocks on the chip taking about 5.0 (4.4) us per 1024 values of
-// K, never under 4 us.  Measured at W[2880,2880], 4 bits: 64 / 128 / 256 / 512 rows 13.1 / 25.0 / 32.4 / 48.2 us (180
-// blocks of 32 weight rows in one round; 360 of 32 in two; 360 of 64 in two; 720 in three) against 18.7 / 22.7 / 37.1 us
-// of the tiled kernel at 192 / 384 / 1024 rows.  The counterpart of the reference's device-specific `qmv_batch_limit`
-// (crates/nuvec-core/src/gpu.rs:1506-1538).
+// Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row kernel
+// runs a block (one per compute unit) per pass of 32 rows and 64 weight rows - 32 weight rows where that leaves fewer
+// than 192 blocks (qmf::row_groups).  A round of blocks on the chip costs a fixed part (the tables of scales, the sum of
+// eight wavefronts' partial tiles) and a part per value of K: fitted to W[2880,2880] at 64 / 128 / 256 / 512 rows
+// (13.1 / 25.0 / 32.4 / 48.2 us: one round of 32 weight rows, two of 32, two of 64, three of 64), W[4096,1024] at 64 rows
+// 13.2 (one round of 32), at 128 / 256 rows with the CPU's weights 24.7 / 47.3 (one and two rounds of 64; with one
+// rounding 13.6 a round), W[2048,2048] 64 / 128 rows 12.7 / 13.0, W[4096,512] 64 rows 9.0.  The tiled kernel of few tiles
+// takes 4.5 us more than its estimate of the steps and the second kernel that adds the splits of K, and was never under
+// 11.7 us: W[4096,512] at 128 rows 11.7 (few-row kernel 17.2), W[4096,1024] at 64 / 96 / 256 rows 15.1 / 15.7 / 20.0
+// (13.1 / 24.3 / 47.2), W[2048,2048] at 64 / 256 rows 16.0 / 17.0 (12.7 / 24.8), W[2880,2880] at 64 rows 19.6 (13.8).  The counterpart
+// of the reference's device-specific `qmv_batch_limit` (crates/nuvec-core/src/gpu.rs:1506-1538).
 static bool tiled_is_faster(const nvq::ProductArgs &a) {
     const double passes = (double)((a.m + 31) / 32) * (double)a.batch;
     const double blocks64 = passes * (double)((a.n + 63) / 64);
     const bool wide = blocks64 >= 192.0;
     const double blocks = wide ? blocks64 : passes * (double)((a.n + 31) / 32);
-    const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * fmax(4.0, (wide ? 5.0e-3 : 4.4e-3) * (double)a.k);
-    return fmax(4.0, nvq::qmm_estimate_us(a)) < few_us;  // (no launch is under 4 us)
+    double round_us = wide ? 12.0 + 1.6e-3 * (double)a.k : 8.5 + 2.0e-3 * (double)a.k;
+    if (a.exact_weights) round_us *= wide ? 1.8 : 1.15;
+    const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * round_us;
+    return fmax(11.5, nvq::qmm_estimate_us(a) + 4.5) < 0.9 * few_us;  // (a near tie stays on the few-row kernel: W[512,2048] at 64 rows 12.5 against 14.8)
 }
 
 // Whether the 16x16x32 kernel with directly loaded weight operands takes a few-row product, from its measured times
