@@ -11,7 +11,7 @@ import nuvec_amd as nv
 from nuvec_amd import ops
 from oracle import ref
 from tests.hip_backend import to_dev, to_host
-from tests.test_gpu_parity import assert_device_arithmetic, assert_rows_close, make_w, make_x
+from tests.test_gpu_parity import _excess, assert_device_arithmetic, assert_rows_close, make_w, make_x
 
 pytestmark = pytest.mark.gpu
 
@@ -73,3 +73,22 @@ def test_bias_epilogue_and_determinism():
     assert torch.equal(plain.view(torch.int16), again.view(torch.int16))
     fused = nv.quantized_matmul(xd, q, bias=bias)
     assert torch.equal(fused.view(torch.int16), (plain + bias).view(torch.int16))
+
+
+def test_margin_over_seeds():
+    """The weights are rounded once, as the tiled kernel's: the worst output of a product stays under the bar for every
+    seed tried, with room (the CPU's first rounding of code * scale is a noise of the same fraction of an output as of a
+    weight; against many outputs per row the row's largest output is large)."""
+    quant = nv.Quant.affine(64, 4)
+    m, n, k = 64, 11008, 4096
+    worst = []
+    for seed in range(10):
+        rng = np.random.default_rng(6300 + seed)
+        w, x = make_w(rng, n, k, ref.BF16), make_x(rng, m, k, ref.BF16)
+        packed, scales, biases = ref.affine_quantize(w, ref.BF16, 64, 4)
+        q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+        want = ref.quantized_matmul(x, packed, scales, biases, group=64, bits=4, dtype=ref.BF16, threads=8)
+        got = to_host(nv.quantized_matmul(to_dev(x), q))
+        worst.append(float(np.max(_excess(got, want, ref.BF16))))
+    print("batched decode, worst output over 10 seeds, x the bar:", " ".join(f"{v:.3f}" for v in worst))
+    assert max(worst) <= 0.95, worst
