@@ -170,24 +170,26 @@ using namespace nvq;
 
 // Whether the tiled kernel beats the passes of the few-row kernel, from their measured behaviour: the few-row kernel
 // runs a block (one per compute unit) per pass of 32 rows and 64 weight rows - 32 weight rows where that leaves fewer
-// than 192 blocks (qmf::row_groups).  A round of blocks on the chip costs a fixed part (the tables of scales, the sum of
-// eight wavefronts' partial tiles) and a part per value of K: fitted to W[2880,2880] at 64 / 128 / 256 / 512 rows
-// (13.1 / 25.0 / 32.4 / 48.2 us: one round of 32 weight rows, two of 32, two of 64, three of 64), W[4096,1024] at 64 rows
-// 13.2 (one round of 32), at 128 / 256 rows with the CPU's weights 24.7 / 47.3 (one and two rounds of 64; with one
-// rounding 13.6 a round), W[2048,2048] 64 / 128 rows 12.7 / 13.0, W[4096,512] 64 rows 9.0.  The tiled kernel of few tiles
-// takes 4.5 us more than its estimate of the steps and the second kernel that adds the splits of K, and was never under
-// 11.7 us: W[4096,512] at 128 rows 11.7 (few-row kernel 17.2), W[4096,1024] at 64 / 96 / 256 rows 15.1 / 15.7 / 20.0
-// (13.1 / 24.3 / 47.2), W[2048,2048] at 64 / 256 rows 16.0 / 17.0 (12.7 / 24.8), W[2880,2880] at 64 rows 19.6 (13.8).  The counterpart
+// than 192 blocks (qmf::row_groups).  Both kernels were timed on 1236 products (fifteen weight shapes from W[4096,128]
+// to W[16384,2048] and W[4096,14336], seven formats, bf16 and f16, 24 to 1024 rows of x) and fitted by least squares:
+// a round of the few-row kernel's blocks costs a fixed part (the tables of scales, the sum of eight wavefronts' partial
+// tiles) and a part per value of K, more of both with the CPU's weights; the tiled kernel takes its estimate of the
+// steps and of the second kernel that adds the splits of K, scaled (MXFP4 expands cheaply, the CPU's weights dearly),
+// plus a fixed part.  The fits are off by 9 to 14 % on average; choosing by them costs 1.7 % against always taking
+// the faster kernel, 30 % at worst (the rule before them, a round at 5 us per 1024 values of K against the bare
+// estimate: 6.3 % and 2.5 x - W[4096,1024] at 256 rows 47.4 us on the few-row kernel against 19.8).  The counterpart
 // of the reference's device-specific `qmv_batch_limit` (crates/nuvec-core/src/gpu.rs:1506-1538).
 static bool tiled_is_faster(const nvq::ProductArgs &a) {
-    const double passes = (double)((a.m + 31) / 32) * (double)a.batch;
+    const double passes = (double)((a.m + 31) / 32) * (double)a.batch, k = (double)a.k;
     const double blocks64 = passes * (double)((a.n + 63) / 64);
-    const bool wide = blocks64 >= 192.0;
+    const bool wide = blocks64 >= 192.0, exact = a.exact_weights != 0, fp4 = a.mode == NVQ_MXFP4;
     const double blocks = wide ? blocks64 : passes * (double)((a.n + 31) / 32);
-    double round_us = wide ? 12.0 + 1.6e-3 * (double)a.k : 8.5 + 2.0e-3 * (double)a.k;
-    if (a.exact_weights) round_us *= wide ? 1.8 : 1.15;
+    const double round_us = wide ? (exact ? 13.5 + 4.4e-3 * k : 7.4 + (fp4 ? 2.16e-3 : 2.45e-3) * k)
+                                 : (exact ? 8.0 + 2.0e-3 * k : 6.0 + 2.05e-3 * k);
     const double few_us = ceil(blocks / fmax(1.0, (double)nvq::compute_units())) * round_us;
-    return fmax(11.5, nvq::qmm_estimate_us(a) + 4.5) < 0.9 * few_us;  // (a near tie stays on the few-row kernel: W[512,2048] at 64 rows 12.5 against 14.8)
+    const double steps_us = nvq::qmm_estimate_us(a);
+    const double tiled_us = exact ? 1.8 + 1.26 * steps_us : fp4 ? 3.2 + 0.73 * steps_us : 3.4 + steps_us;
+    return fmax(7.0, tiled_us) < few_us;  // (its fastest launches, at K = 128, take 6 to 7.4 us)
 }
 
 // Whether the 16x16x32 kernel with directly loaded weight operands takes a few-row product, from its measured times
@@ -260,9 +262,10 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 // (f16: 33 rows 22.9 / 28.9); W[11008,4096] 40 / 64 rows 23.2 / 26.8, 23.3 / 29.8; W[16384,4096] 23.3 / 31.7, 23.7 / 35.1;
 // W[22016,4096] 43.4 / 46.6; W[32768,4096] 47.6 / 52.9; W[14336,8192] 40.9 / 50.1, 42.6 / 51.9; W[28672,8192] 83.8 / 93.3.  It
 // loses below: W[8192,4096] 23.0 against 18.7, W[8192,8192] 36.0 / 30.4, W[14336,4096] at 32 rows 20.2 / 18.7, at 128 rows
-// (two passes) 44.2 / 35.0, W[14336,2048] a tie.
+// (two passes) 44.2 / 35.0, W[14336,2048] a tie; and against very tall weights, whose many tiles fill the tiled kernel's
+// rounds: W[65536,4096] 94.2 / 96.4 and 97.7 / 95.7, W[151936,4096] 228 / 219 and 237 / 227.
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
-    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.k >= 4096 && nvq::qmr_supported(a);
+    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.n <= 65536 && a.k >= 4096 && nvq::qmr_supported(a);
 }
 
 // The kernels' view of a product descriptor.
