@@ -231,9 +231,16 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
         // (5 and 6 bits: the passes' never-rounded weights put one of 139360 half-precision outputs of a 130-row product of
         // 6-bit codes in groups of 128 at 1.06 x the bar against the CPU's doubly rounded ones; the tiles round once)
         if (a.k > 4096 || a.m > 192 || a.bits == 5 || a.bits == 6) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
+        // (K = 512 is one wavefront a block: W[32768,512] at 17 to 192 rows 17 - 22 us against 11.3 - 13 on the tiles)
+        if (a.k < 1024 && rows >= 16384) return false;
         const double passes = (double)((a.m + 15) / 16), mb = (double)rows * (double)a.k * a.bits / 8.0 / 1048576.0;
+        // Timed against the better of the other two kernels on 462 products (us, this kernel / the other): MXFP4
+        // W[4096,4096] at 64 rows 9.0 / 13.4, W[16384,2048] at 64 rows 0.73 of the other, W[11008,4096] at 48 rows 0.93, at
+        // 80 rows 1.11; NVFP4 W[4096,4096] at 64 rows 0.87, at 96 rows 1.08; 4 bits in groups of 32 W[11008,4096] at 17 to
+        // 32 rows 0.74, W[14336,4096] 1.24 - 1.31.
+        if (a.mode != NVQ_AFFINE) return passes * mb <= (a.mode == NVQ_MXFP4 ? 64.0 : 48.0);
         if (a.bits == 8) return passes * mb <= (a.group == 32 ? 34.0 : 40.0);
-        if (a.group == 32) return passes * mb <= 30.0;
+        if (a.group == 32) return passes * mb <= 45.0;
         return passes * mb <= 50.0 || (passes <= 4.0 && mb <= 32.0);
     }
     // One or two rows of 3-bit, up to three or four of 8-bit codes with K beyond 2048: the decode kernel of the vector units (3 bits, us: W[4096,4096]
