@@ -223,6 +223,17 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     if (!nvq::qmd_supported(a)) return false;
     if (a.mode != NVQ_AFFINE && nvq::qmv_block_decode_takes(a)) return false;  // one or two rows (some more): the decode kernel of the vector units
     const int64_t rows = a.n * a.batch;
+    // The kernel's block is one wavefront per 512 values of K, up to eight - the largest divisor of K / 512 where K is
+    // longer and walked in chunks.  Short blocks against many weight rows lose: W[32768,512] (one wavefront) 2 to 4 rows
+    // of 4-bit codes in groups of 32 15 us against 5 - 7 on the short-row decode kernel, 10 to 16 rows 17 - 20 against
+    // 13 - 14 on the few-row kernel; K = 6144 (six wavefronts, two chunks) at 10 to 16 rows 16 - 22 against 13 - 17.
+    if (a.mode == NVQ_AFFINE && a.k < 1024 && rows >= 16384) return false;  // (MXFP4 there: 8.4 - 8.8 us at 4 to 8 rows against 10.4 - 11.2)
+    if (a.k > 4096) {
+        const int64_t all = a.k / 512;
+        int64_t slices = 8;
+        while (all % slices != 0) slices--;
+        if (slices < 7) return false;
+    }
     // The block formats (bf16, new / the few-row kernel of the 32x32x16 instruction): MXFP4 W[14336,4096] 1 row 11.1 / 13.4,
     // 16 rows 11.3 / 14.6; W[4096,4096] 1 row 5.4 / 6.9, 32 rows 7.0 / 14.2; NVFP4 W[14336,4096] 1 row 13.2 / 17.7;
     // MXFP8 W[4096,14336] 16 rows 18.8 / 29.4: every row count up to 16, 32 where K or the matrix is short.
@@ -231,8 +242,7 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
         // (5 and 6 bits: the passes' never-rounded weights put one of 139360 half-precision outputs of a 130-row product of
         // 6-bit codes in groups of 128 at 1.06 x the bar against the CPU's doubly rounded ones; the tiles round once)
         if (a.k > 4096 || a.m > 192 || a.bits == 5 || a.bits == 6) return false;  // (a long K is walked in chunks with x staged per chunk and pass)
-        // (K = 512 is one wavefront a block: W[32768,512] at 17 to 192 rows 17 - 22 us against 11.3 - 13 on the tiles)
-        if (a.k < 1024 && rows >= 16384) return false;
+        // (W[32768,512] at 17 to 192 rows: 17 - 22 us against 11.3 - 13 on the tiles)
         const double passes = (double)((a.m + 15) / 16), mb = (double)rows * (double)a.k * a.bits / 8.0 / 1048576.0;
         // Timed against the better of the other two kernels on 462 products (us, this kernel / the other): MXFP4
         // W[4096,4096] at 64 rows 9.0 / 13.4, W[16384,2048] at 64 rows 0.73 of the other, W[11008,4096] at 48 rows 0.93, at
