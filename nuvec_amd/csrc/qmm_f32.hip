@@ -179,11 +179,18 @@ bool qmm_f32_takes(const ProductArgs &a) {
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.glu != 0) return false;
     if (a.k < kStep || a.k % kStep != 0 || (a.mode == NVQ_AFFINE && a.group != 32 && a.group != 64 && a.group != 128)) return false;
     if (a.m < 8 || a.m > 65535 * (int64_t)kTile || a.n > 0x7FFFFFFF / 64 || (uintptr_t)a.x % 16 != 0) return false;
+    // Both kernels as timed on 1078 products (fourteen weight shapes, seven formats, 8 to 512 rows): this one a step of 64
+    // values at 1.64 us for a lone block and 1.25 us per block sharing a compute unit, the block formats 1.7 times that;
+    // the vector kernel a pass of four rows at 1 us per 2.06 M weights with K counted in its steps of 2048 values (a row
+    // of 512 costs a whole step: W[32768,512] at 8 rows 68.6 us there against 25.4 here), the block formats 2.05 times
+    // that.  Choosing by them is 0.2 % above always taking the faster kernel, 1.4 x at worst.
+    const bool block_format = a.mode != NVQ_AFFINE;
     const double tiles = (double)((a.m + kTile - 1) / kTile) * (double)((a.n + kTile - 1) / kTile);
     const double per_unit = 1.25 * tiles / compute_units();
-    const double here = (double)(a.k / kStep) * (per_unit > 1.64 ? per_unit : 1.64);
-    const double there = (double)((a.m + 3) / 4) * (double)a.n * (double)a.k / 2.2e6;
-    return here < 0.95 * there;
+    const double here = (double)(a.k / kStep) * (per_unit > 1.64 ? per_unit : 1.64) * (block_format ? 1.7 : 1.0);
+    const double k_steps = (double)((a.k + 2047) / 2048) * 2048.0;
+    const double there = (double)((a.m + 3) / 4) * (double)a.n * k_steps / 2.2e6 * (block_format ? 2.05 : 1.07);
+    return here < there;
 }
 
 int32_t launch_qmm_f32(const ProductArgs &a, hipStream_t s) {
