@@ -583,7 +583,16 @@ static Route pick_route(const nvq_qmm_desc *d, const ProductArgs &a) {
     // kernel's 3-, 5-, 6- and 8-bit variants take (wide_decode_takes): the vector kernels too (a row of 3-bit codes at
     // 4096 x 4096: 4.0 us against 10.1 us on the matrix cores, of 8-bit codes in groups of 32 5.8 against 11.7 us).
     // Other few-row products share one weight decode on the matrix cores where those kernels take them.
+    // The CPU's weights (rows of fewer than 1024 outputs) at up to 16 rows: the vector kernel's passes of four rows are
+    // ahead of the few-row kernel's exact variant on matrices this small (us: W[768,2048] 2 to 8 rows 4.6 - 4.9 against
+    // 7.4 - 8.4, W[512,4096] 16 rows 7.8 / 10.7, W[640,8192] 12 rows 13 / 17, 16 rows 21 / 18).
+    if (a.exact_weights && a.m <= 16 && a.m * a.k <= 12 * 8192) return Route::kVector;
     if (!takes_decode(a) && qmf_supported(a)) return Route::kFewRows;
+    // Five rows and more that neither few-row kernel takes (1, 3 and 5 bits with K off whole windows of 128): the tiles
+    // where the vector kernel's passes of four rows add up (3 bits, W[11008,2880]: 5 / 16 rows 42 / 82 us there, 23 here;
+    // W[2880,2880]: 5 to 8 rows, two passes of four, 14 against 16, 12 rows 21 against 16.)
+    if (!takes_decode(a) && a.m >= 5 && (double)((a.m + 3) / 4) * (double)a.n * (double)a.k * (double)a.batch >= 20.0e6 && qmm_supported(a))
+        return Route::kTiled;
     return Route::kVector;
 }
 

@@ -45,7 +45,9 @@ def test_routes_of_the_baseline_configurations():
         assert c4(16, row_exact=False, rows=True) == "qmv_lds_kernel"
     assert ops.quantized_matmul_route(24, 1000, 1024, nv.Quant.affine(64, 6), bf16) == "qmf_kernel"
     assert ops.quantized_matmul_route(96, 4096, 14336, nv.Quant.affine(64, 4), bf16) == "qmm_kernel"  # (a long K: the tiles split it: 41 us against 75; at 24 rows the few-row kernel's one round is ahead, 32 against 38)
-    assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
+    assert ops.quantized_matmul_route(16, 1100, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmf_kernel"  # K off the kernel's slices
+    # (rows of fewer than 1024 outputs, up to 16 rows of x: the vector kernel with the CPU's weights, ahead on matrices this small)
+    assert ops.quantized_matmul_route(16, 1000, 4096 + 128, nv.Quant.affine(64, 3), bf16) == "qmv_lds_kernel"
     assert ops.quantized_matmul_route(64, 2880, 2880, nv.Quant.new(nv.QuantMode.MXFP4), bf16) in ("qmf_kernel", "qmm_kernel")
     # passes of 16 rows where the matrix is small enough to be read again from the caches; the tiles beyond
     # (bfloat16 products of more than 16 rows and fewer than 8192 outputs per row take the kernels that hold the CPU's weights)
@@ -56,7 +58,7 @@ def test_routes_of_the_baseline_configurations():
     assert c2(32) == "qmd_kernel" and c2(96) == "qmm_kernel"
     assert c2(33) == "qmr_kernel" and c2(64) == "qmr_kernel"  # (one pass over this many weight rows: the batched-decode kernel)
     # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
-    for m, n, k, group, bits in ((5, 77, 1152, 64, 3), (16, 130, 2176, 32, 8), (20, 1000, 1024, 64, 6)):
+    for m, n, k, group, bits in ((5, 1077, 1152, 64, 3), (16, 1130, 2176, 32, 8), (20, 1000, 1024, 64, 6)):
         assert ops.quantized_matmul_route(m, n, k, nv.Quant.affine(group, bits), bf16) == "qmf_kernel", (m, n, k, group, bits)
     # (a tiny product of more than 16 rows: the two kernels are within a microsecond of each other, W[4096,128] at 32 rows 6.5 against 7.1 us)
     assert ops.quantized_matmul_route(30, 64, 128, nv.Quant.affine(64, 4), bf16) in ("qmf_kernel", "qmm_kernel")

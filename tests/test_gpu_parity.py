@@ -306,8 +306,9 @@ def test_rows_of_few_outputs_take_the_cpu_weights(dtype):
     0.78 x the bar for a row's largest output)."""
     rng = np.random.default_rng(8800 + dtype)
     tdtype = TORCH[dtype]
-    cases = [(5, 200, 1024, 4, 64, True, "qmf_kernel"), (1, 100, 4096, 4, 64, True, "qmv_lds_kernel"), (3, 64, 480, 8, 32, True, "qmv_lds_kernel"),
-             (2048, 768, 512, 4, 64, True, "qmm_kernel"), (300, 640, 1024, 4, 64, True, None), (260, 257, 192, 3, 64, True, None), (16, 48, 1536, 8, 128, True, "qmf_kernel"),
+    cases = [(24, 200, 1024, 4, 64, True, "qmf_kernel"), (5, 200, 1024, 4, 64, True, "qmv_lds_kernel"), (1, 100, 4096, 4, 64, True, "qmv_lds_kernel"), (3, 64, 480, 8, 32, True, "qmv_lds_kernel"),
+             (2048, 768, 512, 4, 64, True, "qmm_kernel"), (300, 640, 1024, 4, 64, True, None), (260, 257, 192, 3, 64, True, None), (16, 48, 6400, 8, 128, True, "qmf_kernel"),
+             (16, 48, 1536, 8, 128, True, "qmv_lds_kernel"),
              (40, 384, 256, 4, 64, False, "qmn_kernel"), (130, 992, 192, 8, 32, False, "qmn_kernel"), (7, 256, 200, 4, 64, False, "qvm_kernel"),
              (9, 128, 320, 6, 64, False, "qmn_kernel")]
     for m, n, k, bits, group, transpose, kernel in cases:
@@ -538,7 +539,7 @@ def test_few_rows_every_width(dtype, group, bits):
     """The few-row matrix-core kernel at every code width it takes: K of whole and of half windows
     (128 and 64 values), N off the rows per block, passes of 8, 16 and 32 rows of x."""
     rng = np.random.default_rng(900 + 10 * bits + group)
-    for m, n, k in [(1, 200, 256), (5, 77, 1152), (16, 130, 2048 + 128), (33, 64, 128), (2, 96, 576 if group < 128 else 640)]:
+    for m, n, k in [(1, 200, 256), (5, 77, 1152), (16, 130, 2048 + 128), (14, 77, 7168), (33, 64, 128), (2, 96, 576 if group < 128 else 640)]:
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
         packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
         q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), nv.Quant.affine(group, bits))
@@ -547,7 +548,9 @@ def test_few_rows_every_width(dtype, group, bits):
         assert_rows_close(got, want, dtype, f"few rows b{bits} g{group} M={m} N={n} K={k}")
         assert_device_arithmetic(got, x, packed, scales, biases, group, bits, dtype, f"few rows b{bits} g{group} M={m} N={n} K={k}")
         if m >= 5 and k % 128 == 0:  # (a single row of some widths stays on the vector kernels; odd widths need whole windows)
-            assert nv.quantized_matmul_route(m, n, k, q.quant, TORCH[dtype]) in ("qmf_kernel", "qmd_kernel", "qmm_kernel")
+            # (up to 16 rows against rows of fewer than 1024 outputs: the vector kernel with the CPU's weights while m K <= 12 x 8192)
+            few = ("qmv_lds_kernel",) if m <= 16 and m * k <= 12 * 8192 else ("qmf_kernel", "qmd_kernel", "qmm_kernel")
+            assert nv.quantized_matmul_route(m, n, k, q.quant, TORCH[dtype]) in few
 
 
 @pytest.mark.parametrize("bits,group", [(3, 64), (8, 32)])
