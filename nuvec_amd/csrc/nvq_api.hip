@@ -279,10 +279,10 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 // (f16: 33 rows 22.9 / 28.9); W[11008,4096] 40 / 64 rows 23.2 / 26.8, 23.3 / 29.8; W[16384,4096] 23.3 / 31.7, 23.7 / 35.1;
 // W[22016,4096] 43.4 / 46.6; W[32768,4096] 47.6 / 52.9; W[14336,8192] 40.9 / 50.1, 42.6 / 51.9; W[28672,8192] 83.8 / 93.3.  It
 // loses below: W[8192,4096] 23.0 against 18.7, W[8192,8192] 36.0 / 30.4, W[14336,4096] at 32 rows 20.2 / 18.7, at 128 rows
-// (two passes) 44.2 / 35.0, W[14336,2048] a tie; and against very tall weights, whose many tiles fill the tiled kernel's
-// rounds: W[65536,4096] 94.2 / 96.4 and 97.7 / 95.7, W[151936,4096] 228 / 219 and 237 / 227.
+// (two passes) 44.2 / 35.0, W[14336,2048] a tie.  Beyond 16384 weight rows its blocks take 128 of them: W[65536,4096] 88.6
+// against 95.7 on the tiles, W[151936,4096] at 40 / 64 rows 201 / 209 against 219 / 227.
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
-    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.n <= 65536 && a.k >= 4096 && nvq::qmr_supported(a);
+    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.k >= 4096 && nvq::qmr_supported(a);
 }
 
 // The kernels' view of a product descriptor.

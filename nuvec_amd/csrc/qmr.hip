@@ -6,7 +6,8 @@
 // follow nuvec's CPU product (crates/nuvec-core/src/kernels.rs:1091-1142) as the tiled kernel's do: a weight is one
 // rounding of fma(code, scale, bias) to the element type.
 //
-// A block of four wavefronts owns 16 WT weight rows and all rows of the pass; its wavefronts split K: wavefront v takes
+// A block of four wavefronts owns 16 WT weight rows (64, or 128 where the weight has more rows than one round of 64-row
+// blocks covers: x is then read half as often per weight) and all rows of the pass; its wavefronts split K: wavefront v takes
 // the chunks of 512 values v, v + 4, ...  Nothing is shared between them until their partial tiles are added, so the
 // loop has no block barrier.  A wavefront walks its chunks in windows of 128 values:
 //   * weights: lane (row n = lane % 16, quarter q = lane / 16) loads the 32 codes [32 q, 32 q + 32) of the window of its
@@ -62,6 +63,11 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     constexpr int kXLoads = 4 * XT;                   // loads of a window of x per lane: four rows of 256 bytes each
     constexpr int kBuf = qmr_buffer_bytes<XT>();
     constexpr int kOutStride = kCols + 4;             // floats between two rows of a wavefront's partial tile
+    // Eight tiles of weight rows fill the registers: their weights are requested one window ahead instead of two and
+    // expanded in the step that multiplies them.
+    constexpr int kWeightsAhead = WT >= 8 ? 1 : 2;
+    constexpr int kXSets = WT >= 8 ? 1 : 2;           // windows of x on their way in registers
+    constexpr bool kAhead = WT < 8;
     static_assert(kRows * kOutStride * 4 <= 2 * kBuf, "the partial tile reuses the wavefront's x buffers");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -91,18 +97,12 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     // w, scales, biases: this lane's row of each tile (rows past N read row N - 1)
     const uint32_t *wbase = (const uint32_t *)a.w;
     const uint16_t *sbase = (const uint16_t *)a.scales, *bbase = (const uint16_t *)a.biases;
-    int woff[WT], soff[WT];
-#pragma unroll
-    for (int wt = 0; wt < WT; wt++) {
-        const int n = n0 + 16 * wt + nl < N ? n0 + 16 * wt + nl : N - 1;
-        woff[wt] = n * kwords + q * BITS;
-        soff[wt] = n * kgroups;
-    }
+    const int nrow = n0 + nl, wlane = q * BITS;  // (the tiles' offsets are computed at the loads: sixteen registers fewer)
 
-    qmf::u32x4_t xg[2][kXLoads];  // (a native vector: arrays of it stay in registers)
+    qmf::u32x4_t xg[kXSets][kXLoads];  // (a native vector: arrays of it stay in registers)
     uint32_t wq[4][WT][BITS], sq[4][WT], bq[4][WT];
-    auto load_x = [&](int widx, auto set_tag, auto first_tag, auto count_tag) __attribute__((always_inline)) {
-        constexpr int set = decltype(set_tag)::value, first = decltype(first_tag)::value, count = decltype(count_tag)::value;
+    auto load_x = [&](int widx, auto buffer_tag, auto first_tag, auto count_tag) __attribute__((always_inline)) {
+        constexpr int set = kXSets == 2 ? decltype(buffer_tag)::value : 0, first = decltype(first_tag)::value, count = decltype(count_tag)::value;
         const T *src = xbase + k_of(widx);
 #pragma unroll
         for (int j = first; j < first + count; j++) {
@@ -110,9 +110,10 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
             xg[set][j] = *reinterpret_cast<const qmf::u32x4_t *>(src + (r < xrows ? r : xrows - 1) * K);
         }
     };
-    auto store_x = [&](auto set_tag, auto first_tag, auto count_tag) __attribute__((always_inline)) {
-        constexpr int set = decltype(set_tag)::value, first = decltype(first_tag)::value, count = decltype(count_tag)::value;
-        unsigned char *dst = mine + set * kBuf + xdst;
+    auto store_x = [&](auto buffer_tag, auto first_tag, auto count_tag) __attribute__((always_inline)) {
+        constexpr int buffer = decltype(buffer_tag)::value, first = decltype(first_tag)::value, count = decltype(count_tag)::value;
+        constexpr int set = kXSets == 2 ? buffer : 0;
+        unsigned char *dst = mine + buffer * kBuf + xdst;
 #pragma unroll
         for (int j = first; j < first + count; j++) {
             // x on its way lives in the accumulation registers (loads and LDS writes take them), which the loop leaves free
@@ -128,9 +129,10 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
         const int g = (k0 + 32 * q) / GROUP;
 #pragma unroll
         for (int wt = 0; wt < WT; wt++) {
-            qmr_load_codes<BITS>(src + woff[wt], wq[set][wt]);
-            sq[set][wt] = sbase[soff[wt] + g];
-            bq[set][wt] = bbase[soff[wt] + g];
+            const int n = nrow + 16 * wt < N ? nrow + 16 * wt : N - 1;
+            qmr_load_codes<BITS>(src + n * kwords + wlane, wq[set][wt]);
+            sq[set][wt] = sbase[n * kgroups + g];
+            bq[set][wt] = bbase[n * kgroups + g];
         }
     };
 
@@ -151,23 +153,23 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     // requested two windows before its use: requests return in order, so the shortest lead is everyone's.
     load_x(0, I0{}, I0{}, IAll{});
     load_w(0, I0{});
-    load_x(1, I1{}, I0{}, IAll{});
-    load_w(1, I1{});
+    if constexpr (kXSets == 2) load_x(1, I1{}, I0{}, IAll{});
+    if constexpr (kWeightsAhead == 2) load_w(1, I1{});
     __builtin_amdgcn_sched_barrier(0);
     store_x(I0{}, I0{}, IAll{});
-    load_x(2, I0{}, I0{}, IAll{});
+    load_x(kXSets, I0{}, I0{}, IAll{});
     __builtin_amdgcn_sched_barrier(0);
 
     // The weight operands of a step are expanded during the matrix instructions of the step before it (they run on
     // their own pipe): set s % 2 of `wo` holds step s of a window.
-    uint4 wo[2][WT];
+    uint4 wo[kAhead ? 2 : 1][WT];
     float sc[WT], bi[WT];
     auto expand = [&](auto j_tag, auto s_tag, auto wt_tag) __attribute__((always_inline)) {
         constexpr int j = decltype(j_tag)::value, s = decltype(s_tag)::value, wt = decltype(wt_tag)::value;
         if constexpr (s == 0) sc[wt] = Pair<T>::lo(sq[j][wt]), bi[wt] = Pair<T>::lo(bq[j][wt]);  // (the window's last expansion is behind)
-        wo[s & 1][wt] = qmf::expand_piece<T, BITS, qmf::kAffine, s, EXACT>(wq[j][wt], sc[wt], bi[wt]);
+        wo[kAhead ? s & 1 : 0][wt] = qmf::expand_piece<T, BITS, qmf::kAffine, s, EXACT>(wq[j][wt], sc[wt], bi[wt]);
     };
-    qmf::static_for<WT>([&](auto wt_tag) { expand(I0{}, I0{}, wt_tag); });
+    if constexpr (kAhead) qmf::static_for<WT>([&](auto wt_tag) { expand(I0{}, I0{}, wt_tag); });
 
 #pragma unroll 1
     for (int turn = 0; turn < turns; turn++) {
@@ -181,8 +183,8 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
                 // a quarter of the next window of x goes to LDS and its registers take the window two after that one
                 using Next = std::integral_constant<int, (j + 1) & 1>;
                 store_x(Next{}, First{}, IPart{});
-                load_x(widx + 3, Next{}, First{}, IPart{});
-                if constexpr (s == 0) load_w(widx + 2, std::integral_constant<int, (j + 2) & 3>{});
+                load_x(widx + 1 + kXSets, Next{}, First{}, IPart{});
+                if constexpr (s == 0) load_w(widx + kWeightsAhead, std::integral_constant<int, (j + kWeightsAhead) & 3>{});
                 __builtin_amdgcn_sched_barrier(0);  // (the requests keep this order: the waits count them)
                 qmf::u32x4_t xo[XT];
 #pragma unroll
@@ -191,9 +193,10 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
                 using NextS = std::integral_constant<int, (s + 1) & 3>;
                 qmf::static_for<WT>([&](auto wt_tag) {
                     constexpr int wt = decltype(wt_tag)::value;
+                    if constexpr (!kAhead) expand(j_tag, s_tag, wt_tag);
 #pragma unroll
-                    for (int t = 0; t < XT; t++) acc[t][wt] = Mfma16<T>::run(__builtin_bit_cast(uint4, xo[t]), wo[s & 1][wt], acc[t][wt]);
-                    expand(NextJ{}, NextS{}, wt_tag);
+                    for (int t = 0; t < XT; t++) acc[t][wt] = Mfma16<T>::run(__builtin_bit_cast(uint4, xo[t]), wo[kAhead ? s & 1 : 0][wt], acc[t][wt]);
+                    if constexpr (kAhead) expand(NextJ{}, NextS{}, wt_tag);
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -262,10 +265,14 @@ int32_t run_sized(const ProductArgs &a, hipStream_t s) {
 
 template <typename T, int BITS>
 int32_t run_group(const ProductArgs &a, hipStream_t s) {
+    // More weight rows than one round of 64-row blocks covers: blocks of 128 rows, which read x half as often per weight
+    // (us, 64 rows of x: W[28672,4096] 47.9 -> 43.3, W[32768,4096] 50.8 -> 42.5, W[65536,4096] 98.5 -> 88.7, W[28672,8192] 87.3 ->
+    // 79.4; a single round of them is slower, W[14336,4096] 25.2 -> 40.4).
+    const bool tall = a.n > 64 * (int64_t)compute_units();
     switch (a.group) {
-    case 32: return run_sized<T, BITS, 32, 4, 4, false>(a, s);
-    case 64: return run_sized<T, BITS, 64, 4, 4, false>(a, s);
-    default: return run_sized<T, BITS, 128, 4, 4, false>(a, s);
+    case 32: return tall ? run_sized<T, BITS, 32, 4, 8, false>(a, s) : run_sized<T, BITS, 32, 4, 4, false>(a, s);
+    case 64: return tall ? run_sized<T, BITS, 64, 4, 8, false>(a, s) : run_sized<T, BITS, 64, 4, 4, false>(a, s);
+    default: return tall ? run_sized<T, BITS, 128, 4, 8, false>(a, s) : run_sized<T, BITS, 128, 4, 4, false>(a, s);
     }
 }
 

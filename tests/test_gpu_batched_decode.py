@@ -26,6 +26,10 @@ TORCH = {ref.BF16: torch.bfloat16, ref.F16: torch.float16}
     (ref.F16, 32, 50, 11040, 4608),
     (ref.BF16, 128, 47, 11072, 5120),
     (ref.F16, 128, 64, 12288, 4096),
+    # more than 16384 weight rows: blocks of 128 of them; weight rows off the block and off the 16-byte stores
+    (ref.BF16, 64, 64, 16512, 4096),
+    (ref.F16, 32, 37, 16501, 4096),
+    (ref.BF16, 128, 50, 16648, 4608),
 ])
 def test_against_the_cpu_product(dtype, group, m, n, k):
     rng = np.random.default_rng(6100 + group + m)
@@ -42,14 +46,14 @@ def test_against_the_cpu_product(dtype, group, m, n, k):
 
 
 def test_routes():
-    """The rule is measured: 33 to 64 rows, 11008 to 65536 weight rows, K from 4096 in chunks of 512, 4 bits, one
+    """The rule is measured: 33 to 64 rows, at least 11008 weight rows, K from 4096 in chunks of 512, 4 bits, one
     product; everything else stays where it was."""
     q4 = nv.Quant.affine(64, 4)
     route = lambda m, n, k, quant=q4, dtype=torch.bfloat16, **kw: ops.quantized_matmul_route(m, n, k, quant, dtype, **kw)
     assert route(33, 14336, 4096) == "qmr_kernel" and route(64, 14336, 4096) == "qmr_kernel"
     assert route(64, 14336, 4096, dtype=torch.float16) == "qmr_kernel" and route(48, 28672, 8192) == "qmr_kernel"
     assert route(32, 14336, 4096) != "qmr_kernel" and route(65, 14336, 4096) != "qmr_kernel"
-    assert route(64, 8192, 4096) != "qmr_kernel" and route(64, 14336, 2048) != "qmr_kernel" and route(64, 151936, 4096) != "qmr_kernel"
+    assert route(64, 8192, 4096) != "qmr_kernel" and route(64, 14336, 2048) != "qmr_kernel" and route(64, 151936, 4096) == "qmr_kernel"
     assert route(64, 14336, 4096 + 256) != "qmr_kernel"  # K off the chunks of 512
     assert route(64, 14336, 4096, nv.Quant.affine(64, 8)) != "qmr_kernel"
     assert route(64, 14336, 4096, nv.Quant.new(nv.QuantMode.MXFP4)) != "qmr_kernel"
