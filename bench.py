@@ -271,7 +271,7 @@ def all_configs(lib, device, qs):
     # (C1 is one row; 512 rows beside it: float32 on the matrix cores, against the 157.3 TFLOP/s of the float32 matrix instruction)
     products("C1 f32 4-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 4), torch.float32, _lib.F32, [1, 512], 48, 10_485_760,
              matrix_peak=MFMA_F32_PEAK_TFLOPS)
-    products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 64, 2048], 0, WEIGHT_BYTES,
+    products("C2/C3 bf16 4-bit g64 W[14336,4096]", N, K, None, torch.bfloat16, _lib.BF16, [1, 4, 8, 32, 64, 2048], 0, WEIGHT_BYTES,
              weights=qs)
     # Beside C2: the same layer's down projection, whose rows are K = 14336 long
     products("beside C2: bf16 4-bit g64 W[4096,14336]", 4096, 14336, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1], 24, WEIGHT_BYTES)

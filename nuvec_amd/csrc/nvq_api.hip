@@ -273,16 +273,26 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     }
 }
 
-// Whether a product takes the batched-decode kernel: 33 to 64 rows of x against at least 11008 weight rows and K from
-// 4096, where its one pass over the weights beats the passes of 16 rows of the few-row kernel and the tiles of the
-// tiled one.  Measured (bf16, 4 bits in groups of 64, us, new / old): W[14336,4096] 48 rows 24.1 / 30.5, 64 rows 24.0 / 34.1
-// (f16: 33 rows 22.9 / 28.9); W[11008,4096] 40 / 64 rows 23.2 / 26.8, 23.3 / 29.8; W[16384,4096] 23.3 / 31.7, 23.7 / 35.1;
-// W[22016,4096] 43.4 / 46.6; W[32768,4096] 47.6 / 52.9; W[14336,8192] 40.9 / 50.1, 42.6 / 51.9; W[28672,8192] 83.8 / 93.3.  It
-// loses below: W[8192,4096] 23.0 against 18.7, W[8192,8192] 36.0 / 30.4, W[14336,4096] at 32 rows 20.2 / 18.7, at 128 rows
-// (two passes) 44.2 / 35.0, W[14336,2048] a tie.  Beyond 16384 weight rows its blocks take 128 of them: W[65536,4096] 88.6
-// against 95.7 on the tiles, W[151936,4096] at 40 / 64 rows 201 / 209 against 219 / 227.
+// Whether a product takes the batched-decode kernel: 17 to 64 rows of x (passes of 32 rows up to 32, of 64 beyond)
+// against 8192 weight rows or more, where its one pass over the weights beats the passes of 16 rows of the few-row
+// kernels and the tiles of the tiled one.  The bounds are those of 702 products timed on both sides (4 bits, K 512 to
+// 16384, 8192 to 151936 weight rows, 17 to 128 rows, the three group sizes, bf16 and f16): without the kernel they take
+// 18.8 % more time than always the faster of the two, with this rule 0.2 % (worst 1.22 x).  us, this kernel / the other:
+// W[14336,4096] 17 / 32 / 33 / 64 rows 13.8 / 14.1 / 18.8 / 19.2 against 16.4 / 17.5 / 28.8 / 32.9; W[16384,1024] 32 rows
+// 0.53 x, W[32768,4096] 64 rows 32.7 / 52.7, W[11008,8192] in groups of 32 at 32 rows 23.6 / 44.8, W[32768,14336] 64 rows
+// 0.57 x.  It loses, and is not taken: under 11008 weight rows from K = 3072 (one round of 128 blocks: W[8192,4096] 1.2 x at
+// 32 rows), groups of 128 below K = 4096 (W[8192,2048] 1.26 x: the few-row kernel's per-group work is small there), K = 512
+// beyond 16384 weight rows and K = 1024 beyond 32768 (65536 from 33 rows) - one or two of the block's four wavefronts
+// have a chunk of K -, and from 65 rows (two passes: W[14336,4096] 34.4 against 31.7 on the tiles) but for fewer than 11008
+// weight rows at K <= 4096 (W[8192,2048] at 128 rows 12.4 / 17.6).
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
-    return a.m > 32 && a.m <= 64 && a.n >= 11008 && a.k >= 4096 && nvq::qmr_supported(a);
+    if (a.m <= 16 || a.m > 128 || a.n < 8192 || !nvq::qmr_supported(a)) return false;
+    if (a.m > 64) return a.n < 11008 && a.k <= 4096;
+    if (a.group == 128) return a.k >= 4096 && a.n >= 11008;
+    if (a.k >= 3072) return a.n >= 11008;
+    if (a.k >= 2048) return true;
+    if (a.k >= 1024) return a.n <= (a.m <= 32 ? 32768 : 65536);
+    return a.n <= 16384;
 }
 
 // The kernels' view of a product descriptor.

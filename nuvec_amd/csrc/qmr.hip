@@ -1,10 +1,11 @@
-// Batched decode: passes of up to 64 rows of x times 4-bit affine weights stored [N, K], bf16 / f16, on the 16x16x32
-// matrix instruction with every weight fetched and dequantized once per pass.  The regime between the few-row kernels
-// (up to 16 rows a pass: more rows are passes that read the weights again) and the tiled kernel (tiles of 128 or 256
-// rows of x, whose step costs the same however few rows it multiplies).  The reference routes these row counts to its
-// tiled kernel (crates/nuvec-core/src/gpu.rs:6975-7060, crates/nuvec-kernels/src/metal/quantized.h:1358-1485); values
-// follow nuvec's CPU product (crates/nuvec-core/src/kernels.rs:1091-1142) as the tiled kernel's do: a weight is one
-// rounding of fma(code, scale, bias) to the element type.
+// Batched decode: passes of up to 64 rows of x (32 where x has no more) times 4-bit affine weights stored [N, K],
+// bf16 / f16, on the 16x16x32 matrix instruction with every weight fetched and dequantized once per pass.  The regime
+// between the few-row kernels (up to 16 rows a pass: more rows are passes that read the weights again) and the tiled
+// kernel (tiles of 128 or 256 rows of x, whose step costs the same however few rows it multiplies).  The reference routes
+// these row counts to its tiled kernel (crates/nuvec-core/src/gpu.rs:6975-7060,
+// crates/nuvec-kernels/src/metal/quantized.h:1358-1485); values follow nuvec's CPU product
+// (crates/nuvec-core/src/kernels.rs:1091-1142) as the tiled kernel's do: a weight is one rounding of
+// fma(code, scale, bias) to the element type.
 //
 // A block of four wavefronts owns 16 WT weight rows (64, or 128 where the weight has more rows than one round of 64-row
 // blocks covers: x is then read half as often per weight) and all rows of the pass; its wavefronts split K: wavefront v takes
@@ -12,17 +13,22 @@
 // loop has no block barrier.  A wavefront walks its chunks in windows of 128 values:
 //   * weights: lane (row n = lane % 16, quarter q = lane / 16) loads the 32 codes [32 q, 32 q + 32) of the window of its
 //     row of each of the WT tiles (BITS dwords: a wavefront's load is 16 runs of 16 BITS bytes), two windows ahead,
-//     straight into registers; matrix instruction s of a window takes codes [8 s, 8 s + 8) of every quarter.  A lane's
-//     32 codes lie in one group: its scale and bias travel with the codes, a 16-bit load each;
+//     straight into registers; matrix instruction s of a window takes codes [8 s, 8 s + 8) of every quarter;
+//   * scales and biases: a lane's 32 codes lie in one group.  The scales and biases of a chunk's groups of the block's
+//     weight rows are a table in the wavefront's own LDS (a lane brings a weight row's 512 / GROUP values with one load
+//     for the scales and one for the biases, a chunk ahead), and a lane reads its 16-bit pair per tile and window there.
+//     Fetched per lane and window from memory they were 8 of a window's 28 requests, each of 64 two-byte pieces
+//     (W[14336,4096] at 64 rows 24.0 -> 20.5 us, W[151936,4096] 209 -> 156); the 128-row blocks of groups of 32, whose
+//     table does not fit beside x, still fetch them so;
 //   * x: the window of the pass's rows (16 XT rows of 256 bytes) is loaded coalesced (a load is four whole rows) three
 //     windows ahead, written to the wavefront's own LDS a window before its use (rows 272 bytes apart: the 16-byte
 //     operand reads of sixteen rows fall on all 64 banks) and read from there in the instruction's operand layout;
 //   * a window's XT x WT accumulators run over all of the wavefront's K: each dequantized weight operand feeds XT matrix
 //     instructions, each x operand WT; the operands of a step are expanded under the matrix instructions of the step
 //     before it.
-// Every block reads all of x (from the L2): 2 x 16 XT K bytes against the 8 WT K bytes of its weights, which is what
-// bounds it - a window takes the time of its requests, not of its arithmetic (measured: 23 us at K = 4096 for any N up
-// to 16384, one round of blocks).
+// Every block reads all of x (from the L2): 2 x 16 XT K bytes against the 8 WT K bytes of its weights; a window takes
+// the time of its requests, not of its arithmetic (measured: 20 us at K = 4096 for any N up to 16384, one round of
+// blocks).
 #include "qmv_common.h"
 
 namespace nvq {
@@ -34,7 +40,19 @@ constexpr int kQmrChunk = 4 * kQmrWindow;          // values of K per turn of th
 constexpr int kQmrRowBytes = 2 * kQmrWindow + 16;  // a row of a window of x in LDS
 
 template <int XT> constexpr int qmr_buffer_bytes() { return 16 * XT * kQmrRowBytes; }
-template <int XT> constexpr size_t qmr_lds_bytes() { return (size_t)kQmrWaves * 2 * qmr_buffer_bytes<XT>(); }
+// A wavefront's table of the scales and biases of a chunk (its weight rows' groups of 512 values, 16 bits each), where
+// it fits beside the buffers of x; 0: the lanes fetch them from memory window by window.
+template <int WT, int GROUP> constexpr int qmr_table_bytes() {
+    constexpr int bytes = 2 * 16 * WT * (kQmrChunk / GROUP) * 2;
+    return bytes <= 4096 ? bytes : 0;
+}
+template <int XT, int WT, int GROUP> constexpr int qmr_wave_bytes() { return 2 * qmr_buffer_bytes<XT>() + qmr_table_bytes<WT, GROUP>(); }
+template <int XT, int WT, int GROUP> constexpr size_t qmr_lds_bytes() { return (size_t)kQmrWaves * qmr_wave_bytes<XT, WT, GROUP>(); }
+
+// The table of scales is written in dwords and read 16 bits at a time: types that may alias, so that the reads stay
+// behind the writes.
+typedef uint32_t __attribute__((may_alias)) qmr_word_t;
+typedef uint16_t __attribute__((may_alias)) qmr_half_t;
 
 // BITS dwords from p (whole dwords; the widest loads the alignment of every window allows).
 template <int BITS>
@@ -62,6 +80,9 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     constexpr int kRows = 16 * XT, kCols = 16 * WT;
     constexpr int kXLoads = 4 * XT;                   // loads of a window of x per lane: four rows of 256 bytes each
     constexpr int kBuf = qmr_buffer_bytes<XT>();
+    constexpr int kWaveBytes = qmr_wave_bytes<XT, WT, GROUP>();
+    constexpr int kTabRow = kQmrChunk / GROUP * 2;    // bytes of a weight row's scales (or biases) of a chunk
+    constexpr bool kTable = qmr_table_bytes<WT, GROUP>() != 0;
     constexpr int kOutStride = kCols + 4;             // floats between two rows of a wavefront's partial tile
     // Eight tiles of weight rows fill the registers: their weights are requested one window ahead instead of two and
     // expanded in the step that multiplies them.
@@ -78,7 +99,8 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     const int m0 = blockIdx.y * kRows, n0 = blockIdx.x * kCols;
     const int chunks = K / kQmrChunk;
     const int turns = chunks > wave ? (chunks - wave + kQmrWaves - 1) / kQmrWaves : 0;  // chunks of this wavefront
-    unsigned char *mine = lds + wave * 2 * kBuf;
+    unsigned char *mine = lds + wave * kWaveBytes;
+    unsigned char *table = mine + 2 * kBuf;  // [scales, biases][weight row of the block][group of the chunk]
 
     // k of window `widx` of this wavefront; windows past its last one (and a wavefront without chunks) fetch a window
     // that exists, and nothing of it is used: no test around the loads.
@@ -121,18 +143,72 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
             *reinterpret_cast<qmf::u32x4_t *>(dst + 4 * j * kQmrRowBytes) = xg[set][j];
         }
     };
-    // The codes of a window and, per tile, the scale and bias of the group this lane's 32 codes lie in.
-    auto load_w = [&](int widx, auto set_tag) __attribute__((always_inline)) {
+    // The codes of a window and, per tile, the scale and bias of the group this lane's 32 codes lie in: from the
+    // wavefront's table of the chunk, or from memory.
+    auto load_codes = [&](int widx, auto set_tag) __attribute__((always_inline)) {
         constexpr int set = decltype(set_tag)::value;
-        const int k0 = k_of(widx);
-        const uint32_t *src = wbase + k0 / 32 * BITS;
-        const int g = (k0 + 32 * q) / GROUP;
+        const uint32_t *src = wbase + k_of(widx) / 32 * BITS;
 #pragma unroll
         for (int wt = 0; wt < WT; wt++) {
             const int n = nrow + 16 * wt < N ? nrow + 16 * wt : N - 1;
             qmr_load_codes<BITS>(src + n * kwords + wlane, wq[set][wt]);
-            sq[set][wt] = sbase[n * kgroups + g];
-            bq[set][wt] = bbase[n * kgroups + g];
+        }
+    };
+    auto load_groups = [&](int widx, auto set_tag) __attribute__((always_inline)) {
+        constexpr int set = decltype(set_tag)::value;
+        const unsigned char *src = table + nl * kTabRow + ((widx & 3) * kQmrWindow + 32 * q) / GROUP * 2;
+#pragma unroll
+        for (int wt = 0; wt < WT; wt++) {
+            sq[set][wt] = *reinterpret_cast<const qmr_half_t *>(src + 16 * wt * kTabRow);
+            bq[set][wt] = *reinterpret_cast<const qmr_half_t *>(src + (kCols + 16 * wt) * kTabRow);
+        }
+    };
+    auto load_w = [&](int widx, auto set_tag) __attribute__((always_inline)) {
+        if constexpr (kTable) {
+            load_codes(widx, set_tag);
+            load_groups(widx, set_tag);
+        } else {  // (one walk over the tiles: a row's offset serves its codes, scale and bias)
+            constexpr int set = decltype(set_tag)::value;
+            const int k0 = k_of(widx);
+            const uint32_t *src = wbase + k0 / 32 * BITS;
+            const int g = (k0 + 32 * q) / GROUP;
+#pragma unroll
+            for (int wt = 0; wt < WT; wt++) {
+                const int n = nrow + 16 * wt < N ? nrow + 16 * wt : N - 1;
+                qmr_load_codes<BITS>(src + n * kwords + wlane, wq[set][wt]);
+                sq[set][wt] = sbase[n * kgroups + g];
+                bq[set][wt] = bbase[n * kgroups + g];
+            }
+        }
+    };
+    // The table of a chunk: lane L brings the scales and the biases of the chunk's groups of weight rows L, L + 64, ...
+    // of the block (kTabRow bytes each), a chunk ahead; they go to LDS once the last window of the chunk before has
+    // read its own (the wavefront's LDS accesses execute in order: no barrier).
+    constexpr int kTabRows = kCols / 64, kTabWords = kTabRow / 4;
+    uint32_t tq[kTable ? 2 * kTabRows * kTabWords : 1];
+    auto table_load = [&](int turn) __attribute__((always_inline)) {
+        if constexpr (kTable) {
+            int chunk = wave + kQmrWaves * turn;
+            chunk = chunk < chunks ? chunk : chunks - 1;
+#pragma unroll
+            for (int r = 0; r < kTabRows; r++) {
+                const int n = n0 + lane + 64 * r < N ? n0 + lane + 64 * r : N - 1;
+                const int at = n * kgroups + chunk * (kQmrChunk / GROUP);
+                qmr_load_codes<kTabWords>(reinterpret_cast<const uint32_t *>(sbase + at), reinterpret_cast<uint32_t (&)[kTabWords]>(tq[(2 * r) * kTabWords]));
+                qmr_load_codes<kTabWords>(reinterpret_cast<const uint32_t *>(bbase + at), reinterpret_cast<uint32_t (&)[kTabWords]>(tq[(2 * r + 1) * kTabWords]));
+            }
+        }
+    };
+    auto table_store = [&]() __attribute__((always_inline)) {
+        if constexpr (kTable) {
+#pragma unroll
+            for (int r = 0; r < kTabRows; r++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    qmr_word_t *dst = reinterpret_cast<qmr_word_t *>(table + (h * kCols + lane + 64 * r) * kTabRow);
+#pragma unroll
+                    for (int i = 0; i < kTabWords; i++) dst[i] = tq[(2 * r + h) * kTabWords + i];
+                }
         }
     };
 
@@ -151,11 +227,19 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
 
     // Prologue: x of window 0 to LDS; x of windows 1 and 2 and the weights of windows 0 and 1 on their way.  Every load is
     // requested two windows before its use: requests return in order, so the shortest lead is everyone's.
+    table_load(0);
     load_x(0, I0{}, I0{}, IAll{});
-    load_w(0, I0{});
+    if constexpr (kTable) load_codes(0, I0{}); else load_w(0, I0{});
     if constexpr (kXSets == 2) load_x(1, I1{}, I0{}, IAll{});
-    if constexpr (kWeightsAhead == 2) load_w(1, I1{});
+    if constexpr (kWeightsAhead == 2) {
+        if constexpr (kTable) load_codes(1, I1{}); else load_w(1, I1{});
+    }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kTable) {
+        table_store();
+        load_groups(0, I0{});
+        if constexpr (kWeightsAhead == 2) load_groups(1, I1{});
+    }
     store_x(I0{}, I0{}, IAll{});
     load_x(kXSets, I0{}, I0{}, IAll{});
     __builtin_amdgcn_sched_barrier(0);
@@ -184,7 +268,12 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
                 using Next = std::integral_constant<int, (j + 1) & 1>;
                 store_x(Next{}, First{}, IPart{});
                 load_x(widx + 1 + kXSets, Next{}, First{}, IPart{});
-                if constexpr (s == 0) load_w(widx + kWeightsAhead, std::integral_constant<int, (j + kWeightsAhead) & 3>{});
+                if constexpr (s == 0) {
+                    // (the first window ahead that lies in the next chunk finds that chunk's table)
+                    if constexpr (j == 4 - kWeightsAhead) table_store();
+                    load_w(widx + kWeightsAhead, std::integral_constant<int, (j + kWeightsAhead) & 3>{});
+                    if constexpr (j == 0) table_load(turn + 1);
+                }
                 __builtin_amdgcn_sched_barrier(0);  // (the requests keep this order: the waits count them)
                 qmf::u32x4_t xo[XT];
 #pragma unroll
@@ -227,7 +316,7 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
         for (int e = 0; e < 8; e++) v[e] = 0.0f;
 #pragma unroll
         for (int wv = 0; wv < kQmrWaves; wv++) {
-            const floatx4_t *p = reinterpret_cast<const floatx4_t *>(lds + wv * 2 * kBuf + (r * kOutStride + c) * 4);
+            const floatx4_t *p = reinterpret_cast<const floatx4_t *>(lds + wv * kWaveBytes + (r * kOutStride + c) * 4);
             const floatx4_t lo = p[0], hi = p[1];
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] += lo[e], v[4 + e] += hi[e];
@@ -252,7 +341,7 @@ template <typename T, int BITS, int GROUP, int XT, int WT, bool EXACT>
 int32_t run_sized(const ProductArgs &a, hipStream_t s) {
     const dim3 grid((unsigned)((a.n + 16 * WT - 1) / (16 * WT)), (unsigned)((a.m + 16 * XT - 1) / (16 * XT)));
     auto kernel = qmr_kernel<T, BITS, GROUP, XT, WT, EXACT>;
-    constexpr size_t lds_bytes = qmr_lds_bytes<XT>();
+    constexpr size_t lds_bytes = qmr_lds_bytes<XT, WT, GROUP>();
     static std::atomic<bool> configured{false};
     if (lds_bytes > 64 * 1024 && !configured.load()) {
         NVQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
@@ -263,16 +352,24 @@ int32_t run_sized(const ProductArgs &a, hipStream_t s) {
     return NVQ_OK;
 }
 
+template <typename T, int BITS, int GROUP>
+int32_t run_shape(const ProductArgs &a, hipStream_t s, bool tall, bool low) {
+    if (low) return tall ? run_sized<T, BITS, GROUP, 2, 8, false>(a, s) : run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
+    return tall ? run_sized<T, BITS, GROUP, 4, 8, false>(a, s) : run_sized<T, BITS, GROUP, 4, 4, false>(a, s);
+}
+
 template <typename T, int BITS>
 int32_t run_group(const ProductArgs &a, hipStream_t s) {
     // More weight rows than one round of 64-row blocks covers: blocks of 128 rows, which read x half as often per weight
     // (us, 64 rows of x: W[28672,4096] 47.9 -> 43.3, W[32768,4096] 50.8 -> 42.5, W[65536,4096] 98.5 -> 88.7, W[28672,8192] 87.3 ->
     // 79.4; a single round of them is slower, W[14336,4096] 25.2 -> 40.4).
     const bool tall = a.n > 64 * (int64_t)compute_units();
+    // Up to 32 rows of x: passes of 32, which read half as much of x per weight.
+    const bool low = a.m <= 32;
     switch (a.group) {
-    case 32: return tall ? run_sized<T, BITS, 32, 4, 8, false>(a, s) : run_sized<T, BITS, 32, 4, 4, false>(a, s);
-    case 64: return tall ? run_sized<T, BITS, 64, 4, 8, false>(a, s) : run_sized<T, BITS, 64, 4, 4, false>(a, s);
-    default: return tall ? run_sized<T, BITS, 128, 4, 8, false>(a, s) : run_sized<T, BITS, 128, 4, 4, false>(a, s);
+    case 32: return run_shape<T, BITS, 32>(a, s, tall, low);
+    case 64: return run_shape<T, BITS, 64>(a, s, tall, low);
+    default: return run_shape<T, BITS, 128>(a, s, tall, low);
     }
 }
 
@@ -285,7 +382,7 @@ bool qmr_supported(const ProductArgs &a) {
     if (a.dtype == NVQ_F32 || a.mode != NVQ_AFFINE || a.bits != 4 || a.row_exact || a.exact_weights) return false;
     if (a.group != 32 && a.group != 64 && a.group != 128) return false;
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.offsets != nullptr || a.glu != 0) return false;
-    if (a.k < kQmrChunk || a.k % kQmrChunk != 0 || a.k > (1 << 24) || a.m < 1 || (a.m + 63) / 64 > 65535) return false;
+    if (a.k < kQmrChunk || a.k % kQmrChunk != 0 || a.k > (1 << 24) || a.m < 1 || (a.m + 31) / 32 > 65535) return false;
     if (a.n * (a.k / 32 * a.bits) >= (1LL << 31)) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases | (uintptr_t)a.w | (uintptr_t)a.x | (uintptr_t)a.y) % 16 == 0;
 }

@@ -55,7 +55,7 @@ def test_routes_of_the_baseline_configurations():
     assert small(64) == "qmd_kernel" and small(192) == "qmd_kernel" and small(512) in ("qmf_kernel", "qmm_kernel")
     assert small(16, bf16) == "qmd_kernel" and small(64, bf16) in ("qmf_kernel", "qmm_kernel") and small(192, bf16) in ("qmf_kernel", "qmm_kernel")
     assert ops.quantized_matmul_route(64, 8192, 4096, nv.Quant.affine(64, 4), bf16) == "qmd_kernel"
-    assert c2(32) == "qmd_kernel" and c2(96) == "qmm_kernel"
+    assert c2(17) == "qmr_kernel" and c2(32) == "qmr_kernel" and c2(96) == "qmm_kernel"
     assert c2(33) == "qmr_kernel" and c2(64) == "qmr_kernel"  # (one pass over this many weight rows: the batched-decode kernel)
     # the few-row kernel of the 32x32x16 instruction keeps what the direct kernel does not take
     for m, n, k, group, bits in ((5, 1077, 1152, 64, 3), (16, 1130, 2176, 32, 8), (20, 1000, 1024, 64, 6)):
@@ -85,7 +85,9 @@ def test_direct_few_row_kernel_every_width(dtype, bits, group):
         if dtype == ref.BF16 and m > 16 and n < 8192:  # the CPU's weights: not this kernel's, which never materialises one
             assert route in ("qmf_kernel", "qmm_kernel"), f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
             continue
-        assert route == "qmd_kernel", f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
+        # (more than 16 rows against 8192 weight rows or more of 4-bit codes: one pass of the batched-decode kernel)
+        expect = "qmr_kernel" if bits == 4 and m > 16 and n >= 8192 else "qmd_kernel"
+        assert route == expect, f"b{bits} g{group} M={m} N={n} K={k} runs on {route}"
         w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
         packed, scales, biases = ref.affine_quantize(w, dtype, group, bits)
         q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
