@@ -285,8 +285,22 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 // beyond 16384 weight rows and K = 1024 beyond 32768 (65536 from 33 rows) - one or two of the block's four wavefronts
 // have a chunk of K -, and from 65 rows (two passes: W[14336,4096] 34.4 against 31.7 on the tiles) but for fewer than 11008
 // weight rows at K <= 4096 (W[8192,2048] at 128 rows 12.4 / 17.6).
+// Up to 16 rows (a pass of 16), timed the same way on 420 products of 5 to 16 rows (8.2 % -> 0.6 %): from 9 rows against
+// 11008 weight rows or more at K <= 1024 (W[14336,512] at 16 rows 7.0 against 10.2 us, W[65536,512] 11.7 / 27.2,
+// W[32768,1024] 10.6 / 15.6), at K <= 2048 up to 16384 weight rows (W[14336,2048] 7.7 / 9.3) and from K = 8192
+// (W[14336,8192] 19.9 / 25.9, W[32768,14336] 67.5 / 95.9) - at K = 4096 the direct few-row kernel's slices fit and it is
+// level or ahead, and groups of 128 cost it little below K = 8192; from 5 rows at K = 512 against 14336 weight rows or
+// more (W[65536,512] at 8 rows 11.8 / 25.3) and, in groups of 32, at K >= 4096 against 11008 to 16384 weight rows
+// (W[14336,4096] at 8 rows 12.7 / 15.5, W[11008,8192] 20.8 / 31.6; beyond, the 128-row blocks fetch the scales per window).
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
-    if (a.m <= 16 || a.m > 128 || a.n < 8192 || !nvq::qmr_supported(a)) return false;
+    if (a.m < 5 || a.m > 128 || a.n < 8192 || !nvq::qmr_supported(a)) return false;
+    if (a.m <= 16) {
+        if (a.group == 32) return a.k >= 4096 && a.n >= 11008 && a.n <= 16384;
+        if (a.m <= 8) return a.k < 1024 && a.n >= 14336;
+        if (a.n < 11008 || (a.group == 128 && a.k < 8192)) return false;
+        if (a.k <= 1024 || a.k >= 8192) return true;
+        return a.k <= 2048 && a.n <= 16384;
+    }
     if (a.m > 64) return a.n < 11008 && a.k <= 4096;
     if (a.group == 128) return a.k >= 4096 && a.n >= 11008;
     if (a.k >= 3072) return a.n >= 11008;

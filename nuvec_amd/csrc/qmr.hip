@@ -353,8 +353,10 @@ int32_t run_sized(const ProductArgs &a, hipStream_t s) {
 }
 
 template <typename T, int BITS, int GROUP>
-int32_t run_shape(const ProductArgs &a, hipStream_t s, bool tall, bool low) {
-    if (low) return tall ? run_sized<T, BITS, GROUP, 2, 8, false>(a, s) : run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
+int32_t run_shape(const ProductArgs &a, hipStream_t s, bool tall) {
+    // Up to 16 and up to 32 rows of x: passes of 16 and of 32 rows, which read a quarter and half as much of x per weight.
+    if (a.m <= 16) return tall ? run_sized<T, BITS, GROUP, 1, 8, false>(a, s) : run_sized<T, BITS, GROUP, 1, 4, false>(a, s);
+    if (a.m <= 32) return tall ? run_sized<T, BITS, GROUP, 2, 8, false>(a, s) : run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
     return tall ? run_sized<T, BITS, GROUP, 4, 8, false>(a, s) : run_sized<T, BITS, GROUP, 4, 4, false>(a, s);
 }
 
@@ -364,12 +366,10 @@ int32_t run_group(const ProductArgs &a, hipStream_t s) {
     // (us, 64 rows of x: W[28672,4096] 47.9 -> 43.3, W[32768,4096] 50.8 -> 42.5, W[65536,4096] 98.5 -> 88.7, W[28672,8192] 87.3 ->
     // 79.4; a single round of them is slower, W[14336,4096] 25.2 -> 40.4).
     const bool tall = a.n > 64 * (int64_t)compute_units();
-    // Up to 32 rows of x: passes of 32, which read half as much of x per weight.
-    const bool low = a.m <= 32;
     switch (a.group) {
-    case 32: return run_shape<T, BITS, 32>(a, s, tall, low);
-    case 64: return run_shape<T, BITS, 64>(a, s, tall, low);
-    default: return run_shape<T, BITS, 128>(a, s, tall, low);
+    case 32: return run_shape<T, BITS, 32>(a, s, tall);
+    case 64: return run_shape<T, BITS, 64>(a, s, tall);
+    default: return run_shape<T, BITS, 128>(a, s, tall);
     }
 }
 
@@ -382,7 +382,7 @@ bool qmr_supported(const ProductArgs &a) {
     if (a.dtype == NVQ_F32 || a.mode != NVQ_AFFINE || a.bits != 4 || a.row_exact || a.exact_weights) return false;
     if (a.group != 32 && a.group != 64 && a.group != 128) return false;
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.offsets != nullptr || a.glu != 0) return false;
-    if (a.k < kQmrChunk || a.k % kQmrChunk != 0 || a.k > (1 << 24) || a.m < 1 || (a.m + 31) / 32 > 65535) return false;
+    if (a.k < kQmrChunk || a.k % kQmrChunk != 0 || a.k > (1 << 24) || a.m < 1 || (a.m + 15) / 16 > 65535) return false;
     if (a.n * (a.k / 32 * a.bits) >= (1LL << 31)) return false;
     return ((uintptr_t)a.scales | (uintptr_t)a.biases | (uintptr_t)a.w | (uintptr_t)a.x | (uintptr_t)a.y) % 16 == 0;
 }

@@ -1,5 +1,6 @@
 """Batched decode (`qmr_kernel`): 17 to 64 rows of x (up to 128 against few weight rows) against 4-bit affine weights
-stored [N, K] with 8192 rows or more, every weight fetched and dequantized once per pass.  The reference takes these row counts on its tiled kernel
+stored [N, K] with 8192 rows or more - and fewer rows where the direct few-row kernel's slices of K do not fit -, every
+weight fetched and dequantized once per pass.  The reference takes these row counts on its tiled kernel
 (crates/nuvec-core/src/gpu.rs:6975-7060, crates/nuvec-kernels/src/metal/quantized.h:1358-1485); the values are held to the
 CPU product (crates/nuvec-core/src/kernels.rs:1091-1142) at the bar of the element type (1e-2 of a row's largest output
 in bfloat16, 1e-3 in float16) and to the device arithmetic of a once-rounded weight at half of it."""
@@ -39,6 +40,12 @@ TORCH = {ref.BF16: torch.bfloat16, ref.F16: torch.float16}
     (ref.F16, 64, 128, 9001, 1536),
     (ref.BF16, 64, 29, 16448, 2560),
     (ref.BF16, 32, 20, 16500, 1024),
+    # passes of 16 rows: a short K, the 128-row blocks, groups of 32 and of 128, five and seven rows
+    (ref.BF16, 64, 9, 11008, 512),
+    (ref.F16, 64, 16, 16500, 8192),
+    (ref.BF16, 32, 5, 11050, 4096),
+    (ref.BF16, 128, 13, 11008, 8192),
+    (ref.BF16, 64, 7, 14350, 512),
 ])
 def test_against_the_cpu_product(dtype, group, m, n, k):
     rng = np.random.default_rng(6100 + group + m + k)
@@ -64,6 +71,11 @@ def test_routes():
     assert route(64, 14336, 4096, dtype=torch.float16) == "qmr_kernel" and route(48, 28672, 8192) == "qmr_kernel"
     assert route(17, 14336, 4096) == "qmr_kernel" and route(32, 14336, 4096) == "qmr_kernel"
     assert route(16, 14336, 4096) != "qmr_kernel" and route(65, 14336, 4096) != "qmr_kernel"
+    # up to 16 rows: where the direct few-row kernel's slices of K do not fit
+    assert route(16, 14336, 512) == "qmr_kernel" and route(9, 14336, 8192) == "qmr_kernel" and route(9, 14336, 2048) == "qmr_kernel"
+    assert route(8, 14336, 8192) != "qmr_kernel" and route(8, 14336, 512) == "qmr_kernel" and route(4, 14336, 512) != "qmr_kernel"
+    assert route(12, 32768, 2048) != "qmr_kernel" and route(12, 8192, 512) != "qmr_kernel"
+    assert route(8, 14336, 4096, nv.Quant.affine(32, 4)) == "qmr_kernel" and route(8, 32768, 4096, nv.Quant.affine(32, 4)) != "qmr_kernel"
     assert route(64, 8192, 4096) != "qmr_kernel" and route(64, 8192, 2048) == "qmr_kernel" and route(128, 8192, 4096) == "qmr_kernel"
     assert route(129, 8192, 4096) != "qmr_kernel" and route(128, 8192, 8192) != "qmr_kernel"
     assert route(64, 14336, 2048) == "qmr_kernel" and route(64, 151936, 4096) == "qmr_kernel"
