@@ -34,8 +34,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_235_140
-QMM_TRAFFIC_BYTES = 297_181_108
+QMV_TRAFFIC_BYTES = 33_235_170
+QMM_TRAFFIC_BYTES = 297_180_512
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
