@@ -290,12 +290,13 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 // W[32768,1024] 10.6 / 15.6), at K <= 2048 up to 16384 weight rows (W[14336,2048] 7.7 / 9.3) and from K = 8192
 // (W[14336,8192] 19.9 / 25.9, W[32768,14336] 67.5 / 95.9) - at K = 4096 the direct few-row kernel's slices fit and it is
 // level or ahead, and groups of 128 cost it little below K = 8192; from 5 rows at K = 512 against 14336 weight rows or
-// more (W[65536,512] at 8 rows 11.8 / 25.3) and, in groups of 32, at K >= 4096 against 11008 to 16384 weight rows
-// (W[14336,4096] at 8 rows 12.7 / 15.5, W[11008,8192] 20.8 / 31.6; beyond, the 128-row blocks fetch the scales per window).
+// more (W[65536,512] at 8 rows 11.8 / 25.3) and, in groups of 32, at K >= 4096 against 11008 to 16384 or from 28672 weight rows
+// (W[14336,4096] at 8 rows 12.7 / 15.5, W[11008,8192] 20.8 / 31.6, W[32768,4096] at 16 rows 25.0 / 30.0, W[28672,8192] 46.2 /
+// 72.0; between 16384 and 28672 weight rows the 128-row blocks leave compute units idle: W[20480,4096] 20.8 / 19.2).
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
     if (a.m < 5 || a.m > 128 || a.n < 8192 || !nvq::qmr_supported(a)) return false;
     if (a.m <= 16) {
-        if (a.group == 32) return a.k >= 4096 && a.n >= 11008 && a.n <= 16384;
+        if (a.group == 32) return a.k >= 4096 && a.n >= 11008 && (a.n <= 16384 || a.n >= 28672);
         if (a.m <= 8) return a.k < 1024 && a.n >= 14336;
         if (a.n < 11008 || (a.group == 128 && a.k < 8192)) return false;
         if (a.k <= 1024 || a.k >= 8192) return true;

@@ -18,8 +18,8 @@
 //     weight rows are a table in the wavefront's own LDS (a lane brings a weight row's 512 / GROUP values with one load
 //     for the scales and one for the biases, a chunk ahead), and a lane reads its 16-bit pair per tile and window there.
 //     Fetched per lane and window from memory they were 8 of a window's 28 requests, each of 64 two-byte pieces
-//     (W[14336,4096] at 64 rows 24.0 -> 20.5 us, W[151936,4096] 209 -> 156); the 128-row blocks of groups of 32, whose
-//     table does not fit beside x, still fetch them so;
+//     (W[14336,4096] at 64 rows 24.0 -> 20.5 us, W[151936,4096] 209 -> 156); passes of 64 rows on 128-row blocks of groups of
+//     32, whose table does not fit beside x, still fetch them so;
 //   * x: the window of the pass's rows (16 XT rows of 256 bytes) is loaded coalesced (a load is four whole rows) three
 //     windows ahead, written to the wavefront's own LDS a window before its use (rows 272 bytes apart: the 16-byte
 //     operand reads of sixteen rows fall on all 64 banks) and read from there in the instruction's operand layout;
@@ -42,11 +42,11 @@ constexpr int kQmrRowBytes = 2 * kQmrWindow + 16;  // a row of a window of x in 
 template <int XT> constexpr int qmr_buffer_bytes() { return 16 * XT * kQmrRowBytes; }
 // A wavefront's table of the scales and biases of a chunk (its weight rows' groups of 512 values, 16 bits each), where
 // it fits beside the buffers of x; 0: the lanes fetch them from memory window by window.
-template <int WT, int GROUP> constexpr int qmr_table_bytes() {
+template <int XT, int WT, int GROUP> constexpr int qmr_table_bytes() {
     constexpr int bytes = 2 * 16 * WT * (kQmrChunk / GROUP) * 2;
-    return bytes <= 4096 ? bytes : 0;
+    return 2 * qmr_buffer_bytes<XT>() + bytes <= 160 * 1024 / kQmrWaves ? bytes : 0;  // (all but passes of 64 rows on 128 weight rows in groups of 32)
 }
-template <int XT, int WT, int GROUP> constexpr int qmr_wave_bytes() { return 2 * qmr_buffer_bytes<XT>() + qmr_table_bytes<WT, GROUP>(); }
+template <int XT, int WT, int GROUP> constexpr int qmr_wave_bytes() { return 2 * qmr_buffer_bytes<XT>() + qmr_table_bytes<XT, WT, GROUP>(); }
 template <int XT, int WT, int GROUP> constexpr size_t qmr_lds_bytes() { return (size_t)kQmrWaves * qmr_wave_bytes<XT, WT, GROUP>(); }
 
 // The table of scales is written in dwords and read 16 bits at a time: types that may alias, so that the reads stay
@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     constexpr int kBuf = qmr_buffer_bytes<XT>();
     constexpr int kWaveBytes = qmr_wave_bytes<XT, WT, GROUP>();
     constexpr int kTabRow = kQmrChunk / GROUP * 2;    // bytes of a weight row's scales (or biases) of a chunk
-    constexpr bool kTable = qmr_table_bytes<WT, GROUP>() != 0;
+    constexpr bool kTable = qmr_table_bytes<XT, WT, GROUP>() != 0;
     constexpr int kOutStride = kCols + 4;             // floats between two rows of a wavefront's partial tile
     // Eight tiles of weight rows fill the registers: their weights are requested one window ahead instead of two and
     // expanded in the step that multiplies them.

@@ -46,6 +46,7 @@ TORCH = {ref.BF16: torch.bfloat16, ref.F16: torch.float16}
     (ref.BF16, 32, 5, 11050, 4096),
     (ref.BF16, 128, 13, 11008, 8192),
     (ref.BF16, 64, 7, 14350, 512),
+    (ref.BF16, 32, 11, 28700, 4096),
 ])
 def test_against_the_cpu_product(dtype, group, m, n, k):
     rng = np.random.default_rng(6100 + group + m + k)
@@ -75,7 +76,7 @@ def test_routes():
     assert route(16, 14336, 512) == "qmr_kernel" and route(9, 14336, 8192) == "qmr_kernel" and route(9, 14336, 2048) == "qmr_kernel"
     assert route(8, 14336, 8192) != "qmr_kernel" and route(8, 14336, 512) == "qmr_kernel" and route(4, 14336, 512) != "qmr_kernel"
     assert route(12, 32768, 2048) != "qmr_kernel" and route(12, 8192, 512) != "qmr_kernel"
-    assert route(8, 14336, 4096, nv.Quant.affine(32, 4)) == "qmr_kernel" and route(8, 32768, 4096, nv.Quant.affine(32, 4)) != "qmr_kernel"
+    assert route(8, 14336, 4096, nv.Quant.affine(32, 4)) == "qmr_kernel" and route(8, 32768, 4096, nv.Quant.affine(32, 4)) == "qmr_kernel" and route(8, 20480, 4096, nv.Quant.affine(32, 4)) != "qmr_kernel"
     assert route(64, 8192, 4096) != "qmr_kernel" and route(64, 8192, 2048) == "qmr_kernel" and route(128, 8192, 4096) == "qmr_kernel"
     assert route(129, 8192, 4096) != "qmr_kernel" and route(128, 8192, 8192) != "qmr_kernel"
     assert route(64, 14336, 2048) == "qmr_kernel" and route(64, 151936, 4096) == "qmr_kernel"
