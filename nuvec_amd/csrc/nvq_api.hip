@@ -273,7 +273,7 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
     }
 }
 
-// Whether a product takes the batched-decode kernel: 17 to 64 rows of x (passes of 32 rows up to 32, of 64 beyond)
+// Whether a product of 4- or 8-bit affine codes takes the batched-decode kernel.  4 bits: 17 to 64 rows of x (passes of 32 rows up to 32, of 64 beyond)
 // against 8192 weight rows or more, where its one pass over the weights beats the passes of 16 rows of the few-row
 // kernels and the tiles of the tiled one.  The bounds are those of 702 products timed on both sides (4 bits, K 512 to
 // 16384, 8192 to 151936 weight rows, 17 to 128 rows, the three group sizes, bf16 and f16): without the kernel they take
@@ -295,6 +295,15 @@ static bool takes_few_rows_direct(const nvq::ProductArgs &a) {
 // 72.0; between 16384 and 28672 weight rows the 128-row blocks leave compute units idle: W[20480,4096] 20.8 / 19.2).
 static bool takes_batched_decode(const nvq::ProductArgs &a) {
     if (a.m < 5 || a.m > 128 || a.n < 8192 || !nvq::qmr_supported(a)) return false;
+    // 8-bit codes (blocks of 64 weight rows only; a window of codes one window ahead): 418 products of 8 to 128 rows timed
+    // on both sides, 19.5 % -> 0.5 %.  W[14336,4096] at 16 / 32 / 64 rows 13.6-15.6 / 17.9 / 23.2 us against 15.0 / 20.3 /
+    // 38.3; W[11008,8192] in groups of 32 at 32 rows 32.0 / 53.6; W[32768,4096] at 64 rows 51 / 61-62.
+    if (a.bits == 8) {
+        if (a.m < 8 || a.k < 1024) return false;  // (fewer rows and shorter K were not timed)
+        if (a.m > 64) return a.n < 11008;
+        if (a.m <= 16) return a.n >= 11008 && (a.k >= 8192 || a.n <= 16384 || (a.k <= 1024 && a.n <= 32768));
+        return !(a.k <= 1024 && a.n >= 28672 && a.m >= 33);
+    }
     if (a.m <= 16) {
         if (a.group == 32) return a.k >= 4096 && a.n >= 11008 && (a.n <= 16384 || a.n >= 28672);
         if (a.m <= 8) return a.k < 1024 && a.n >= 14336;

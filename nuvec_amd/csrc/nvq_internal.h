@@ -126,7 +126,7 @@ double qmm_estimate_us(const ProductArgs &a);  // estimated duration of the tile
 // float32 products of many rows on v_mfma_f32_32x32x2_f32 (affine codes, weights stored [N, K]).
 bool qmm_f32_takes(const ProductArgs &a);
 int32_t launch_qmm_f32(const ProductArgs &a, hipStream_t s);
-// Batched decode: passes of up to 64 rows of x (5 to 128 rows routed there, where it measured faster), every weight fetched and dequantized once per pass (4-bit affine codes).
+// Batched decode: passes of up to 64 rows of x (5 to 128 rows routed there, where it measured faster), every weight fetched and dequantized once per pass (4- and 8-bit affine codes).
 bool qmr_supported(const ProductArgs &a);
 int32_t launch_qmr(const ProductArgs &a, hipStream_t s);
 // The few-row matrix-core kernel (up to 32 rows of x per pass; also the grouped gathered product).

@@ -1,4 +1,4 @@
-// Batched decode: passes of up to 64 rows of x (32 where x has no more) times 4-bit affine weights stored [N, K],
+// Batched decode: passes of up to 64 rows of x (16 or 32 where x has no more) times 4- or 8-bit affine weights stored [N, K],
 // bf16 / f16, on the 16x16x32 matrix instruction with every weight fetched and dequantized once per pass.  The regime
 // between the few-row kernels (up to 16 rows a pass: more rows are passes that read the weights again) and the tiled
 // kernel (tiles of 128 or 256 rows of x, whose step costs the same however few rows it multiplies).  The reference routes
@@ -86,7 +86,7 @@ __global__ void __launch_bounds__(64 * kQmrWaves) qmr_kernel(const ProductArgs a
     constexpr int kOutStride = kCols + 4;             // floats between two rows of a wavefront's partial tile
     // Eight tiles of weight rows fill the registers: their weights are requested one window ahead instead of two and
     // expanded in the step that multiplies them.
-    constexpr int kWeightsAhead = WT >= 8 ? 1 : 2;
+    constexpr int kWeightsAhead = WT >= 8 || BITS >= 8 ? 1 : 2;  // (8-bit codes: a window of them is twice the registers)
     constexpr int kXSets = WT >= 8 ? 1 : 2;           // windows of x on their way in registers
     constexpr bool kAhead = WT < 8;
     static_assert(kRows * kOutStride * 4 <= 2 * kBuf, "the partial tile reuses the wavefront's x buffers");
@@ -355,9 +355,15 @@ int32_t run_sized(const ProductArgs &a, hipStream_t s) {
 template <typename T, int BITS, int GROUP>
 int32_t run_shape(const ProductArgs &a, hipStream_t s, bool tall) {
     // Up to 16 and up to 32 rows of x: passes of 16 and of 32 rows, which read a quarter and half as much of x per weight.
-    if (a.m <= 16) return tall ? run_sized<T, BITS, GROUP, 1, 8, false>(a, s) : run_sized<T, BITS, GROUP, 1, 4, false>(a, s);
-    if (a.m <= 32) return tall ? run_sized<T, BITS, GROUP, 2, 8, false>(a, s) : run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
-    return tall ? run_sized<T, BITS, GROUP, 4, 8, false>(a, s) : run_sized<T, BITS, GROUP, 4, 4, false>(a, s);
+    if constexpr (BITS == 4) {
+        if (a.m <= 16) return tall ? run_sized<T, BITS, GROUP, 1, 8, false>(a, s) : run_sized<T, BITS, GROUP, 1, 4, false>(a, s);
+        if (a.m <= 32) return tall ? run_sized<T, BITS, GROUP, 2, 8, false>(a, s) : run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
+        return tall ? run_sized<T, BITS, GROUP, 4, 8, false>(a, s) : run_sized<T, BITS, GROUP, 4, 4, false>(a, s);
+    } else {  // (8-bit codes: blocks of 64 weight rows only, the registers hold no more)
+        if (a.m <= 16) return run_sized<T, BITS, GROUP, 1, 4, false>(a, s);
+        if (a.m <= 32) return run_sized<T, BITS, GROUP, 2, 4, false>(a, s);
+        return run_sized<T, BITS, GROUP, 4, 4, false>(a, s);
+    }
 }
 
 template <typename T, int BITS>
@@ -376,10 +382,10 @@ int32_t run_group(const ProductArgs &a, hipStream_t s) {
 }  // namespace
 
 // Whether the kernel takes the product (the routes decide by its shape whether it should): a single product of bf16 / f16
-// rows and 4-bit affine codes whose weights take one rounding, K in chunks of 512, every operand 16-byte aligned,
+// rows and 4- or 8-bit affine codes whose weights take one rounding, K in chunks of 512, every operand 16-byte aligned,
 // offsets within 32 bits.
 bool qmr_supported(const ProductArgs &a) {
-    if (a.dtype == NVQ_F32 || a.mode != NVQ_AFFINE || a.bits != 4 || a.row_exact || a.exact_weights) return false;
+    if (a.dtype == NVQ_F32 || a.mode != NVQ_AFFINE || (a.bits != 4 && a.bits != 8) || a.row_exact || a.exact_weights) return false;
     if (a.group != 32 && a.group != 64 && a.group != 128) return false;
     if (a.batch != 1 || a.batch_ndim != 0 || a.rhs != nullptr || a.lhs != nullptr || a.offsets != nullptr || a.glu != 0) return false;
     if (a.k < kQmrChunk || a.k % kQmrChunk != 0 || a.k > (1 << 24) || a.m < 1 || (a.m + 15) / 16 > 65535) return false;
@@ -389,6 +395,7 @@ bool qmr_supported(const ProductArgs &a) {
 
 int32_t launch_qmr(const ProductArgs &a, hipStream_t s) {
     if (!qmr_supported(a)) return fail(NVQ_UNSUPPORTED, "quantized_matmul: the batched-decode kernel does not take this product");
+    if (a.bits == 8) return a.dtype == NVQ_BF16 ? run_group<bf16_t, 8>(a, s) : run_group<f16_t, 8>(a, s);
     return a.dtype == NVQ_BF16 ? run_group<bf16_t, 4>(a, s) : run_group<f16_t, 4>(a, s);
 }
 

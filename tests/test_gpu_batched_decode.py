@@ -1,4 +1,4 @@
-"""Batched decode (`qmr_kernel`): 17 to 64 rows of x (up to 128 against few weight rows) against 4-bit affine weights
+"""Batched decode (`qmr_kernel`): 17 to 64 rows of x (up to 128 against few weight rows) against 4- and 8-bit affine weights
 stored [N, K] with 8192 rows or more - and fewer rows where the direct few-row kernel's slices of K do not fit -, every
 weight fetched and dequantized once per pass.  The reference takes these row counts on its tiled kernel
 (crates/nuvec-core/src/gpu.rs:6975-7060, crates/nuvec-kernels/src/metal/quantized.h:1358-1485); the values are held to the
@@ -62,6 +62,30 @@ def test_against_the_cpu_product(dtype, group, m, n, k):
     assert_device_arithmetic(got, x, packed, scales, biases, group, 4, dtype, what)
 
 
+# 8-bit codes: blocks of 64 weight rows, the codes of a window one window ahead; passes of 16, 32 and 64 rows, two passes,
+# every group size, tails of rows and of weight rows, K of three chunks.
+@pytest.mark.parametrize("dtype,group,m,n,k", [
+    (ref.BF16, 64, 64, 11008, 4096),
+    (ref.F16, 32, 33, 11017, 2048),
+    (ref.BF16, 128, 24, 8192, 1536),
+    (ref.BF16, 64, 12, 14336, 1024),
+    (ref.F16, 64, 100, 8200, 2048),
+    (ref.BF16, 32, 50, 16648, 4608),
+])
+def test_eight_bit_codes_against_the_cpu_product(dtype, group, m, n, k):
+    rng = np.random.default_rng(6500 + group + m + k)
+    quant = nv.Quant.affine(group, 8)
+    assert ops.quantized_matmul_route(m, n, k, quant, TORCH[dtype]) == "qmr_kernel"
+    w, x = make_w(rng, n, k, dtype), make_x(rng, m, k, dtype)
+    packed, scales, biases = ref.affine_quantize(w, dtype, group, 8)
+    q = nv.Quantized(to_dev(packed), to_dev(scales), to_dev(biases), quant)
+    want = ref.quantized_matmul(x, packed, scales, biases, group=group, bits=8, dtype=dtype, threads=8)
+    got = to_host(nv.quantized_matmul(to_dev(x), q))
+    what = f"batched decode b8 g{group} M={m} N={n} K={k}"
+    assert_rows_close(got, want, dtype, what)
+    assert_device_arithmetic(got, x, packed, scales, biases, group, 8, dtype, what)
+
+
 def test_routes():
     """The rule is measured: 17 to 64 rows against 8192 weight rows or more (11008 from K = 3072 and for groups of 128,
     which also need K from 4096; short K only up to a number of weight rows), up to 128 rows against fewer than 11008
@@ -86,7 +110,11 @@ def test_routes():
     assert route(64, 14336, 4096, q128) == "qmr_kernel" and route(64, 14336, 2048, q128) != "qmr_kernel"
     assert route(64, 4096, 4096, dtype=torch.float16) != "qmr_kernel"
     assert route(64, 14336, 4096 + 256) != "qmr_kernel"  # K off the chunks of 512
-    assert route(64, 14336, 4096, nv.Quant.affine(64, 8)) != "qmr_kernel"
+    q8 = nv.Quant.affine(64, 8)
+    assert route(64, 14336, 4096, q8) == "qmr_kernel" and route(17, 8192, 2048, q8) == "qmr_kernel" and route(16, 14336, 4096, q8) == "qmr_kernel"
+    assert route(7, 14336, 4096, q8) != "qmr_kernel" and route(16, 8192, 4096, q8) != "qmr_kernel" and route(16, 32768, 4096, q8) != "qmr_kernel"
+    assert route(128, 8192, 4096, q8) == "qmr_kernel" and route(128, 14336, 4096, q8) != "qmr_kernel" and route(64, 32768, 1024, q8) != "qmr_kernel"
+    assert route(32, 14336, 512, q8) != "qmr_kernel" and route(64, 14336, 4096, nv.Quant.affine(64, 6)) != "qmr_kernel"
     assert route(64, 14336, 4096, nv.Quant.new(nv.QuantMode.MXFP4)) != "qmr_kernel"
     assert route(64, 14336, 4096, dtype=torch.float32) != "qmr_kernel"
     assert route(64, 14336, 4096, batch=2) != "qmr_kernel"
