@@ -34,8 +34,8 @@ GROUP, BITS = 64, 4
 WEIGHT_BYTES = N * K * BITS // 8 + 2 * (N * (K // GROUP) * 2)  # 33,030,144
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by
 # what the same counters read for a plain device copy of known size; None until measured.
-QMV_TRAFFIC_BYTES = 33_235_170
-QMM_TRAFFIC_BYTES = 297_180_512
+QMV_TRAFFIC_BYTES = 33_235_175
+QMM_TRAFFIC_BYTES = 297_181_328
 METRIC = "QMV weight GB/s (% HBM peak) at M=1; QMM TFLOP/s (% MFMA peak) at M=2048"
 
 
@@ -275,6 +275,9 @@ def all_configs(lib, device, qs):
              weights=qs)
     # Beside C2: the same layer's down projection, whose rows are K = 14336 long
     products("beside C2: bf16 4-bit g64 W[4096,14336]", 4096, 14336, nv.Quant.affine(64, 4), torch.bfloat16, _lib.BF16, [1], 24, WEIGHT_BYTES)
+    # ... and C2's shape in 8-bit codes at the rows of batched decode
+    products("beside C2: bf16 8-bit g64 W[14336,4096]", N, K, nv.Quant.affine(64, 8), torch.bfloat16, _lib.BF16, [16, 64], 12,
+             N * K + 2 * (N * (K // 64) * 2))
     products("C4 bf16 3-bit g64 W[4096,4096]", 4096, 4096, nv.Quant.affine(64, 3), torch.bfloat16, _lib.BF16, [1, 16, 512], 48,
              7_340_032)
     products("C4 bf16 8-bit g32 W[4096,4096]", 4096, 4096, nv.Quant.affine(32, 8), torch.bfloat16, _lib.BF16, [1, 16, 512], 32,
